@@ -1,0 +1,153 @@
+/*
+ * libnxrt_ep_rocm.so — MI355X (gfx950) execution provider for com.microsoft::MatMulNBits, bits=4.
+ *
+ * Three groups of C entry points:
+ *   1. the nxrt plugin exports (nxrt_abi.h) and the nxmem allocator exports (nxmem_abi.h);
+ *   2. a C mirror of the reference's ExecutionProvider / KernelFactory / Kernel traits for this one
+ *      operator, because NxrtKernelVtable.execute (vtable.rs:108-122) carries raw pointers only —
+ *      no shapes, dtypes or attributes — and the reference's own nxrt wrapper still leaves
+ *      get_capability / compile / get_allocator unwired (vtable.rs:355-398);
+ *   3. entry points for the pieces the parity contract names one by one (dequantized weights,
+ *      activation codes, int32 block accumulators) and for timing on the provider's stream.
+ *
+ * Every pointer named "device" is device memory obtained from nxrt_rocm_ep_allocate (or any HIP
+ * allocation on the provider's GPU). Nothing here takes or returns a torch / C++ type. All calls on
+ * one provider are issued on that provider's single HIP stream, in call order; host-visible results
+ * require nxrt_rocm_ep_sync or a copy_to_host (which synchronises).
+ */
+#ifndef NXRT_EP_ROCM_H
+#define NXRT_EP_ROCM_H
+
+#include "nxmem_abi.h"
+#include "nxrt_abi.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct NxrtRocmEp NxrtRocmEp;                     /* one provider = one GPU + one stream */
+typedef struct NxrtRocmMatMulNBits NxrtRocmMatMulNBits;   /* one kernel = one MatMulNBits node */
+
+/* ---- ExecutionProvider (crates/onnx-runtime-ep-api/src/provider.rs:708-1600) ------------------ */
+
+/* initialize(&EpConfig) — provider.rs:93 (string map). keys/values: n_config NUL-terminated pairs.
+ * Known keys: "acc4_rounding" = "mlas" (ties to even, default) | "native" (ties away);
+ *             "decode_waves", "decode_col_groups" = launch overrides for the decode GEMV. */
+NxrtStatus nxrt_rocm_ep_create(uint32_t device_ordinal, const char* const* config_keys,
+                               const char* const* config_values, uint32_t n_config, NxrtRocmEp** out_ep);
+/* shutdown + drop. Frees the stream and every buffer the provider still owns. */
+void nxrt_rocm_ep_release(NxrtRocmEp* ep);
+/* name() / device_type() / device_id() / memory_vendor_id() — provider.rs:708-731. */
+const char* nxrt_rocm_ep_name(const NxrtRocmEp* ep);                   /* "RocmExecutionProvider" */
+uint32_t nxrt_rocm_ep_device_type(const NxrtRocmEp* ep);               /* NXRT_DEVICE_ROCM */
+uint32_t nxrt_rocm_ep_device_id(const NxrtRocmEp* ep);
+uint32_t nxrt_rocm_ep_memory_vendor_id(const NxrtRocmEp* ep);          /* 0x1002 */
+/* Architecture string ("gfx950..."), compute units, bytes of device memory. */
+NxrtStatus nxrt_rocm_ep_device_info(const NxrtRocmEp* ep, char* arch, size_t arch_len, uint32_t* compute_units, uint64_t* total_memory);
+/* allocate(size, align) / deallocate — provider.rs (DeviceBuffer); align <= 256 is always met. */
+NxrtStatus nxrt_rocm_ep_allocate(NxrtRocmEp* ep, size_t size, size_t align, void** out_device);
+NxrtStatus nxrt_rocm_ep_deallocate(NxrtRocmEp* ep, void* device);
+/* copy_from_host / copy_to_host (provider.rs:1434,1502), copy (device to device), sync. */
+NxrtStatus nxrt_rocm_ep_copy_from_host(NxrtRocmEp* ep, void* dst_device, const void* src_host, size_t bytes);
+NxrtStatus nxrt_rocm_ep_copy_to_host(NxrtRocmEp* ep, void* dst_host, const void* src_device, size_t bytes);
+NxrtStatus nxrt_rocm_ep_copy(NxrtRocmEp* ep, void* dst_device, const void* src_device, size_t bytes);
+NxrtStatus nxrt_rocm_ep_sync(NxrtRocmEp* ep);
+/* The nxrt EP vtable whose ctx is this provider (what NxrtEpFactoryVtable.create_ep hands out);
+ * the inverse recovers the provider from a vtable obtained through the plugin exports. */
+NxrtRocmEp* nxrt_rocm_ep_from_vtable(const NxrtEpVtable* vtable);
+
+/* ---- KernelFactory + Kernel (registry.rs:39-45, kernel.rs:548-706) ----------------------------- */
+
+/* Node attributes of MatMulNBits. `present` has bit i set when attribute i was on the node:
+ * 0=K 1=N 2=bits 3=block_size 4=accuracy_level 5=weight_prepacked
+ * (onnx-runtime-ep-cpu/src/kernels/matmul_nbits.rs:1410-1481). */
+typedef struct NxrtRocmMatMulNBitsAttrs {
+  uint32_t struct_size;
+  uint32_t present;
+  int64_t K, N, bits, block_size, accuracy_level, weight_prepacked;
+} NxrtRocmMatMulNBitsAttrs;
+
+/* C layout of TensorView / TensorMut (crates/onnx-runtime-ep-api/src/tensor.rs:132-143, 241).
+ * data == NULL marks an absent optional input (tensor.rs:173-192). strides are in elements;
+ * NULL means contiguous row-major. */
+typedef struct NxrtRocmTensorView {
+  void* data;
+  uint32_t dtype;        /* NXRT_DT_* */
+  uint32_t ndim;
+  const uint64_t* shape;
+  const int64_t* strides;
+  uint64_t byte_offset;
+  uint32_t device_type;  /* NXRT_DEVICE_* */
+  uint32_t device_index;
+} NxrtRocmTensorView;
+
+/* kernel.rs:508-524 */
+typedef struct NxrtRocmWorkspaceRequirement {
+  uint64_t bytes;
+  uint64_t alignment;
+} NxrtRocmWorkspaceRequirement;
+
+/* supports_op(node, opset, shapes, dtypes, layouts) -> KernelMatch (kernel.rs:118-130).
+ * Returns 1 when the provider takes the node; otherwise 0 with an actionable reason. */
+int nxrt_rocm_ep_supports_matmul_nbits(const NxrtRocmEp* ep, const NxrtRocmMatMulNBitsAttrs* attrs,
+                                       const NxrtTensorDesc* inputs, uint32_t n_inputs, char* reason, size_t reason_len);
+
+/* get_kernel -> KernelFactory::create (matmul_nbits.rs:1410-1481): attribute checks, same messages. */
+NxrtStatus nxrt_rocm_matmul_nbits_create(NxrtRocmEp* ep, const NxrtRocmMatMulNBitsAttrs* attrs,
+                                         const NxrtTensorDesc* input_shapes, uint32_t n_inputs,
+                                         NxrtRocmMatMulNBits** out_kernel);
+/* Kernel::set_constant_inputs (kernel.rs:548-, matmul_nbits.rs:1483-1488). */
+void nxrt_rocm_matmul_nbits_set_constant_inputs(NxrtRocmMatMulNBits* kernel, const uint8_t* is_constant, uint32_t n);
+/* Kernel::workspace_requirement: scratch for these input shapes (accuracy_level 4 activation codes). */
+NxrtStatus nxrt_rocm_matmul_nbits_workspace_requirement(const NxrtRocmMatMulNBits* kernel, const NxrtTensorDesc* inputs,
+                                                        uint32_t n_inputs, NxrtRocmWorkspaceRequirement* out);
+/* Kernel::execute / execute_with_workspace (matmul_nbits.rs:1490-1600, 2320-2330).
+ * inputs: A, B, scales, [zero_points], [g_idx], [bias]; outputs: Y. workspace may be NULL: the
+ * kernel then keeps its own scratch, grown on demand (an allocation inside the call). */
+NxrtStatus nxrt_rocm_matmul_nbits_execute(NxrtRocmMatMulNBits* kernel, const NxrtRocmTensorView* inputs, uint32_t n_inputs,
+                                          NxrtRocmTensorView* outputs, uint32_t n_outputs,
+                                          void* workspace_device, uint64_t workspace_bytes);
+/* Kernel::estimated_flops (matmul_nbits.rs:2338): 2*M*N*K, 0 when M is not known from the shapes. */
+uint64_t nxrt_rocm_matmul_nbits_estimated_flops(const NxrtRocmMatMulNBits* kernel);
+/* record_kernel_variant (kernel.rs:361): which kernel served the last execute. */
+const char* nxrt_rocm_matmul_nbits_last_variant(const NxrtRocmMatMulNBits* kernel);
+void nxrt_rocm_matmul_nbits_release(NxrtRocmMatMulNBits* kernel);
+/* The same kernel behind the nxrt kernel vtable (raw pointers only: the shapes are those given at
+ * create time, M taken from input_shapes[0]). The host calls release(ctx) once. */
+NxrtStatus nxrt_rocm_matmul_nbits_as_vtable(NxrtRocmMatMulNBits* kernel, NxrtKernelVtable** out_vtable);
+
+/* ---- pieces of the operator the parity contract checks one by one ------------------------------ */
+
+/* w[n,k] = (q - zp) * scale as f32 [N, K] (matmul_nbits.rs:1360-1363, 3502-3661; the CUDA sibling's
+ * matmul_nbits_dequant_f32, ep-cuda matmul_nbits.rs:414-455). scales dtype: f32 / f16 / bf16. */
+NxrtStatus nxrt_rocm_matmul_nbits_dequantize(NxrtRocmEp* ep, const void* b_device, const void* scales_device, uint32_t scale_dtype,
+                                             const void* zero_points_device, uint64_t n, uint64_t k, uint32_t block_size,
+                                             float* out_nk_device);
+/* accuracy_level=4 activation quantizer (simd_quant.rs:131-143 / sqnbitgemm_kernel_avx512.cpp:349-426).
+ * rounding: 0 = ties to even (MLAS), 1 = ties away from zero (native). qa: int8 [M, kb*bs];
+ * qscale: f32 [M, kb]. */
+NxrtStatus nxrt_rocm_matmul_nbits_quantize_a(NxrtRocmEp* ep, const void* a_device, uint32_t a_dtype, uint64_t m, uint64_t k,
+                                             uint32_t block_size, uint32_t rounding, int8_t* qa_device, float* qscale_device);
+/* acc[m,n,b] = sum_{k in block b} qa[m,k] * (q[n,k] - zp[n,b]), int32 [M, N, kb]
+ * (matmul_nbits.rs:3360-3412 + 9159-9177; qnbitgemm.cpp:727-893). */
+NxrtStatus nxrt_rocm_matmul_nbits_block_acc(NxrtRocmEp* ep, const int8_t* qa_device, const void* b_device,
+                                            const void* zero_points_device, uint64_t m, uint64_t n, uint64_t k,
+                                            uint32_t block_size, int32_t* acc_device);
+
+/* ---- timing on the provider's stream (HIP events) ---------------------------------------------- */
+
+typedef struct NxrtRocmEvent NxrtRocmEvent;
+NxrtStatus nxrt_rocm_ep_event_create(NxrtRocmEp* ep, NxrtRocmEvent** out_event);
+NxrtStatus nxrt_rocm_ep_event_record(NxrtRocmEp* ep, NxrtRocmEvent* event);
+NxrtStatus nxrt_rocm_ep_event_elapsed_ms(NxrtRocmEp* ep, NxrtRocmEvent* start, NxrtRocmEvent* stop, float* out_ms);
+void nxrt_rocm_ep_event_destroy(NxrtRocmEp* ep, NxrtRocmEvent* event);
+
+/* Counters a harness reads to prove the provider, not a fallback, did the work
+ * (the role of nxrt_ep_compiled_node_count in ep-cuda-plugin/src/lib.rs:345-372). */
+uint64_t nxrt_rocm_ep_kernel_launch_count(const NxrtRocmEp* ep);
+uint64_t nxrt_rocm_live_provider_count(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NXRT_EP_ROCM_H */

@@ -1,0 +1,508 @@
+// KernelFactory + Kernel for com.microsoft::MatMulNBits on the ROCm provider.
+// Attribute parsing, input validation and their messages follow the reference's CPU kernel
+// (crates/onnx-runtime-ep-cpu/src/kernels/matmul_nbits.rs:1410-1600, helpers at :10254-10378);
+// the contiguity rule follows its CUDA sibling (crates/onnx-runtime-ep-cuda/src/kernels/matmul_nbits.rs:7089-7106).
+#include <string>
+#include <vector>
+
+#include "provider.h"
+
+using namespace nxrt_rocm;
+
+namespace {
+
+enum AttrBit { kAttrK = 0, kAttrN = 1, kAttrBits = 2, kAttrBlockSize = 3, kAttrAccuracy = 4, kAttrPrepacked = 5 };
+
+std::string err(const std::string& message) { return "MatMulNBits: " + message; }   // matmul_nbits.rs:10376
+
+const char* dtype_name(uint32_t dt)
+{
+    switch (dt) {
+        case 0: return "Undefined";
+        case 1: return "Float32";
+        case 2: return "Uint8";
+        case 3: return "Int8";
+        case 4: return "Uint16";
+        case 5: return "Int16";
+        case 6: return "Int32";
+        case 7: return "Int64";
+        case 8: return "String";
+        case 9: return "Bool";
+        case 10: return "Float16";
+        case 11: return "Float64";
+        case 12: return "Uint32";
+        case 13: return "Uint64";
+        case 16: return "BFloat16";
+        default: return "Unknown";
+    }
+}
+
+std::string shape_str(const uint64_t* shape, uint32_t ndim)
+{
+    std::string s = "[";
+    for (uint32_t i = 0; i < ndim; ++i) {
+        if (i) s += ", ";
+        s += std::to_string(shape[i]);
+    }
+    return s + "]";
+}
+
+std::string shape_str(const std::vector<uint64_t>& v) { return shape_str(v.data(), static_cast<uint32_t>(v.size())); }
+
+bool is_float_compute(uint32_t dt) { return dt == NXRT_DT_FLOAT32 || dt == NXRT_DT_FLOAT16 || dt == NXRT_DT_BFLOAT16; }
+
+bool shape_is(const NxrtRocmTensorView& v, const std::vector<uint64_t>& want)
+{
+    if (v.ndim != want.size()) return false;
+    for (uint32_t i = 0; i < v.ndim; ++i)
+        if (v.shape[i] != want[i]) return false;
+    return true;
+}
+
+bool is_contiguous(const NxrtRocmTensorView& v)
+{
+    if (!v.strides) return true;
+    int64_t expect = 1;
+    for (int i = static_cast<int>(v.ndim) - 1; i >= 0; --i) {
+        if (v.shape[i] != 1 && v.strides[i] != expect) return false;
+        expect *= static_cast<int64_t>(v.shape[i]);
+    }
+    return true;
+}
+
+struct Check {
+    std::string message;
+    bool failed = false;
+    void fail(const std::string& m)
+    {
+        if (!failed) {
+            failed = true;
+            message = err(m);
+        }
+    }
+};
+
+// matmul_nbits.rs:10258-10277 + 1410-1445
+void check_attrs(const NxrtRocmMatMulNBitsAttrs& a, Check& c)
+{
+    auto required_positive = [&](int bit, const char* name, int64_t value) {
+        if (!(a.present & (1u << bit))) return c.fail(std::string("missing required integer attribute '") + name + "'");
+        if (value <= 0) c.fail(std::string("attribute '") + name + "' must be positive, got " + std::to_string(value));
+    };
+    required_positive(kAttrK, "K", a.K);
+    if (c.failed) return;
+    required_positive(kAttrN, "N", a.N);
+    if (c.failed) return;
+    const int64_t bits = (a.present & (1u << kAttrBits)) ? a.bits : 4;
+    if (bits != 4) {
+        c.failed = true;
+        c.message = "MatMulNBits ROCm supports bits=4, got bits=" + std::to_string(bits) +
+                    ". Why: only the 4-bit packed layout has a validated gfx950 kernel. How to fix: export bits=4, "
+                    "or select the CPU execution provider for this node";
+        return;
+    }
+    const int64_t prepacked = (a.present & (1u << kAttrPrepacked)) ? a.weight_prepacked : 0;
+    if (prepacked != 0 && prepacked != 1)
+        return c.fail("weight_prepacked must be 0 (standard ONNX layout) or 1 (MLAS SQNBit packed layout), got " + std::to_string(prepacked));
+    if (prepacked == 1)
+        return c.fail("weight_prepacked=1 holds the MLAS SQNBit CPU layout; the ROCm execution provider takes the standard ONNX layout (weight_prepacked=0)");
+    required_positive(kAttrBlockSize, "block_size", a.block_size);
+    if (c.failed) return;
+    if (a.block_size < 16 || (a.block_size & (a.block_size - 1)) != 0)
+        c.fail("block_size must be a power of two and at least 16, got " + std::to_string(a.block_size));
+}
+
+}  // namespace
+
+struct NxrtRocmMatMulNBits {
+    NxrtRocmEp* ep = nullptr;
+    int64_t k = 0, n = 0, block_size = 0, accuracy_level = 0;
+    int64_t rows_hint = -1;              // M when the create-time shape of A was static
+    bool constant_inputs[6] = {false, false, false, false, false, false};
+    std::string variant = "none";
+    void* scratch = nullptr;             // kernel-owned workspace, grown on demand
+    size_t scratch_bytes = 0;
+    NxrtKernelVtable vtable;
+    uint32_t vt_a_dtype = 0, vt_scale_dtype = 0, vt_y_dtype = 0;
+
+    ~NxrtRocmMatMulNBits()
+    {
+        if (scratch && ep && ep->bind().code == NXRT_OK) {
+            rocm_ffi_stream_sync(ep->stream);
+            rocm_ffi_free(scratch);
+        }
+    }
+};
+
+namespace {
+
+// Bytes of scratch accuracy_level=4 needs for M rows: int8 codes, f32 scales, int32 code sums.
+uint64_t acc4_workspace_bytes(const NxrtRocmMatMulNBits& kn, uint64_t m)
+{
+    const uint64_t kb = (kn.k + kn.block_size - 1) / kn.block_size;
+    const uint64_t codes = (m * kb * kn.block_size + 255) / 256 * 256;
+    const uint64_t scales = (m * kb * 4 + 255) / 256 * 256;
+    return codes + 2 * scales;
+}
+
+NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, uint32_t n_in, NxrtRocmTensorView* out, uint32_t n_out,
+                        void* workspace, uint64_t workspace_bytes)
+{
+    // kernels/mod.rs:1898-1919 (check_arity)
+    if (n_in < 3 || n_in > 6) return make_status(NXRT_INVALID_ARGUMENT, "MatMulNBits: expected 3..=6 inputs, got " + std::to_string(n_in));
+    if (n_out < 1) return make_status(NXRT_INVALID_ARGUMENT, "MatMulNBits: expected at least 1 output(s), got " + std::to_string(n_out));
+    if (!in || !out) return make_status(NXRT_INVALID_ARGUMENT, "MatMulNBits: null tensor view array");
+
+    Check c;
+    auto require_float = [&](const char* name, uint32_t dt) {
+        if (!is_float_compute(dt)) c.fail(std::string(name) + " must have dtype Float32, Float16, or BFloat16, got " + dtype_name(dt));
+    };
+    auto require_dtype = [&](const char* name, uint32_t got, uint32_t want) {
+        if (got != want) c.fail(std::string(name) + " must have dtype " + dtype_name(want) + ", got " + dtype_name(got));
+    };
+    auto optional = [&](uint32_t i) -> const NxrtRocmTensorView* { return (i < n_in && in[i].data != nullptr) ? &in[i] : nullptr; };
+    auto flat_or_matrix = [&](const char* name, const NxrtRocmTensorView& v, uint64_t rows, uint64_t cols) {
+        if (!shape_is(v, {rows * cols}) && !shape_is(v, {rows, cols}))
+            c.fail(std::string(name) + " must have shape [" + std::to_string(rows * cols) + "] or [" + std::to_string(rows) + ", " + std::to_string(cols) +
+                   "], got " + shape_str(v.shape, v.ndim));
+    };
+
+    const NxrtRocmTensorView& A = in[0];
+    const NxrtRocmTensorView& B = in[1];
+    const NxrtRocmTensorView& S = in[2];
+    NxrtRocmTensorView& Y = out[0];
+    require_float("A", A.dtype);
+    require_dtype("B", B.dtype, NXRT_DT_UINT8);
+    require_float("scales", S.dtype);
+    require_float("Y", Y.dtype);
+    if (c.failed) return make_status(NXRT_INVALID_ARGUMENT, c.message);
+
+    const uint64_t K = static_cast<uint64_t>(kn.k), N = static_cast<uint64_t>(kn.n), BS = static_cast<uint64_t>(kn.block_size);
+    if (A.ndim == 0 || A.shape[A.ndim - 1] != K)
+        return make_status(NXRT_INVALID_ARGUMENT, err("A must have rank >= 1 and last dimension K=" + std::to_string(K) + ", got " + shape_str(A.shape, A.ndim)));
+    std::vector<uint64_t> y_shape(A.shape, A.shape + A.ndim - 1);
+    y_shape.push_back(N);
+    if (!shape_is(Y, y_shape))
+        return make_status(NXRT_INVALID_ARGUMENT, err("Y must have shape " + shape_str(y_shape) + ", got " + shape_str(Y.shape, Y.ndim)));
+
+    const uint64_t kb = (K + BS - 1) / BS;
+    const uint64_t blob = BS / 2;
+    flat_or_matrix("scales", S, N, kb);
+    const NxrtRocmTensorView* ZP = optional(3);
+    if (ZP && !c.failed) {
+        require_dtype("zero_points", ZP->dtype, NXRT_DT_UINT8);
+        if (!c.failed) flat_or_matrix("zero_points", *ZP, N, (kb + 1) / 2);
+    }
+    const NxrtRocmTensorView* G = optional(4);
+    if (G && !c.failed) {
+        require_dtype("g_idx", G->dtype, NXRT_DT_INT32);
+        if (!c.failed && !shape_is(*G, {K}) && !shape_is(*G, {kb * BS}))
+            c.fail("g_idx must have shape [" + std::to_string(K) + "] or [" + std::to_string(kb * BS) + "], got " + shape_str(G->shape, G->ndim));
+        if (!c.failed)
+            c.fail("g_idx is not supported on the ROCm execution provider. Why: its kernels stream contiguous K blocks. "
+                   "How to fix: export the weight without act-order, or run this node on the CPU execution provider");
+    }
+    if (!c.failed && !shape_is(B, {N, kb, blob}))
+        c.fail("B must have shape " + shape_str({N, kb, blob}) + ", got " + shape_str(B.shape, B.ndim));
+    const NxrtRocmTensorView* BIAS = optional(5);
+    if (BIAS && !c.failed) {
+        require_float("bias", BIAS->dtype);
+        if (!c.failed && !shape_is(*BIAS, {N})) c.fail("bias must have shape " + shape_str({N}) + ", got " + shape_str(BIAS->shape, BIAS->ndim));
+    }
+    if (c.failed) return make_status(NXRT_INVALID_ARGUMENT, c.message);
+
+    struct Named { const char* name; const NxrtRocmTensorView* v; };
+    const Named all[] = {{"A", &A}, {"B", &B}, {"scales", &S}, {"zero_points", ZP}, {"bias", BIAS}, {"Y", &Y}};
+    for (const Named& t : all) {
+        if (!t.v) continue;
+        if (!is_contiguous(*t.v)) return make_status(NXRT_INVALID_ARGUMENT, err(std::string(t.name) + " must be contiguous on the ROCm execution provider"));
+        if (t.v->device_type != NXRT_DEVICE_ROCM || t.v->device_index != kn.ep->device)
+            return make_status(NXRT_INVALID_ARGUMENT, err(std::string(t.name) + " must live on ROCm device " + std::to_string(kn.ep->device) +
+                                                          " (allocate it with this provider and copy the data in)"));
+    }
+
+    uint64_t M = 1;
+    for (uint32_t i = 0; i + 1 < A.ndim; ++i) M *= A.shape[i];
+    if (M == 0) return ok();
+
+    NxrtStatus st = kn.ep->bind();
+    if (st.code != NXRT_OK) return st;
+
+    auto at = [](const NxrtRocmTensorView& v) { return static_cast<void*>(static_cast<uint8_t*>(v.data) + v.byte_offset); };
+    RocmMatMulNBitsArgs args;
+    args.a = at(A);
+    args.b = static_cast<const uint8_t*>(at(B));
+    args.scales = at(S);
+    args.zp = ZP ? static_cast<const uint8_t*>(at(*ZP)) : nullptr;
+    args.bias = BIAS ? at(*BIAS) : nullptr;
+    args.y = at(Y);
+    args.a_dtype = static_cast<int>(A.dtype);
+    args.scale_dtype = static_cast<int>(S.dtype);
+    args.bias_dtype = BIAS ? static_cast<int>(BIAS->dtype) : ROCM_DT_F32;
+    args.y_dtype = static_cast<int>(Y.dtype);
+    args.m = static_cast<int64_t>(M);
+    args.n = kn.n;
+    args.k = kn.k;
+    args.block_size = static_cast<int>(kn.block_size);
+
+    rocm_stream_t stream = kn.ep->stream;
+    int rc = 0;
+    if (kn.accuracy_level == 4) {
+        const uint64_t need = acc4_workspace_bytes(kn, M);
+        uint8_t* ws = static_cast<uint8_t*>(workspace);
+        if (!ws || workspace_bytes < need) {
+            if (kn.scratch_bytes < need) {
+                if (kn.scratch) {
+                    rocm_ffi_stream_sync(stream);
+                    rocm_ffi_free(kn.scratch);
+                    kn.scratch = nullptr;
+                    kn.scratch_bytes = 0;
+                }
+                const int e = rocm_ffi_malloc(&kn.scratch, need);
+                if (e != 0) return hip_status(e, "MatMulNBits: workspace hipMalloc");
+                kn.scratch_bytes = need;
+            }
+            ws = static_cast<uint8_t*>(kn.scratch);
+        }
+        const uint64_t codes = (M * kb * BS + 255) / 256 * 256;
+        const uint64_t scl = (M * kb * 4 + 255) / 256 * 256;
+        int8_t* qa = reinterpret_cast<int8_t*>(ws);
+        float* qscale = reinterpret_cast<float*>(ws + codes);
+        int32_t* qsum = reinterpret_cast<int32_t*>(ws + codes + scl);
+        rc = rocm_launch_quantize_a(args.a, args.a_dtype, args.m, args.k, args.block_size, kn.ep->acc4_rounding, qa, qscale, qsum, stream);
+        if (rc == 0) {
+            if (rocm_acc4_mfma_eligible(&args)) {
+                rc = rocm_launch_acc4_mfma(&args, qa, qscale, qsum, stream);
+                kn.variant = "acc4_mfma_i8";
+            } else {
+                rc = rocm_launch_acc4_gemv(&args, qa, qscale, qsum, stream);
+                kn.variant = "acc4_gemv_dot4";
+            }
+        }
+    } else if (M <= 16 && rocm_decode_mfma_eligible(&args)) {
+        rc = rocm_launch_decode_mfma(&args, kn.ep->decode_waves, kn.ep->decode_col_groups, stream);
+        kn.variant = "decode_mfma_splitk";
+    } else if (M > 16 && rocm_prefill_mfma_eligible(&args)) {
+        rc = rocm_launch_prefill_mfma(&args, stream);
+        kn.variant = "prefill_mfma_lds";
+    } else {
+        rc = rocm_launch_gemv_generic(&args, stream);
+        kn.variant = "gemv_generic_f32";
+    }
+    kn.ep->launches.fetch_add(1);
+    return hip_status(rc, "MatMulNBits: kernel launch");
+}
+
+NxrtStatus vtable_execute(void* ctx, const void* const* inputs, uint32_t n_in, void** outputs, uint32_t n_out)
+{
+    return fenced([&]() -> NxrtStatus {
+        auto* kn = static_cast<NxrtRocmMatMulNBits*>(ctx);
+        if (!kn || !inputs || !outputs) return make_status(NXRT_INVALID_ARGUMENT, "MatMulNBits: null pointer in kernel vtable execute");
+        if (kn->rows_hint < 0)
+            return make_status(NXRT_INVALID_ARGUMENT, err("the kernel vtable carries no shapes; create the kernel with a static shape for A"));
+        const uint64_t K = kn->k, N = kn->n, BS = kn->block_size, kb = (K + BS - 1) / BS;
+        const uint64_t a_shape[2] = {static_cast<uint64_t>(kn->rows_hint), K}, b_shape[3] = {N, kb, BS / 2}, s_shape[2] = {N, kb},
+                       z_shape[2] = {N, (kb + 1) / 2}, bias_shape[1] = {N}, y_shape[2] = {static_cast<uint64_t>(kn->rows_hint), N};
+        NxrtRocmTensorView in[6];
+        std::memset(in, 0, sizeof(in));
+        auto set = [&](NxrtRocmTensorView& v, const void* p, uint32_t dt, uint32_t nd, const uint64_t* sh) {
+            v.data = const_cast<void*>(p);
+            v.dtype = dt;
+            v.ndim = nd;
+            v.shape = sh;
+            v.device_type = NXRT_DEVICE_ROCM;
+            v.device_index = kn->ep->device;
+        };
+        set(in[0], n_in > 0 ? inputs[0] : nullptr, kn->vt_a_dtype, 2, a_shape);
+        set(in[1], n_in > 1 ? inputs[1] : nullptr, NXRT_DT_UINT8, 3, b_shape);
+        set(in[2], n_in > 2 ? inputs[2] : nullptr, kn->vt_scale_dtype, 2, s_shape);
+        set(in[3], n_in > 3 ? inputs[3] : nullptr, NXRT_DT_UINT8, 2, z_shape);
+        set(in[4], n_in > 4 ? inputs[4] : nullptr, NXRT_DT_INT32, 0, nullptr);
+        set(in[5], n_in > 5 ? inputs[5] : nullptr, kn->vt_a_dtype, 1, bias_shape);
+        NxrtRocmTensorView y;
+        std::memset(&y, 0, sizeof(y));
+        set(y, n_out > 0 ? outputs[0] : nullptr, kn->vt_y_dtype, 2, y_shape);
+        return execute_impl(*kn, in, n_in, &y, n_out, nullptr, 0);
+    });
+}
+
+void vtable_release(void* ctx)
+{
+    try {
+        delete static_cast<NxrtRocmMatMulNBits*>(ctx);
+    } catch (...) {
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+int nxrt_rocm_ep_supports_matmul_nbits(const NxrtRocmEp* ep, const NxrtRocmMatMulNBitsAttrs* attrs, const NxrtTensorDesc* inputs, uint32_t n_inputs,
+                                       char* reason, size_t reason_len)
+{
+    auto decline = [&](const std::string& why) {
+        if (reason && reason_len) {
+            std::strncpy(reason, why.c_str(), reason_len - 1);
+            reason[reason_len - 1] = 0;
+        }
+        return 0;
+    };
+    if (reason && reason_len) reason[0] = 0;
+    if (!attrs) return decline("MatMulNBits: null attributes");
+    Check c;
+    check_attrs(*attrs, c);
+    if (c.failed) return decline(c.message);
+    if (inputs) {
+        if (n_inputs < 3 || n_inputs > 6) return decline("MatMulNBits: expected 3..=6 inputs, got " + std::to_string(n_inputs));
+        if (!is_float_compute(inputs[0].dtype)) return decline(err(std::string("A must have dtype Float32, Float16, or BFloat16, got ") + dtype_name(inputs[0].dtype)));
+        if (inputs[1].dtype != NXRT_DT_UINT8) return decline(err(std::string("B must have dtype Uint8, got ") + dtype_name(inputs[1].dtype)));
+        if (!is_float_compute(inputs[2].dtype)) return decline(err(std::string("scales must have dtype Float32, Float16, or BFloat16, got ") + dtype_name(inputs[2].dtype)));
+        if (n_inputs > 4 && inputs[4].dtype != 0)
+            return decline(err("g_idx is not supported on the ROCm execution provider. Why: its kernels stream contiguous K blocks. "
+                               "How to fix: export the weight without act-order, or run this node on the CPU execution provider"));
+    }
+    return 1;
+}
+
+NxrtStatus nxrt_rocm_matmul_nbits_create(NxrtRocmEp* ep, const NxrtRocmMatMulNBitsAttrs* attrs, const NxrtTensorDesc* input_shapes, uint32_t n_inputs,
+                                         NxrtRocmMatMulNBits** out_kernel)
+{
+    return fenced([&]() -> NxrtStatus {
+        if (!out_kernel) return make_status(NXRT_INVALID_ARGUMENT, "MatMulNBits: null out_kernel");
+        *out_kernel = nullptr;
+        if (!attrs) return make_status(NXRT_INVALID_ARGUMENT, "MatMulNBits: null attributes");
+        Check c;
+        check_attrs(*attrs, c);
+        if (c.failed) return make_status(NXRT_INVALID_ARGUMENT, c.message);
+        if (!ep) return make_status(NXRT_INVALID_ARGUMENT, "MatMulNBits: null provider");
+        auto* kn = new NxrtRocmMatMulNBits();
+        kn->ep = ep;
+        kn->k = attrs->K;
+        kn->n = attrs->N;
+        kn->block_size = attrs->block_size;
+        kn->accuracy_level = (attrs->present & (1u << kAttrAccuracy)) ? attrs->accuracy_level : 0;
+        // flops::leading_rows: product of A's leading dims when all are static
+        if (input_shapes && n_inputs >= 1 && input_shapes[0].ndim >= 1 && input_shapes[0].dims) {
+            int64_t rows = 1;
+            for (uint32_t i = 0; i + 1 < input_shapes[0].ndim; ++i) {
+                const int64_t d = input_shapes[0].dims[i];
+                if (d < 0) { rows = -1; break; }
+                rows *= d;
+            }
+            kn->rows_hint = rows;
+            kn->vt_a_dtype = input_shapes[0].dtype;
+            kn->vt_y_dtype = input_shapes[0].dtype;
+            kn->vt_scale_dtype = n_inputs >= 3 ? input_shapes[2].dtype : input_shapes[0].dtype;
+        }
+        std::memset(&kn->vtable, 0, sizeof(kn->vtable));
+        kn->vtable.struct_size = sizeof(NxrtKernelVtable);
+        kn->vtable.execute = vtable_execute;
+        kn->vtable.release = vtable_release;
+        kn->vtable.ctx = kn;
+        *out_kernel = kn;
+        return ok();
+    });
+}
+
+void nxrt_rocm_matmul_nbits_set_constant_inputs(NxrtRocmMatMulNBits* kernel, const uint8_t* is_constant, uint32_t n)
+{
+    if (!kernel) return;
+    for (uint32_t i = 0; i < 6; ++i) kernel->constant_inputs[i] = (is_constant && i < n) ? is_constant[i] != 0 : false;
+}
+
+NxrtStatus nxrt_rocm_matmul_nbits_workspace_requirement(const NxrtRocmMatMulNBits* kernel, const NxrtTensorDesc* inputs, uint32_t n_inputs,
+                                                        NxrtRocmWorkspaceRequirement* out)
+{
+    return fenced([&]() -> NxrtStatus {
+        if (!kernel || !out) return make_status(NXRT_INVALID_ARGUMENT, "MatMulNBits: null pointer in workspace_requirement");
+        out->bytes = 0;
+        out->alignment = 1;
+        if (kernel->accuracy_level != 4) return ok();
+        if (!inputs || n_inputs < 1 || inputs[0].ndim < 1 || !inputs[0].dims) return make_status(NXRT_INVALID_ARGUMENT, err("workspace_requirement needs the shape of A"));
+        uint64_t m = 1;
+        for (uint32_t i = 0; i + 1 < inputs[0].ndim; ++i) {
+            if (inputs[0].dims[i] < 0) return make_status(NXRT_INVALID_ARGUMENT, err("workspace_requirement needs static leading dimensions of A"));
+            m *= static_cast<uint64_t>(inputs[0].dims[i]);
+        }
+        out->bytes = acc4_workspace_bytes(*kernel, m);
+        out->alignment = 256;
+        return ok();
+    });
+}
+
+NxrtStatus nxrt_rocm_matmul_nbits_execute(NxrtRocmMatMulNBits* kernel, const NxrtRocmTensorView* inputs, uint32_t n_inputs, NxrtRocmTensorView* outputs,
+                                          uint32_t n_outputs, void* workspace_device, uint64_t workspace_bytes)
+{
+    return fenced([&]() -> NxrtStatus {
+        if (!kernel) return make_status(NXRT_INVALID_ARGUMENT, "MatMulNBits: null kernel");
+        return execute_impl(*kernel, inputs, n_inputs, outputs, n_outputs, workspace_device, workspace_bytes);
+    });
+}
+
+uint64_t nxrt_rocm_matmul_nbits_estimated_flops(const NxrtRocmMatMulNBits* kernel)
+{
+    if (!kernel || kernel->rows_hint < 0) return 0;
+    return 2ull * static_cast<uint64_t>(kernel->rows_hint) * static_cast<uint64_t>(kernel->n) * static_cast<uint64_t>(kernel->k);
+}
+
+const char* nxrt_rocm_matmul_nbits_last_variant(const NxrtRocmMatMulNBits* kernel) { return kernel ? kernel->variant.c_str() : ""; }
+
+void nxrt_rocm_matmul_nbits_release(NxrtRocmMatMulNBits* kernel) { vtable_release(kernel); }
+
+NxrtStatus nxrt_rocm_matmul_nbits_as_vtable(NxrtRocmMatMulNBits* kernel, NxrtKernelVtable** out_vtable)
+{
+    if (!kernel || !out_vtable) return make_status(NXRT_INVALID_ARGUMENT, "MatMulNBits: null pointer in as_vtable");
+    *out_vtable = &kernel->vtable;
+    return ok();
+}
+
+NxrtStatus nxrt_rocm_matmul_nbits_dequantize(NxrtRocmEp* ep, const void* b, const void* scales, uint32_t scale_dtype, const void* zp, uint64_t n, uint64_t k,
+                                             uint32_t block_size, float* out_nk)
+{
+    return fenced([&]() -> NxrtStatus {
+        if (!ep || !b || !scales || !out_nk) return make_status(NXRT_INVALID_ARGUMENT, "MatMulNBits dequantize: null pointer");
+        if (!is_float_compute(scale_dtype)) return make_status(NXRT_INVALID_ARGUMENT, err(std::string("scales must have dtype Float32, Float16, or BFloat16, got ") + dtype_name(scale_dtype)));
+        if (block_size < 16 || (block_size & (block_size - 1)) != 0) return make_status(NXRT_INVALID_ARGUMENT, err("block_size must be a power of two and at least 16, got " + std::to_string(block_size)));
+        NxrtStatus st = ep->bind();
+        if (st.code != NXRT_OK) return st;
+        ep->launches.fetch_add(1);
+        return hip_status(rocm_launch_dequant_f32(static_cast<const uint8_t*>(b), scales, static_cast<int>(scale_dtype), static_cast<const uint8_t*>(zp),
+                                                  static_cast<int64_t>(n), static_cast<int64_t>(k), static_cast<int>(block_size), out_nk, ep->stream),
+                          "MatMulNBits dequantize launch");
+    });
+}
+
+NxrtStatus nxrt_rocm_matmul_nbits_quantize_a(NxrtRocmEp* ep, const void* a, uint32_t a_dtype, uint64_t m, uint64_t k, uint32_t block_size, uint32_t rounding,
+                                             int8_t* qa, float* qscale)
+{
+    return fenced([&]() -> NxrtStatus {
+        if (!ep || !a || !qa || !qscale) return make_status(NXRT_INVALID_ARGUMENT, "MatMulNBits quantize_a: null pointer");
+        if (!is_float_compute(a_dtype)) return make_status(NXRT_INVALID_ARGUMENT, err(std::string("A must have dtype Float32, Float16, or BFloat16, got ") + dtype_name(a_dtype)));
+        if (rounding > 1) return make_status(NXRT_INVALID_ARGUMENT, err("rounding must be 0 (ties to even) or 1 (ties away from zero)"));
+        if (block_size < 16 || (block_size & (block_size - 1)) != 0) return make_status(NXRT_INVALID_ARGUMENT, err("block_size must be a power of two and at least 16, got " + std::to_string(block_size)));
+        NxrtStatus st = ep->bind();
+        if (st.code != NXRT_OK) return st;
+        ep->launches.fetch_add(1);
+        return hip_status(rocm_launch_quantize_a(a, static_cast<int>(a_dtype), static_cast<int64_t>(m), static_cast<int64_t>(k), static_cast<int>(block_size),
+                                                 static_cast<int>(rounding), qa, qscale, nullptr, ep->stream),
+                          "MatMulNBits quantize_a launch");
+    });
+}
+
+NxrtStatus nxrt_rocm_matmul_nbits_block_acc(NxrtRocmEp* ep, const int8_t* qa, const void* b, const void* zp, uint64_t m, uint64_t n, uint64_t k,
+                                            uint32_t block_size, int32_t* acc)
+{
+    return fenced([&]() -> NxrtStatus {
+        if (!ep || !qa || !b || !acc) return make_status(NXRT_INVALID_ARGUMENT, "MatMulNBits block_acc: null pointer");
+        if (block_size < 16 || (block_size & (block_size - 1)) != 0) return make_status(NXRT_INVALID_ARGUMENT, err("block_size must be a power of two and at least 16, got " + std::to_string(block_size)));
+        NxrtStatus st = ep->bind();
+        if (st.code != NXRT_OK) return st;
+        ep->launches.fetch_add(1);
+        return hip_status(rocm_launch_block_acc_i32(qa, static_cast<const uint8_t*>(b), static_cast<const uint8_t*>(zp), static_cast<int64_t>(m),
+                                                    static_cast<int64_t>(n), static_cast<int64_t>(k), static_cast<int>(block_size), acc, ep->stream),
+                          "MatMulNBits block_acc launch");
+    });
+}
+
+}  // extern "C"

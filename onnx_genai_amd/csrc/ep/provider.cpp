@@ -1,0 +1,229 @@
+// ExecutionProvider side of the C ABI: lifecycle, device memory, copies, events.
+// Mirrors crates/onnx-runtime-ep-api/src/provider.rs:708-1600 for one ROCm device.
+#include "provider.h"
+
+#include <cstdlib>
+
+namespace nxrt_rocm {
+std::atomic<uint64_t> g_live_providers{0};
+}
+
+using namespace nxrt_rocm;
+
+NxrtRocmEp::NxrtRocmEp() { g_live_providers.fetch_add(1); }
+
+NxrtRocmEp::~NxrtRocmEp()
+{
+    if (rocm_ffi_set_device(static_cast<int>(device)) == 0) {
+        if (stream) rocm_ffi_stream_sync(stream);
+        for (auto& kv : live) rocm_ffi_free(kv.first);
+        if (stream) rocm_ffi_stream_destroy(stream);
+    }
+    g_live_providers.fetch_sub(1);
+}
+
+NxrtStatus NxrtRocmEp::bind() const { return hip_status(rocm_ffi_set_device(static_cast<int>(device)), "hipSetDevice"); }
+
+static int parse_int(const std::string& v, int fallback)
+{
+    char* end = nullptr;
+    const long x = std::strtol(v.c_str(), &end, 10);
+    return (end && *end == 0 && !v.empty()) ? static_cast<int>(x) : fallback;
+}
+
+extern "C" {
+
+NxrtStatus nxrt_rocm_ep_create(uint32_t device_ordinal, const char* const* keys, const char* const* values, uint32_t n_config, NxrtRocmEp** out_ep)
+{
+    return fenced([&]() -> NxrtStatus {
+        if (!out_ep) return make_status(NXRT_INVALID_ARGUMENT, "nxrt_rocm_ep_create: null out_ep");
+        *out_ep = nullptr;
+        int count = 0;
+        int err = rocm_ffi_device_count(&count);
+        if (err != 0 || count <= 0)
+            return make_status(NXRT_DEVICE_ERROR, "RocmExecutionProvider: no HIP device is visible. Why: hipGetDeviceCount found none. "
+                                                  "How to fix: run on a host with an AMD GPU and the ROCm driver loaded");
+        if (device_ordinal >= static_cast<uint32_t>(count))
+            return make_status(NXRT_INVALID_ARGUMENT, "RocmExecutionProvider: device ordinal " + std::to_string(device_ordinal) + " out of range (" + std::to_string(count) + " visible)");
+        auto* ep = new NxrtRocmEp();
+        ep->device = device_ordinal;
+        for (uint32_t i = 0; i < n_config; ++i)
+            if (keys && values && keys[i] && values[i]) ep->config[keys[i]] = values[i];
+        if (const char* env = std::getenv("NXRT_ROCM_ACC4_ROUNDING")) ep->config.emplace("acc4_rounding", env);
+        if (const char* env = std::getenv("NXRT_ROCM_DECODE_WAVES")) ep->config.emplace("decode_waves", env);
+        if (const char* env = std::getenv("NXRT_ROCM_DECODE_COL_GROUPS")) ep->config.emplace("decode_col_groups", env);
+        auto it = ep->config.find("acc4_rounding");
+        if (it != ep->config.end()) {
+            if (it->second == "native") ep->acc4_rounding = 1;
+            else if (it->second == "mlas") ep->acc4_rounding = 0;
+            else {
+                delete ep;
+                return make_status(NXRT_INVALID_ARGUMENT, "RocmExecutionProvider: acc4_rounding must be 'mlas' or 'native'");
+            }
+        }
+        if ((it = ep->config.find("decode_waves")) != ep->config.end()) ep->decode_waves = parse_int(it->second, 0);
+        if ((it = ep->config.find("decode_col_groups")) != ep->config.end()) ep->decode_col_groups = parse_int(it->second, 0);
+        NxrtStatus st = ep->bind();
+        if (st.code == NXRT_OK) st = hip_status(rocm_ffi_stream_create(&ep->stream), "hipStreamCreate");
+        if (st.code != NXRT_OK) {
+            delete ep;
+            return st;
+        }
+        init_ep_vtable(ep);
+        *out_ep = ep;
+        return ok();
+    });
+}
+
+void nxrt_rocm_ep_release(NxrtRocmEp* ep)
+{
+    try {
+        delete ep;
+    } catch (...) {
+    }
+}
+
+const char* nxrt_rocm_ep_name(const NxrtRocmEp* ep) { return ep ? ep->name.c_str() : ""; }
+uint32_t nxrt_rocm_ep_device_type(const NxrtRocmEp*) { return NXRT_DEVICE_ROCM; }
+uint32_t nxrt_rocm_ep_device_id(const NxrtRocmEp* ep) { return ep ? ep->device : 0; }
+uint32_t nxrt_rocm_ep_memory_vendor_id(const NxrtRocmEp*) { return 0x1002u; }
+
+NxrtStatus nxrt_rocm_ep_device_info(const NxrtRocmEp* ep, char* arch, size_t arch_len, uint32_t* compute_units, uint64_t* total_memory)
+{
+    return fenced([&]() -> NxrtStatus {
+        if (!ep) return make_status(NXRT_INVALID_ARGUMENT, "null provider");
+        int cus = 0;
+        size_t mem = 0;
+        const int err = rocm_ffi_device_info(static_cast<int>(ep->device), arch, arch_len, &cus, &mem);
+        if (compute_units) *compute_units = static_cast<uint32_t>(cus);
+        if (total_memory) *total_memory = mem;
+        return hip_status(err, "hipGetDeviceProperties");
+    });
+}
+
+NxrtStatus nxrt_rocm_ep_allocate(NxrtRocmEp* ep, size_t size, size_t align, void** out_device)
+{
+    return fenced([&]() -> NxrtStatus {
+        if (!ep || !out_device) return make_status(NXRT_INVALID_ARGUMENT, "nxrt_rocm_ep_allocate: null pointer");
+        *out_device = nullptr;
+        if (align > 256 || (align & (align - 1)) != 0)
+            return make_status(NXRT_INVALID_ARGUMENT, "nxrt_rocm_ep_allocate: alignment must be a power of two <= 256, got " + std::to_string(align));
+        NxrtStatus st = ep->bind();
+        if (st.code != NXRT_OK) return st;
+        void* p = nullptr;
+        const int err = rocm_ffi_malloc(&p, size ? size : 1);
+        if (err != 0) return hip_status(err, "hipMalloc");
+        std::lock_guard<std::mutex> lock(ep->mu);
+        ep->live[p] = size;
+        *out_device = p;
+        return ok();
+    });
+}
+
+NxrtStatus nxrt_rocm_ep_deallocate(NxrtRocmEp* ep, void* device)
+{
+    return fenced([&]() -> NxrtStatus {
+        if (!ep) return make_status(NXRT_INVALID_ARGUMENT, "nxrt_rocm_ep_deallocate: null provider");
+        if (!device) return ok();
+        {
+            std::lock_guard<std::mutex> lock(ep->mu);
+            auto it = ep->live.find(device);
+            if (it == ep->live.end()) return make_status(NXRT_INVALID_ARGUMENT, "nxrt_rocm_ep_deallocate: pointer was not allocated by this provider");
+            ep->live.erase(it);
+        }
+        NxrtStatus st = ep->bind();
+        if (st.code != NXRT_OK) return st;
+        rocm_ffi_stream_sync(ep->stream);   // work queued on the stream may still read the buffer
+        return hip_status(rocm_ffi_free(device), "hipFree");
+    });
+}
+
+NxrtStatus nxrt_rocm_ep_copy_from_host(NxrtRocmEp* ep, void* dst, const void* src, size_t bytes)
+{
+    return fenced([&]() -> NxrtStatus {
+        if (!ep || (bytes && (!dst || !src))) return make_status(NXRT_INVALID_ARGUMENT, "copy_from_host: null pointer");
+        if (!bytes) return ok();
+        NxrtStatus st = ep->bind();
+        if (st.code != NXRT_OK) return st;
+        return hip_status(rocm_ffi_memcpy_h2d(dst, src, bytes, ep->stream), "hipMemcpy host to device");
+    });
+}
+
+NxrtStatus nxrt_rocm_ep_copy_to_host(NxrtRocmEp* ep, void* dst, const void* src, size_t bytes)
+{
+    return fenced([&]() -> NxrtStatus {
+        if (!ep || (bytes && (!dst || !src))) return make_status(NXRT_INVALID_ARGUMENT, "copy_to_host: null pointer");
+        if (!bytes) return ok();
+        NxrtStatus st = ep->bind();
+        if (st.code != NXRT_OK) return st;
+        return hip_status(rocm_ffi_memcpy_d2h(dst, src, bytes, ep->stream), "hipMemcpy device to host");
+    });
+}
+
+NxrtStatus nxrt_rocm_ep_copy(NxrtRocmEp* ep, void* dst, const void* src, size_t bytes)
+{
+    return fenced([&]() -> NxrtStatus {
+        if (!ep || (bytes && (!dst || !src))) return make_status(NXRT_INVALID_ARGUMENT, "copy: null pointer");
+        if (!bytes) return ok();
+        NxrtStatus st = ep->bind();
+        if (st.code != NXRT_OK) return st;
+        return hip_status(rocm_ffi_memcpy_d2d(dst, src, bytes, ep->stream), "hipMemcpy device to device");
+    });
+}
+
+NxrtStatus nxrt_rocm_ep_sync(NxrtRocmEp* ep)
+{
+    return fenced([&]() -> NxrtStatus {
+        if (!ep) return make_status(NXRT_INVALID_ARGUMENT, "sync: null provider");
+        NxrtStatus st = ep->bind();
+        if (st.code != NXRT_OK) return st;
+        return hip_status(rocm_ffi_stream_sync(ep->stream), "hipStreamSynchronize");
+    });
+}
+
+NxrtStatus nxrt_rocm_ep_event_create(NxrtRocmEp* ep, NxrtRocmEvent** out_event)
+{
+    return fenced([&]() -> NxrtStatus {
+        if (!ep || !out_event) return make_status(NXRT_INVALID_ARGUMENT, "event_create: null pointer");
+        NxrtStatus st = ep->bind();
+        if (st.code != NXRT_OK) return st;
+        auto* e = new NxrtRocmEvent();
+        const int err = rocm_ffi_event_create(&e->ev);
+        if (err != 0) {
+            delete e;
+            return hip_status(err, "hipEventCreate");
+        }
+        *out_event = e;
+        return ok();
+    });
+}
+
+NxrtStatus nxrt_rocm_ep_event_record(NxrtRocmEp* ep, NxrtRocmEvent* event)
+{
+    return fenced([&]() -> NxrtStatus {
+        if (!ep || !event) return make_status(NXRT_INVALID_ARGUMENT, "event_record: null pointer");
+        return hip_status(rocm_ffi_event_record(event->ev, ep->stream), "hipEventRecord");
+    });
+}
+
+NxrtStatus nxrt_rocm_ep_event_elapsed_ms(NxrtRocmEp* ep, NxrtRocmEvent* start, NxrtRocmEvent* stop, float* out_ms)
+{
+    return fenced([&]() -> NxrtStatus {
+        if (!ep || !start || !stop || !out_ms) return make_status(NXRT_INVALID_ARGUMENT, "event_elapsed_ms: null pointer");
+        int err = rocm_ffi_event_sync(stop->ev);
+        if (err == 0) err = rocm_ffi_event_elapsed_ms(start->ev, stop->ev, out_ms);
+        return hip_status(err, "hipEventElapsedTime");
+    });
+}
+
+void nxrt_rocm_ep_event_destroy(NxrtRocmEp*, NxrtRocmEvent* event)
+{
+    if (!event) return;
+    rocm_ffi_event_destroy(event->ev);
+    delete event;
+}
+
+uint64_t nxrt_rocm_ep_kernel_launch_count(const NxrtRocmEp* ep) { return ep ? ep->launches.load() : 0; }
+uint64_t nxrt_rocm_live_provider_count(void) { return g_live_providers.load(); }
+
+}  // extern "C"

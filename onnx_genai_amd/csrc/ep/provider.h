@@ -1,0 +1,38 @@
+// The execution provider object: one GPU, one HIP stream, the buffers it handed out.
+#pragma once
+
+#include <atomic>
+#include <cstdint>
+#include <map>
+#include <mutex>
+#include <string>
+#include <unordered_map>
+
+#include "status.h"
+
+struct NxrtRocmEp {
+    uint32_t device = 0;
+    rocm_stream_t stream = nullptr;
+    std::string name = "RocmExecutionProvider";
+    std::map<std::string, std::string> config;   // EpConfig: a string map
+    int acc4_rounding = 0;                        // 0 = ties to even (MLAS), 1 = ties away (native)
+    int decode_waves = 0;                         // 0 = chosen per shape
+    int decode_col_groups = 0;
+    std::mutex mu;
+    std::unordered_map<void*, size_t> live;       // allocations handed out and not yet returned
+    std::atomic<uint64_t> launches{0};
+    NxrtEpVtable vtable;                          // ctx points back at this object
+
+    NxrtRocmEp();
+    ~NxrtRocmEp();
+    NxrtStatus bind() const;                      // make this provider's GPU current on the calling thread
+};
+
+struct NxrtRocmEvent {
+    rocm_event_t ev = nullptr;
+};
+
+namespace nxrt_rocm {
+extern std::atomic<uint64_t> g_live_providers;
+void init_ep_vtable(NxrtRocmEp* ep);
+}  // namespace nxrt_rocm

@@ -1,0 +1,87 @@
+/*
+ * The only doorway from the execution provider's host code to HIP: device memory, one stream,
+ * events, and one launcher per hand-written gfx950 kernel. Plain C types only. Every function
+ * returns 0 on success or the hipError_t value; rocm_ffi_error_string() names it.
+ */
+#ifndef NXRT_ROCM_HIP_FFI_H
+#define NXRT_ROCM_HIP_FFI_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* rocm_stream_t;
+typedef void* rocm_event_t;
+
+/* element dtypes on the wire (onnx-runtime-ir DataType discriminants) */
+enum { ROCM_DT_F32 = 1, ROCM_DT_U8 = 2, ROCM_DT_I32 = 6, ROCM_DT_F16 = 10, ROCM_DT_BF16 = 16 };
+
+const char* rocm_ffi_error_string(int err);
+int rocm_ffi_device_count(int* count);
+int rocm_ffi_set_device(int device);
+int rocm_ffi_device_info(int device, char* arch, size_t arch_len, int* compute_units, size_t* total_mem);
+int rocm_ffi_malloc(void** ptr, size_t bytes);
+int rocm_ffi_free(void* ptr);
+int rocm_ffi_memcpy_h2d(void* dst, const void* src, size_t bytes, rocm_stream_t stream);
+int rocm_ffi_memcpy_d2h(void* dst, const void* src, size_t bytes, rocm_stream_t stream);
+int rocm_ffi_memcpy_d2d(void* dst, const void* src, size_t bytes, rocm_stream_t stream);
+int rocm_ffi_stream_create(rocm_stream_t* stream);
+int rocm_ffi_stream_destroy(rocm_stream_t stream);
+int rocm_ffi_stream_sync(rocm_stream_t stream);
+int rocm_ffi_event_create(rocm_event_t* event);
+int rocm_ffi_event_destroy(rocm_event_t event);
+int rocm_ffi_event_record(rocm_event_t event, rocm_stream_t stream);
+int rocm_ffi_event_sync(rocm_event_t event);
+int rocm_ffi_event_elapsed_ms(rocm_event_t start, rocm_event_t stop, float* ms);
+int rocm_ffi_fill_u32(void* dst, uint32_t value, size_t count, rocm_stream_t stream);
+
+/* Operands of one MatMulNBits call, all device pointers, all contiguous. */
+typedef struct RocmMatMulNBitsArgs {
+  const void* a;        /* [M, K] a_dtype */
+  const uint8_t* b;     /* [N, kb, bs/2] */
+  const void* scales;   /* [N, kb] scale_dtype */
+  const uint8_t* zp;    /* [N, ceil(kb/2)] or NULL (zero point 8) */
+  const void* bias;     /* [N] bias_dtype or NULL */
+  void* y;              /* [M, N] y_dtype */
+  int a_dtype, scale_dtype, bias_dtype, y_dtype;
+  int64_t m, n, k;
+  int block_size;
+} RocmMatMulNBitsArgs;
+
+/* w[n,k] = (q - zp) * scale as f32 [N, K]. */
+int rocm_launch_dequant_f32(const uint8_t* b, const void* scales, int scale_dtype, const uint8_t* zp,
+                            int64_t n, int64_t k, int block_size, float* out_nk, rocm_stream_t stream);
+
+/* Any dtype mix, any K, any block size: f32 math, one wave per output column. */
+int rocm_launch_gemv_generic(const RocmMatMulNBitsArgs* args, rocm_stream_t stream);
+
+/* Decode (M <= 16), f16/bf16 activations: split-K MFMA GEMV. Returns -1 when the shape is not eligible.
+ * waves/col_groups = 0 lets the launcher choose. */
+int rocm_decode_mfma_eligible(const RocmMatMulNBitsArgs* args);
+int rocm_launch_decode_mfma(const RocmMatMulNBitsArgs* args, int waves, int col_groups, rocm_stream_t stream);
+
+/* Prefill (M > 16), f16/bf16 activations: B tiles dequantized into LDS, 32x32x16 MFMA. */
+int rocm_prefill_mfma_eligible(const RocmMatMulNBitsArgs* args);
+int rocm_launch_prefill_mfma(const RocmMatMulNBitsArgs* args, rocm_stream_t stream);
+
+/* accuracy_level 4. rounding: 0 = ties to even (MLAS rule), 1 = ties away (native Rust rule).
+ * qa: int8 [M, kb*bs]; qscale: f32 [M, kb]; qsum: int32 [M, kb] (sum of codes per block). */
+int rocm_launch_quantize_a(const void* a, int a_dtype, int64_t m, int64_t k, int block_size, int rounding,
+                           int8_t* qa, float* qscale, int32_t* qsum, rocm_stream_t stream);
+/* acc[m,n,b] = sum_k qa[m,k] * (q[n,k] - zp[n,b]), int32 [M, N, kb]. */
+int rocm_launch_block_acc_i32(const int8_t* qa, const uint8_t* b, const uint8_t* zp,
+                              int64_t m, int64_t n, int64_t k, int block_size, int32_t* acc, rocm_stream_t stream);
+/* y = sum_b f32(acc_b) * (sa_b * sb_b) + bias, from already quantized activations. */
+int rocm_launch_acc4_gemv(const RocmMatMulNBitsArgs* args, const int8_t* qa, const float* qscale, const int32_t* qsum,
+                          rocm_stream_t stream);
+int rocm_acc4_mfma_eligible(const RocmMatMulNBitsArgs* args);
+int rocm_launch_acc4_mfma(const RocmMatMulNBitsArgs* args, const int8_t* qa, const float* qscale, const int32_t* qsum,
+                          rocm_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

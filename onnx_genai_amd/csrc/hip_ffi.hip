@@ -1,0 +1,90 @@
+// HIP runtime half of hip_ffi.h: device memory, the stream, events. No kernels live here.
+#include <hip/hip_runtime.h>
+
+#include <cstring>
+
+#include "hip_ffi.h"
+
+namespace {
+__global__ void fill_u32_kernel(uint32_t* dst, uint32_t value, size_t count)
+{
+    for (size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; i < count; i += static_cast<size_t>(gridDim.x) * blockDim.x) dst[i] = value;
+}
+}  // namespace
+
+extern "C" {
+
+const char* rocm_ffi_error_string(int err) { return err < 0 ? "shape not eligible for this kernel" : hipGetErrorString(static_cast<hipError_t>(err)); }
+int rocm_ffi_device_count(int* count) { return static_cast<int>(hipGetDeviceCount(count)); }
+int rocm_ffi_set_device(int device) { return static_cast<int>(hipSetDevice(device)); }
+
+int rocm_ffi_device_info(int device, char* arch, size_t arch_len, int* compute_units, size_t* total_mem)
+{
+    hipDeviceProp_t prop;
+    const hipError_t e = hipGetDeviceProperties(&prop, device);
+    if (e != hipSuccess) return static_cast<int>(e);
+    if (arch && arch_len) {
+        std::strncpy(arch, prop.gcnArchName, arch_len - 1);
+        arch[arch_len - 1] = 0;
+    }
+    if (compute_units) *compute_units = prop.multiProcessorCount;
+    if (total_mem) *total_mem = prop.totalGlobalMem;
+    return 0;
+}
+
+int rocm_ffi_malloc(void** ptr, size_t bytes) { return static_cast<int>(hipMalloc(ptr, bytes)); }
+int rocm_ffi_free(void* ptr) { return static_cast<int>(hipFree(ptr)); }
+
+int rocm_ffi_memcpy_h2d(void* dst, const void* src, size_t bytes, rocm_stream_t stream)
+{
+    hipError_t e = hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, static_cast<hipStream_t>(stream));
+    if (e == hipSuccess) e = hipStreamSynchronize(static_cast<hipStream_t>(stream));
+    return static_cast<int>(e);
+}
+
+int rocm_ffi_memcpy_d2h(void* dst, const void* src, size_t bytes, rocm_stream_t stream)
+{
+    hipError_t e = hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, static_cast<hipStream_t>(stream));
+    if (e == hipSuccess) e = hipStreamSynchronize(static_cast<hipStream_t>(stream));
+    return static_cast<int>(e);
+}
+
+int rocm_ffi_memcpy_d2d(void* dst, const void* src, size_t bytes, rocm_stream_t stream)
+{
+    return static_cast<int>(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, static_cast<hipStream_t>(stream)));
+}
+
+int rocm_ffi_stream_create(rocm_stream_t* stream)
+{
+    hipStream_t s = nullptr;
+    const hipError_t e = hipStreamCreateWithFlags(&s, hipStreamNonBlocking);   // default priority
+    *stream = s;
+    return static_cast<int>(e);
+}
+
+int rocm_ffi_stream_destroy(rocm_stream_t stream) { return static_cast<int>(hipStreamDestroy(static_cast<hipStream_t>(stream))); }
+int rocm_ffi_stream_sync(rocm_stream_t stream) { return static_cast<int>(hipStreamSynchronize(static_cast<hipStream_t>(stream))); }
+
+int rocm_ffi_event_create(rocm_event_t* event)
+{
+    hipEvent_t e = nullptr;
+    const hipError_t r = hipEventCreate(&e);
+    *event = e;
+    return static_cast<int>(r);
+}
+
+int rocm_ffi_event_destroy(rocm_event_t event) { return static_cast<int>(hipEventDestroy(static_cast<hipEvent_t>(event))); }
+int rocm_ffi_event_record(rocm_event_t event, rocm_stream_t stream) { return static_cast<int>(hipEventRecord(static_cast<hipEvent_t>(event), static_cast<hipStream_t>(stream))); }
+int rocm_ffi_event_sync(rocm_event_t event) { return static_cast<int>(hipEventSynchronize(static_cast<hipEvent_t>(event))); }
+int rocm_ffi_event_elapsed_ms(rocm_event_t start, rocm_event_t stop, float* ms) { return static_cast<int>(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop))); }
+
+int rocm_ffi_fill_u32(void* dst, uint32_t value, size_t count, rocm_stream_t stream)
+{
+    if (count == 0) return 0;
+    size_t blocks = (count + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(fill_u32_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, static_cast<hipStream_t>(stream), static_cast<uint32_t*>(dst), value, count);
+    return static_cast<int>(hipGetLastError());
+}
+
+}  // extern "C"

@@ -1,0 +1,172 @@
+// accuracy_level = 4: activations quantized per K-block to symmetric int8, integer block dot
+// products, one f32 scale-and-add per block.
+//
+//   scale = max|a| / 127, inv = 127 / max|a| (0 for an all-zero block), code = round(a * inv)
+//   acc[m,n,b] = sum_{k in b} code[m,k] * (q[n,k] - zp[n,b])                       (int32, exact)
+//   y[m,n]     = sum_b f32(acc[m,n,b]) * (scale_a[m,b] * scale_b[n,b]) + bias[n]   (f32)
+//
+// Two rounding rules exist in the reference's CPU code and both are implemented: ties to even (its
+// MLAS kernels) and ties away from zero with a clamp to +-127 (its native Rust kernels).
+#include "common.hiph"
+
+namespace mnb {
+
+// One wave per (row, block). Division and multiply are single correctly rounded f32 operations.
+__global__ __launch_bounds__(256) void quantize_a_kernel(
+    const void* __restrict__ a, int a_dtype, int64_t m, int64_t k, int bs, int64_t kb, int rounding,
+    int8_t* __restrict__ qa, float* __restrict__ qscale, int32_t* __restrict__ qsum)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t item = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+    if (item >= m * kb) return;
+    const int64_t row = item / kb, blk = item - row * kb;
+    const int64_t k0 = blk * bs;
+    const int64_t valid = (k - k0 < bs) ? (k - k0) : bs;
+    float vmax = 0.0f;
+    for (int i = lane; i < valid; i += 64) vmax = fmaxf(vmax, fabsf(load_as_f32(a, a_dtype, row * k + k0 + i)));
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) vmax = fmaxf(vmax, __shfl_xor(vmax, off, 64));
+    const float scale = __fdiv_rn(vmax, 127.0f);
+    const float inv = vmax != 0.0f ? __fdiv_rn(127.0f, vmax) : 0.0f;
+    int sum = 0;
+    for (int i = lane; i < bs; i += 64) {
+        int code = 0;
+        if (i < valid) {
+            const float scaled = __fmul_rn(load_as_f32(a, a_dtype, row * k + k0 + i), inv);
+            float r = rounding == 1 ? roundf(scaled) : rintf(scaled);
+            r = fminf(fmaxf(r, -127.0f), 127.0f);
+            code = static_cast<int>(r);
+        }
+        qa[(row * kb + blk) * bs + i] = static_cast<int8_t>(code);
+        sum += code;
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    if (lane == 0) {
+        qscale[row * kb + blk] = scale;
+        if (qsum) qsum[row * kb + blk] = sum;
+    }
+}
+
+// Parity probe: one thread per (m, n, block), straight integer loop.
+__global__ __launch_bounds__(256) void block_acc_i32_kernel(
+    const int8_t* __restrict__ qa, const uint8_t* __restrict__ b, const uint8_t* __restrict__ zp,
+    int64_t m, int64_t n, int64_t k, int bs, int64_t kb, int32_t* __restrict__ acc)
+{
+    const int64_t total = m * n * kb;
+    for (int64_t idx = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; idx < total; idx += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+        const int64_t blk = idx % kb;
+        const int64_t col = (idx / kb) % n;
+        const int64_t row = idx / (kb * n);
+        const int z = zero_point_of(zp ? zp + col * ((kb + 1) >> 1) : nullptr, blk);
+        const uint8_t* wb = b + (col * kb + blk) * (bs / 2);
+        const int8_t* q = qa + (row * kb + blk) * bs;
+        const int64_t valid = (k - blk * bs < bs) ? (k - blk * bs) : bs;
+        int s = 0;
+        for (int i = 0; i < valid; ++i) s += static_cast<int>(q[i]) * (static_cast<int>((wb[i >> 1] >> ((i & 1) * 4)) & 0xf) - z);
+        acc[idx] = s;
+    }
+}
+
+// One wave per output column; a lane takes one packed dword (8 weights) at a time, dots it against the
+// 8 matching activation codes with v_dot4_i32_i8, and the bs/8 lanes of a block add up with shuffles.
+template <int ROWS>
+__global__ __launch_bounds__(256) void acc4_gemv_kernel(RocmMatMulNBitsArgs p, const int8_t* __restrict__ qa, const float* __restrict__ qscale,
+                                                        const int32_t* __restrict__ qsum, int bs_log2, int64_t kb, int64_t row0)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t col = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+    if (col >= p.n) return;
+    const int bs = 1 << bs_log2;
+    const int lanes_per_block = bs >> 3;                       // 2 .. 32 lanes share a block
+    const int64_t row_dwords = (kb << bs_log2) >> 3;
+    const uint32_t* brow = reinterpret_cast<const uint32_t*>(p.b) + col * row_dwords;
+    const uint8_t* zrow = p.zp ? p.zp + col * ((kb + 1) >> 1) : nullptr;
+    const int rows = static_cast<int>(p.m - row0 < ROWS ? p.m - row0 : ROWS);
+    const int64_t padded_k = kb << bs_log2;
+
+    float acc[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) acc[r] = 0.0f;
+
+    const int64_t steps = (row_dwords + 63) / 64;
+    for (int64_t it = 0; it < steps; ++it) {
+        const int64_t d = it * 64 + lane;
+        const bool ok = d < row_dwords;
+        const int64_t blk = ok ? ((d << 3) >> bs_log2) : 0;
+        const uint32_t w = ok ? brow[d] : 0u;
+        const int lo = static_cast<int>(w & 0x0f0f0f0fu);          // elements 0,2,4,6
+        const int hi = static_cast<int>((w >> 4) & 0x0f0f0f0fu);   // elements 1,3,5,7
+        const int z = zero_point_of(zrow, blk);
+        const float sb = ok ? load_as_f32(p.scales, p.scale_dtype, col * kb + blk) : 0.0f;
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) {
+            int dot = 0;
+            if (ok && r < rows) {
+                const uint2 c = *reinterpret_cast<const uint2*>(qa + (row0 + r) * padded_k + (d << 3));
+                const int even = static_cast<int>(__builtin_amdgcn_perm(c.y, c.x, 0x06040200u));
+                const int odd = static_cast<int>(__builtin_amdgcn_perm(c.y, c.x, 0x07050301u));
+                dot = __builtin_amdgcn_sdot4(even, lo, 0, false);
+                dot = __builtin_amdgcn_sdot4(odd, hi, dot, false);
+            }
+            for (int off = 1; off < lanes_per_block; off <<= 1) dot += __shfl_xor(dot, off, 64);
+            if (ok && r < rows && (lane & (lanes_per_block - 1)) == 0) {
+                const int block_acc = dot - z * qsum[(row0 + r) * kb + blk];
+                acc[r] += static_cast<float>(block_acc) * __fmul_rn(qscale[(row0 + r) * kb + blk], sb);
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+        const float total = wave_sum(acc[r]);
+        if (lane == 0 && r < rows) {
+            const float bias = p.bias ? load_as_f32(p.bias, p.bias_dtype, col) : 0.0f;
+            store_from_f32(p.y, p.y_dtype, (row0 + r) * p.n + col, total + bias);
+        }
+    }
+}
+
+}  // namespace mnb
+
+extern "C" int rocm_launch_quantize_a(const void* a, int a_dtype, int64_t m, int64_t k, int block_size, int rounding,
+                                      int8_t* qa, float* qscale, int32_t* qsum, rocm_stream_t stream)
+{
+    if (m <= 0 || k <= 0) return 0;
+    const int64_t kb = (k + block_size - 1) / block_size;
+    const int64_t items = m * kb;
+    hipLaunchKernelGGL(mnb::quantize_a_kernel, dim3(static_cast<unsigned>((items + 3) / 4)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       a, a_dtype, m, k, block_size, kb, rounding, qa, qscale, qsum);
+    return static_cast<int>(hipGetLastError());
+}
+
+extern "C" int rocm_launch_block_acc_i32(const int8_t* qa, const uint8_t* b, const uint8_t* zp, int64_t m, int64_t n, int64_t k,
+                                         int block_size, int32_t* acc, rocm_stream_t stream)
+{
+    if (m <= 0 || n <= 0 || k <= 0) return 0;
+    const int64_t kb = (k + block_size - 1) / block_size;
+    int64_t blocks = (m * n * kb + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    hipLaunchKernelGGL(mnb::block_acc_i32_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       qa, b, zp, m, n, k, block_size, kb, acc);
+    return static_cast<int>(hipGetLastError());
+}
+
+extern "C" int rocm_launch_acc4_gemv(const RocmMatMulNBitsArgs* args, const int8_t* qa, const float* qscale, const int32_t* qsum,
+                                     rocm_stream_t stream)
+{
+    if (args->m <= 0 || args->n <= 0) return 0;
+    const int bs_log2 = __builtin_ctz(static_cast<unsigned>(args->block_size));
+    const int64_t kb = (args->k + args->block_size - 1) / args->block_size;
+    const dim3 grid(static_cast<unsigned>((args->n + 3) / 4));
+    constexpr int kRows = 4;
+    for (int64_t row0 = 0; row0 < args->m; row0 += kRows) {
+        if (args->m - row0 == 1)
+            hipLaunchKernelGGL(mnb::acc4_gemv_kernel<1>, grid, dim3(256), 0, static_cast<hipStream_t>(stream), *args, qa, qscale, qsum, bs_log2, kb, row0);
+        else
+            hipLaunchKernelGGL(mnb::acc4_gemv_kernel<kRows>, grid, dim3(256), 0, static_cast<hipStream_t>(stream), *args, qa, qscale, qsum, bs_log2, kb, row0);
+    }
+    return static_cast<int>(hipGetLastError());
+}
+
+extern "C" int rocm_acc4_mfma_eligible(const RocmMatMulNBitsArgs*) { return 0; }
+extern "C" int rocm_launch_acc4_mfma(const RocmMatMulNBitsArgs*, const int8_t*, const float*, const int32_t*, rocm_stream_t) { return -1; }

@@ -1,0 +1,41 @@
+import os
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
+
+
+@pytest.fixture(scope="session")
+def port():
+    import oracle
+    return oracle.Port()
+
+
+@pytest.fixture(scope="session")
+def ref():
+    """The reference's own compiled CPU path (oracle/_ref). Built here from /root/reference; prebuilt on the GPU box."""
+    import oracle
+    if not oracle.Ref.available():
+        if os.path.isdir("/root/reference/crates/mlas-sys/vendor"):
+            oracle.build(ref=True)
+        else:
+            pytest.skip("oracle/_ref/libmlas_ref.so is not built and /root/reference is absent")
+    return oracle.Ref()
+
+
+@pytest.fixture(scope="session")
+def ep():
+    """One provider for the whole GPU session. No fallback: a missing library or GPU is a hard failure."""
+    from onnx_genai_amd.ep import RocmExecutionProvider
+    provider = RocmExecutionProvider(0)
+    info = provider.device_info()
+    assert info["arch"].startswith("gfx950"), info
+    yield provider
+    provider.shutdown()

@@ -1,0 +1,442 @@
+"""Parity of the HIP path with the CPU oracle, called through the C ABI of libnxrt_ep_rocm.so.
+
+Bars (from the parity contract of this build):
+  * dequantized weights ........................ bit-exact
+  * accuracy_level=4 codes and int32 block sums  bit-exact
+  * outputs, f32 activations ................... rel-L2 <= 1e-5
+  * outputs, f16/bf16 activations .............. rel-L2 <= 5e-3
+"""
+import numpy as np
+import pytest
+
+import oracle
+from onnx_genai_amd import ep as E
+from onnx_genai_amd import synth
+from tests import helpers
+
+pytestmark = pytest.mark.gpu
+
+TOL_F32 = 1e-5
+TOL_HALF = 5e-3
+NPDT = {E.F32: np.float32, E.F16: np.float16, E.BF16: np.uint16}
+
+
+def run_op(ep, a, a_dt, b, s, s_dt, zp, n, k, bs, **kw):
+    return E.matmul_nbits(ep, a, a_dt, b, s, s_dt, zp, n, k, bs, **kw)
+
+
+def oracle_f64(port, a, a_dt, b, s, s_dt, zp, n, k, bs, bias=None, bias_dt=E.F32):
+    af = synth.to_f32(a, a_dt)
+    sf = synth.to_f32(s, s_dt)
+    bf = None if bias is None else synth.to_f32(bias, bias_dt)
+    return port.matmul_f64(af, b, sf, zp, n, k, bs, bias=bf)
+
+
+# ---------------------------------------------------------------------------------------------
+# dequantization: bit-exact
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("bs", [16, 32, 64, 128, 256])
+@pytest.mark.parametrize("zero_points", [False, True])
+@pytest.mark.parametrize("s_dt", [E.F32, E.F16, E.BF16])
+def test_dequantize_bit_exact(ep, port, bs, zero_points, s_dt):
+    n, k = 75, 3 * bs + (bs // 2 if bs >= 32 else 0)      # ragged N, partial last block
+    b, s, zp = synth.make_weights(n, k, bs, 11 + bs, zero_points=zero_points, scale_lo=0.002, scale_hi=0.02, scale_dtype=s_dt)
+    want = port.dequantize_nk(b, synth.to_f32(s, s_dt), zp, n, k, bs)
+    bb, sb = ep.upload(b), ep.upload(s)
+    zb = ep.upload(zp) if zp is not None else None
+    out = ep.allocate(n * k * 4)
+    ep.dequantize(bb, sb, s_dt, zb, n, k, bs, out)
+    got = ep.download(out, (n, k), np.float32)
+    for buf in (bb, sb, zb, out):
+        if buf is not None:
+            ep.deallocate(buf)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_dequantize_all_nibble_zero_point_pairs(ep, port):
+    """Every (q, zp) pair against scales with awkward bit patterns."""
+    bs, kb = 16, 16
+    n = 16
+    q = np.tile(np.arange(16, dtype=np.uint8), (n, kb, 1))
+    b = synth.pack_nibbles(q)
+    zq = np.tile(np.arange(16, dtype=np.uint8)[:, None], (1, kb))
+    zp = synth.pack_nibbles(zq)
+    rng = np.random.default_rng(5)
+    s = rng.uniform(1e-4, 3.0, size=(n, kb)).astype(np.float32)
+    s.view(np.uint32)[:, ::2] |= 0x7FF                      # low mantissa bits set: products must round once
+    want = port.dequantize_nk(b, s, zp, n, kb * bs, bs)
+    bb, sb, zb, out = ep.upload(b), ep.upload(s), ep.upload(zp), ep.allocate(n * kb * bs * 4)
+    ep.dequantize(bb, sb, E.F32, zb, n, kb * bs, bs, out)
+    got = ep.download(out, (n, kb * bs), np.float32)
+    for buf in (bb, sb, zb, out):
+        ep.deallocate(buf)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+# ---------------------------------------------------------------------------------------------
+# known answers held by the reference's own tests
+# ---------------------------------------------------------------------------------------------
+def test_low_nibble_before_high_nibble(ep):
+    """matmul_nbits.rs:18702-18722: packed[0]=0xe1, A=[1,10,0...] -> (1-8)*1 + (14-8)*10 = 53."""
+    k = 16
+    a = np.zeros((1, k), np.float32)
+    a[0, 0], a[0, 1] = 1.0, 10.0
+    b = np.full((1, 1, 8), 0x88, np.uint8)
+    b[0, 0, 0] = 0xE1
+    y, _ = run_op(ep, a, E.F32, b, np.ones((1, 1), np.float32), E.F32, None, 1, k, 16)
+    assert y.tolist() == [[53.0]]
+
+
+def test_accuracy_envelope_against_f64(ep, port):
+    """matmul_nbits.rs:10986-11068: level 0 error < 1e-5, level 4 error inside [1e-4, 1e-2)."""
+    k, n, bs, weights, act = helpers.envelope_fixture()
+    b, s, zp, _ = helpers.quantize_blockwise(weights, bs, True)
+    want = port.matmul_f64(act, b, s, zp, n, k, bs)
+    assert np.abs(want).max() > 1.0
+    y0, _ = run_op(ep, act, E.F32, b, s, E.F32, zp, n, k, bs, accuracy_level=0)
+    y4, _ = run_op(ep, act, E.F32, b, s, E.F32, zp, n, k, bs, accuracy_level=4)
+    exact, reduced = helpers.max_rel_to_peak(y0, want), helpers.max_rel_to_peak(y4, want)
+    assert exact < 1e-5
+    assert reduced > 10 * exact
+    assert 1e-4 <= reduced < 1e-2
+
+
+# ---------------------------------------------------------------------------------------------
+# f32 activations (generic kernel): rel-L2 <= 1e-5
+# ---------------------------------------------------------------------------------------------
+def test_config1_qwen_mlp_shape_f32(ep, port, ref):
+    m, k, n, bs = 1, 896, 4864, 32
+    b, s, _ = synth.make_weights(n, k, bs, 1, zero_points=False, scale_lo=0.005, scale_hi=0.02, scale_dtype=E.F32)
+    a = synth.make_activation(m, k, 1, E.F32, dist="uniform")
+    y, variant = run_op(ep, a, E.F32, b, s, E.F32, None, n, k, bs)
+    assert variant == "gemv_generic_f32"
+    want = port.matmul_f64(a, b, s, None, n, k, bs)
+    assert helpers.rel_l2(y, want) <= TOL_F32
+    y_ref = ref.matmul(a, b, s, None, n, k, bs, ref.COMP_FP32)
+    assert helpers.rel_l2(y, y_ref) <= TOL_F32
+
+
+@pytest.mark.parametrize("m", [1, 5])
+@pytest.mark.parametrize("bs", [32, 64, 128])
+@pytest.mark.parametrize("asym", [False, True])
+def test_sqnbit_grid_f32(ep, port, ref, m, bs, asym):
+    """mlas-sys/src/lib.rs:3268-3285 grid: n=96, k=256."""
+    n, k = 96, 256
+    w, a, bias = helpers.sqnbit_fixture(m, n, k)
+    b, s, zp, deq = helpers.quantize_blockwise(w, bs, asym)
+    y, _ = run_op(ep, a, E.F32, b, s, E.F32, zp, n, k, bs, bias=bias)
+    want = port.matmul_f64(a, b, s, zp, n, k, bs, bias=bias)
+    assert helpers.rel_l2(y, want) <= TOL_F32
+    y_ref = ref.matmul(a, b, s, zp, n, k, bs, ref.COMP_FP32, bias=bias)
+    assert helpers.rel_l2(y, y_ref) <= TOL_F32
+    assert np.abs(y - port.matmul_dequant_f32(a, deq, bias)).max() <= 2e-2       # the reference test's own tolerance
+
+
+@pytest.mark.parametrize("k,bs", [(40, 16), (100, 32), (72, 64), (130, 128)])
+def test_ragged_k_f32(ep, port, k, bs):
+    """K not a multiple of the block size (partial last block) and of 8."""
+    n, m = 37, 3
+    b, s, zp = synth.make_weights(n, k, bs, 3, zero_points=True, scale_lo=0.01, scale_hi=0.05, scale_dtype=E.F32)
+    a = synth.make_activation(m, k, 3, E.F32)
+    y, _ = run_op(ep, a, E.F32, b, s, E.F32, zp, n, k, bs)
+    assert helpers.rel_l2(y, port.matmul_f64(a, b, s, zp, n, k, bs)) <= TOL_F32
+
+
+# ---------------------------------------------------------------------------------------------
+# decode path (f16 / bf16 activations, M <= 16)
+# ---------------------------------------------------------------------------------------------
+DECODE_CASES = [
+    # a_dt, s_dt, bs, zp, m, n, k
+    (E.BF16, E.BF16, 128, True, 1, 512, 3584),
+    (E.BF16, E.BF16, 128, True, 4, 500, 3584),
+    (E.BF16, E.BF16, 128, True, 8, 96, 1024),
+    (E.BF16, E.BF16, 128, True, 16, 1000, 2048),
+    (E.BF16, E.F32, 128, False, 3, 64, 512),
+    (E.F16, E.F16, 32, True, 1, 896, 896),
+    (E.F16, E.F16, 32, True, 1, 128, 896),
+    (E.F16, E.F16, 32, False, 7, 130, 4864),
+    (E.F16, E.F16, 64, True, 2, 257, 1024),
+    (E.BF16, E.BF16, 64, True, 16, 48, 8192),
+    (E.F16, E.F32, 256, True, 5, 80, 1536),
+    (E.BF16, E.BF16, 256, False, 1, 33, 768),
+    (E.F16, E.F16, 32, True, 9, 17, 72),        # K = 72: multiple of 8, not of the block size
+    (E.BF16, E.BF16, 128, True, 2, 20, 200),    # partial last block
+    (E.F16, E.F16, 64, True, 1, 1, 64),
+]
+
+
+@pytest.mark.parametrize("a_dt,s_dt,bs,zero_points,m,n,k", DECODE_CASES)
+def test_decode_matches_oracle(ep, port, a_dt, s_dt, bs, zero_points, m, n, k):
+    b, s, zp = synth.make_weights(n, k, bs, 100 + n + k, zero_points=zero_points, scale_lo=0.002, scale_hi=0.01, scale_dtype=s_dt)
+    a = synth.make_activation(m, k, n, a_dt)
+    bias = synth.to_dtype(np.random.default_rng(n).standard_normal(n).astype(np.float32), a_dt)
+    want64 = oracle_f64(port, a, a_dt, b, s, s_dt, zp, n, k, bs, bias, a_dt)
+
+    # f32 output: the arithmetic itself, before any narrowing
+    y32, variant = run_op(ep, a, a_dt, b, s, s_dt, zp, n, k, bs, bias=bias, bias_dtype=a_dt, y_dtype=E.F32)
+    assert variant == "decode_mfma_splitk"
+    # The kernel carries each weight as (2^10 + q) in f16 or (2^7 + q) in bf16 and cancels the offset inside the
+    # f32 accumulator, which costs 10 (7) of its 24 bits: a few 1e-5 on outputs that themselves cancel.
+    assert helpers.rel_l2(y32, want64) <= 1e-4
+
+    # output in the activation dtype, against the oracle's whole-operator result
+    y, _ = run_op(ep, a, a_dt, b, s, s_dt, zp, n, k, bs, bias=bias, bias_dtype=a_dt)
+    want = port.matmul_nbits(a, a_dt, b, s, s_dt, zp, bias, a_dt, a_dt, m, n, k, bs)
+    assert helpers.rel_l2(synth.to_f32(y, a_dt), synth.to_f32(want, a_dt)) <= TOL_HALF
+    assert helpers.rel_l2(synth.to_f32(y, a_dt), want64) <= TOL_HALF
+
+    # dtype contract (matmul_nbits.rs:17197-17281): compute in f32, narrow once
+    assert np.array_equal(np.asarray(y).view(np.uint16), np.asarray(port.narrow(y32, a_dt)).view(np.uint16))
+
+
+@pytest.mark.parametrize("waves,cg", [(1, 1), (3, 2), (16, 4), (7, 1)])
+def test_decode_launch_shapes_agree(port, waves, cg):
+    """Every split of the work over waves and column groups gives the same answer (to f32 rounding)."""
+    provider = E.RocmExecutionProvider(0, {"decode_waves": waves, "decode_col_groups": cg})
+    try:
+        a_dt, bs, m, n, k = E.BF16, 128, 6, 200, 3584
+        b, s, zp = synth.make_weights(n, k, bs, 77, zero_points=True, scale_lo=0.002, scale_hi=0.01, scale_dtype=a_dt)
+        a = synth.make_activation(m, k, 77, a_dt)
+        y32, variant = run_op(provider, a, a_dt, b, s, a_dt, zp, n, k, bs, y_dtype=E.F32)
+        assert variant == "decode_mfma_splitk"
+        assert helpers.rel_l2(y32, oracle_f64(port, a, a_dt, b, s, a_dt, zp, n, k, bs)) <= 2e-5
+    finally:
+        provider.shutdown()
+
+
+def test_decode_is_deterministic(ep):
+    a_dt, bs, m, n, k = E.F16, 32, 4, 300, 4864
+    b, s, zp = synth.make_weights(n, k, bs, 9, zero_points=True, scale_lo=0.002, scale_hi=0.01, scale_dtype=a_dt)
+    a = synth.make_activation(m, k, 9, a_dt)
+    y1, _ = run_op(ep, a, a_dt, b, s, a_dt, zp, n, k, bs)
+    y2, _ = run_op(ep, a, a_dt, b, s, a_dt, zp, n, k, bs)
+    assert np.array_equal(y1.view(np.uint16), y2.view(np.uint16))
+
+
+def test_linearity_at_full_7b_shape(ep):
+    """Size-independent property at a full 7B decode shape: Y(A1 + A2) = Y(A1) + Y(A2) when the sum is exact."""
+    a_dt, bs, n, k = E.BF16, 128, 4608, 3584
+    b, s, zp = synth.make_weights(n, k, bs, 21, zero_points=True, scale_lo=0.002, scale_hi=0.01, scale_dtype=a_dt)
+    rng = np.random.default_rng(21)
+    a1 = rng.integers(-8, 9, size=(1, k)).astype(np.float32)          # small integers: sums stay exact in bf16
+    a2 = rng.integers(-8, 9, size=(1, k)).astype(np.float32)
+    ys = []
+    for a in (a1, a2, a1 + a2):
+        y, _ = run_op(ep, synth.to_dtype(a, a_dt), a_dt, b, s, a_dt, zp, n, k, bs, y_dtype=E.F32)
+        ys.append(y.astype(np.float64))
+    assert helpers.rel_l2(ys[0] + ys[1], ys[2]) <= 1e-5
+
+
+# ---------------------------------------------------------------------------------------------
+# accuracy_level = 4
+# ---------------------------------------------------------------------------------------------
+def _tie_heavy_activation(m, k, bs, seed, dtype):
+    """N(0,1) rows plus blocks built to hit exact .5 ties, all-zero blocks and +-max codes."""
+    rng = np.random.default_rng(seed)
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    blocks = k // bs
+    if blocks >= 3:
+        a[0, 0:bs] = 0.0                                              # all-zero block: scale 0, codes 0
+        a[0, bs:2 * bs] = (rng.integers(-253, 254, size=bs) * 0.5).astype(np.float32)
+        a[0, bs] = 127.0                                              # max = 127 -> inv = 1 -> halves are exact ties
+        a[0, bs + 1] = -127.0
+        a[0, 2 * bs:3 * bs] = np.float32(3.0)                         # every element is the maximum
+    return synth.to_dtype(a, dtype)
+
+
+@pytest.mark.parametrize("a_dt", [E.F32, E.F16, E.BF16])
+@pytest.mark.parametrize("bs", [16, 32, 64, 128])
+@pytest.mark.parametrize("rounding", [oracle.ROUND_HALF_EVEN, oracle.ROUND_HALF_AWAY])
+def test_quantize_a_bit_exact(ep, port, ref, a_dt, bs, rounding):
+    m, k = 5, 4 * bs + (bs // 2)
+    a = _tie_heavy_activation(m, k, bs, 40 + bs, a_dt)
+    af = synth.to_f32(a, a_dt)
+    kb = -(-k // bs)
+    want_q, want_s = port.quantize_a(af, k, bs, rounding)
+    ab, qb, sb = ep.upload(a), ep.allocate(m * kb * bs), ep.allocate(m * kb * 4)
+    ep.quantize_a(ab, a_dt, m, k, bs, rounding, qb, sb)
+    got_q = ep.download(qb, (m, kb * bs), np.int8)
+    got_s = ep.download(sb, (m, kb), np.float32)
+    for buf in (ab, qb, sb):
+        ep.deallocate(buf)
+    assert np.array_equal(got_q, want_q)
+    assert np.array_equal(got_s.view(np.uint32), want_s.view(np.uint32))
+    if rounding == oracle.ROUND_HALF_EVEN:                            # the reference's compiled MLAS quantizer
+        r = ref.quantize_a(af, k, bs)
+        assert r is not None
+        assert np.array_equal(got_q, r[0]) and np.array_equal(got_s.view(np.uint32), r[1].view(np.uint32))
+    assert (want_q != port.quantize_a(af, k, bs, 1 - rounding)[0]).any()   # the fixture does separate the two rules
+
+
+@pytest.mark.parametrize("bs,zero_points", [(16, True), (32, False), (64, True), (128, True)])
+def test_block_accumulators_bit_exact(ep, port, bs, zero_points):
+    m, n, k = 6, 50, 5 * bs
+    b, _, zp = synth.make_weights(n, k, bs, 60 + bs, zero_points=zero_points, scale_lo=0.01, scale_hi=0.02, scale_dtype=E.F32)
+    a = synth.make_activation(m, k, 60, E.F32)
+    qa, _ = port.quantize_a(a, k, bs, oracle.ROUND_HALF_EVEN)
+    want = port.block_acc_i32(qa, b, zp, n, k, bs)
+    kb = k // bs
+    qb, bb = ep.upload(qa), ep.upload(b)
+    zb = ep.upload(zp) if zp is not None else None
+    acc = ep.allocate(m * n * kb * 4)
+    ep.block_acc(qb, bb, zb, m, n, k, bs, acc)
+    got = ep.download(acc, (m, n, kb), np.int32)
+    for buf in (qb, bb, zb, acc):
+        if buf is not None:
+            ep.deallocate(buf)
+    assert np.array_equal(got, want)
+    # independent integer check of the oracle itself on the same operands
+    q = synth.unpack_nibbles(b.reshape(n, kb, bs // 2), bs).astype(np.int64)
+    z = synth.unpack_nibbles(zp, kb).astype(np.int64) if zp is not None else np.full((n, kb), 8, np.int64)
+    brute = np.einsum("mbk,nbk->mnb", qa.reshape(m, kb, bs).astype(np.int64), q - z[:, :, None])
+    assert np.array_equal(want.astype(np.int64), brute)
+
+
+ACC4_CASES = [
+    (E.F16, 64, True, 1, 160, 1024),
+    (E.F16, 64, True, 5, 96, 512),
+    (E.F32, 32, False, 1, 128, 1024),
+    (E.BF16, 128, True, 3, 77, 1024),
+    (E.F16, 32, True, 20, 64, 256),
+    (E.F32, 16, True, 2, 40, 80),
+]
+
+
+@pytest.mark.parametrize("a_dt,bs,zero_points,m,n,k", ACC4_CASES)
+@pytest.mark.parametrize("rounding", ["mlas", "native"])
+def test_acc4_outputs(port, ref, a_dt, bs, zero_points, m, n, k, rounding):
+    provider = E.RocmExecutionProvider(0, {"acc4_rounding": rounding})
+    try:
+        b, s, zp = synth.make_weights(n, k, bs, 80 + n, zero_points=zero_points, scale_lo=0.002, scale_hi=0.01, scale_dtype=a_dt)
+        a = synth.make_activation(m, k, 80, a_dt)
+        bias = synth.to_dtype(np.linspace(-1, 1, n).astype(np.float32), a_dt)
+        y32, variant = run_op(provider, a, a_dt, b, s, a_dt, zp, n, k, bs, accuracy_level=4, bias=bias, bias_dtype=a_dt, y_dtype=E.F32)
+        assert variant.startswith("acc4")
+        rnd = oracle.ROUND_HALF_EVEN if rounding == "mlas" else oracle.ROUND_HALF_AWAY
+        af, sf, bf = synth.to_f32(a, a_dt), synth.to_f32(s, a_dt), synth.to_f32(bias, a_dt)
+        want = port.matmul_acc4_f32(af, b, sf, zp, n, k, bs, rnd, bias=bf)
+        assert helpers.rel_l2(y32, want) <= TOL_F32                   # same codes, same integers: only f32 summation order differs
+        if rounding == "mlas":
+            y_ref = ref.matmul(af, b, sf, zp, n, k, bs, ref.COMP_INT8, bias=bf)
+            if y_ref is not None:
+                assert helpers.rel_l2(y32, y_ref) <= TOL_F32
+        y, _ = run_op(provider, a, a_dt, b, s, a_dt, zp, n, k, bs, accuracy_level=4, bias=bias, bias_dtype=a_dt)
+        assert np.array_equal(np.asarray(y).view(NPDT[a_dt] if a_dt != E.F32 else np.float32), np.asarray(port.narrow(y32, a_dt)))
+    finally:
+        provider.shutdown()
+
+
+def test_acc4_with_caller_workspace(ep, port):
+    a_dt, bs, m, n, k = E.F16, 64, 4, 64, 512
+    b, s, zp = synth.make_weights(n, k, bs, 91, zero_points=True, scale_lo=0.002, scale_hi=0.01, scale_dtype=a_dt)
+    a = synth.make_activation(m, k, 91, a_dt)
+    ops = E.DeviceOperands(ep, b, s, a_dt, zp, n, k, bs, accuracy_level=4)
+    need, align = ops.kernel.workspace_requirement([((m, k), a_dt)])
+    assert need > 0 and align == 256
+    ws, ab, yb = ep.allocate(need), ep.upload(a), ep.allocate(m * n * 2)
+    ops.kernel.execute(ops.views(ab, a_dt, m), [E.TensorView(yb.ptr, a_dt, (m, n))], workspace=ws)
+    y = ep.download(yb, (m, n), np.float16)
+    want = port.matmul_nbits(a, a_dt, b, s, a_dt, zp, None, E.F32, a_dt, m, n, k, bs, accuracy_level=4, rounding=oracle.ROUND_HALF_EVEN)
+    assert helpers.rel_l2(y.astype(np.float32), want.astype(np.float32)) <= TOL_HALF
+    for buf in (ws, ab, yb):
+        ep.deallocate(buf)
+    ops.free()
+
+
+# ---------------------------------------------------------------------------------------------
+# interface behaviour through the C ABI
+# ---------------------------------------------------------------------------------------------
+def test_provider_identity(ep):
+    assert ep.name() == "RocmExecutionProvider"
+    assert ep.device_type() == 2 and ep.device_id() == 0 and ep.memory_vendor_id() == 0x1002
+    info = ep.device_info()
+    assert info["arch"].startswith("gfx950") and info["compute_units"] >= 200
+
+
+def test_execute_validation_messages(ep):
+    """Same checks, same words as the reference's Kernel::execute (matmul_nbits.rs:1490-1572)."""
+    n, k, bs = 8, 64, 32
+    b, s, zp = synth.make_weights(n, k, bs, 1, zero_points=True, scale_lo=0.01, scale_hi=0.02, scale_dtype=E.F32)
+    ops = E.DeviceOperands(ep, b, s, E.F32, zp, n, k, bs)
+    ab, yb = ep.upload(np.zeros((2, k), np.float32)), ep.allocate(2 * n * 4)
+    good_in = ops.views(ab, E.F32, 2)
+    good_out = [E.TensorView(yb.ptr, E.F32, (2, n))]
+
+    def fails(inputs, outputs, text):
+        with pytest.raises(E.EpError) as e:
+            ops.kernel.execute(inputs, outputs)
+        assert text in str(e.value), str(e.value)
+
+    fails(good_in[:2], good_out, "MatMulNBits: expected 3..=6 inputs, got 2")
+    bad = list(good_in)
+    bad[0] = E.TensorView(ab.ptr, E.F32, (2, k - 1))
+    fails(bad, good_out, f"MatMulNBits: A must have rank >= 1 and last dimension K={k}, got [2, {k - 1}]")
+    bad = list(good_in)
+    bad[1] = E.TensorView(ops.b.ptr, E.I8, (n, 2, 16))
+    fails(bad, good_out, "MatMulNBits: B must have dtype Uint8, got Int8")
+    bad = list(good_in)
+    bad[1] = E.TensorView(ops.b.ptr, E.U8, (n, 2, 15))
+    fails(bad, good_out, f"MatMulNBits: B must have shape [{n}, 2, 16], got [{n}, 2, 15]")
+    bad = list(good_in)
+    bad[2] = E.TensorView(ops.scales.ptr, E.F32, (n, 3))
+    fails(bad, good_out, f"MatMulNBits: scales must have shape [{n * 2}] or [{n}, 2], got [{n}, 3]")
+    fails(good_in, [E.TensorView(yb.ptr, E.F32, (2, n + 1))], f"MatMulNBits: Y must have shape [2, {n}], got [2, {n + 1}]")
+    fails(good_in, [E.TensorView(yb.ptr, E.I32, (2, n))], "MatMulNBits: Y must have dtype Float32, Float16, or BFloat16, got Int32")
+    bad = list(good_in)
+    bad[0] = E.TensorView(ab.ptr, E.F32, (2, k), strides=(2 * k, 1))
+    fails(bad, good_out, "MatMulNBits: A must be contiguous on the ROCm execution provider")
+    bad = list(good_in) + [E.TensorView(ab.ptr, E.I32, (k,))]
+    fails(bad, good_out, "g_idx is not supported on the ROCm execution provider")
+    bad = list(good_in)
+    bad[0] = E.TensorView(ab.ptr, E.F32, (2, k), device_type=0)
+    fails(bad, good_out, "must live on ROCm device 0")
+
+    # flat scales / zero points are accepted, as in the reference
+    flat = list(good_in)
+    flat[2] = E.TensorView(ops.scales.ptr, E.F32, (n * 2,))
+    flat[3] = E.TensorView(ops.zp.ptr, E.U8, (n * 1,))
+    ops.kernel.execute(flat, good_out)
+    # rank-3 A: Y = A.shape[:-1] + [N]
+    ops.kernel.execute([E.TensorView(ab.ptr, E.F32, (2, 1, k))] + good_in[1:], [E.TensorView(yb.ptr, E.F32, (2, 1, n))])
+    # empty A is a no-op
+    ops.kernel.execute([E.TensorView(ab.ptr, E.F32, (0, k))] + good_in[1:], [E.TensorView(yb.ptr, E.F32, (0, n))])
+    ep.sync()
+    for buf in (ab, yb):
+        ep.deallocate(buf)
+    ops.free()
+
+
+def test_kernel_vtable_execute(ep, port):
+    """The nxrt kernel vtable (raw pointers only) runs the same kernel with the create-time shapes."""
+    import ctypes as C
+    a_dt, bs, m, n, k = E.F16, 32, 2, 64, 256
+    b, s, zp = synth.make_weights(n, k, bs, 33, zero_points=True, scale_lo=0.002, scale_hi=0.01, scale_dtype=a_dt)
+    a = synth.make_activation(m, k, 33, a_dt)
+    ops = E.DeviceOperands(ep, b, s, a_dt, zp, n, k, bs, rows=m, a_dtype=a_dt)
+    assert ops.kernel.estimated_flops() == 2 * m * n * k
+    ab, yb = ep.upload(a), ep.allocate(m * n * 2)
+
+    class KernelVtable(C.Structure):
+        _fields_ = [("struct_size", C.c_uint32), ("_pad", C.c_uint32),
+                    ("execute", C.CFUNCTYPE(E.NxrtStatus, C.c_void_p, C.POINTER(C.c_void_p), C.c_uint32, C.POINTER(C.c_void_p), C.c_uint32)),
+                    ("release", C.CFUNCTYPE(None, C.c_void_p)), ("ctx", C.c_void_p)]
+
+    vt = C.c_void_p()
+    ep.lib.nxrt_rocm_matmul_nbits_as_vtable(ops.kernel.handle, C.byref(vt)).check()
+    table = C.cast(vt, C.POINTER(KernelVtable)).contents
+    assert table.struct_size == C.sizeof(KernelVtable)
+    ins = (C.c_void_p * 4)(ab.ptr, ops.b.ptr, ops.scales.ptr, ops.zp.ptr)
+    outs = (C.c_void_p * 1)(yb.ptr)
+    table.execute(table.ctx, ins, 4, outs, 1).check()
+    y = ep.download(yb, (m, n), np.float16)
+    want = port.matmul_nbits(a, a_dt, b, s, a_dt, zp, None, E.F32, a_dt, m, n, k, bs)
+    assert helpers.rel_l2(y.astype(np.float32), want.astype(np.float32)) <= TOL_HALF
+    for buf in (ab, yb):
+        ep.deallocate(buf)
+    ops.free()
+
+
+def test_launch_counter_proves_native_path(ep):
+    before = ep.kernel_launch_count()
+    test_low_nibble_before_high_nibble(ep)
+    assert ep.kernel_launch_count() == before + 1
