@@ -1,0 +1,362 @@
+#!/usr/bin/env python3
+"""Benchmark of the int4 MatMulNBits hot path on one MI355X.
+
+A step is one decode step's worth of MatMulNBits calls for a Qwen2.5-7B-shaped stack (28 layers of
+qkv 3584->4608, o 3584->3584, gate/up 3584->37888, down 18944->3584, plus lm_head 3584->152064):
+bf16 activations, block_size 128, packed 4-bit zero points, M rows (default 1). Every layer has its
+own weight buffers (3.7 GB in all), so each step streams its weights from HBM. The calls of one step
+are recorded once into a HIP graph through the provider's C ABI and replayed; the timed region is K
+replays between two HIP events on the provider's stream.
+
+Prints one JSON line: value = algorithmic GB/s of the whole step, plus `roofline` for the decode
+kernel on the gate/up shape, `cpu_baseline` (the reference's MLAS path on this host's cores), and
+`sweep` / `prefill` tables.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+from onnx_genai_amd import ep as E  # noqa: E402
+from onnx_genai_amd import synth  # noqa: E402
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA, published
+MFMA_I8_PEAK_TOPS = 5000.0
+
+LAYERS = 28
+HIDDEN, INTER, VOCAB = 3584, 18944, 152064
+LAYER_SHAPES = [("qkv", HIDDEN, 4608), ("o", HIDDEN, HIDDEN), ("gate_up", HIDDEN, 2 * INTER), ("down", INTER, HIDDEN)]
+LM_HEAD = ("lm_head", HIDDEN, VOCAB)
+BS = 128
+A_DT = E.BF16
+
+
+def _device_random_weights(ep, n, k, bs, seed, scale_lo, scale_hi, dtype, zero_points=True, reuse=None):
+    """Packed nibbles, scales and zero points for one node, resident on the GPU. Random bytes ARE uniform
+    nibbles; to keep set-up short the byte pattern of large tensors is generated once per shape and
+    shifted per layer (the values do not affect timing, only the buffers must be distinct)."""
+    kb = -(-k // bs)
+    rng = np.random.default_rng(seed)
+    if reuse is None:
+        b = rng.integers(0, 256, size=(n, kb, bs // 2), dtype=np.uint8)
+    else:
+        b = np.roll(reuse, seed % 251 + 1, axis=0)
+    scales = synth.to_dtype(rng.uniform(scale_lo, scale_hi, size=(n, kb)).astype(np.float32), dtype)
+    zp = rng.integers(0, 256, size=(n, (kb + 1) // 2), dtype=np.uint8) if zero_points else None
+    return b, scales, zp
+
+
+class Node:
+    def __init__(self, ep, name, k, n, bs, seed, a_dt, m, *, zero_points=True, scale_range=(0.002, 0.01), accuracy_level=0, reuse=None):
+        self.name, self.k, self.n, self.bs, self.m, self.a_dt = name, k, n, bs, m, a_dt
+        b, s, zp = _device_random_weights(ep, n, k, bs, seed, scale_range[0], scale_range[1], a_dt, zero_points, reuse)
+        self.host_b = b
+        self.ops = E.DeviceOperands(ep, b, s, a_dt, zp, n, k, bs, accuracy_level=accuracy_level, rows=m, a_dtype=a_dt)
+        self.y = ep.allocate(m * n * 2)
+        self.bytes = synth.algorithmic_bytes(m, n, k, bs, a_dtype=a_dt, scale_dtype=a_dt, zero_points=zero_points)
+        self.flops = synth.matmul_flops(m, n, k)
+        self.workspace = None
+        if accuracy_level == 4:
+            need, _ = self.ops.kernel.workspace_requirement([((m, k), a_dt)])
+            self.workspace = ep.allocate(need)
+
+    def run(self, a_buf):
+        out = [E.TensorView(self.y.ptr, self.a_dt, (self.m, self.n), device_index=self.ops.ep.device_index)]
+        self.ops.kernel.execute(self.ops.views(a_buf, self.a_dt, self.m), out, workspace=self.workspace)
+
+    def free(self, ep):
+        ep.deallocate(self.y)
+        if self.workspace:
+            ep.deallocate(self.workspace)
+        self.ops.free()
+
+
+def time_graph(ep, graph, reps, warmup):
+    for _ in range(warmup):
+        graph.replay()
+    ep.sync()
+    start, stop = ep.event(), ep.event()
+    start.record()
+    for _ in range(reps):
+        graph.replay()
+    stop.record()
+    ms = start.elapsed_ms(stop)
+    return ms / reps
+
+
+def capture(ep, fn):
+    ep.sync()
+    ep.capture_begin()
+    try:
+        fn()
+    finally:
+        graph = ep.capture_end()
+    return graph
+
+
+def build_decode_stack(ep, m, layers):
+    a_bufs = {k: ep.upload(synth.make_activation(m, k, 5, A_DT)) for k in (HIDDEN, INTER)}
+    nodes, reuse = [], {}
+    for layer in range(layers):
+        for name, k, n in LAYER_SHAPES:
+            node = Node(ep, f"{name}.{layer}", k, n, BS, 1000 * layer + len(nodes), A_DT, m, reuse=reuse.get(name))
+            reuse.setdefault(name, node.host_b)
+            node.host_b = None
+            nodes.append(node)
+    nodes.append(Node(ep, LM_HEAD[0], LM_HEAD[1], LM_HEAD[2], BS, 99, A_DT, m))
+    nodes[-1].host_b = None
+    return nodes, a_bufs
+
+
+def cpu_baseline(seconds_budget=20.0, threads=None):
+    """The reference's CPU path (vendored MLAS through its plain-C shim, oracle/_ref) on this host, on a bounded
+    sample of the workload: the gate/up projection (3584 -> 37888), bf16 activations widened to f32 before and
+    the output narrowed after each call inside the timed region, weights packed once outside it."""
+    import oracle
+    from concurrent.futures import ThreadPoolExecutor
+    if not oracle.Ref.available():
+        return None
+    ref, port = oracle.Ref(), oracle.Port()
+    threads = threads or min(16, os.cpu_count() or 1)
+    k, n, m = HIDDEN, 2 * INTER, 1
+    copies = 3                                         # 3 x 68 MB of packed weights: larger than the last-level cache
+    shard = -(-n // threads)
+    shard = (shard + 15) // 16 * 16
+    packs = []
+    for c in range(copies):
+        b, s, zp = synth.make_weights(n, k, BS, 300 + c, zero_points=True, scale_lo=0.002, scale_hi=0.01, scale_dtype=A_DT)
+        sf = synth.to_f32(s, A_DT)
+        shards = []
+        for lo in range(0, n, shard):
+            hi = min(lo + shard, n)
+            pk = ref.pack(b[lo:hi], sf[lo:hi], zp[lo:hi], hi - lo, k, BS, ref.COMP_FP32)
+            if pk is None:
+                return None
+            pk["ws"] = ref.workspace(pk, m)
+            pk["lo"], pk["hi"] = lo, hi
+            shards.append(pk)
+        whole = ref.pack(b, sf, zp, n, k, BS, ref.COMP_FP32)
+        whole["ws"] = ref.workspace(whole, m)
+        packs.append((shards, whole))
+    a16 = synth.make_activation(m, k, 5, A_DT)
+    nbytes = synth.algorithmic_bytes(m, n, k, BS, a_dtype=A_DT, scale_dtype=A_DT, zero_points=True)
+    out = np.empty((m, n), np.float32)
+
+    def one_thread(i):
+        _, whole = packs[i % copies]
+        a = port.widen(a16, A_DT)
+        ref.gemm(whole, a, out=out, workspace=whole["ws"])
+        return port.narrow(out, A_DT)
+
+    pool = ThreadPoolExecutor(max_workers=threads)
+    outs = [np.empty((m, pk["hi"] - pk["lo"]), np.float32) for pk in packs[0][0]]
+
+    def all_threads(i):
+        shards, _ = packs[i % copies]
+        a = port.widen(a16, A_DT)
+        list(pool.map(lambda t: ref.gemm(shards[t], a, out=outs[t], workspace=shards[t]["ws"]), range(len(shards))))
+        return port.narrow(np.concatenate(outs, axis=1), A_DT)
+
+    result = {}
+    for label, fn in (("1", one_thread), (str(threads), all_threads)):
+        for i in range(3):
+            fn(i)
+        t0, calls = time.perf_counter(), 0
+        while time.perf_counter() - t0 < seconds_budget / 2 and calls < 400:
+            fn(calls)
+            calls += 1
+        dt = (time.perf_counter() - t0) / calls
+        result[label] = {"gbs": nbytes / dt / 1e9, "us": dt * 1e6, "calls": calls}
+    pool.shutdown()
+    cpu_model = ""
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    cpu_model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    best = result[str(threads)]
+    return {"value": round(best["gbs"], 2), "unit": "GB/s", "cores": threads, "kind": "reference",
+            "sample": f"MLAS SQNBit CompFp32 (oracle/_ref), gate_up 3584->37888, M=1, bf16 in/out widened+narrowed in the timed region, "
+                      f"block 128 with zero points, {best['calls']} calls rotating over {copies} weight copies, N-sharded over {threads} threads",
+            "us_per_call": round(best["us"], 1), "single_thread_gbs": round(result["1"]["gbs"], 2),
+            "dispatch": ref.dispatch_id(), "cpu": cpu_model}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--m", type=int, default=1, help="rows of the decode batch (1..16)")
+    ap.add_argument("--layers", type=int, default=LAYERS)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-sweep", action="store_true", help="skip the per-shape sweep and the prefill table")
+    ap.add_argument("--cpu-seconds", type=float, default=20.0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only (no collectives exist on the MatMulNBits path); use --gpus 1")
+
+    ep = E.RocmExecutionProvider(0)
+    info = ep.device_info()
+    nodes, a_bufs = build_decode_stack(ep, args.m, args.layers)
+    step_bytes = sum(n.bytes for n in nodes)
+    step_flops = sum(n.flops for n in nodes)
+
+    def one_step():
+        for node in nodes:
+            node.run(a_bufs[node.k])
+
+    one_step()                       # eager once: every kernel resolves its variant and reports errors here
+    ep.sync()
+    variants = sorted({n.ops.kernel.last_variant() for n in nodes})
+    graph = capture(ep, one_step)
+    for _ in range(args.warmup):
+        graph.replay()
+    ep.sync()
+    start, stop = ep.event(), ep.event()
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(args.steps):
+        graph.replay()
+    stop.record()
+    ms_total = start.elapsed_ms(stop)
+    ep.sync()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    ms_per_step = ms_total / args.steps
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+
+    # roofline of the dominant kernel: decode GEMV on the gate/up shape (58% of the step's bytes), one launch
+    # per layer buffer, recorded as a graph of `layers` launches and timed with events on the same stream.
+    gate_up = [n for n in nodes if n.name.startswith("gate_up")]
+    g2 = capture(ep, lambda: [n.run(a_bufs[n.k]) for n in gate_up])
+    ms = time_graph(ep, g2, max(10, args.steps // 2), 3)
+    launch_us = ms * 1e3 / len(gate_up)
+    achieved = gate_up[0].bytes / (launch_us * 1e-6) / 1e9
+    roofline = {"bound": "hbm", "kernel": "decode_mfma_kernel<bf16, block 128> on gate_up 3584->37888, M=%d" % args.m,
+                "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                "bytes_per_launch": gate_up[0].bytes, "us_per_launch": round(launch_us, 2), "traffic": None}
+    g2.release()
+
+    result = {
+        "metric": "int4 MatMulNBits decode GB/s (% HBM peak) + prefill TFLOPS, 7B shapes, 1 GPU",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"Qwen2.5-7B decode-step MatMulNBits sweep (configs[2]): {args.layers} layers x (qkv, o, gate_up, down) + lm_head, "
+                               f"M={args.m}, bf16, block_size 128, zero points; {len(nodes)} calls per step replayed as one HIP graph",
+                   "m": args.m, "calls_per_step": len(nodes), "bytes_per_step": step_bytes, "flops_per_step": step_flops},
+        "hbm_frac": round(value / HBM_PEAK_GBS, 4), "wall_ms_per_step": round(wall_ms / args.steps, 4),
+        "kernel_variants": variants, "device": info, "roofline": roofline,
+    }
+    graph.release()
+
+    if not args.no_sweep:
+        result["sweep"] = sweep(ep, nodes, a_bufs, args)
+    for node in nodes:
+        node.free(ep)
+    for buf in a_bufs.values():
+        ep.deallocate(buf)
+    if not args.no_sweep:
+        result["prefill"] = prefill_table(ep)
+        result["acc4"] = acc4_table(ep)
+    ep.shutdown()
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(args.cpu_seconds)
+    print(json.dumps(result), flush=True)
+
+
+def sweep(ep, nodes, a_bufs, args):
+    """Per-shape decode figures at M in {1, 4, 8, 16}: the launches of one shape across all layer buffers in one graph."""
+    table = []
+    by_shape = {}
+    for n in nodes:
+        by_shape.setdefault(n.name.split(".")[0], []).append(n)
+    for m in (1, 4, 8, 16):
+        a_m = {k: ep.upload(synth.make_activation(m, k, 6, A_DT)) for k in (HIDDEN, INTER)}
+        for shape, group in by_shape.items():
+            group = list(group)
+            if shape == "lm_head":
+                pass
+            saved = [(g.m, g.y) for g in group]
+            ys = []
+            for g in group:
+                g.m = m
+                g.y = ep.allocate(m * g.n * 2)
+                ys.append(g.y)
+            group[0].run(a_m[group[0].k])
+            ep.sync()
+            graph = capture(ep, lambda: [g.run(a_m[g.k]) for g in group])
+            ms = time_graph(ep, graph, 20, 3)
+            graph.release()
+            us = ms * 1e3 / len(group)
+            nbytes = synth.algorithmic_bytes(m, group[0].n, group[0].k, BS, a_dtype=A_DT, scale_dtype=A_DT, zero_points=True)
+            table.append({"shape": shape, "k": group[0].k, "n": group[0].n, "m": m, "us": round(us, 2),
+                          "gbs": round(nbytes / (us * 1e-6) / 1e9, 1), "hbm_frac": round(nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+                          "variant": group[0].ops.kernel.last_variant()})
+            for g, (m0, y0) in zip(group, saved):
+                ep.deallocate(g.y)
+                g.m, g.y = m0, y0
+        for buf in a_m.values():
+            ep.deallocate(buf)
+    return table
+
+
+def prefill_table(ep):
+    """Prefill GEMM at Llama-3-8B MLP shapes (configs[3]): fp16, block 32, no zero points."""
+    table = []
+    for k, n in ((4096, 14336), (14336, 4096)):
+        for m in (512, 2048, 8192):
+            node = Node(ep, "prefill", k, n, 32, 7, E.F16, m, zero_points=False, scale_range=(0.001, 0.01))
+            a = ep.upload(synth.make_activation(m, k, 8, E.F16))
+            node.run(a)
+            ep.sync()
+            variant = node.ops.kernel.last_variant()
+            if not variant.startswith("prefill") and m > 512:      # the catch-all kernel is not a prefill path: one row of the table is enough
+                ep.deallocate(a)
+                node.free(ep)
+                continue
+            reps = 10 if variant.startswith("prefill") else 1
+            graph = capture(ep, lambda: node.run(a))
+            ms = time_graph(ep, graph, reps, 1)
+            graph.release()
+            tflops = node.flops / (ms * 1e-3) / 1e12
+            table.append({"k": k, "n": n, "m": m, "us": round(ms * 1e3, 1), "tflops": round(tflops, 1),
+                          "mfma_frac": round(tflops / MFMA_F16_PEAK_TFLOPS, 4), "variant": variant})
+            ep.deallocate(a)
+            node.free(ep)
+    return table
+
+
+def acc4_table(ep):
+    """accuracy_level=4 at 70B-class shapes (configs[4]): fp16, block 64, zero points; M=1 rows only here."""
+    table = []
+    for k, n in ((8192, 28672), (28672, 8192), (8192, 10240)):
+        for m in (1,):
+            node = Node(ep, "acc4", k, n, 64, 9, E.F16, m, accuracy_level=4)
+            a = ep.upload(synth.make_activation(m, k, 8, E.F16))
+            node.run(a)
+            ep.sync()
+            graph = capture(ep, lambda: node.run(a))
+            ms = time_graph(ep, graph, 20, 2)
+            graph.release()
+            table.append({"k": k, "n": n, "m": m, "us": round(ms * 1e3, 1), "gbs": round(node.bytes / (ms * 1e-3) / 1e9, 1),
+                          "hbm_frac": round(node.bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "variant": node.ops.kernel.last_variant()})
+            ep.deallocate(a)
+            node.free(ep)
+    return table
+
+
+if __name__ == "__main__":
+    main()

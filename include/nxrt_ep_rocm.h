@@ -142,6 +142,17 @@ NxrtStatus nxrt_rocm_ep_event_record(NxrtRocmEp* ep, NxrtRocmEvent* event);
 NxrtStatus nxrt_rocm_ep_event_elapsed_ms(NxrtRocmEp* ep, NxrtRocmEvent* start, NxrtRocmEvent* stop, float* out_ms);
 void nxrt_rocm_ep_event_destroy(NxrtRocmEp* ep, NxrtRocmEvent* event);
 
+/* ---- graph capture (Kernel::capture_support in kernel.rs; the CUDA sibling's capture-safe decode path,
+ * ep-cuda matmul_nbits.rs:11136-11162) ---------------------------------------------------------
+ * Between begin and end, execute calls on this provider are recorded instead of run. Only calls that
+ * allocate nothing may be recorded: accuracy_level 0 always, accuracy_level 4 with a caller workspace.
+ * A recorded graph replays the same launches on the same device pointers. */
+typedef struct NxrtRocmGraph NxrtRocmGraph;
+NxrtStatus nxrt_rocm_ep_capture_begin(NxrtRocmEp* ep);
+NxrtStatus nxrt_rocm_ep_capture_end(NxrtRocmEp* ep, NxrtRocmGraph** out_graph, uint64_t* out_num_nodes);
+NxrtStatus nxrt_rocm_ep_graph_replay(NxrtRocmEp* ep, NxrtRocmGraph* graph);
+void nxrt_rocm_ep_graph_release(NxrtRocmEp* ep, NxrtRocmGraph* graph);
+
 /* Counters a harness reads to prove the provider, not a fallback, did the work
  * (the role of nxrt_ep_compiled_node_count in ep-cuda-plugin/src/lib.rs:345-372). */
 uint64_t nxrt_rocm_ep_kernel_launch_count(const NxrtRocmEp* ep);

@@ -252,6 +252,9 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
         uint8_t* ws = static_cast<uint8_t*>(workspace);
         if (!ws || workspace_bytes < need) {
             if (kn.scratch_bytes < need) {
+                if (kn.ep->capturing)
+                    return make_status(NXRT_INVALID_ARGUMENT, err("accuracy_level=4 under graph capture needs a caller workspace of " + std::to_string(need) +
+                                                                  " bytes (see workspace_requirement); the kernel may not allocate while a capture is open"));
                 if (kn.scratch) {
                     rocm_ffi_stream_sync(stream);
                     rocm_ffi_free(kn.scratch);

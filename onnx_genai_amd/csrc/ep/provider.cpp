@@ -223,6 +223,54 @@ void nxrt_rocm_ep_event_destroy(NxrtRocmEp*, NxrtRocmEvent* event)
     delete event;
 }
 
+NxrtStatus nxrt_rocm_ep_capture_begin(NxrtRocmEp* ep)
+{
+    return fenced([&]() -> NxrtStatus {
+        if (!ep) return make_status(NXRT_INVALID_ARGUMENT, "capture_begin: null provider");
+        NxrtStatus st = ep->bind();
+        if (st.code != NXRT_OK) return st;
+        if (ep->capturing) return make_status(NXRT_INVALID_ARGUMENT, "capture_begin: a capture is already open on this provider");
+        st = hip_status(rocm_ffi_capture_begin(ep->stream), "hipStreamBeginCapture");
+        if (st.code == NXRT_OK) ep->capturing = true;
+        return st;
+    });
+}
+
+NxrtStatus nxrt_rocm_ep_capture_end(NxrtRocmEp* ep, NxrtRocmGraph** out_graph, uint64_t* out_num_nodes)
+{
+    return fenced([&]() -> NxrtStatus {
+        if (!ep || !out_graph) return make_status(NXRT_INVALID_ARGUMENT, "capture_end: null pointer");
+        *out_graph = nullptr;
+        if (!ep->capturing) return make_status(NXRT_INVALID_ARGUMENT, "capture_end: no capture is open on this provider");
+        ep->capturing = false;
+        rocm_graph_exec_t exec = nullptr;
+        size_t nodes = 0;
+        const int err = rocm_ffi_capture_end(ep->stream, &exec, &nodes);
+        if (err != 0) return hip_status(err, "hipStreamEndCapture");
+        auto* g = new NxrtRocmGraph();
+        g->exec = exec;
+        if (out_num_nodes) *out_num_nodes = nodes;
+        *out_graph = g;
+        return ok();
+    });
+}
+
+NxrtStatus nxrt_rocm_ep_graph_replay(NxrtRocmEp* ep, NxrtRocmGraph* graph)
+{
+    return fenced([&]() -> NxrtStatus {
+        if (!ep || !graph) return make_status(NXRT_INVALID_ARGUMENT, "graph_replay: null pointer");
+        return hip_status(rocm_ffi_graph_launch(graph->exec, ep->stream), "hipGraphLaunch");
+    });
+}
+
+void nxrt_rocm_ep_graph_release(NxrtRocmEp* ep, NxrtRocmGraph* graph)
+{
+    if (!graph) return;
+    if (ep && ep->bind().code == NXRT_OK) rocm_ffi_stream_sync(ep->stream);
+    rocm_ffi_graph_destroy(graph->exec);
+    delete graph;
+}
+
 uint64_t nxrt_rocm_ep_kernel_launch_count(const NxrtRocmEp* ep) { return ep ? ep->launches.load() : 0; }
 uint64_t nxrt_rocm_live_provider_count(void) { return g_live_providers.load(); }
 

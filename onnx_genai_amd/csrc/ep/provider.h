@@ -21,11 +21,16 @@ struct NxrtRocmEp {
     std::mutex mu;
     std::unordered_map<void*, size_t> live;       // allocations handed out and not yet returned
     std::atomic<uint64_t> launches{0};
+    bool capturing = false;                       // a stream capture is open: nothing may allocate or synchronise
     NxrtEpVtable vtable;                          // ctx points back at this object
 
     NxrtRocmEp();
     ~NxrtRocmEp();
     NxrtStatus bind() const;                      // make this provider's GPU current on the calling thread
+};
+
+struct NxrtRocmGraph {
+    rocm_graph_exec_t exec = nullptr;
 };
 
 struct NxrtRocmEvent {

@@ -38,6 +38,13 @@ int rocm_ffi_event_sync(rocm_event_t event);
 int rocm_ffi_event_elapsed_ms(rocm_event_t start, rocm_event_t stop, float* ms);
 int rocm_ffi_fill_u32(void* dst, uint32_t value, size_t count, rocm_stream_t stream);
 
+/* Stream capture into an executable HIP graph, and its replay on a stream. */
+typedef void* rocm_graph_exec_t;
+int rocm_ffi_capture_begin(rocm_stream_t stream);
+int rocm_ffi_capture_end(rocm_stream_t stream, rocm_graph_exec_t* exec, size_t* num_nodes);
+int rocm_ffi_graph_launch(rocm_graph_exec_t exec, rocm_stream_t stream);
+int rocm_ffi_graph_destroy(rocm_graph_exec_t exec);
+
 /* Operands of one MatMulNBits call, all device pointers, all contiguous. */
 typedef struct RocmMatMulNBitsArgs {
   const void* a;        /* [M, K] a_dtype */

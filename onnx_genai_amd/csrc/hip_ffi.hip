@@ -87,4 +87,33 @@ int rocm_ffi_fill_u32(void* dst, uint32_t value, size_t count, rocm_stream_t str
     return static_cast<int>(hipGetLastError());
 }
 
+int rocm_ffi_capture_begin(rocm_stream_t stream)
+{
+    return static_cast<int>(hipStreamBeginCapture(static_cast<hipStream_t>(stream), hipStreamCaptureModeThreadLocal));
+}
+
+int rocm_ffi_capture_end(rocm_stream_t stream, rocm_graph_exec_t* exec, size_t* num_nodes)
+{
+    hipGraph_t graph = nullptr;
+    hipError_t e = hipStreamEndCapture(static_cast<hipStream_t>(stream), &graph);
+    if (e != hipSuccess) return static_cast<int>(e);
+    if (num_nodes) {
+        size_t n = 0;
+        (void)hipGraphGetNodes(graph, nullptr, &n);
+        *num_nodes = n;
+    }
+    hipGraphExec_t ge = nullptr;
+    e = hipGraphInstantiate(&ge, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    *exec = ge;
+    return static_cast<int>(e);
+}
+
+int rocm_ffi_graph_launch(rocm_graph_exec_t exec, rocm_stream_t stream)
+{
+    return static_cast<int>(hipGraphLaunch(static_cast<hipGraphExec_t>(exec), static_cast<hipStream_t>(stream)));
+}
+
+int rocm_ffi_graph_destroy(rocm_graph_exec_t exec) { return static_cast<int>(hipGraphExecDestroy(static_cast<hipGraphExec_t>(exec))); }
+
 }  // extern "C"

@@ -131,6 +131,14 @@ def load_library() -> C.CDLL:
     L.nxrt_rocm_ep_event_elapsed_ms.argtypes = [v, v, v, C.POINTER(C.c_float)]
     L.nxrt_rocm_ep_event_destroy.restype = None
     L.nxrt_rocm_ep_event_destroy.argtypes = [v, v]
+    L.nxrt_rocm_ep_capture_begin.restype = S
+    L.nxrt_rocm_ep_capture_begin.argtypes = [v]
+    L.nxrt_rocm_ep_capture_end.restype = S
+    L.nxrt_rocm_ep_capture_end.argtypes = [v, C.POINTER(v), C.POINTER(u64)]
+    L.nxrt_rocm_ep_graph_replay.restype = S
+    L.nxrt_rocm_ep_graph_replay.argtypes = [v, v]
+    L.nxrt_rocm_ep_graph_release.restype = None
+    L.nxrt_rocm_ep_graph_release.argtypes = [v, v]
     L.nxrt_rocm_ep_kernel_launch_count.restype = u64
     L.nxrt_rocm_ep_kernel_launch_count.argtypes = [v]
     L.nxrt_rocm_live_provider_count.restype = u64
@@ -308,6 +316,15 @@ class RocmExecutionProvider:
     def block_acc(self, qa: DeviceBuffer, b: DeviceBuffer, zp: DeviceBuffer | None, m, n, k, bs, acc: DeviceBuffer) -> None:
         self.lib.nxrt_rocm_matmul_nbits_block_acc(self.handle, qa.ptr, b.ptr, zp.ptr if zp else None, m, n, k, bs, acc.ptr).check()
 
+    # -- graph capture ----------------------------------------------------------------------------
+    def capture_begin(self) -> None:
+        self.lib.nxrt_rocm_ep_capture_begin(self.handle).check()
+
+    def capture_end(self) -> "Graph":
+        h, nodes = C.c_void_p(), C.c_uint64()
+        self.lib.nxrt_rocm_ep_capture_end(self.handle, C.byref(h), C.byref(nodes)).check()
+        return Graph(self, h, nodes.value)
+
     # -- timing -----------------------------------------------------------------------------------
     def event(self) -> "Event":
         return Event(self)
@@ -323,6 +340,27 @@ class RocmExecutionProvider:
     def __del__(self):
         try:
             self.shutdown()
+        except Exception:
+            pass
+
+
+class Graph:
+    """A recorded sequence of launches on the provider's stream (a HIP graph)."""
+
+    def __init__(self, ep, handle, num_nodes):
+        self.ep, self.handle, self.num_nodes = ep, handle, num_nodes
+
+    def replay(self) -> None:
+        self.ep.lib.nxrt_rocm_ep_graph_replay(self.ep.handle, self.handle).check()
+
+    def release(self) -> None:
+        if self.handle and self.ep.handle:
+            self.ep.lib.nxrt_rocm_ep_graph_release(self.ep.handle, self.handle)
+        self.handle = None
+
+    def __del__(self):
+        try:
+            self.release()
         except Exception:
             pass
 
