@@ -7,12 +7,19 @@
 // column c: 32 nibbles that never leave registers. Each of its four dwords becomes the eight
 // 16-bit operands one v_mfma_f32_16x16x32 wants from that lane, by OR-ing the nibble under a
 // constant exponent ("magic" value: 1024+q as f16, 128+q as bf16 - both exact). The activation
-// rows are the other MFMA operand (rows beyond M are zero). A second MFMA per dword, whose weight
-// operand is the constant -(magic+zp), removes magic and zero point inside the f32 accumulator, so
-// the accumulator holds sum a*(q-zp) for the block and is scaled once per block:
+// rows are the other MFMA operand (rows beyond M read as zero). A second MFMA per dword, whose
+// weight operand is the constant -(magic+zp), removes magic and zero point inside the f32
+// accumulator, so the accumulator holds sum a*(q-zp) for the block and is scaled once per block:
 //     y += scale[n, block] * acc.
 // For block sizes below 128 the four lane groups first swap dwords (two v_permlane*_swap stages,
 // a 4x4 transpose) so that one MFMA never mixes two blocks.
+//
+// Memory. All global loads are buffer loads with hardware range checking, so ragged edges
+// (columns beyond N, rows beyond M, the end of K) cost no branches: they read zeros. A wave keeps
+// two groups of tiles in registers: while the MFMAs consume one, the loads of the next are in
+// flight. Activations travel with their tile in the most compact form (one 16-byte piece per lane
+// per four rows) and are turned into MFMA operand order through a small wave-private LDS buffer,
+// whose reads are counted separately from global loads and so never drain the prefetch queue.
 #include "common.hiph"
 
 namespace mnb {
@@ -20,6 +27,7 @@ namespace mnb {
 typedef __attribute__((ext_vector_type(8))) _Float16 half8_t;
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float float4_t;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
 
 struct DecodeParams {
     const uint16_t* a;
@@ -31,14 +39,31 @@ struct DecodeParams {
     int64_t m, n, k, kb;
     int64_t row_bytes;      // packed bytes of one column: kb * BS / 2
     int64_t zp_row;         // ceil(kb / 2)
-    int tiles;              // ceil(kb * BS / 128)
-    int tiles_per_wave;     // multiple of max(1, BS / 128)
+    int tiles;              // ceil(K / 128)
+    int tiles_per_wave;     // multiple of the group size
     int bias_dtype, y_dtype;
+    uint32_t nibble_mask;   // 0x000F000F
+    uint32_t magic;         // two 16-bit magic exponents (see Magic<>::pos); passed in so that the compiler keeps it in a register
 };
 
 template <bool BF16> struct Magic;
 template <> struct Magic<false> { static constexpr uint32_t pos = 0x64006400u, neg = 0xE400E400u; };
 template <> struct Magic<true> { static constexpr uint32_t pos = 0x43004300u, neg = 0xC300C300u; };
+
+constexpr uint32_t kOutOfRange = 0x7ffffff0u;   // an offset beyond any range this kernel sets up: the load returns zeros
+constexpr int kRowPitch = 272;                   // bytes between activation rows in LDS: 256 + 16, so 16 rows hit 64 distinct banks
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_srd(const void* base, uint64_t bytes)
+{
+    const uint32_t range = bytes > 0x7fffffffull ? 0x7fffffffu : static_cast<uint32_t>(bytes);
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, static_cast<int>(range), 0x00020000);
+}
+
+__device__ __forceinline__ uint4 load16(__amdgpu_buffer_rsrc_t srd, uint32_t voffset, uint32_t soffset)
+{
+    const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(srd, static_cast<int>(voffset), static_cast<int>(soffset), 0);
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
 
 template <bool BF16>
 __device__ __forceinline__ float4_t mfma16(const uint4& act, const uint4& wgt, float4_t acc)
@@ -50,18 +75,21 @@ __device__ __forceinline__ float4_t mfma16(const uint4& act, const uint4& wgt, f
     }
 }
 
+__device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t mask, uint32_t bits)
+{
+    return (x & mask) | bits;   // v_and_or_b32: both constants arrive as kernel arguments, so neither is a literal
+}
+
 // Eight nibbles of `w` (k ascending from bit 0) -> four registers of two 16-bit floats (magic + q),
 // element 2i in the low half and 2i+1 in the high half: the order activations lie in memory.
-template <bool BF16>
-__device__ __forceinline__ uint4 unpack8(uint32_t w)
+__device__ __forceinline__ uint4 unpack8(uint32_t w, uint32_t mask, uint32_t magic)
 {
     const uint32_t w4 = w >> 4;
-    constexpr uint32_t mask = 0x000F000Fu, mg = Magic<BF16>::pos;
     uint4 r;
-    r.x = (__builtin_amdgcn_perm(w4, w, 0x0c040c00u) & mask) | mg;
-    r.y = (__builtin_amdgcn_perm(w4, w, 0x0c050c01u) & mask) | mg;
-    r.z = (__builtin_amdgcn_perm(w4, w, 0x0c060c02u) & mask) | mg;
-    r.w = (__builtin_amdgcn_perm(w4, w, 0x0c070c03u) & mask) | mg;
+    r.x = and_or(__builtin_amdgcn_perm(w4, w, 0x0c040c00u), mask, magic);
+    r.y = and_or(__builtin_amdgcn_perm(w4, w, 0x0c050c01u), mask, magic);
+    r.z = and_or(__builtin_amdgcn_perm(w4, w, 0x0c060c02u), mask, magic);
+    r.w = and_or(__builtin_amdgcn_perm(w4, w, 0x0c070c03u), mask, magic);
     return r;
 }
 
@@ -79,39 +107,75 @@ __device__ __forceinline__ void transpose_groups(uint4& v)
     v.w = t1[1];
 }
 
-template <typename ST> __device__ __forceinline__ float scale_to_f32(ST s, bool bf16);
-template <> __device__ __forceinline__ float scale_to_f32<float>(float s, bool) { return s; }
-template <> __device__ __forceinline__ float scale_to_f32<uint16_t>(uint16_t s, bool bf16) { return bf16 ? bf16_bits_to_f32(s) : f16_bits_to_f32(s); }
+template <typename ST> struct ScaleIo;
+template <> struct ScaleIo<float> {
+    static __device__ __forceinline__ uint32_t load(__amdgpu_buffer_rsrc_t srd, uint32_t v, uint32_t s) { return __builtin_amdgcn_raw_buffer_load_b32(srd, static_cast<int>(v), static_cast<int>(s), 0); }
+    static __device__ __forceinline__ float to_f32(uint32_t raw, bool) { return __uint_as_float(raw); }
+};
+template <> struct ScaleIo<uint16_t> {
+    static __device__ __forceinline__ uint32_t load(__amdgpu_buffer_rsrc_t srd, uint32_t v, uint32_t s) { return __builtin_amdgcn_raw_buffer_load_b16(srd, static_cast<int>(v), static_cast<int>(s), 0); }
+    static __device__ __forceinline__ float to_f32(uint32_t raw, bool bf16) { return bf16 ? __uint_as_float(raw << 16) : f16_bits_to_f32(static_cast<uint16_t>(raw)); }
+};
 
-// BF16: activation element type. BS: block size (32, 64, 128, 256). CG: 16-column groups per workgroup.
-// ST: storage type of the scales (uint16_t = same 16-bit type as the activations, float = f32).
-template <bool BF16, int BS, int CG, typename ST, int U>
-__global__ __launch_bounds__(1024) void decode_mfma_kernel(DecodeParams p)
+// One group of U tiles: packed weights, scales, zero points of CG column groups, and the activation tile
+// in compact form (piece p = lane % 16 of row lane / 16 + 4 i).
+template <int U, int CG, int AR>
+struct Group {
+    uint4 w[U][CG];
+    uint32_t s[U][CG];
+    uint32_t z[U][CG];
+    uint4 a[U][AR];
+};
+
+// BF16: activation element type. BS: block size (32, 64, 128). CG: 16-column groups per workgroup.
+// MR: rows staged (1, 4, 8 or 16; M <= MR). ST: storage type of the scales (uint16_t = the activations'
+// 16-bit type, float = f32).
+template <bool BF16, int BS, int CG, int MR, typename ST>
+__global__ __launch_bounds__(512) void decode_mfma_kernel(DecodeParams p)
 {
-    constexpr bool kTranspose = BS < 128;      // several blocks inside one 128-element tile
-    constexpr int kBsLog2 = BS == 32 ? 5 : BS == 64 ? 6 : BS == 128 ? 7 : 8;
-    extern __shared__ float red[];             // [waves][CG][4][64]
+    constexpr bool kTranspose = BS < 128;              // several blocks inside one 128-element tile
+    constexpr int kBsLog2 = BS == 32 ? 5 : BS == 64 ? 6 : 7;
+    constexpr int kBlocksPerTile = 128 / BS;
+    constexpr int AR = (MR + 3) / 4;                    // 16-byte activation pieces per lane per tile
+    constexpr int U = (CG == 1 && MR <= 4) ? 4 : 2;     // tiles per prefetch group
+    constexpr int kStageBytes = MR * kRowPitch;         // one activation tile in LDS
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const int waves = blockDim.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform by construction; say so, or every
+    const int waves = blockDim.x >> 6;                                   // tile offset below is treated as divergent
     const int c = lane & 15;
     const int g = lane >> 4;
     const int64_t n_base = static_cast<int64_t>(blockIdx.x) * (16 * CG);
+    const int64_t cols_left = p.n - n_base;
+    const bool has_zp = p.zp != nullptr;
+    const bool full_k = (p.k & 127) == 0;
 
-    const uint8_t* brow[CG];
-    const ST* srow[CG];
-    const uint8_t* zrow[CG];
+    const __amdgpu_buffer_rsrc_t srd_b = make_srd(p.b + n_base * p.row_bytes, static_cast<uint64_t>(cols_left * p.row_bytes));
+    const __amdgpu_buffer_rsrc_t srd_s = make_srd(static_cast<const ST*>(p.scales) + n_base * p.kb, static_cast<uint64_t>(cols_left * p.kb) * sizeof(ST));
+    const __amdgpu_buffer_rsrc_t srd_z = make_srd(has_zp ? p.zp + n_base * p.zp_row : p.b, has_zp ? static_cast<uint64_t>(cols_left * p.zp_row) : 0);
+    const __amdgpu_buffer_rsrc_t srd_a = make_srd(p.a, static_cast<uint64_t>(p.m * p.k) * 2);
+
+    // Per-lane byte offsets; the tile-dependent part is wave-uniform and travels in the scalar offset.
+    uint32_t b_off[CG], s_off[CG], z_off[CG];
+    const uint32_t lane_blk = kTranspose ? static_cast<uint32_t>((g * 32) >> kBsLog2) : 0u;   // block of this lane's piece inside a tile
 #pragma unroll
     for (int cg = 0; cg < CG; ++cg) {
-        int64_t col = n_base + cg * 16 + c;
-        if (col >= p.n) col = p.n - 1;          // stay inside the tensor; the store is masked
-        brow[cg] = p.b + col * p.row_bytes;
-        srow[cg] = static_cast<const ST*>(p.scales) + col * p.kb;
-        zrow[cg] = p.zp ? p.zp + col * p.zp_row : nullptr;
+        const uint32_t col = static_cast<uint32_t>(cg * 16 + c);
+        b_off[cg] = col * static_cast<uint32_t>(p.row_bytes) + static_cast<uint32_t>(g * 16);
+        s_off[cg] = (col * static_cast<uint32_t>(p.kb) + lane_blk) * static_cast<uint32_t>(sizeof(ST));
+        z_off[cg] = col * static_cast<uint32_t>(p.zp_row) + (lane_blk >> 1);
     }
-    const bool row_ok = c < p.m;
-    const uint16_t* arow = p.a + static_cast<int64_t>(row_ok ? c : 0) * p.k;
+    // compact activation load: row g (+4i), piece c
+    const uint32_t a_off = static_cast<uint32_t>(g) * static_cast<uint32_t>(p.k) * 2u + static_cast<uint32_t>(c * 16);
+    const uint32_t a_row_step = 4u * static_cast<uint32_t>(p.k) * 2u;
+    // LDS: this wave's two staging tiles; write at (row g + 4i, piece c), read at (row c % MR, piece of MFMA j)
+    unsigned char* stage = smem + wave * (2 * kStageBytes);
+    const uint32_t st_write = static_cast<uint32_t>(g * kRowPitch + c * 16);
+    const uint32_t st_read = static_cast<uint32_t>((c & (MR - 1)) * kRowPitch + (kTranspose ? g * 16 : g * 64));
+    // v_and_or_b32 may read one scalar operand only: keep the mask in a vector register (an identity DPP move
+    // makes it one), the magic in a scalar register.
+    const uint32_t mask = __builtin_amdgcn_mov_dpp(p.nibble_mask, 0xE4, 0xf, 0xf, false), magic = p.magic;
 
     float4_t y[CG];
     float4_t acc[CG];
@@ -124,73 +188,90 @@ __global__ __launch_bounds__(1024) void decode_mfma_kernel(DecodeParams p)
     const int t_begin = wave * p.tiles_per_wave;
     const int t_end = min(t_begin + p.tiles_per_wave, p.tiles);
 
-    for (int t0 = t_begin; t0 < t_end; t0 += U) {
-        uint4 wq[U][CG];
-        uint4 av[U][4];
-        ST sc[U][CG];
-        uint32_t zq[U][CG];
-        // ---- issue every load of this batch before touching any of them ----
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int kt = t0 + u;
-            const bool tile_ok = kt < t_end;
-            const int64_t boff = static_cast<int64_t>(kt) * 64 + g * 16;
-            const bool w_ok = tile_ok && boff < p.row_bytes;
-            const int64_t blk = (static_cast<int64_t>(kt) * 128 + g * 32) >> kBsLog2;
-#pragma unroll
-            for (int cg = 0; cg < CG; ++cg) {
-                wq[u][cg] = w_ok ? *reinterpret_cast<const uint4*>(brow[cg] + boff) : make_uint4(0, 0, 0, 0);
-                sc[u][cg] = w_ok ? srow[cg][blk] : ST(0);
-                zq[u][cg] = (w_ok && zrow[cg]) ? ((zrow[cg][blk >> 1] >> ((blk & 1) * 4)) & 0xfu) : 8u;
-            }
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int64_t k0 = static_cast<int64_t>(kt) * 128 + (kTranspose ? j * 32 + g * 8 : g * 32 + j * 8);
-                av[u][j] = (tile_ok && row_ok && k0 + 8 <= p.k) ? *reinterpret_cast<const uint4*>(arow + k0) : make_uint4(0, 0, 0, 0);
-            }
-        }
-        // ---- compute ----
+    using Grp = Group<U, CG, AR>;
+    auto fetch_group = [&](Grp& grp, int t0) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int kt = t0 + u;
             if (kt < t_end) {
+                const uint32_t blk0 = static_cast<uint32_t>(kt) * kBlocksPerTile;
+#pragma unroll
+                for (int cg = 0; cg < CG; ++cg) grp.w[u][cg] = load16(srd_b, b_off[cg], static_cast<uint32_t>(kt) * 64u);
+#pragma unroll
+                for (int i = 0; i < AR; ++i) {
+                    uint32_t off = a_off + static_cast<uint32_t>(i) * a_row_step;
+                    if (!full_k && static_cast<int64_t>(kt) * 128 + c * 8 + 8 > p.k) off = kOutOfRange;
+                    if (MR < 4 && g >= MR) off = kOutOfRange;
+                    grp.a[u][i] = load16(srd_a, off, static_cast<uint32_t>(kt) * 256u);
+                }
 #pragma unroll
                 for (int cg = 0; cg < CG; ++cg) {
-                    uint4 w = wq[u][cg];
-                    if constexpr (kTranspose) transpose_groups(w);
-                    const uint32_t wd[4] = {w.x, w.y, w.z, w.w};
+                    grp.s[u][cg] = ScaleIo<ST>::load(srd_s, s_off[cg], blk0 * static_cast<uint32_t>(sizeof(ST)));
+                    grp.z[u][cg] = has_zp ? static_cast<uint32_t>(__builtin_amdgcn_raw_buffer_load_b8(srd_z, static_cast<int>(z_off[cg]), static_cast<int>(blk0 >> 1), 0)) : 0x88u;
+                }
+            }
+        }
+    };
+    auto compute_tile = [&](const Grp& grp, int u, int kt) {
+        // activations: compact registers -> LDS -> MFMA operand order
+        unsigned char* st = stage + (u & 1) * kStageBytes;
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        // zero point and scale of the block MFMA j works on
-                        uint32_t z = zq[u][cg];
-                        ST s = sc[u][cg];
-                        if constexpr (kTranspose) {
-                            const int src = c + 16 * ((j * 32) / BS) * (BS / 32);
-                            z = __shfl(z, src, kWave);
-                            if constexpr (sizeof(ST) == 4) s = __shfl(s, src, kWave);
-                            else s = static_cast<ST>(__shfl(static_cast<uint32_t>(s), src, kWave));
-                        }
-                        const uint32_t zpair = Magic<BF16>::neg | (z * 0x00010001u);
-                        const uint4 zc = make_uint4(zpair, zpair, zpair, zpair);
-                        acc[cg] = mfma16<BF16>(av[u][j], unpack8<BF16>(wd[j]), acc[cg]);
-                        acc[cg] = mfma16<BF16>(av[u][j], zc, acc[cg]);
-                        const int k_done = kt * 128 + (j + 1) * 32;
-                        const bool flush = kTranspose ? (k_done % BS == 0) : (j == 3 && (k_done % BS == 0 || kt + 1 == t_end));
-                        if (flush) {
-                            const float sf = scale_to_f32<ST>(s, BF16);
+        for (int i = 0; i < AR; ++i)
+            if (MR >= 4 || g < MR) *reinterpret_cast<uint4*>(st + st_write + i * 4 * kRowPitch) = grp.a[u][i];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        uint4 av[4];
 #pragma unroll
-                            for (int r = 0; r < 4; ++r) {
-                                y[cg][r] = fmaf(sf, acc[cg][r], y[cg][r]);
-                                acc[cg][r] = 0.f;
-                            }
-                        }
+        for (int j = 0; j < 4; ++j) av[j] = *reinterpret_cast<const uint4*>(st + st_read + (kTranspose ? j * 64 : j * 16));
+#pragma unroll
+        for (int cg = 0; cg < CG; ++cg) {
+            uint4 w = grp.w[u][cg];
+            if constexpr (kTranspose) transpose_groups(w);
+            const uint32_t wd[4] = {w.x, w.y, w.z, w.w};
+            // zero-point nibble and scale of the block this lane's own piece belongs to
+            const uint32_t z_lane = (grp.z[u][cg] >> ((kTranspose ? (lane_blk & 1u) : (static_cast<uint32_t>(kt) & 1u)) * 4u)) & 0xfu;
+            const uint32_t s_lane = grp.s[u][cg];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                uint32_t z = z_lane, s = s_lane;
+                if constexpr (kTranspose) {
+                    const int src = c + 16 * (((j * 32) / BS) * (BS / 32));   // a lane whose piece lies in MFMA j's block
+                    z = __shfl(z, src, kWave);
+                    s = __shfl(s, src, kWave);
+                }
+                const uint32_t zpair = Magic<BF16>::neg | (z * 0x00010001u);
+                const uint4 zc = make_uint4(zpair, zpair, zpair, zpair);
+                acc[cg] = mfma16<BF16>(av[j], unpack8(wd[j], mask, magic), acc[cg]);
+                acc[cg] = mfma16<BF16>(av[j], zc, acc[cg]);
+                if (kTranspose ? (((j + 1) * 32) % BS == 0) : (j == 3)) {
+                    const float sf = ScaleIo<ST>::to_f32(s, BF16);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        y[cg][r] = fmaf(sf, acc[cg][r], y[cg][r]);
+                        acc[cg][r] = 0.f;
                     }
                 }
             }
         }
+    };
+    auto run_group = [&](const Grp& cur, Grp& next, int t0) {
+        fetch_group(next, t0 + U);
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            if (t0 + u < t_end) compute_tile(cur, u, t0 + u);
+    };
+
+    Grp ga, gb;
+    fetch_group(ga, t_begin);
+    for (int t0 = t_begin; t0 < t_end; t0 += 2 * U) {
+        run_group(ga, gb, t0);
+        if (t0 + U < t_end) run_group(gb, ga, t0 + U);
     }
 
     // ---- split-K reduction across the waves of this workgroup, in wave order ----
+    __syncthreads();                                   // every wave is done with its staging tiles
+    float* red = reinterpret_cast<float*>(smem);       // [waves][CG][4][64]
 #pragma unroll
     for (int cg = 0; cg < CG; ++cg)
 #pragma unroll
@@ -211,34 +292,41 @@ __global__ __launch_bounds__(1024) void decode_mfma_kernel(DecodeParams p)
     }
 }
 
-template <bool BF16, int BS, int CG, typename ST>
+template <int CG, int MR> constexpr int group_tiles() { return (CG == 1 && MR <= 4) ? 4 : 2; }
+
+template <bool BF16, int BS, int CG, int MR, typename ST>
 static int launch_cfg(const DecodeParams& p, int waves, hipStream_t stream)
 {
-    constexpr int U = CG >= 4 ? 1 : (CG == 2 ? 2 : 4);
     const unsigned grid = static_cast<unsigned>((p.n + 16 * CG - 1) / (16 * CG));
-    const size_t lds = static_cast<size_t>(waves) * CG * 256 * sizeof(float);
-    hipLaunchKernelGGL((decode_mfma_kernel<BF16, BS, CG, ST, U>), dim3(grid), dim3(waves * 64), lds, stream, p);
+    const size_t stage = static_cast<size_t>(waves) * 2 * MR * kRowPitch;
+    const size_t red = static_cast<size_t>(waves) * CG * 256 * sizeof(float);
+    hipLaunchKernelGGL((decode_mfma_kernel<BF16, BS, CG, MR, ST>), dim3(grid), dim3(waves * 64), stage > red ? stage : red, stream, p);
     return static_cast<int>(hipGetLastError());
 }
 
-template <bool BF16, int BS, typename ST>
-static int launch_cg(const DecodeParams& p, int waves, int cg, hipStream_t stream)
+template <bool BF16, int BS, int CG, typename ST>
+static int launch_mr(const DecodeParams& p, int waves, hipStream_t stream)
 {
-    switch (cg) {
-        case 1: return launch_cfg<BF16, BS, 1, ST>(p, waves, stream);
-        case 2: return launch_cfg<BF16, BS, 2, ST>(p, waves, stream);
-        default: return launch_cfg<BF16, BS, 4, ST>(p, waves, stream);
-    }
+    if (p.m <= 1) return launch_cfg<BF16, BS, CG, 1, ST>(p, waves, stream);
+    if (p.m <= 4) return launch_cfg<BF16, BS, CG, 4, ST>(p, waves, stream);
+    if (p.m <= 8) return launch_cfg<BF16, BS, CG, 8, ST>(p, waves, stream);
+    return launch_cfg<BF16, BS, CG, 16, ST>(p, waves, stream);
 }
 
 template <bool BF16, typename ST>
 static int launch_bs(const DecodeParams& p, int bs, int waves, int cg, hipStream_t stream)
 {
+    if (cg == 1) {
+        switch (bs) {
+            case 32: return launch_mr<BF16, 32, 1, ST>(p, waves, stream);
+            case 64: return launch_mr<BF16, 64, 1, ST>(p, waves, stream);
+            default: return launch_mr<BF16, 128, 1, ST>(p, waves, stream);
+        }
+    }
     switch (bs) {
-        case 32: return launch_cg<BF16, 32, ST>(p, waves, cg, stream);
-        case 64: return launch_cg<BF16, 64, ST>(p, waves, cg, stream);
-        case 128: return launch_cg<BF16, 128, ST>(p, waves, cg, stream);
-        default: return launch_cg<BF16, 256, ST>(p, waves, cg, stream);
+        case 32: return launch_mr<BF16, 32, 2, ST>(p, waves, stream);
+        case 64: return launch_mr<BF16, 64, 2, ST>(p, waves, stream);
+        default: return launch_mr<BF16, 128, 2, ST>(p, waves, stream);
     }
 }
 
@@ -248,9 +336,13 @@ extern "C" int rocm_decode_mfma_eligible(const RocmMatMulNBitsArgs* a)
 {
     const bool half_in = a->a_dtype == ROCM_DT_F16 || a->a_dtype == ROCM_DT_BF16;
     const bool scale_ok = a->scale_dtype == a->a_dtype || a->scale_dtype == ROCM_DT_F32;
-    const bool bs_ok = a->block_size == 32 || a->block_size == 64 || a->block_size == 128 || a->block_size == 256;
-    return half_in && scale_ok && bs_ok && a->m >= 1 && a->m <= 16 && a->n >= 1 && a->k % 8 == 0 &&
-           (reinterpret_cast<uintptr_t>(a->a) & 15) == 0 && (reinterpret_cast<uintptr_t>(a->b) & 15) == 0;
+    const bool bs_ok = a->block_size == 32 || a->block_size == 64 || a->block_size == 128;
+    if (!(half_in && scale_ok && bs_ok && a->m >= 1 && a->m <= 16 && a->n >= 1 && a->k % 8 == 0)) return 0;
+    // 32-bit offsets inside one workgroup's 32-column window of B, and inside A
+    const int64_t kb = (a->k + a->block_size - 1) / a->block_size;
+    if (kb * a->block_size / 2 * 32 >= 0x7fffffff || a->m * a->k * 2 >= 0x7ffffff0) return 0;
+    return (reinterpret_cast<uintptr_t>(a->a) & 15) == 0 && (reinterpret_cast<uintptr_t>(a->b) & 15) == 0 &&
+           (reinterpret_cast<uintptr_t>(a->scales) & 3) == 0;
 }
 
 extern "C" int rocm_launch_decode_mfma(const RocmMatMulNBitsArgs* a, int waves, int col_groups, rocm_stream_t stream)
@@ -269,29 +361,33 @@ extern "C" int rocm_launch_decode_mfma(const RocmMatMulNBitsArgs* a, int waves, 
     p.kb = (a->k + a->block_size - 1) / a->block_size;
     p.row_bytes = p.kb * a->block_size / 2;
     p.zp_row = (p.kb + 1) / 2;
-    p.tiles = static_cast<int>((p.kb * a->block_size + 127) / 128);
+    p.tiles = static_cast<int>((a->k + 127) / 128);
     p.bias_dtype = a->bias_dtype;
     p.y_dtype = a->y_dtype;
+    p.nibble_mask = 0x000F000Fu;
+    p.magic = a->a_dtype == ROCM_DT_BF16 ? mnb::Magic<true>::pos : mnb::Magic<false>::pos;
 
-    const int tiles_per_block = a->block_size > 128 ? a->block_size / 128 : 1;
-    // Heuristic: enough waves to cover the chip several times, at least ~4 tiles of work each.
     int cg = col_groups;
-    if (cg != 1 && cg != 2 && cg != 4) {
+    if (cg != 1 && cg != 2) {
         const int64_t groups = (a->n + 15) / 16;
-        cg = (a->m > 4 && groups >= 4096) ? 2 : 1;
+        cg = (a->m > 8 && groups >= 2048) ? 2 : 1;
     }
+    const int group_tiles = (cg == 1 && a->m <= 4) ? 4 : 2;   // U of the kernel: wave ranges are whole groups
     int w = waves;
     if (w <= 0) {
         const int64_t wgs = (a->n + 16 * cg - 1) / (16 * cg);
-        int want = static_cast<int>((8192 + wgs - 1) / wgs);   // waves per workgroup to reach ~8k waves
-        int by_work = p.tiles / (4 * tiles_per_block);          // keep >= 4 tiles per wave
+        const int want = static_cast<int>((8192 + wgs - 1) / wgs);   // waves per workgroup to reach ~8k waves
+        int by_work = p.tiles / group_tiles;                          // at least one full group per wave
         if (by_work < 1) by_work = 1;
         w = want < by_work ? want : by_work;
         if (w < 1) w = 1;
     }
-    if (w > 16) w = 16;
+    if (w > 8) w = 8;
+    const int mr = a->m <= 1 ? 1 : a->m <= 4 ? 4 : a->m <= 8 ? 8 : 16;
+    const int lds_cap = 65536 / (2 * mr * mnb::kRowPitch);           // staging tiles must fit the default LDS window
+    if (w > lds_cap) w = lds_cap;
     int tpw = (p.tiles + w - 1) / w;
-    tpw = (tpw + tiles_per_block - 1) / tiles_per_block * tiles_per_block;
+    tpw = (tpw + group_tiles - 1) / group_tiles * group_tiles;
     w = (p.tiles + tpw - 1) / tpw;
     p.tiles_per_wave = tpw;
 

@@ -20,7 +20,7 @@ F32, U8, I8, I32, F16, BF16 = 1, 2, 3, 6, 10, 16
 DEVICE_ROCM = 2
 _ITEM = {F32: 4, U8: 1, I8: 1, I32: 4, F16: 2, BF16: 2}
 
-LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libnxrt_ep_rocm.so")
+LIB_PATH = os.environ.get("NXRT_ROCM_LIBRARY") or os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libnxrt_ep_rocm.so")
 
 
 class EpError(RuntimeError):

@@ -157,8 +157,10 @@ DECODE_CASES = [
     (E.F16, E.F16, 32, False, 7, 130, 4864),
     (E.F16, E.F16, 64, True, 2, 257, 1024),
     (E.BF16, E.BF16, 64, True, 16, 48, 8192),
-    (E.F16, E.F32, 256, True, 5, 80, 1536),
-    (E.BF16, E.BF16, 256, False, 1, 33, 768),
+    (E.F16, E.F32, 128, True, 5, 80, 1536),
+    (E.BF16, E.BF16, 32, False, 1, 33, 768),
+    (E.BF16, E.BF16, 32, True, 13, 100, 1000),
+    (E.F16, E.F16, 128, True, 12, 40, 18944),
     (E.F16, E.F16, 32, True, 9, 17, 72),        # K = 72: multiple of 8, not of the block size
     (E.BF16, E.BF16, 128, True, 2, 20, 200),    # partial last block
     (E.F16, E.F16, 64, True, 1, 1, 64),
