@@ -117,28 +117,37 @@ template <> struct ScaleIo<uint16_t> {
     static __device__ __forceinline__ float to_f32(uint32_t raw, bool bf16) { return bf16 ? __uint_as_float(raw << 16) : f16_bits_to_f32(static_cast<uint16_t>(raw)); }
 };
 
-// One group of U tiles: packed weights, scales, zero points of CG column groups, and the activation tile
-// in compact form (piece p = lane % 16 of row lane / 16 + 4 i).
-template <int U, int CG, int AR>
+// One group of U tiles held in registers: packed weights of CG column groups, the activations in compact
+// form, scales and zero points. NA / NS count the activation / scale loads of a group (see the kernel).
+template <int U, int CG, int NA, int NS>
 struct Group {
     uint4 w[U][CG];
-    uint32_t s[U][CG];
-    uint32_t z[U][CG];
-    uint4 a[U][AR];
+    uint4 a[NA];
+    uint32_t s[NS][CG];
+    uint32_t z[NS][CG];
 };
 
 // BF16: activation element type. BS: block size (32, 64, 128). CG: 16-column groups per workgroup.
 // MR: rows staged (1, 4, 8 or 16; M <= MR). ST: storage type of the scales (uint16_t = the activations'
 // 16-bit type, float = f32).
+//
+// Vector memory instructions, not bytes, are what this kernel runs out of first, so everything except the
+// weights is fetched as rarely as possible: with one row (MR = 1) the activations of a whole group arrive in
+// one 16-byte-per-lane load; with block size 128 the scale and zero point of tile t0 + g are loaded once per
+// group by lane group g and handed to the other lanes with a lane shuffle.
 template <bool BF16, int BS, int CG, int MR, typename ST>
 __global__ __launch_bounds__(512) void decode_mfma_kernel(DecodeParams p)
 {
     constexpr bool kTranspose = BS < 128;              // several blocks inside one 128-element tile
     constexpr int kBsLog2 = BS == 32 ? 5 : BS == 64 ? 6 : 7;
     constexpr int kBlocksPerTile = 128 / BS;
-    constexpr int AR = (MR + 3) / 4;                    // 16-byte activation pieces per lane per tile
+    constexpr int AR = (MR + 3) / 4;                    // 16-byte activation pieces per lane per tile (MR > 1)
     constexpr int U = (CG == 1 && MR <= 4) ? 4 : 2;     // tiles per prefetch group
-    constexpr int kStageBytes = MR * kRowPitch;         // one activation tile in LDS
+    constexpr bool kGroupA = MR == 1;                   // one activation load per group
+    constexpr int NA = kGroupA ? 1 : U * AR;
+    constexpr bool kGroupS = !kTranspose;               // one scale / zero-point load per group
+    constexpr int NS = kGroupS ? 1 : U;
+    constexpr int kStageBytes = kGroupA ? 1024 : MR * kRowPitch;   // one staging buffer in LDS (a group / a tile)
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
     const int lane = threadIdx.x & 63;
@@ -158,7 +167,8 @@ __global__ __launch_bounds__(512) void decode_mfma_kernel(DecodeParams p)
 
     // Per-lane byte offsets; the tile-dependent part is wave-uniform and travels in the scalar offset.
     uint32_t b_off[CG], s_off[CG], z_off[CG];
-    const uint32_t lane_blk = kTranspose ? static_cast<uint32_t>((g * 32) >> kBsLog2) : 0u;   // block of this lane's piece inside a tile
+    // block (inside a tile, or inside a group when scales are loaded per group) whose scale this lane fetches
+    const uint32_t lane_blk = kTranspose ? static_cast<uint32_t>((g * 32) >> kBsLog2) : static_cast<uint32_t>(g);
 #pragma unroll
     for (int cg = 0; cg < CG; ++cg) {
         const uint32_t col = static_cast<uint32_t>(cg * 16 + c);
@@ -166,13 +176,15 @@ __global__ __launch_bounds__(512) void decode_mfma_kernel(DecodeParams p)
         s_off[cg] = (col * static_cast<uint32_t>(p.kb) + lane_blk) * static_cast<uint32_t>(sizeof(ST));
         z_off[cg] = col * static_cast<uint32_t>(p.zp_row) + (lane_blk >> 1);
     }
-    // compact activation load: row g (+4i), piece c
-    const uint32_t a_off = static_cast<uint32_t>(g) * static_cast<uint32_t>(p.k) * 2u + static_cast<uint32_t>(c * 16);
+    // compact activation load. MR > 1: row g (+4i), piece c of one tile. MR = 1: piece c of tile g of the group.
+    const uint32_t a_off = kGroupA ? static_cast<uint32_t>(g * 256 + c * 16)
+                                   : static_cast<uint32_t>(g) * static_cast<uint32_t>(p.k) * 2u + static_cast<uint32_t>(c * 16);
     const uint32_t a_row_step = 4u * static_cast<uint32_t>(p.k) * 2u;
-    // LDS: this wave's two staging tiles; write at (row g + 4i, piece c), read at (row c % MR, piece of MFMA j)
+    // LDS: this wave's two staging buffers. MR > 1: written at (row g + 4i, piece c), read at (row c % MR, piece of
+    // MFMA j). MR = 1: written at (tile g, piece c), every lane reads the piece of MFMA j of the tile at hand.
     unsigned char* stage = smem + wave * (2 * kStageBytes);
-    const uint32_t st_write = static_cast<uint32_t>(g * kRowPitch + c * 16);
-    const uint32_t st_read = static_cast<uint32_t>((c & (MR - 1)) * kRowPitch + (kTranspose ? g * 16 : g * 64));
+    const uint32_t st_write = kGroupA ? static_cast<uint32_t>(lane * 16) : static_cast<uint32_t>(g * kRowPitch + c * 16);
+    const uint32_t st_read = (kGroupA ? 0u : static_cast<uint32_t>((c & (MR - 1)) * kRowPitch)) + static_cast<uint32_t>(kTranspose ? g * 16 : g * 64);
     // v_and_or_b32 may read one scalar operand only: keep the mask in a vector register (an identity DPP move
     // makes it one), the magic in a scalar register.
     const uint32_t mask = __builtin_amdgcn_mov_dpp(p.nibble_mask, 0xE4, 0xf, 0xf, false), magic = p.magic;
@@ -188,57 +200,94 @@ __global__ __launch_bounds__(512) void decode_mfma_kernel(DecodeParams p)
     const int t_begin = wave * p.tiles_per_wave;
     const int t_end = min(t_begin + p.tiles_per_wave, p.tiles);
 
-    using Grp = Group<U, CG, AR>;
+    using Grp = Group<U, CG, NA, NS>;
     auto fetch_group = [&](Grp& grp, int t0) {
+        if (t0 >= t_end) return;
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int kt = t0 + u;
-            if (kt < t_end) {
-                const uint32_t blk0 = static_cast<uint32_t>(kt) * kBlocksPerTile;
+            if (t0 + u < t_end) {
 #pragma unroll
-                for (int cg = 0; cg < CG; ++cg) grp.w[u][cg] = load16(srd_b, b_off[cg], static_cast<uint32_t>(kt) * 64u);
+                for (int cg = 0; cg < CG; ++cg) grp.w[u][cg] = load16(srd_b, b_off[cg], static_cast<uint32_t>(t0 + u) * 64u);
+            }
+        }
+        if constexpr (kGroupA) {
+            uint32_t off = a_off;
+            if (g >= U || t0 + g >= t_end || (!full_k && static_cast<int64_t>(t0 + g) * 128 + c * 8 + 8 > p.k)) off = kOutOfRange;
+            grp.a[0] = load16(srd_a, off, static_cast<uint32_t>(t0) * 256u);
+        } else {
 #pragma unroll
-                for (int i = 0; i < AR; ++i) {
-                    uint32_t off = a_off + static_cast<uint32_t>(i) * a_row_step;
-                    if (!full_k && static_cast<int64_t>(kt) * 128 + c * 8 + 8 > p.k) off = kOutOfRange;
-                    if (MR < 4 && g >= MR) off = kOutOfRange;
-                    grp.a[u][i] = load16(srd_a, off, static_cast<uint32_t>(kt) * 256u);
+            for (int u = 0; u < U; ++u) {
+                if (t0 + u < t_end) {
+#pragma unroll
+                    for (int i = 0; i < AR; ++i) {
+                        uint32_t off = a_off + static_cast<uint32_t>(i) * a_row_step;
+                        if (!full_k && static_cast<int64_t>(t0 + u) * 128 + c * 8 + 8 > p.k) off = kOutOfRange;
+                        if (MR < 4 && g >= MR) off = kOutOfRange;
+                        grp.a[u * AR + i] = load16(srd_a, off, static_cast<uint32_t>(t0 + u) * 256u);
+                    }
                 }
+            }
+        }
+        if constexpr (kGroupS) {
+            // lane group g fetches scale and zero point of tile t0 + g (t0 is even, so the nibble is g & 1)
+            const bool mine = g < U && t0 + g < t_end;
 #pragma unroll
-                for (int cg = 0; cg < CG; ++cg) {
-                    grp.s[u][cg] = ScaleIo<ST>::load(srd_s, s_off[cg], blk0 * static_cast<uint32_t>(sizeof(ST)));
-                    grp.z[u][cg] = has_zp ? static_cast<uint32_t>(__builtin_amdgcn_raw_buffer_load_b8(srd_z, static_cast<int>(z_off[cg]), static_cast<int>(blk0 >> 1), 0)) : 0x88u;
+            for (int cg = 0; cg < CG; ++cg) {
+                grp.s[0][cg] = ScaleIo<ST>::load(srd_s, mine ? s_off[cg] : kOutOfRange, static_cast<uint32_t>(t0) * static_cast<uint32_t>(sizeof(ST)));
+                grp.z[0][cg] = has_zp ? static_cast<uint32_t>(__builtin_amdgcn_raw_buffer_load_b8(srd_z, static_cast<int>(mine ? z_off[cg] : kOutOfRange), static_cast<int>(t0 >> 1), 0)) : 0x88u;
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                if (t0 + u < t_end) {
+                    const uint32_t blk0 = static_cast<uint32_t>(t0 + u) * kBlocksPerTile;
+#pragma unroll
+                    for (int cg = 0; cg < CG; ++cg) {
+                        grp.s[u][cg] = ScaleIo<ST>::load(srd_s, s_off[cg], blk0 * static_cast<uint32_t>(sizeof(ST)));
+                        grp.z[u][cg] = has_zp ? static_cast<uint32_t>(__builtin_amdgcn_raw_buffer_load_b8(srd_z, static_cast<int>(z_off[cg]), static_cast<int>(blk0 >> 1), 0)) : 0x88u;
+                    }
                 }
             }
         }
     };
-    auto compute_tile = [&](const Grp& grp, int u, int kt) {
-        // activations: compact registers -> LDS -> MFMA operand order
-        unsigned char* st = stage + (u & 1) * kStageBytes;
-#pragma unroll
-        for (int i = 0; i < AR; ++i)
-            if (MR >= 4 || g < MR) *reinterpret_cast<uint4*>(st + st_write + i * 4 * kRowPitch) = grp.a[u][i];
+    // LDS operations of one wave execute in issue order; the fences only keep the compiler from reordering them.
+    auto lds_order = [&]() {
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
+    auto compute_tile = [&](const Grp& grp, int u, int parity) {
+        // activations: compact registers -> LDS -> MFMA operand order
+        unsigned char* st = stage + (kGroupA ? parity : (u & 1)) * kStageBytes;
+        if constexpr (!kGroupA) {
+#pragma unroll
+            for (int i = 0; i < AR; ++i)
+                if (MR >= 4 || g < MR) *reinterpret_cast<uint4*>(st + st_write + i * 4 * kRowPitch) = grp.a[u * AR + i];
+            lds_order();
+        }
         uint4 av[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) av[j] = *reinterpret_cast<const uint4*>(st + st_read + (kTranspose ? j * 64 : j * 16));
+        for (int j = 0; j < 4; ++j) av[j] = *reinterpret_cast<const uint4*>(st + st_read + (kGroupA ? u * 256 : 0) + (kTranspose ? j * 64 : j * 16));
 #pragma unroll
         for (int cg = 0; cg < CG; ++cg) {
             uint4 w = grp.w[u][cg];
             if constexpr (kTranspose) transpose_groups(w);
             const uint32_t wd[4] = {w.x, w.y, w.z, w.w};
-            // zero-point nibble and scale of the block this lane's own piece belongs to
-            const uint32_t z_lane = (grp.z[u][cg] >> ((kTranspose ? (lane_blk & 1u) : (static_cast<uint32_t>(kt) & 1u)) * 4u)) & 0xfu;
-            const uint32_t s_lane = grp.s[u][cg];
+            // scale and zero-point nibble this lane fetched: of its own block (BS < 128) or of tile g (BS = 128)
+            const uint32_t z_lane = (grp.z[kGroupS ? 0 : u][cg] >> ((lane_blk & 1u) * 4u)) & 0xfu;
+            const uint32_t s_lane = grp.s[kGroupS ? 0 : u][cg];
+            uint32_t z_tile = z_lane, s_tile = s_lane;
+            if constexpr (kGroupS) {
+                z_tile = __shfl(z_lane, c + 16 * u, kWave);
+                s_tile = __shfl(s_lane, c + 16 * u, kWave);
+            }
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                uint32_t z = z_lane, s = s_lane;
+                uint32_t z = z_tile, s = s_tile;
                 if constexpr (kTranspose) {
                     const int src = c + 16 * (((j * 32) / BS) * (BS / 32));   // a lane whose piece lies in MFMA j's block
-                    z = __shfl(z, src, kWave);
-                    s = __shfl(s, src, kWave);
+                    z = __shfl(z_lane, src, kWave);
+                    s = __shfl(s_lane, src, kWave);
                 }
                 const uint32_t zpair = Magic<BF16>::neg | (z * 0x00010001u);
                 const uint4 zc = make_uint4(zpair, zpair, zpair, zpair);
@@ -255,18 +304,22 @@ __global__ __launch_bounds__(512) void decode_mfma_kernel(DecodeParams p)
             }
         }
     };
-    auto run_group = [&](const Grp& cur, Grp& next, int t0) {
+    auto run_group = [&](const Grp& cur, Grp& next, int t0, int parity) {
         fetch_group(next, t0 + U);
+        if constexpr (kGroupA) {
+            *reinterpret_cast<uint4*>(stage + parity * kStageBytes + st_write) = cur.a[0];
+            lds_order();
+        }
 #pragma unroll
         for (int u = 0; u < U; ++u)
-            if (t0 + u < t_end) compute_tile(cur, u, t0 + u);
+            if (t0 + u < t_end) compute_tile(cur, u, parity);
     };
 
     Grp ga, gb;
     fetch_group(ga, t_begin);
     for (int t0 = t_begin; t0 < t_end; t0 += 2 * U) {
-        run_group(ga, gb, t0);
-        if (t0 + U < t_end) run_group(gb, ga, t0 + U);
+        run_group(ga, gb, t0, 0);
+        if (t0 + U < t_end) run_group(gb, ga, t0 + U, 1);
     }
 
     // ---- split-K reduction across the waves of this workgroup, in wave order ----
@@ -298,7 +351,7 @@ template <bool BF16, int BS, int CG, int MR, typename ST>
 static int launch_cfg(const DecodeParams& p, int waves, hipStream_t stream)
 {
     const unsigned grid = static_cast<unsigned>((p.n + 16 * CG - 1) / (16 * CG));
-    const size_t stage = static_cast<size_t>(waves) * 2 * MR * kRowPitch;
+    const size_t stage = static_cast<size_t>(waves) * 2 * (MR == 1 ? 1024 : MR * kRowPitch);
     const size_t red = static_cast<size_t>(waves) * CG * 256 * sizeof(float);
     hipLaunchKernelGGL((decode_mfma_kernel<BF16, BS, CG, MR, ST>), dim3(grid), dim3(waves * 64), stage > red ? stage : red, stream, p);
     return static_cast<int>(hipGetLastError());
@@ -384,7 +437,7 @@ extern "C" int rocm_launch_decode_mfma(const RocmMatMulNBitsArgs* a, int waves, 
     }
     if (w > 8) w = 8;
     const int mr = a->m <= 1 ? 1 : a->m <= 4 ? 4 : a->m <= 8 ? 8 : 16;
-    const int lds_cap = 65536 / (2 * mr * mnb::kRowPitch);           // staging tiles must fit the default LDS window
+    const int lds_cap = 65536 / (2 * (mr == 1 ? 1024 : mr * mnb::kRowPitch));   // staging buffers must fit the default LDS window
     if (w > lds_cap) w = lds_cap;
     int tpw = (p.tiles + w - 1) / w;
     tpw = (tpw + group_tiles - 1) / group_tiles * group_tiles;
