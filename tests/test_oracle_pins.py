@@ -1,0 +1,212 @@
+"""Pins for the CPU oracle (oracle/matmul_nbits_oracle.c): every function is checked against something that is not
+a retyping of its own formula — the reference's known answers, golden vectors taken from the reference's compiled
+MLAS, the compiled MLAS itself where it is built, library conversions, or brute force."""
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from onnx_genai_amd import synth
+from tests import helpers
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "mlas_vectors.npz")
+
+
+@pytest.fixture(scope="module")
+def golden():
+    return np.load(GOLDEN, allow_pickle=False)
+
+
+# ---- layout ---------------------------------------------------------------------------------------------------
+def test_known_answer_low_nibble_first(port):
+    """matmul_nbits.rs:18702-18722: packed[0] = 0xe1, A = [1, 10, 0, ...], scale 1, default zero point 8 -> 53."""
+    k = 16
+    a = np.zeros((1, k), np.float32)
+    a[0, 0], a[0, 1] = 1.0, 10.0
+    b = np.full((1, 1, 8), 0x88, np.uint8)
+    b[0, 0, 0] = 0xE1
+    s = np.ones((1, 1), np.float32)
+    assert port.matmul_blocksum_f32(a, b, s, None, 1, k, 16).tolist() == [[53.0]]
+    assert port.matmul_f64(a, b, s, None, 1, k, 16).tolist() == [[53.0]]
+    assert port.matmul_dequant_f32(a, port.dequantize_nk(b, s, None, 1, k, 16)).tolist() == [[53.0]]
+    qa, qs = port.quantize_a(a, k, 16, oracle.ROUND_HALF_EVEN)
+    assert port.block_acc_i32(qa, b, None, 1, k, 16).tolist() == [[[int(qa[0, 0]) * -7 + int(qa[0, 1]) * 6]]]
+
+
+def test_zero_point_nibble_order(port):
+    """Zero points are packed like the weights: even block in the low nibble (matmul_nbits.rs:1317-1321)."""
+    n, bs, kb = 1, 16, 3
+    b = synth.pack_nibbles(np.zeros((n, kb, bs), np.uint8))
+    zp = np.array([[0x21, 0x03]], np.uint8)                 # blocks 0,1,2 -> 1,2,3
+    w = port.dequantize_nk(b, np.ones((n, kb), np.float32), zp, n, kb * bs, bs)
+    assert w[0, 0] == -1.0 and w[0, bs] == -2.0 and w[0, 2 * bs] == -3.0
+
+
+# ---- conversions ----------------------------------------------------------------------------------------------
+def test_f16_widen_matches_numpy_on_every_pattern(port):
+    bits = np.arange(65536, dtype=np.uint16)
+    got = port.widen(bits.view(np.float16), oracle.F16)
+    want = bits.view(np.float16).astype(np.float32)
+    assert np.array_equal(got.view(np.uint32)[~np.isnan(want)], want.view(np.uint32)[~np.isnan(want)])
+    assert np.isnan(got[np.isnan(want)]).all()
+
+
+def test_f16_narrow_matches_numpy(port):
+    rng = np.random.default_rng(0)
+    x = np.concatenate([rng.standard_normal(200000).astype(np.float32) * np.float32(10.0) ** rng.integers(-9, 6, 200000).astype(np.float32),
+                        np.array([0.0, -0.0, 65504.0, 65519.9, 65520.0, 1e-8, 5.96e-8, 2.98e-8, 2.9802322e-8, 6.1e-5, np.inf, -np.inf], np.float32)])
+    halves = (np.arange(0, 65535, dtype=np.uint16).view(np.float16).astype(np.float32)[:31000])
+    mid = ((halves[:-1].astype(np.float64) + halves[1:].astype(np.float64)) / 2).astype(np.float32)   # exact ties between neighbours
+    x = np.concatenate([x, mid])
+    got = port.narrow(x, oracle.F16)
+    with np.errstate(over="ignore"):
+        want = x.astype(np.float16)
+    assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+
+
+def test_bf16_round_trip_matches_torch(port):
+    torch = pytest.importorskip("torch")
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal(100000).astype(np.float32) * np.float32(3.0) ** rng.integers(-40, 40, 100000).astype(np.float32)
+    ties = (np.arange(1, 20000, dtype=np.uint32) << 16 | 0x8000).view(np.float32)                       # exactly half way
+    x = np.concatenate([x, ties, np.array([0.0, -0.0, np.inf, -np.inf, 3.4e38], np.float32)])
+    want = torch.from_numpy(x).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(port.narrow(x, oracle.BF16), want)
+    assert np.array_equal(synth.f32_to_bf16_bits(x), want)
+    back = port.widen(want, oracle.BF16)
+    assert np.array_equal(back.view(np.uint32), want.astype(np.uint32) << 16)
+
+
+# ---- dequantization and the float routes ----------------------------------------------------------------------
+def test_three_float_routes_agree(port):
+    """f64 literal reading, block-sum form and dequantize-then-GEMM are three different computations of one operator."""
+    rng = np.random.default_rng(3)
+    for bs, zero_points, k in ((16, True, 80), (32, False, 256), (64, True, 200), (128, True, 384)):
+        n, m = 33, 3
+        b, s, zp = synth.make_weights(n, k, bs, bs, zero_points=zero_points, scale_lo=0.005, scale_hi=0.02, scale_dtype=synth.F32)
+        a = rng.standard_normal((m, k)).astype(np.float32)
+        bias = rng.standard_normal(n).astype(np.float32)
+        y64 = port.matmul_f64(a, b, s, zp, n, k, bs, bias=bias)
+        assert helpers.rel_l2(port.matmul_blocksum_f32(a, b, s, zp, n, k, bs, bias=bias), y64) < 2e-6
+        assert helpers.rel_l2(port.matmul_dequant_f32(a, port.dequantize_nk(b, s, zp, n, k, bs), bias), y64) < 2e-6
+        # brute force with numpy on unpacked operands
+        kb = -(-k // bs)
+        q = synth.unpack_nibbles(b.reshape(n, kb, bs // 2), bs).reshape(n, kb * bs)[:, :k].astype(np.float64)
+        z = (synth.unpack_nibbles(zp, kb) if zp is not None else np.full((n, kb), 8)).astype(np.float64)
+        w = (q - np.repeat(z, bs, axis=1)[:, :k]) * np.repeat(s.astype(np.float64), bs, axis=1)[:, :k]
+        assert helpers.rel_l2(a.astype(np.float64) @ w.T + bias, y64) < 1e-12
+
+
+def test_golden_mlas_fp32_outputs(port, golden):
+    """The reference's compiled MLAS CompFp32 on its own check_sqnbit grid (mlas-sys/src/lib.rs:3268-3285)."""
+    for tag in golden["cases"]:
+        tag = str(tag)
+        parts = {p[0]: p[1:] for p in tag.split("_")[:4]}
+        m, n, k, bs = int(parts["m"]), int(parts["n"]), int(parts["k"]), int(parts["b"])
+        b, s, a = golden[tag + "_b"], golden[tag + "_s"], golden[tag + "_a"]
+        zp = golden[tag + "_zp"] if tag + "_zp" in golden.files else None
+        bias = golden[tag + "_bias"] if tag + "_bias" in golden.files else None
+        y = port.matmul_blocksum_f32(a, b, s, zp, n, k, bs, bias=bias)
+        assert helpers.rel_l2(y, golden[tag + "_y_fp32"]) < 2e-6, tag
+        assert m * n == y.size
+
+
+def test_golden_mlas_int8_outputs(port, golden):
+    """The reference's compiled MLAS CompInt8: same codes and integers, another f32 summation order."""
+    for tag in golden["cases"]:
+        tag = str(tag)
+        parts = {p[0]: p[1:] for p in tag.split("_")[:4]}
+        n, k, bs = int(parts["n"]), int(parts["k"]), int(parts["b"])
+        b, s, a = golden[tag + "_b"], golden[tag + "_s"], golden[tag + "_a"]
+        zp = golden[tag + "_zp"] if tag + "_zp" in golden.files else None
+        bias = golden[tag + "_bias"] if tag + "_bias" in golden.files else None
+        y = port.matmul_acc4_f32(a, b, s, zp, n, k, bs, oracle.ROUND_HALF_EVEN, bias=bias)
+        assert helpers.rel_l2(y, golden[tag + "_y_int8"]) < 2e-6, tag
+        y_away = port.matmul_acc4_f32(a, b, s, zp, n, k, bs, oracle.ROUND_HALF_AWAY, bias=bias)
+        assert helpers.rel_l2(y_away, golden[tag + "_y_int8"]) < 2e-3, tag      # the two rules differ on ties only
+
+
+def test_envelope_pinned_against_f64(port):
+    """matmul_nbits.rs:10986-11068 with the oracle's two routes in place of the reference kernel."""
+    k, n, bs, weights, act = helpers.envelope_fixture()
+    b, s, zp, _ = helpers.quantize_blockwise(weights, bs, True)
+    want = port.matmul_f64(act, b, s, zp, n, k, bs)
+    assert np.abs(want).max() > 1.0
+    exact = helpers.max_rel_to_peak(port.matmul_blocksum_f32(act, b, s, zp, n, k, bs), want)
+    assert exact < 1e-5
+    for rounding in (oracle.ROUND_HALF_EVEN, oracle.ROUND_HALF_AWAY):
+        reduced = helpers.max_rel_to_peak(port.matmul_acc4_f32(act, b, s, zp, n, k, bs, rounding), want)
+        assert reduced > 10 * exact and 1e-4 <= reduced < 1e-2
+
+
+# ---- activation quantizer -------------------------------------------------------------------------------------
+def test_golden_mlas_quantizer_codes(port, golden):
+    """Ties-to-even rule: bit-exact against the codes and scales the reference's compiled MLAS produced."""
+    for bs in (32, 64, 128):
+        a = golden[f"quant_b{bs}_a"]
+        qa, qs = port.quantize_a(a, a.shape[1], bs, oracle.ROUND_HALF_EVEN)
+        assert np.array_equal(qa, golden[f"quant_b{bs}_codes"])
+        assert np.array_equal(qs.view(np.uint32), golden[f"quant_b{bs}_scales"].view(np.uint32))
+        blksum = qs * qa.reshape(a.shape[0], -1, bs).sum(axis=2).astype(np.float32)
+        assert np.array_equal(blksum.view(np.uint32), golden[f"quant_b{bs}_blksum"].view(np.uint32))
+        assert (qa != port.quantize_a(a, a.shape[1], bs, oracle.ROUND_HALF_AWAY)[0]).any()
+
+
+def test_quantizer_closed_form_cases(port):
+    """simd_quant.rs:131-143 by hand: max 127 makes inv exactly 1, so the codes are the rounded inputs."""
+    bs = 16
+    a = np.zeros((1, 3 * bs), np.float32)
+    a[0, :8] = [127.0, -127.0, 0.5, -0.5, 1.5, 2.5, -2.5, 126.5]
+    a[0, 2 * bs:] = 3.0
+    even, s_even = port.quantize_a(a, 3 * bs, bs, oracle.ROUND_HALF_EVEN)
+    away, s_away = port.quantize_a(a, 3 * bs, bs, oracle.ROUND_HALF_AWAY)
+    assert even[0, :8].tolist() == [127, -127, 0, 0, 2, 2, -2, 126]
+    assert away[0, :8].tolist() == [127, -127, 1, -1, 2, 3, -3, 127]
+    assert s_even[0].tolist() == [1.0, 0.0, np.float32(3.0) / np.float32(127.0)] and np.array_equal(s_even, s_away)
+    assert not even[0, bs:2 * bs].any() and not away[0, bs:2 * bs].any()          # all-zero block: scale 0, codes 0
+    assert (even[0, 2 * bs:] == 127).all() and (away[0, 2 * bs:] == 127).all()    # every element is the maximum
+    # partial last block: the tail is zero
+    q, s = port.quantize_a(np.ones((1, bs + 3), np.float32), bs + 3, bs, oracle.ROUND_HALF_EVEN)
+    assert q.shape == (1, 2 * bs) and q[0, bs:bs + 3].tolist() == [127] * 3 and not q[0, bs + 3:].any()
+
+
+def test_block_accumulators_brute_force(port):
+    rng = np.random.default_rng(7)
+    for bs, zero_points in ((16, True), (32, False), (128, True)):
+        m, n, k = 4, 21, 3 * bs
+        kb = k // bs
+        b, _, zp = synth.make_weights(n, k, bs, bs, zero_points=zero_points, scale_lo=0.01, scale_hi=0.02, scale_dtype=synth.F32)
+        qa = rng.integers(-127, 128, size=(m, k), dtype=np.int8)
+        got = port.block_acc_i32(qa, b, zp, n, k, bs).astype(np.int64)
+        q = synth.unpack_nibbles(b.reshape(n, kb, bs // 2), bs).astype(np.int64)
+        z = synth.unpack_nibbles(zp, kb).astype(np.int64) if zp is not None else np.full((n, kb), 8, np.int64)
+        want = np.einsum("mbk,nbk->mnb", qa.reshape(m, kb, bs).astype(np.int64), q - z[:, :, None])
+        assert np.array_equal(got, want)
+        assert np.abs(got).max() <= bs * 127 * 15
+
+
+# ---- the compiled reference itself, where it is built ---------------------------------------------------------
+def test_compiled_mlas_agrees_with_golden_and_oracle(port, ref, golden):
+    """Re-derives the golden vectors from oracle/_ref on this host and checks the oracle's dequantization through
+    one-hot activations (each output is then a single dequantized weight)."""
+    tag = "m5_n96_k256_b64_asym"
+    b, s, a, zp = golden[tag + "_b"], golden[tag + "_s"], golden[tag + "_a"], golden[tag + "_zp"]
+    y = ref.matmul(a, b, s, zp, 96, 256, 64, ref.COMP_FP32)
+    assert helpers.rel_l2(y, golden[tag + "_y_fp32"]) < 1e-6
+    for bs in (16, 32, 64, 128, 256):
+        for zero_points in (False, True):
+            n, k = 48, 2 * max(bs, 64)
+            bb, ss, zz = synth.make_weights(n, k, bs, 5 + bs, zero_points=zero_points, scale_lo=0.003, scale_hi=0.05, scale_dtype=synth.F32)
+            w = port.dequantize_nk(bb, ss, zz, n, k, bs)
+            for kk in (0, 1, bs - 1, bs, k - 1):
+                onehot = np.zeros((1, k), np.float32)
+                onehot[0, kk] = 1.0
+                row = ref.matmul(onehot, bb, ss, zz, n, k, bs, ref.COMP_FP32)
+                assert row is not None and np.array_equal(row[0].view(np.uint32), w[:, kk].view(np.uint32)), (bs, zero_points, kk)
+    rng = np.random.default_rng(11)
+    a = rng.standard_normal((7, 512)).astype(np.float16).astype(np.float32)
+    for bs in (16, 32, 64, 128):
+        r = ref.quantize_a(a, 512, bs)
+        qa, qs = port.quantize_a(a, 512, bs, oracle.ROUND_HALF_EVEN)
+        assert np.array_equal(r[0], qa) and np.array_equal(r[1].view(np.uint32), qs.view(np.uint32))
