@@ -1,4 +1,289 @@
-// Prefill path placeholder: filled in by the LDS-staged dequant + MFMA GEMM.
+// Prefill path of MatMulNBits (M > 16, f16/bf16 activations): Y[M,N] = A[M,K] . dequant(B)[N,K]^T on the matrix cores.
+//
+// A workgroup of four waves owns a BM x 128 tile of Y and walks K in steps of 64. Per step it
+//   * copies a BM x 64 tile of A from global memory to LDS (16 bytes per lane, rows padded to 144 bytes so that
+//     the 32 lanes of an MFMA operand read hit different banks);
+//   * reads 128 x 64 packed 4-bit weights (one 16-byte piece = 32 nibbles = one lane), dequantizes them in registers
+//     and writes them to LDS as 16-bit floats. f16 with f16 scales: (0x6400|q) is 1024+q, a packed subtract of 1024+zp
+//     is exact and one packed multiply by the scale rounds once - the tile is bit-identical to f16((q-zp)*scale).
+//     Otherwise (bf16, or f32 scales): (q-zp)*scale in f32, rounded to nearest even;
+//   * runs v_mfma_f32_32x32x16 on 2 x 2 waves, each owning a (BM/2) x 64 sub-tile, f32 accumulators.
+// LDS is double buffered: the global loads of step t+1 are in flight while the MFMAs of step t run, and one barrier
+// per step separates the two buffers. Edges in M and N are handled by range-checked buffer loads and masked stores.
+#include <hip/hip_fp16.h>
+
 #include "common.hiph"
-extern "C" int rocm_prefill_mfma_eligible(const RocmMatMulNBitsArgs*) { return 0; }
-extern "C" int rocm_launch_prefill_mfma(const RocmMatMulNBitsArgs*, rocm_stream_t) { return -1; }
+
+namespace mnb {
+
+typedef __attribute__((ext_vector_type(8))) _Float16 half8_t;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(16))) float float16_t;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
+typedef __attribute__((ext_vector_type(2))) _Float16 half2_t;
+
+struct PrefillParams {
+    const uint16_t* a;
+    const uint8_t* b;
+    const void* scales;
+    const uint8_t* zp;
+    const void* bias;
+    void* y;
+    int64_t m, n, k, kb;
+    int64_t row_bytes, zp_row;
+    int bs_log2;
+    int scale_dtype, bias_dtype, y_dtype;
+};
+
+constexpr int kBN = 128;
+constexpr int kBK = 64;
+constexpr int kPitch = 144;            // bytes per LDS row: 64 halfs + 8 of padding
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_srd_p(const void* base, uint64_t bytes)
+{
+    const uint32_t range = bytes > 0x7fffffffull ? 0x7fffffffu : static_cast<uint32_t>(bytes);
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, static_cast<int>(range), 0x00020000);
+}
+
+__device__ __forceinline__ uint4 load16_p(__amdgpu_buffer_rsrc_t srd, uint32_t voffset, uint32_t soffset)
+{
+    const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(srd, static_cast<int>(voffset), static_cast<int>(soffset), 0);
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+
+template <bool BF16>
+__device__ __forceinline__ float16_t mfma32(const uint4& a, const uint4& b, float16_t c)
+{
+    if constexpr (BF16) return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+    else return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, b), c, 0, 0, 0);
+}
+
+// Two nibbles (elements 2i, 2i+1 of a packed dword) as a pair of 16-bit floats carrying magic + q.
+__device__ __forceinline__ uint32_t magic_pair(uint32_t w, uint32_t w4, uint32_t sel, uint32_t magic)
+{
+    return (__builtin_amdgcn_perm(w4, w, sel) & 0x000F000Fu) | magic;
+}
+
+// f16, f16 scale: exact subtract, one rounding multiply.
+__device__ __forceinline__ uint32_t finish_f16(uint32_t pair, half2_t neg_off, half2_t scale)
+{
+    const half2_t v = (__builtin_bit_cast(half2_t, pair) + neg_off) * scale;
+    return __builtin_bit_cast(uint32_t, v);
+}
+
+// (q - zp) * scale in f32 for both halves of a magic pair (bf16 magic 0x4300 or f16 magic 0x6400), rounded to 16 bits.
+template <bool BF16>
+__device__ __forceinline__ uint32_t finish_f32(uint32_t pair, float off, float scale)
+{
+    float lo, hi;
+    if constexpr (BF16) {
+        lo = __uint_as_float(pair << 16);
+        hi = __uint_as_float(pair & 0xffff0000u);
+    } else {
+        const half2_t h = __builtin_bit_cast(half2_t, pair);
+        lo = static_cast<float>(h.x);
+        hi = static_cast<float>(h.y);
+    }
+    lo = __fmul_rn(lo - off, scale);
+    hi = __fmul_rn(hi - off, scale);
+    if constexpr (BF16) return static_cast<uint32_t>(f32_to_bf16_bits(lo)) | (static_cast<uint32_t>(f32_to_bf16_bits(hi)) << 16);
+    else return static_cast<uint32_t>(f32_to_f16_bits(lo)) | (static_cast<uint32_t>(f32_to_f16_bits(hi)) << 16);
+}
+
+// BF16: element type. BM: rows of Y per workgroup (128 or 256). F32MATH: dequantize in f32 (bf16, or f32 scales).
+template <bool BF16, int BM, bool F32MATH>
+__global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillParams p)
+{
+    constexpr int WM = BM / 2;             // wave sub-tile rows
+    constexpr int TM = WM / 32;            // 32x32 MFMA tiles per wave along M
+    constexpr int TN = 2;                  // and along N (64 columns)
+    constexpr int A_LOADS = BM / 32;       // 16-byte pieces of A per lane per step
+    constexpr uint32_t kMagic = BF16 ? 0x43004300u : 0x64006400u;
+    constexpr float kMagicF = BF16 ? 128.0f : 1024.0f;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    unsigned char* lds_a = smem;                                   // [2][BM][kPitch]
+    unsigned char* lds_b = smem + 2 * BM * kPitch;                 // [2][kBN][kPitch]
+
+    const int t = threadIdx.x;
+    const int lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int64_t m_base = static_cast<int64_t>(blockIdx.x) * BM;
+    const int64_t n_base = static_cast<int64_t>(blockIdx.y) * kBN;
+    const int64_t rows_left = p.m - m_base, cols_left = p.n - n_base;
+
+    const __amdgpu_buffer_rsrc_t srd_a = make_srd_p(p.a + m_base * p.k, static_cast<uint64_t>(rows_left * p.k) * 2);
+    const __amdgpu_buffer_rsrc_t srd_b = make_srd_p(p.b + n_base * p.row_bytes, static_cast<uint64_t>(cols_left * p.row_bytes));
+
+    // A: lane -> (row t/8 + 32 i, piece t%8). B: lane -> (column t/2, half t%2 of the 64-element step).
+    const uint32_t a_goff = static_cast<uint32_t>(t >> 3) * static_cast<uint32_t>(p.k) * 2u + static_cast<uint32_t>((t & 7) * 16);
+    const uint32_t a_gstep = 32u * static_cast<uint32_t>(p.k) * 2u;
+    const uint32_t a_loff = static_cast<uint32_t>((t >> 3) * kPitch + (t & 7) * 16);
+    const int bcol = t >> 1, bhalf = t & 1;
+    const uint32_t b_goff = static_cast<uint32_t>(bcol) * static_cast<uint32_t>(p.row_bytes) + static_cast<uint32_t>(bhalf * 16);
+    const uint32_t b_loff = static_cast<uint32_t>(bcol * kPitch + bhalf * 64);
+    const bool col_ok = bcol < cols_left;
+    const int64_t gcol = n_base + (col_ok ? bcol : 0);
+    const uint8_t* zrow = p.zp ? p.zp + gcol * p.zp_row : nullptr;
+
+    // MFMA operand reads: lane (r = lane % 32, kg = lane / 32) reads 8 consecutive k of row r.
+    const uint32_t frag_off = static_cast<uint32_t>((lane & 31) * kPitch + (lane >> 5) * 16);
+
+    float16_t acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    const int steps = static_cast<int>(p.k / kBK);
+    uint4 ra[A_LOADS];
+    uint4 rb;
+    float rs;
+    int rz;
+
+    auto load_global = [&](int kt) {
+#pragma unroll
+        for (int i = 0; i < A_LOADS; ++i) ra[i] = load16_p(srd_a, a_goff + static_cast<uint32_t>(i) * a_gstep, static_cast<uint32_t>(kt) * 128u);
+        rb = load16_p(srd_b, b_goff, static_cast<uint32_t>(kt) * 32u);
+        const int64_t blk = (static_cast<int64_t>(kt) * kBK + bhalf * 32) >> p.bs_log2;
+        rs = col_ok ? load_as_f32(p.scales, p.scale_dtype, gcol * p.kb + blk) : 0.f;
+        rz = zero_point_of(zrow, blk);
+    };
+    auto store_lds = [&](int buf) {
+        unsigned char* la = lds_a + buf * (BM * kPitch) + a_loff;
+#pragma unroll
+        for (int i = 0; i < A_LOADS; ++i) *reinterpret_cast<uint4*>(la + i * 32 * kPitch) = ra[i];
+        unsigned char* lb = lds_b + buf * (kBN * kPitch) + b_loff;
+        const uint32_t wd[4] = {rb.x, rb.y, rb.z, rb.w};
+        half2_t neg_off, sc2;
+        if constexpr (!F32MATH) {
+            const _Float16 o = static_cast<_Float16>(-(1024.0f + static_cast<float>(rz)));
+            const _Float16 s = static_cast<_Float16>(rs);          // exact: the scale is stored as f16
+            neg_off = half2_t{o, o};
+            sc2 = half2_t{s, s};
+        }
+        const float off = kMagicF + static_cast<float>(rz);
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            const uint32_t w = wd[d], w4 = w >> 4;
+            uint32_t pr[4];
+            pr[0] = magic_pair(w, w4, 0x0c040c00u, kMagic);
+            pr[1] = magic_pair(w, w4, 0x0c050c01u, kMagic);
+            pr[2] = magic_pair(w, w4, 0x0c060c02u, kMagic);
+            pr[3] = magic_pair(w, w4, 0x0c070c03u, kMagic);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if constexpr (F32MATH) pr[i] = finish_f32<BF16>(pr[i], off, rs);
+                else pr[i] = finish_f16(pr[i], neg_off, sc2);
+            }
+            *reinterpret_cast<uint4*>(lb + d * 16) = make_uint4(pr[0], pr[1], pr[2], pr[3]);
+        }
+    };
+    auto compute = [&](int buf) {
+        const unsigned char* la = lds_a + buf * (BM * kPitch) + wm * (WM * kPitch) + frag_off;
+        const unsigned char* lb = lds_b + buf * (kBN * kPitch) + wn * (64 * kPitch) + frag_off;
+#pragma unroll
+        for (int kk = 0; kk < kBK / 16; ++kk) {
+            uint4 fa[TM], fb[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i) fa[i] = *reinterpret_cast<const uint4*>(la + i * 32 * kPitch + kk * 32);
+#pragma unroll
+            for (int j = 0; j < TN; ++j) fb[j] = *reinterpret_cast<const uint4*>(lb + j * 32 * kPitch + kk * 32);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) acc[i][j] = mfma32<BF16>(fa[i], fb[j], acc[i][j]);
+        }
+    };
+
+    load_global(0);
+    store_lds(0);
+    __syncthreads();
+    for (int kt = 0; kt < steps; ++kt) {
+        const int buf = kt & 1;
+        if (kt + 1 < steps) load_global(kt + 1);
+        compute(buf);
+        if (kt + 1 < steps) store_lds(buf ^ 1);
+        __syncthreads();
+    }
+
+    // Epilogue. A 32x32 accumulator holds, in lane l, column l % 32 and rows 8 q + 4 (l / 32) + r (q, r = 0..3).
+    const int col_in_tile = lane & 31;
+    const int row_group = (lane >> 5) * 4;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const int64_t col = n_base + wn * 64 + j * 32 + col_in_tile;
+        if (col >= p.n) continue;
+        const float bias = p.bias ? load_as_f32(p.bias, p.bias_dtype, col) : 0.f;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int64_t row = m_base + wm * WM + i * 32 + q * 8 + row_group + r;
+                    if (row < p.m) store_from_f32(p.y, p.y_dtype, row * p.n + col, acc[i][j][q * 4 + r] + bias);
+                }
+            }
+        }
+    }
+}
+
+template <bool BF16, int BM, bool F32MATH>
+static int launch_prefill(const PrefillParams& p, hipStream_t stream)
+{
+    const dim3 grid(static_cast<unsigned>((p.m + BM - 1) / BM), static_cast<unsigned>((p.n + kBN - 1) / kBN));
+    const size_t lds = 2 * static_cast<size_t>(BM + kBN) * kPitch;
+    auto kernel = prefill_mfma_kernel<BF16, BM, F32MATH>;
+    if (lds > 65536) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+        if (e != hipSuccess) return static_cast<int>(e);
+    }
+    hipLaunchKernelGGL(kernel, grid, dim3(256), lds, stream, p);
+    return static_cast<int>(hipGetLastError());
+}
+
+}  // namespace mnb
+
+extern "C" int rocm_prefill_mfma_eligible(const RocmMatMulNBitsArgs* a)
+{
+    const bool half_in = a->a_dtype == ROCM_DT_F16 || a->a_dtype == ROCM_DT_BF16;
+    const bool bs_ok = a->block_size >= 32;                            // a 16-byte piece must lie inside one block
+    if (!(half_in && bs_ok && a->m > 16 && a->n >= 1 && a->k >= 64 && a->k % 64 == 0)) return 0;
+    const int64_t kb = (a->k + a->block_size - 1) / a->block_size;
+    if (kb * a->block_size / 2 * 128 >= 0x7fffffff || 256 * a->k * 2 >= 0x7fffffff) return 0;   // 32-bit offsets inside one tile
+    return (reinterpret_cast<uintptr_t>(a->a) & 15) == 0 && (reinterpret_cast<uintptr_t>(a->b) & 15) == 0;
+}
+
+extern "C" int rocm_launch_prefill_mfma(const RocmMatMulNBitsArgs* a, rocm_stream_t stream)
+{
+    if (!rocm_prefill_mfma_eligible(a)) return -1;
+    mnb::PrefillParams p;
+    p.a = static_cast<const uint16_t*>(a->a);
+    p.b = a->b;
+    p.scales = a->scales;
+    p.zp = a->zp;
+    p.bias = a->bias;
+    p.y = a->y;
+    p.m = a->m;
+    p.n = a->n;
+    p.k = a->k;
+    p.kb = (a->k + a->block_size - 1) / a->block_size;
+    p.row_bytes = p.kb * a->block_size / 2;
+    p.zp_row = (p.kb + 1) / 2;
+    p.bs_log2 = __builtin_ctz(static_cast<unsigned>(a->block_size));
+    p.scale_dtype = a->scale_dtype;
+    p.bias_dtype = a->bias_dtype;
+    p.y_dtype = a->y_dtype;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const bool bf16 = a->a_dtype == ROCM_DT_BF16;
+    const bool f32math = bf16 || a->scale_dtype != ROCM_DT_F16;
+    // 256-row tiles once there are enough of them to fill the chip; 128-row tiles otherwise.
+    const int64_t wg256 = ((a->m + 255) / 256) * ((a->n + 127) / 128);
+    const bool big = a->m >= 256 && wg256 >= 256;
+    if (bf16) return big ? mnb::launch_prefill<true, 256, true>(p, s) : mnb::launch_prefill<true, 128, true>(p, s);
+    if (f32math) return big ? mnb::launch_prefill<false, 256, true>(p, s) : mnb::launch_prefill<false, 128, true>(p, s);
+    return big ? mnb::launch_prefill<false, 256, false>(p, s) : mnb::launch_prefill<false, 128, false>(p, s);
+}

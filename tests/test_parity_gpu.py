@@ -230,6 +230,52 @@ def test_linearity_at_full_7b_shape(ep):
 
 
 # ---------------------------------------------------------------------------------------------
+# prefill path (f16 / bf16 activations, M > 16)
+# ---------------------------------------------------------------------------------------------
+PREFILL_CASES = [
+    # a_dt, s_dt, bs, zp, m, n, k
+    (E.F16, E.F16, 32, False, 512, 256, 4096),
+    (E.F16, E.F16, 32, True, 300, 200, 512),
+    (E.F16, E.F16, 64, True, 17, 128, 64),
+    (E.F16, E.F16, 128, True, 64, 130, 1024),
+    (E.F16, E.F32, 32, True, 100, 96, 256),
+    (E.BF16, E.BF16, 128, True, 257, 384, 3584),
+    (E.BF16, E.BF16, 32, False, 33, 100, 128),
+    (E.BF16, E.F32, 64, True, 1030, 128, 512),
+]
+
+
+@pytest.mark.parametrize("a_dt,s_dt,bs,zero_points,m,n,k", PREFILL_CASES)
+def test_prefill_matches_oracle(ep, port, a_dt, s_dt, bs, zero_points, m, n, k):
+    b, s, zp = synth.make_weights(n, k, bs, 200 + n + k, zero_points=zero_points, scale_lo=0.001, scale_hi=0.01, scale_dtype=s_dt)
+    a = synth.make_activation(m, k, n, a_dt)
+    bias = synth.to_dtype(np.random.default_rng(n).standard_normal(n).astype(np.float32), a_dt)
+    want64 = oracle_f64(port, a, a_dt, b, s, s_dt, zp, n, k, bs, bias, a_dt)
+    y32, variant = run_op(ep, a, a_dt, b, s, s_dt, zp, n, k, bs, bias=bias, bias_dtype=a_dt, y_dtype=E.F32)
+    assert variant == "prefill_mfma_lds"
+    assert helpers.rel_l2(y32, want64) <= TOL_HALF
+    y, _ = run_op(ep, a, a_dt, b, s, s_dt, zp, n, k, bs, bias=bias, bias_dtype=a_dt)
+    assert helpers.rel_l2(synth.to_f32(y, a_dt), want64) <= TOL_HALF
+    assert np.array_equal(np.asarray(y).view(np.uint16), np.asarray(port.narrow(y32, a_dt)).view(np.uint16))
+
+
+@pytest.mark.parametrize("bs,zero_points", [(32, True), (64, False), (128, True)])
+def test_prefill_weight_tiles_are_f16_of_f32_dequant(ep, port, bs, zero_points):
+    """One-hot activation rows read single weights back out of the GEMM: with f16 scales each must equal the f32
+    dequantized weight rounded once to f16, bit for bit."""
+    m, n, k = 64, 256, 256
+    b, s, zp = synth.make_weights(n, k, bs, 300 + bs, zero_points=zero_points, scale_lo=0.001, scale_hi=0.01, scale_dtype=E.F16)
+    ks = (np.arange(m) * 37) % k
+    a = np.zeros((m, k), np.float16)
+    a[np.arange(m), ks] = 1.0
+    y, variant = run_op(ep, a, E.F16, b, s, E.F16, zp, n, k, bs)
+    assert variant == "prefill_mfma_lds"
+    w = port.dequantize_nk(b, synth.to_f32(s, E.F16), zp, n, k, bs)            # f32 [N, K], bit-exact reference definition
+    want = port.narrow(np.ascontiguousarray(w[:, ks].T), oracle.F16)
+    assert np.array_equal(y.view(np.uint16), want.view(np.uint16))
+
+
+# ---------------------------------------------------------------------------------------------
 # accuracy_level = 4
 # ---------------------------------------------------------------------------------------------
 def _tie_heavy_activation(m, k, bs, seed, dtype):
