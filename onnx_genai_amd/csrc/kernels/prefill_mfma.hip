@@ -90,10 +90,12 @@ __device__ __forceinline__ uint32_t finish_f32(uint32_t pair, float off, float s
     else return static_cast<uint32_t>(f32_to_f16_bits(lo)) | (static_cast<uint32_t>(f32_to_f16_bits(hi)) << 16);
 }
 
-// BF16: element type. BM: rows of Y per workgroup (128 or 256). F32MATH: dequantize in f32 (bf16, or f32 scales).
-template <bool BF16, int BM, bool F32MATH>
+// BF16: element type. BM: rows of Y per workgroup (128 or 256). SF32: scales are stored as f32 (otherwise in the
+// activations' 16-bit type). f16 activations with f16 scales dequantize in packed f16, everything else in f32.
+template <bool BF16, int BM, bool SF32>
 __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillParams p)
 {
+    constexpr bool F32MATH = BF16 || SF32;
     constexpr int WM = BM / 2;             // wave sub-tile rows
     constexpr int TM = WM / 32;            // 32x32 MFMA tiles per wave along M
     constexpr int TN = 2;                  // and along N (64 columns)
@@ -108,12 +110,19 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillParams p)
     const int lane = t & 63;
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const int wm = wave >> 1, wn = wave & 1;
-    const int64_t m_base = static_cast<int64_t>(blockIdx.x) * BM;
-    const int64_t n_base = static_cast<int64_t>(blockIdx.y) * kBN;
+    // Column blocks vary fastest: the workgroups running at one time share a few row blocks of A (each XCD's L2 then
+    // holds them once) and sweep the small packed B.
+    const int64_t m_base = static_cast<int64_t>(blockIdx.y) * BM;
+    const int64_t n_base = static_cast<int64_t>(blockIdx.x) * kBN;
     const int64_t rows_left = p.m - m_base, cols_left = p.n - n_base;
 
     const __amdgpu_buffer_rsrc_t srd_a = make_srd_p(p.a + m_base * p.k, static_cast<uint64_t>(rows_left * p.k) * 2);
     const __amdgpu_buffer_rsrc_t srd_b = make_srd_p(p.b + n_base * p.row_bytes, static_cast<uint64_t>(cols_left * p.row_bytes));
+    constexpr uint32_t kScaleBytes = SF32 ? 4 : 2;
+    const __amdgpu_buffer_rsrc_t srd_s = make_srd_p(static_cast<const unsigned char*>(p.scales) + n_base * p.kb * kScaleBytes,
+                                                    static_cast<uint64_t>(cols_left * p.kb) * kScaleBytes);
+    const bool has_zp = p.zp != nullptr;
+    const __amdgpu_buffer_rsrc_t srd_z = make_srd_p(has_zp ? p.zp + n_base * p.zp_row : p.b, has_zp ? static_cast<uint64_t>(cols_left * p.zp_row) : 0);
 
     // A: lane -> (row t/8 + 32 i, piece t%8). B: lane -> (column t/2, half t%2 of the 64-element step).
     const uint32_t a_goff = static_cast<uint32_t>(t >> 3) * static_cast<uint32_t>(p.k) * 2u + static_cast<uint32_t>((t & 7) * 16);
@@ -122,9 +131,8 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillParams p)
     const int bcol = t >> 1, bhalf = t & 1;
     const uint32_t b_goff = static_cast<uint32_t>(bcol) * static_cast<uint32_t>(p.row_bytes) + static_cast<uint32_t>(bhalf * 16);
     const uint32_t b_loff = static_cast<uint32_t>(bcol * kPitch + bhalf * 64);
-    const bool col_ok = bcol < cols_left;
-    const int64_t gcol = n_base + (col_ok ? bcol : 0);
-    const uint8_t* zrow = p.zp ? p.zp + gcol * p.zp_row : nullptr;
+    const uint32_t s_goff = static_cast<uint32_t>(bcol) * static_cast<uint32_t>(p.kb) * kScaleBytes;
+    const uint32_t z_goff = static_cast<uint32_t>(bcol) * static_cast<uint32_t>(p.zp_row);
 
     // MFMA operand reads: lane (r = lane % 32, kg = lane / 32) reads 8 consecutive k of row r.
     const uint32_t frag_off = static_cast<uint32_t>((lane & 31) * kPitch + (lane >> 5) * 16);
@@ -138,75 +146,103 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillParams p)
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
     const int steps = static_cast<int>(p.k / kBK);
-    uint4 ra[A_LOADS];
-    uint4 rb;
-    float rs;
-    int rz;
-
-    auto load_global = [&](int kt) {
-#pragma unroll
-        for (int i = 0; i < A_LOADS; ++i) ra[i] = load16_p(srd_a, a_goff + static_cast<uint32_t>(i) * a_gstep, static_cast<uint32_t>(kt) * 128u);
-        rb = load16_p(srd_b, b_goff, static_cast<uint32_t>(kt) * 32u);
-        const int64_t blk = (static_cast<int64_t>(kt) * kBK + bhalf * 32) >> p.bs_log2;
-        rs = col_ok ? load_as_f32(p.scales, p.scale_dtype, gcol * p.kb + blk) : 0.f;
-        rz = zero_point_of(zrow, blk);
+    // Global loads run D-1 steps ahead of the MFMAs, in D register sets; step x lives in set x % D from its load
+    // (issued while step x-D+1 is being multiplied) to its dequantize-and-store into LDS (while step x-1 is).
+    constexpr int D = 4;
+    struct Regs {
+        uint4 a[A_LOADS];
+        uint4 b;
+        uint32_t s;      // raw scale bits; converted when the step is dequantized, so that no load is waited for early
+        uint32_t z;      // raw zero-point byte and the nibble to take from it
     };
-    auto store_lds = [&](int buf) {
+    Regs regs[D];
+
+    auto load_global = [&](Regs& r, int kt) {
+#pragma unroll
+        for (int i = 0; i < A_LOADS; ++i) r.a[i] = load16_p(srd_a, a_goff + static_cast<uint32_t>(i) * a_gstep, static_cast<uint32_t>(kt) * 128u);
+        r.b = load16_p(srd_b, b_goff, static_cast<uint32_t>(kt) * 32u);
+        const uint32_t blk = static_cast<uint32_t>((kt * kBK + bhalf * 32) >> p.bs_log2);
+        if constexpr (SF32) r.s = __builtin_amdgcn_raw_buffer_load_b32(srd_s, static_cast<int>(s_goff + blk * 4u), 0, 0);
+        else r.s = __builtin_amdgcn_raw_buffer_load_b16(srd_s, static_cast<int>(s_goff + blk * 2u), 0, 0);
+        const uint32_t zbyte = has_zp ? static_cast<uint32_t>(__builtin_amdgcn_raw_buffer_load_b8(srd_z, static_cast<int>(z_goff + (blk >> 1)), 0, 0)) : 0x88u;
+        r.z = zbyte | ((blk & 1u) << 8);
+    };
+    // Quarter `part` (0..3) of one step's trip from registers to LDS: A pieces part, part+4, ... and packed dword `part`
+    // of B, dequantized. Four quarters make a step; they are issued between the MFMA batches of the step before, so
+    // that their VALU and LDS-write work runs while the matrix cores are busy.
+    auto store_part = [&](const Regs& r, int buf, int part) {
         unsigned char* la = lds_a + buf * (BM * kPitch) + a_loff;
 #pragma unroll
-        for (int i = 0; i < A_LOADS; ++i) *reinterpret_cast<uint4*>(la + i * 32 * kPitch) = ra[i];
+        for (int i = part; i < A_LOADS; i += 4) *reinterpret_cast<uint4*>(la + i * 32 * kPitch) = r.a[i];
         unsigned char* lb = lds_b + buf * (kBN * kPitch) + b_loff;
-        const uint32_t wd[4] = {rb.x, rb.y, rb.z, rb.w};
-        half2_t neg_off, sc2;
-        if constexpr (!F32MATH) {
-            const _Float16 o = static_cast<_Float16>(-(1024.0f + static_cast<float>(rz)));
-            const _Float16 s = static_cast<_Float16>(rs);          // exact: the scale is stored as f16
-            neg_off = half2_t{o, o};
-            sc2 = half2_t{s, s};
-        }
-        const float off = kMagicF + static_cast<float>(rz);
+        const uint32_t w = part == 0 ? r.b.x : part == 1 ? r.b.y : part == 2 ? r.b.z : r.b.w, w4 = w >> 4;
+        uint32_t pr[4];
+        pr[0] = magic_pair(w, w4, 0x0c040c00u, kMagic);
+        pr[1] = magic_pair(w, w4, 0x0c050c01u, kMagic);
+        pr[2] = magic_pair(w, w4, 0x0c060c02u, kMagic);
+        pr[3] = magic_pair(w, w4, 0x0c070c03u, kMagic);
+        const uint32_t zq = (r.z >> ((r.z >> 8) * 4u)) & 0xfu;
+        if constexpr (F32MATH) {
+            const float off = kMagicF + static_cast<float>(zq);
+            const float sc = SF32 ? __uint_as_float(r.s) : (BF16 ? __uint_as_float(r.s << 16) : f16_bits_to_f32(static_cast<uint16_t>(r.s)));
 #pragma unroll
-        for (int d = 0; d < 4; ++d) {
-            const uint32_t w = wd[d], w4 = w >> 4;
-            uint32_t pr[4];
-            pr[0] = magic_pair(w, w4, 0x0c040c00u, kMagic);
-            pr[1] = magic_pair(w, w4, 0x0c050c01u, kMagic);
-            pr[2] = magic_pair(w, w4, 0x0c060c02u, kMagic);
-            pr[3] = magic_pair(w, w4, 0x0c070c03u, kMagic);
+            for (int i = 0; i < 4; ++i) pr[i] = finish_f32<BF16>(pr[i], off, sc);
+        } else {
+            const uint32_t o2 = 0xE400E400u | (zq * 0x00010001u);   // -(1024 + zp) twice, exact in f16
+            const uint32_t s2 = r.s * 0x00010001u;                  // the f16 scale twice
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                if constexpr (F32MATH) pr[i] = finish_f32<BF16>(pr[i], off, rs);
-                else pr[i] = finish_f16(pr[i], neg_off, sc2);
-            }
-            *reinterpret_cast<uint4*>(lb + d * 16) = make_uint4(pr[0], pr[1], pr[2], pr[3]);
+            for (int i = 0; i < 4; ++i) pr[i] = finish_f16(pr[i], __builtin_bit_cast(half2_t, o2), __builtin_bit_cast(half2_t, s2));
         }
+        *reinterpret_cast<uint4*>(lb + part * 16) = make_uint4(pr[0], pr[1], pr[2], pr[3]);
     };
-    auto compute = [&](int buf) {
+    auto store_lds = [&](const Regs& r, int buf) {
+#pragma unroll
+        for (int part = 0; part < 4; ++part) store_part(r, buf, part);
+    };
+    // MFMAs of one 64-element step out of LDS buffer `buf`; the operand fragments of the next 16 elements are read
+    // while these run, and (when asked) the following step moves from registers into the other buffer.
+    auto compute = [&](int buf, const Regs& next, bool store_next) {
         const unsigned char* la = lds_a + buf * (BM * kPitch) + wm * (WM * kPitch) + frag_off;
         const unsigned char* lb = lds_b + buf * (kBN * kPitch) + wn * (64 * kPitch) + frag_off;
+        uint4 fa[2][TM], fb[2][TN];
+#pragma unroll
+        for (int i = 0; i < TM; ++i) fa[0][i] = *reinterpret_cast<const uint4*>(la + i * 32 * kPitch);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) fb[0][j] = *reinterpret_cast<const uint4*>(lb + j * 32 * kPitch);
 #pragma unroll
         for (int kk = 0; kk < kBK / 16; ++kk) {
-            uint4 fa[TM], fb[TN];
+            const int cur = kk & 1, nxt = cur ^ 1;
+            if (kk + 1 < kBK / 16) {
 #pragma unroll
-            for (int i = 0; i < TM; ++i) fa[i] = *reinterpret_cast<const uint4*>(la + i * 32 * kPitch + kk * 32);
+                for (int i = 0; i < TM; ++i) fa[nxt][i] = *reinterpret_cast<const uint4*>(la + i * 32 * kPitch + (kk + 1) * 32);
 #pragma unroll
-            for (int j = 0; j < TN; ++j) fb[j] = *reinterpret_cast<const uint4*>(lb + j * 32 * kPitch + kk * 32);
+                for (int j = 0; j < TN; ++j) fb[nxt][j] = *reinterpret_cast<const uint4*>(lb + j * 32 * kPitch + (kk + 1) * 32);
+            }
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
-                for (int j = 0; j < TN; ++j) acc[i][j] = mfma32<BF16>(fa[i], fb[j], acc[i][j]);
+                for (int j = 0; j < TN; ++j) acc[i][j] = mfma32<BF16>(fa[cur][i], fb[cur][j], acc[i][j]);
+            if (store_next) store_part(next, buf ^ 1, kk);
         }
     };
 
-    load_global(0);
-    store_lds(0);
+    // Every load below is issued unconditionally (past the end of K it reads in-range garbage or range-checked zeros
+    // that are never stored): with a fixed number of loads per step the compiler can wait for exactly the step it
+    // needs and leave the newer ones in flight.
+#pragma unroll
+    for (int s0 = 0; s0 < D - 1; ++s0) load_global(regs[s0], s0);
+    store_lds(regs[0], 0);
     __syncthreads();
-    for (int kt = 0; kt < steps; ++kt) {
-        const int buf = kt & 1;
-        if (kt + 1 < steps) load_global(kt + 1);
-        compute(buf);
-        if (kt + 1 < steps) store_lds(buf ^ 1);
-        __syncthreads();
+    for (int kt0 = 0; kt0 < steps; kt0 += D) {
+#pragma unroll
+        for (int s0 = 0; s0 < D; ++s0) {
+            const int kt = kt0 + s0;
+            load_global(regs[(s0 + D - 1) % D], kt + D - 1);
+            if (kt < steps) {
+                compute(s0 & 1, regs[(s0 + 1) % D], kt + 1 < steps);
+                __syncthreads();
+            }
+        }
     }
 
     // Epilogue. A 32x32 accumulator holds, in lane l, column l % 32 and rows 8 q + 4 (l / 32) + r (q, r = 0..3).
@@ -231,12 +267,12 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillParams p)
     }
 }
 
-template <bool BF16, int BM, bool F32MATH>
+template <bool BF16, int BM, bool SF32>
 static int launch_prefill(const PrefillParams& p, hipStream_t stream)
 {
-    const dim3 grid(static_cast<unsigned>((p.m + BM - 1) / BM), static_cast<unsigned>((p.n + kBN - 1) / kBN));
+    const dim3 grid(static_cast<unsigned>((p.n + kBN - 1) / kBN), static_cast<unsigned>((p.m + BM - 1) / BM));
     const size_t lds = 2 * static_cast<size_t>(BM + kBN) * kPitch;
-    auto kernel = prefill_mfma_kernel<BF16, BM, F32MATH>;
+    auto kernel = prefill_mfma_kernel<BF16, BM, SF32>;
     if (lds > 65536) {
         const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
         if (e != hipSuccess) return static_cast<int>(e);
@@ -251,7 +287,8 @@ extern "C" int rocm_prefill_mfma_eligible(const RocmMatMulNBitsArgs* a)
 {
     const bool half_in = a->a_dtype == ROCM_DT_F16 || a->a_dtype == ROCM_DT_BF16;
     const bool bs_ok = a->block_size >= 32;                            // a 16-byte piece must lie inside one block
-    if (!(half_in && bs_ok && a->m > 16 && a->n >= 1 && a->k >= 64 && a->k % 64 == 0)) return 0;
+    const bool scale_ok = a->scale_dtype == a->a_dtype || a->scale_dtype == ROCM_DT_F32;
+    if (!(half_in && bs_ok && scale_ok && a->m > 16 && a->n >= 1 && a->k >= 64 && a->k % 64 == 0)) return 0;
     const int64_t kb = (a->k + a->block_size - 1) / a->block_size;
     if (kb * a->block_size / 2 * 128 >= 0x7fffffff || 256 * a->k * 2 >= 0x7fffffff) return 0;   // 32-bit offsets inside one tile
     return (reinterpret_cast<uintptr_t>(a->a) & 15) == 0 && (reinterpret_cast<uintptr_t>(a->b) & 15) == 0;
@@ -279,11 +316,12 @@ extern "C" int rocm_launch_prefill_mfma(const RocmMatMulNBitsArgs* a, rocm_strea
     p.y_dtype = a->y_dtype;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool bf16 = a->a_dtype == ROCM_DT_BF16;
-    const bool f32math = bf16 || a->scale_dtype != ROCM_DT_F16;
+    const bool sf32 = a->scale_dtype == ROCM_DT_F32;
     // 256-row tiles once there are enough of them to fill the chip; 128-row tiles otherwise.
     const int64_t wg256 = ((a->m + 255) / 256) * ((a->n + 127) / 128);
     const bool big = a->m >= 256 && wg256 >= 256;
-    if (bf16) return big ? mnb::launch_prefill<true, 256, true>(p, s) : mnb::launch_prefill<true, 128, true>(p, s);
-    if (f32math) return big ? mnb::launch_prefill<false, 256, true>(p, s) : mnb::launch_prefill<false, 128, true>(p, s);
+    if (bf16 && sf32) return big ? mnb::launch_prefill<true, 256, true>(p, s) : mnb::launch_prefill<true, 128, true>(p, s);
+    if (bf16) return big ? mnb::launch_prefill<true, 256, false>(p, s) : mnb::launch_prefill<true, 128, false>(p, s);
+    if (sf32) return big ? mnb::launch_prefill<false, 256, true>(p, s) : mnb::launch_prefill<false, 128, true>(p, s);
     return big ? mnb::launch_prefill<false, 256, false>(p, s) : mnb::launch_prefill<false, 128, false>(p, s);
 }
