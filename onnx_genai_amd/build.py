@@ -19,6 +19,7 @@ HIP_SOURCES = [
     "kernels/decode_mfma.hip",
     "kernels/prefill_mfma.hip",
     "kernels/acc4.hip",
+    "kernels/acc4_mfma.hip",
 ]
 HOST_SOURCES = ["ep/provider.cpp", "ep/matmul_nbits.cpp", "ep/nxrt_plugin.cpp", "ep/nxmem_plugin.cpp"]
 

@@ -136,14 +136,20 @@ struct NxrtRocmMatMulNBits {
 
 namespace {
 
-// Bytes of scratch accuracy_level=4 needs for M rows: int8 codes, f32 scales, int32 code sums.
-uint64_t acc4_workspace_bytes(const NxrtRocmMatMulNBits& kn, uint64_t m)
+// Scratch of accuracy_level=4 for M rows: int8 codes, (scale, code sum) pairs, and a block-major copy of the
+// pairs (M <= 16) or of the scales (M > 16) for the matrix-core kernels.
+struct Acc4Layout { uint64_t codes, pairs, aux, total; };
+Acc4Layout acc4_layout(const NxrtRocmMatMulNBits& kn, uint64_t m)
 {
     const uint64_t kb = (kn.k + kn.block_size - 1) / kn.block_size;
-    const uint64_t codes = (m * kb * kn.block_size + 255) / 256 * 256;
-    const uint64_t scales = (m * kb * 4 + 255) / 256 * 256;
-    return codes + 2 * scales;
+    Acc4Layout l;
+    l.codes = (m * kb * kn.block_size + 255) / 256 * 256;
+    l.pairs = (m * kb * 8 + 255) / 256 * 256;
+    l.aux = (kb * (m > 32 ? m : 32) * 4 + 255) / 256 * 256;
+    l.total = l.codes + l.pairs + l.aux;
+    return l;
 }
+uint64_t acc4_workspace_bytes(const NxrtRocmMatMulNBits& kn, uint64_t m) { return acc4_layout(kn, m).total; }
 
 NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, uint32_t n_in, NxrtRocmTensorView* out, uint32_t n_out,
                         void* workspace, uint64_t workspace_bytes)
@@ -267,18 +273,18 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
             }
             ws = static_cast<uint8_t*>(kn.scratch);
         }
-        const uint64_t codes = (M * kb * BS + 255) / 256 * 256;
-        const uint64_t scl = (M * kb * 4 + 255) / 256 * 256;
-        int8_t* qa = reinterpret_cast<int8_t*>(ws);
-        float* qscale = reinterpret_cast<float*>(ws + codes);
-        int32_t* qsum = reinterpret_cast<int32_t*>(ws + codes + scl);
-        rc = rocm_launch_quantize_a(args.a, args.a_dtype, args.m, args.k, args.block_size, kn.ep->acc4_rounding, qa, qscale, qsum, stream);
+        const Acc4Layout lay = acc4_layout(kn, M);
+        RocmAcc4Workspace w4;
+        w4.qa = reinterpret_cast<int8_t*>(ws);
+        w4.aq = reinterpret_cast<float*>(ws + lay.codes);
+        w4.aux = reinterpret_cast<float*>(ws + lay.codes + lay.pairs);
+        rc = rocm_launch_quantize_a_workspace(args.a, args.a_dtype, args.m, args.k, args.block_size, kn.ep->acc4_rounding, &w4, stream);
         if (rc == 0) {
             if (rocm_acc4_mfma_eligible(&args)) {
-                rc = rocm_launch_acc4_mfma(&args, qa, qscale, qsum, stream);
+                rc = rocm_launch_acc4_mfma(&args, &w4, kn.ep->decode_waves, stream);
                 kn.variant = "acc4_mfma_i8";
             } else {
-                rc = rocm_launch_acc4_gemv(&args, qa, qscale, qsum, stream);
+                rc = rocm_launch_acc4_gemv(&args, &w4, stream);
                 kn.variant = "acc4_gemv_dot4";
             }
         }

@@ -81,12 +81,22 @@ int rocm_launch_quantize_a(const void* a, int a_dtype, int64_t m, int64_t k, int
 /* acc[m,n,b] = sum_k qa[m,k] * (q[n,k] - zp[n,b]), int32 [M, N, kb]. */
 int rocm_launch_block_acc_i32(const int8_t* qa, const uint8_t* b, const uint8_t* zp,
                               int64_t m, int64_t n, int64_t k, int block_size, int32_t* acc, rocm_stream_t stream);
-/* y = sum_b f32(acc_b) * (sa_b * sb_b) + bias, from already quantized activations. */
-int rocm_launch_acc4_gemv(const RocmMatMulNBitsArgs* args, const int8_t* qa, const float* qscale, const int32_t* qsum,
-                          rocm_stream_t stream);
+/* Workspace of one accuracy_level 4 call (device memory, each part 256-byte aligned):
+ * qa: int8 [M, kb*bs], inside every run of 8 the elements 0,2,4,6 then 1,3,5,7; aq: f32 [M, kb, 2] = (scale, sum of codes);
+ * aux: for M <= 16, f32 [kb, 16, 2], the same pairs block-major; for M > 16, f32 [kb, M], the scales block-major. */
+typedef struct RocmAcc4Workspace {
+  int8_t* qa;
+  float* aq;
+  float* aux;
+} RocmAcc4Workspace;
+int rocm_launch_quantize_a_workspace(const void* a, int a_dtype, int64_t m, int64_t k, int block_size, int rounding,
+                                     const RocmAcc4Workspace* ws, rocm_stream_t stream);
+/* y = sum_b f32(acc_b) * (sa_b * sb_b) + bias, from a filled workspace. Any block size, any M (4 rows per launch). */
+int rocm_launch_acc4_gemv(const RocmMatMulNBitsArgs* args, const RocmAcc4Workspace* ws, rocm_stream_t stream);
+/* The same on the int8 matrix cores: M <= 16 with block size 32/64/128 (split-K; waves = 0 lets the launcher choose),
+ * M > 16 with any block size >= 32 (tiled). */
 int rocm_acc4_mfma_eligible(const RocmMatMulNBitsArgs* args);
-int rocm_launch_acc4_mfma(const RocmMatMulNBitsArgs* args, const int8_t* qa, const float* qscale, const int32_t* qsum,
-                          rocm_stream_t stream);
+int rocm_launch_acc4_mfma(const RocmMatMulNBitsArgs* args, const RocmAcc4Workspace* ws, int waves, rocm_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -13,8 +13,8 @@ namespace mnb {
 
 // One wave per (row, block). Division and multiply are single correctly rounded f32 operations.
 __global__ __launch_bounds__(256) void quantize_a_kernel(
-    const void* __restrict__ a, int a_dtype, int64_t m, int64_t k, int bs, int64_t kb, int rounding,
-    int8_t* __restrict__ qa, float* __restrict__ qscale, int32_t* __restrict__ qsum)
+    const void* __restrict__ a, int a_dtype, int64_t m, int64_t k, int bs, int64_t kb, int rounding, int interleave,
+    int8_t* __restrict__ qa, float* __restrict__ qscale, int32_t* __restrict__ qsum, float* __restrict__ aq, float* __restrict__ aux16, float* __restrict__ sa_t)
 {
     const int lane = threadIdx.x & 63;
     const int64_t item = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
@@ -37,14 +37,25 @@ __global__ __launch_bounds__(256) void quantize_a_kernel(
             r = fminf(fmaxf(r, -127.0f), 127.0f);
             code = static_cast<int>(r);
         }
-        qa[(row * kb + blk) * bs + i] = static_cast<int8_t>(code);
+        // interleaved: inside every run of 8, elements 0,2,4,6 then 1,3,5,7
+        const int pos = interleave ? ((i & ~7) | ((i & 1) << 2) | ((i & 7) >> 1)) : i;
+        qa[(row * kb + blk) * bs + pos] = static_cast<int8_t>(code);
         sum += code;
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
     if (lane == 0) {
-        qscale[row * kb + blk] = scale;
+        if (qscale) qscale[row * kb + blk] = scale;
         if (qsum) qsum[row * kb + blk] = sum;
+        if (aq) {
+            aq[(row * kb + blk) * 2] = scale;
+            aq[(row * kb + blk) * 2 + 1] = static_cast<float>(sum);   // |sum| <= 127 * bs: exact
+        }
+        if (sa_t) sa_t[blk * m + row] = scale;
+        if (aux16 && row < 16) {
+            aux16[(blk * 16 + row) * 2] = scale;
+            aux16[(blk * 16 + row) * 2 + 1] = static_cast<float>(sum);
+        }
     }
 }
 
@@ -70,9 +81,10 @@ __global__ __launch_bounds__(256) void block_acc_i32_kernel(
 
 // One wave per output column; a lane takes one packed dword (8 weights) at a time, dots it against the
 // 8 matching activation codes with v_dot4_i32_i8, and the bs/8 lanes of a block add up with shuffles.
+// Codes are in the interleaved order and (scale, code sum) pairs in `aq`, as the workspace holds them.
 template <int ROWS>
-__global__ __launch_bounds__(256) void acc4_gemv_kernel(RocmMatMulNBitsArgs p, const int8_t* __restrict__ qa, const float* __restrict__ qscale,
-                                                        const int32_t* __restrict__ qsum, int bs_log2, int64_t kb, int64_t row0)
+__global__ __launch_bounds__(256) void acc4_gemv_kernel(RocmMatMulNBitsArgs p, const int8_t* __restrict__ qa, const float* __restrict__ aq,
+                                                        int bs_log2, int64_t kb, int64_t row0)
 {
     const int lane = threadIdx.x & 63;
     const int64_t col = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
@@ -103,16 +115,15 @@ __global__ __launch_bounds__(256) void acc4_gemv_kernel(RocmMatMulNBitsArgs p, c
         for (int r = 0; r < ROWS; ++r) {
             int dot = 0;
             if (ok && r < rows) {
-                const uint2 c = *reinterpret_cast<const uint2*>(qa + (row0 + r) * padded_k + (d << 3));
-                const int even = static_cast<int>(__builtin_amdgcn_perm(c.y, c.x, 0x06040200u));
-                const int odd = static_cast<int>(__builtin_amdgcn_perm(c.y, c.x, 0x07050301u));
-                dot = __builtin_amdgcn_sdot4(even, lo, 0, false);
-                dot = __builtin_amdgcn_sdot4(odd, hi, dot, false);
+                const uint2 c = *reinterpret_cast<const uint2*>(qa + (row0 + r) * padded_k + (d << 3));   // interleaved: evens, odds
+                dot = __builtin_amdgcn_sdot4(static_cast<int>(c.x), lo, 0, false);
+                dot = __builtin_amdgcn_sdot4(static_cast<int>(c.y), hi, dot, false);
             }
             for (int off = 1; off < lanes_per_block; off <<= 1) dot += __shfl_xor(dot, off, 64);
             if (ok && r < rows && (lane & (lanes_per_block - 1)) == 0) {
-                const int block_acc = dot - z * qsum[(row0 + r) * kb + blk];
-                acc[r] += static_cast<float>(block_acc) * __fmul_rn(qscale[(row0 + r) * kb + blk], sb);
+                const float2 pair = *reinterpret_cast<const float2*>(aq + ((row0 + r) * kb + blk) * 2);
+                const int block_acc = dot - z * static_cast<int>(pair.y);
+                acc[r] += static_cast<float>(block_acc) * __fmul_rn(pair.x, sb);
             }
         }
     }
@@ -128,15 +139,27 @@ __global__ __launch_bounds__(256) void acc4_gemv_kernel(RocmMatMulNBitsArgs p, c
 
 }  // namespace mnb
 
-extern "C" int rocm_launch_quantize_a(const void* a, int a_dtype, int64_t m, int64_t k, int block_size, int rounding,
-                                      int8_t* qa, float* qscale, int32_t* qsum, rocm_stream_t stream)
+static int launch_quantize(const void* a, int a_dtype, int64_t m, int64_t k, int block_size, int rounding, int interleave,
+                           int8_t* qa, float* qscale, int32_t* qsum, float* aq, float* aux16, float* sa_t, rocm_stream_t stream)
 {
     if (m <= 0 || k <= 0) return 0;
     const int64_t kb = (k + block_size - 1) / block_size;
     const int64_t items = m * kb;
     hipLaunchKernelGGL(mnb::quantize_a_kernel, dim3(static_cast<unsigned>((items + 3) / 4)), dim3(256), 0, static_cast<hipStream_t>(stream),
-                       a, a_dtype, m, k, block_size, kb, rounding, qa, qscale, qsum);
+                       a, a_dtype, m, k, block_size, kb, rounding, interleave, qa, qscale, qsum, aq, aux16, sa_t);
     return static_cast<int>(hipGetLastError());
+}
+
+extern "C" int rocm_launch_quantize_a(const void* a, int a_dtype, int64_t m, int64_t k, int block_size, int rounding,
+                                      int8_t* qa, float* qscale, int32_t* qsum, rocm_stream_t stream)
+{
+    return launch_quantize(a, a_dtype, m, k, block_size, rounding, 0, qa, qscale, qsum, nullptr, nullptr, nullptr, stream);
+}
+
+extern "C" int rocm_launch_quantize_a_workspace(const void* a, int a_dtype, int64_t m, int64_t k, int block_size, int rounding,
+                                                const RocmAcc4Workspace* ws, rocm_stream_t stream)
+{
+    return launch_quantize(a, a_dtype, m, k, block_size, rounding, 1, ws->qa, nullptr, nullptr, ws->aq, m <= 16 ? ws->aux : nullptr, m > 16 ? ws->aux : nullptr, stream);
 }
 
 extern "C" int rocm_launch_block_acc_i32(const int8_t* qa, const uint8_t* b, const uint8_t* zp, int64_t m, int64_t n, int64_t k,
@@ -151,8 +174,7 @@ extern "C" int rocm_launch_block_acc_i32(const int8_t* qa, const uint8_t* b, con
     return static_cast<int>(hipGetLastError());
 }
 
-extern "C" int rocm_launch_acc4_gemv(const RocmMatMulNBitsArgs* args, const int8_t* qa, const float* qscale, const int32_t* qsum,
-                                     rocm_stream_t stream)
+extern "C" int rocm_launch_acc4_gemv(const RocmMatMulNBitsArgs* args, const RocmAcc4Workspace* ws, rocm_stream_t stream)
 {
     if (args->m <= 0 || args->n <= 0) return 0;
     const int bs_log2 = __builtin_ctz(static_cast<unsigned>(args->block_size));
@@ -161,12 +183,9 @@ extern "C" int rocm_launch_acc4_gemv(const RocmMatMulNBitsArgs* args, const int8
     constexpr int kRows = 4;
     for (int64_t row0 = 0; row0 < args->m; row0 += kRows) {
         if (args->m - row0 == 1)
-            hipLaunchKernelGGL(mnb::acc4_gemv_kernel<1>, grid, dim3(256), 0, static_cast<hipStream_t>(stream), *args, qa, qscale, qsum, bs_log2, kb, row0);
+            hipLaunchKernelGGL(mnb::acc4_gemv_kernel<1>, grid, dim3(256), 0, static_cast<hipStream_t>(stream), *args, ws->qa, ws->aq, bs_log2, kb, row0);
         else
-            hipLaunchKernelGGL(mnb::acc4_gemv_kernel<kRows>, grid, dim3(256), 0, static_cast<hipStream_t>(stream), *args, qa, qscale, qsum, bs_log2, kb, row0);
+            hipLaunchKernelGGL(mnb::acc4_gemv_kernel<kRows>, grid, dim3(256), 0, static_cast<hipStream_t>(stream), *args, ws->qa, ws->aq, bs_log2, kb, row0);
     }
     return static_cast<int>(hipGetLastError());
 }
-
-extern "C" int rocm_acc4_mfma_eligible(const RocmMatMulNBitsArgs*) { return 0; }
-extern "C" int rocm_launch_acc4_mfma(const RocmMatMulNBitsArgs*, const int8_t*, const float*, const int32_t*, rocm_stream_t) { return -1; }

@@ -1,0 +1,595 @@
+// accuracy_level = 4 on the int8 matrix cores.
+//
+// The activations arrive already quantized (see quantize_a_kernel): int8 codes, one f32 scale and
+// the sum of codes per (row, block). A 4-bit weight is used as the unsigned int8 0..15; the zero
+// point leaves through the code sums:
+//     acc[m,n,b] = sum_k code[m,k] * q[n,k]  -  zp[n,b] * sum_k code[m,k]          (exact integers)
+//     y[m,n]     = sum_b f32(acc[m,n,b]) * (scale_a[m,b] * scale_b[n,b]) + bias[n]
+// Both integer terms stay below 2^24 for every block size up to 256, so the subtraction is done in
+// f32 without rounding.
+//
+// Codes are stored "even/odd interleaved" inside every run of 8: positions 0..3 hold elements
+// 0,2,4,6 and positions 4..7 hold 1,3,5,7. That is the order in which `w & 0x0f0f0f0f` and
+// `(w >> 4) & 0x0f0f0f0f` deliver the eight weights of one packed dword, so unpacking costs three
+// instructions per dword and no byte shuffles.
+#include "mfma_common.hiph"
+
+namespace mnb {
+
+typedef __attribute__((ext_vector_type(4))) int int4_t;
+typedef __attribute__((ext_vector_type(16))) int int16_t_v;
+
+__device__ __forceinline__ long pack64(uint32_t lo, uint32_t hi)
+{
+    return static_cast<long>(static_cast<uint64_t>(lo) | (static_cast<uint64_t>(hi) << 32));
+}
+
+// ---------------------------------------------------------------------------------------------
+// Decode (M <= 16): split-K over the waves of a workgroup, v_mfma_i32_16x16x32_i8.
+// ---------------------------------------------------------------------------------------------
+
+struct Acc4DecodeParams {
+    const int8_t* qa;       // [M, padded_k] interleaved codes
+    const float* aq;        // [M, kb, 2]: scale_a, f32(sum of codes)
+    const float* aux16;     // [kb, 16, 2]: the same pairs, block-major, rows beyond M unspecified (M > 1 only)
+    const uint8_t* b;
+    const void* scales;
+    const uint8_t* zp;
+    const void* bias;
+    void* y;
+    int64_t m, n, kb;
+    int64_t padded_k;       // kb * BS
+    int64_t row_bytes;      // padded_k / 2
+    int64_t zp_row;         // ceil(kb / 2)
+    int tiles;              // ceil(padded_k / 128)
+    int tiles_per_wave;     // multiple of the group size
+    int bias_dtype, y_dtype;
+    int scales_bf16;        // 16-bit scales are bf16 (else f16)
+};
+
+constexpr int kCodePitch = 144;   // bytes between activation rows of one tile in LDS: 128 + 16
+
+template <int U, int NA, int NS, int NZ>
+struct Acc4Group {
+    uint4 w[U];
+    uint4 a[NA];
+    uint32_t s[NS];
+    uint32_t z[NZ];
+    uint4 x;     // MR = 1: .x/.y = (scale_a, code sum) of block `lane` of the group; MR = 16: 16 bytes of the group's aux16 rows
+};
+
+// BS: block size (32, 64, 128). MR: rows staged (1 or 16; M <= MR). ST: storage type of the scales.
+//
+// Lane (c = lane % 16, g = lane / 16) streams column c in 16-byte pieces, as the float decode kernel does.
+// A group is U tiles of 128 elements and NB = U * 128 / BS blocks. Per group a lane issues U weight loads,
+// one load of codes (MR = 1) or two per tile (MR = 16), NS scale loads (lane group g fetches block 4i + g),
+// NZ zero-point loads (lane group g fetches the byte of blocks 8i + 2g and 8i + 2g + 1) and one load of
+// the activation-side pairs; scale and zero point reach the other lane groups by shuffle when a block ends.
+template <int BS, int MR, typename ST>
+__global__ __launch_bounds__(512) void acc4_decode_kernel(Acc4DecodeParams p)
+{
+    constexpr bool kTranspose = BS < 128;
+    constexpr int NBT = 128 / BS;                       // blocks per tile
+    constexpr int U = MR == 1 ? 4 : 2;
+    constexpr int NB = U * NBT;                         // blocks per group
+    constexpr int NS = (NB + 3) / 4;
+    constexpr int NZ = (NB + 7) / 8;
+    constexpr int NA = MR == 1 ? 1 : 2 * U;
+    constexpr int kCodeStage = MR == 1 ? 1024 : 16 * kCodePitch;   // one staging buffer of codes (a group / a tile)
+    constexpr int kAuxStage = MR == 1 ? 0 : 1024;                  // one staging buffer of aux16 rows (a group)
+    constexpr int kWaveBytes = 2 * kCodeStage + 2 * kAuxStage;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int waves = blockDim.x >> 6;
+    const int c = lane & 15;
+    const int g = lane >> 4;
+    const int64_t n_base = static_cast<int64_t>(blockIdx.x) * 16;
+    const int64_t cols_left = p.n - n_base;
+    const bool has_zp = p.zp != nullptr;
+    const bool full_k = (p.padded_k & 127) == 0;
+    const bool bf16_scales = p.scales_bf16 != 0;
+
+    const __amdgpu_buffer_rsrc_t srd_b = make_srd(p.b + n_base * p.row_bytes, static_cast<uint64_t>(cols_left * p.row_bytes));
+    const __amdgpu_buffer_rsrc_t srd_s = make_srd(static_cast<const ST*>(p.scales) + n_base * p.kb, static_cast<uint64_t>(cols_left * p.kb) * sizeof(ST));
+    const __amdgpu_buffer_rsrc_t srd_z = make_srd(has_zp ? p.zp + n_base * p.zp_row : p.b, has_zp ? static_cast<uint64_t>(cols_left * p.zp_row) : 0);
+    const __amdgpu_buffer_rsrc_t srd_a = make_srd(p.qa, static_cast<uint64_t>(p.m * p.padded_k));
+    const __amdgpu_buffer_rsrc_t srd_x = MR == 1 ? make_srd(p.aq, static_cast<uint64_t>(p.kb) * 8) : make_srd(p.aux16, static_cast<uint64_t>(p.kb) * 128);
+
+    const uint32_t b_off = static_cast<uint32_t>(c) * static_cast<uint32_t>(p.row_bytes) + static_cast<uint32_t>(g * 16);
+    const uint32_t s_off = (static_cast<uint32_t>(c) * static_cast<uint32_t>(p.kb) + static_cast<uint32_t>(g)) * static_cast<uint32_t>(sizeof(ST));
+    const uint32_t z_off = static_cast<uint32_t>(c) * static_cast<uint32_t>(p.zp_row) + static_cast<uint32_t>(g);
+    // codes. MR = 1: piece `lane` (16 bytes) of the group's 512. MR = 16: row lane / 8 (+8), piece lane % 8 of a tile.
+    const uint32_t a_off = MR == 1 ? static_cast<uint32_t>(lane * 16)
+                                   : static_cast<uint32_t>(lane >> 3) * static_cast<uint32_t>(p.padded_k) + static_cast<uint32_t>((lane & 7) * 16);
+    unsigned char* stage = smem + wave * kWaveBytes;
+    unsigned char* aux_stage = stage + 2 * kCodeStage;
+    const uint32_t st_write = MR == 1 ? static_cast<uint32_t>(lane * 16) : static_cast<uint32_t>((lane >> 3) * kCodePitch + (lane & 7) * 16);
+    // operand of MFMA j: 8 codes at element j*32 + g*8 of the tile (transposed weights) or g*32 + j*8
+    const uint32_t st_read = (MR == 1 ? 0u : static_cast<uint32_t>(c * kCodePitch)) + static_cast<uint32_t>(kTranspose ? g * 8 : g * 32);
+    constexpr int kReadStep = kTranspose ? 32 : 8;
+
+    float y[4] = {0.f, 0.f, 0.f, 0.f};
+    int4_t acc = {0, 0, 0, 0};
+
+    const int t_begin = wave * p.tiles_per_wave;
+    const int t_end = min(t_begin + p.tiles_per_wave, p.tiles);
+
+    using Grp = Acc4Group<U, NA, NS, NZ>;
+    auto fetch_group = [&](Grp& grp, int t0) {
+        if (t0 >= t_end) return;
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            if (t0 + u < t_end) grp.w[u] = load16(srd_b, b_off, static_cast<uint32_t>(t0 + u) * 64u);
+        if constexpr (MR == 1) {
+            // the range check of srd_a ends the row at padded_k; tiles beyond this wave's share are not read
+            uint32_t off = a_off;
+            if (lane >= U * 8 || t0 + (lane >> 3) >= t_end) off = kOutOfRange;
+            grp.a[0] = load16(srd_a, off, static_cast<uint32_t>(t0) * 128u);
+            const int blocks = (min(t0 + U, t_end) - t0) * NBT;
+            const auto v = __builtin_amdgcn_raw_buffer_load_b64(srd_x, static_cast<int>(lane < blocks ? lane * 8 : kOutOfRange), static_cast<int>(t0 * NBT * 8), 0);
+            grp.x.x = v[0];
+            grp.x.y = v[1];
+        } else {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                if (t0 + u < t_end) {
+#pragma unroll
+                    for (int i = 0; i < 2; ++i) {
+                        uint32_t off = a_off + static_cast<uint32_t>(i * 8) * static_cast<uint32_t>(p.padded_k);
+                        if (!full_k && static_cast<int64_t>(t0 + u) * 128 + (lane & 7) * 16 >= p.padded_k) off = kOutOfRange;
+                        grp.a[u * 2 + i] = load16(srd_a, off, static_cast<uint32_t>(t0 + u) * 128u);
+                    }
+                }
+            }
+            grp.x = load16(srd_x, lane < NB * 8 ? static_cast<uint32_t>(lane * 16) : kOutOfRange, static_cast<uint32_t>(t0 * NBT) * 128u);
+        }
+#pragma unroll
+        for (int i = 0; i < NS; ++i)
+            grp.s[i] = ScaleIo<ST>::load(srd_s, (4 * i + g < NB) ? s_off : kOutOfRange, static_cast<uint32_t>(t0 * NBT + 4 * i) * static_cast<uint32_t>(sizeof(ST)));
+#pragma unroll
+        for (int i = 0; i < NZ; ++i)
+            grp.z[i] = has_zp ? static_cast<uint32_t>(__builtin_amdgcn_raw_buffer_load_b8(srd_z, static_cast<int>((8 * i + 2 * g < NB) ? z_off : kOutOfRange),
+                                                                                            static_cast<int>((t0 * NBT) / 2 + 4 * i), 0))
+                              : 0x88u;
+    };
+
+    // End of block `bi` of the group: y += f32(acc - zp * code_sum) * (scale_a * scale_b).
+    auto flush = [&](const Grp& grp, int bi, int t0, int parity) {
+        if (static_cast<int64_t>(t0) * NBT + bi >= p.kb) return;            // a block beyond K (wave-uniform)
+        const uint32_t s_raw = __shfl(grp.s[bi / 4], c + 16 * (bi % 4), kWave);
+        const uint32_t z_raw = __shfl(grp.z[bi / 8], c + 16 * ((bi / 2) % 4), kWave);
+        const float sb = ScaleIo<ST>::to_f32(s_raw, bf16_scales);
+        const float zf = static_cast<float>((z_raw >> ((bi & 1) * 4)) & 0xfu);
+        if constexpr (MR == 1) {
+            const float sa = __int_as_float(__builtin_amdgcn_readlane(static_cast<int>(grp.x.x), bi));
+            const float qs = __int_as_float(__builtin_amdgcn_readlane(static_cast<int>(grp.x.y), bi));
+            const float f = fmaf(-zf, qs, static_cast<float>(acc[0]));
+            y[0] = fmaf(f, __fmul_rn(sa, sb), y[0]);
+        } else {
+            const float4* rows = reinterpret_cast<const float4*>(aux_stage + parity * kAuxStage + bi * 128 + g * 32);
+            const float4 r01 = rows[0], r23 = rows[1];
+            const float sa[4] = {r01.x, r01.z, r23.x, r23.z};
+            const float qs[4] = {r01.y, r01.w, r23.y, r23.w};
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float f = fmaf(-zf, qs[r], static_cast<float>(acc[r]));
+                y[r] = fmaf(f, __fmul_rn(sa[r], sb), y[r]);
+            }
+        }
+    };
+
+    auto compute_tile = [&](const Grp& grp, int u, int t0, int parity) {
+        unsigned char* st = stage + (MR == 1 ? parity : (u & 1)) * kCodeStage;
+        if constexpr (MR != 1) {
+#pragma unroll
+            for (int i = 0; i < 2; ++i) *reinterpret_cast<uint4*>(st + st_write + i * 8 * kCodePitch) = grp.a[u * 2 + i];
+            lds_order();
+        }
+        long av[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) av[j] = *reinterpret_cast<const long*>(st + st_read + (MR == 1 ? u * 128 : 0) + j * kReadStep);
+        uint4 w = grp.w[u];
+        if constexpr (kTranspose) transpose_groups(w);
+        const uint32_t wd[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const bool first = kTranspose ? ((j * 32) % BS == 0) : (j == 0);
+            const bool last = kTranspose ? (((j + 1) * 32) % BS == 0) : (j == 3);
+            const long bw = pack64(wd[j] & 0x0f0f0f0fu, (wd[j] >> 4) & 0x0f0f0f0fu);
+            const int4_t zero = {0, 0, 0, 0};
+            acc = __builtin_amdgcn_mfma_i32_16x16x32_i8(av[j], bw, first ? zero : acc, 0, 0, 0);
+            if (last) flush(grp, u * NBT + (kTranspose ? (j * 32) / BS : 0), t0, parity);
+        }
+    };
+    auto run_group = [&](const Grp& cur, Grp& next, int t0, int parity) {
+        fetch_group(next, t0 + U);
+        if constexpr (MR == 1) {
+            *reinterpret_cast<uint4*>(stage + parity * kCodeStage + st_write) = cur.a[0];
+        } else {
+            *reinterpret_cast<uint4*>(aux_stage + parity * kAuxStage + lane * 16) = cur.x;
+        }
+        lds_order();
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            if (t0 + u < t_end) compute_tile(cur, u, t0, parity);
+    };
+
+    Grp ga, gb;
+    fetch_group(ga, t_begin);
+    for (int t0 = t_begin; t0 < t_end; t0 += 2 * U) {
+        run_group(ga, gb, t0, 0);
+        if (t0 + U < t_end) run_group(gb, ga, t0 + U, 1);
+    }
+
+    // ---- split-K reduction across the waves of this workgroup, in wave order ----
+    __syncthreads();
+    float* red = reinterpret_cast<float*>(smem);       // [waves][4][64]
+#pragma unroll
+    for (int r = 0; r < 4; ++r) red[(wave * 4 + r) * 64 + lane] = y[r];
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < 256; idx += blockDim.x) {
+        const int r = idx >> 6;
+        const int l = idx & 63;
+        const int row = 4 * (l >> 4) + r;
+        const int64_t col = n_base + (l & 15);
+        if (row < p.m && col < p.n) {
+            float total = 0.f;
+            for (int w = 0; w < waves; ++w) total += red[(w * 4 + r) * 64 + l];
+            if (p.bias) total += load_as_f32(p.bias, p.bias_dtype, col);
+            store_from_f32(p.y, p.y_dtype, static_cast<int64_t>(row) * p.n + col, total);
+        }
+    }
+}
+
+template <int BS, int MR, typename ST>
+static int launch_acc4_decode(const Acc4DecodeParams& p, int waves, hipStream_t stream)
+{
+    const unsigned grid = static_cast<unsigned>((p.n + 15) / 16);
+    const size_t stage = static_cast<size_t>(waves) * (MR == 1 ? 2048 : 2 * 16 * kCodePitch + 2048);
+    const size_t red = static_cast<size_t>(waves) * 1024;
+    hipLaunchKernelGGL((acc4_decode_kernel<BS, MR, ST>), dim3(grid), dim3(waves * 64), stage > red ? stage : red, stream, p);
+    return static_cast<int>(hipGetLastError());
+}
+
+template <typename ST>
+static int launch_acc4_decode_bs(const Acc4DecodeParams& p, int bs, int waves, hipStream_t stream)
+{
+    if (p.m <= 1) {
+        switch (bs) {
+            case 32: return launch_acc4_decode<32, 1, ST>(p, waves, stream);
+            case 64: return launch_acc4_decode<64, 1, ST>(p, waves, stream);
+            default: return launch_acc4_decode<128, 1, ST>(p, waves, stream);
+        }
+    }
+    switch (bs) {
+        case 32: return launch_acc4_decode<32, 16, ST>(p, waves, stream);
+        case 64: return launch_acc4_decode<64, 16, ST>(p, waves, stream);
+        default: return launch_acc4_decode<128, 16, ST>(p, waves, stream);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Prefill (M > 16): 128 x 128 tiles of Y, K in steps of 64 codes, v_mfma_i32_32x32x32_i8.
+// ---------------------------------------------------------------------------------------------
+//
+// Per step a workgroup of four waves copies 128 x 64 activation codes to LDS and unpacks 128 x 64 weights into
+// signed int8 (q - zp) beside them: with c = 0x80 - zp in every byte, (q + c) ^ 0x80 is q - zp in two's
+// complement and no byte ever borrows from its neighbour. The zero point therefore costs two instructions per
+// four weights here instead of one per accumulator. Each wave owns a 64 x 64 sub-tile (2 x 2 MFMA tiles). When a
+// block ends, every int32 accumulator is converted, scaled by scale_a[row] * scale_b[column] and added to the
+// f32 result: three VALU instructions per accumulator per block, which - not the matrix cores - bound this kernel.
+// Activation scales come block-major ([kb, M]) so that a step's 128 of them are one contiguous run.
+
+struct Acc4PrefillParams {
+    const int8_t* qa;       // [M, padded_k] interleaved codes
+    const float* sa_t;      // [kb, M] activation scales, block-major
+    const uint8_t* b;
+    const void* scales;
+    const uint8_t* zp;
+    const void* bias;
+    void* y;
+    int64_t m, n, kb;
+    int64_t padded_k, row_bytes, zp_row;
+    int bs_log2;
+    int scales_bf16;
+    int bias_dtype, y_dtype;
+};
+
+constexpr int kTile = 128;           // rows and columns of Y per workgroup
+constexpr int kStep = 64;            // codes of K per step
+constexpr int kPitch8 = 80;          // bytes per LDS row: 64 codes + 16 of padding (16 rows then cover all 64 banks)
+
+// NBS: blocks per step - 2 (block size 32), 1 (block size 64) or 0 (block size >= 128: a block spans several steps).
+// SF32: scales stored as f32 (else 16 bits, f16 or bf16 by a run-time flag).
+template <int NBS, bool SF32>
+__global__ __launch_bounds__(256) void acc4_prefill_kernel(Acc4PrefillParams p)
+{
+    constexpr int kSlots = NBS == 2 ? 2 : 1;                   // scale slots per step
+    constexpr int kBufBytes = 2 * kTile * kPitch8 + 2 * kSlots * kTile * 4;
+    constexpr int TM = 2, TN = 2;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+    const int t = threadIdx.x;
+    const int lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int64_t m_base = static_cast<int64_t>(blockIdx.y) * kTile;
+    const int64_t n_base = static_cast<int64_t>(blockIdx.x) * kTile;
+    const int64_t rows_left = p.m - m_base, cols_left = p.n - n_base;
+    const bool has_zp = p.zp != nullptr;
+    const bool ragged_k = (p.padded_k & 63) != 0;
+    constexpr uint32_t kScaleBytes = SF32 ? 4 : 2;
+
+    const __amdgpu_buffer_rsrc_t srd_a = make_srd(p.qa + m_base * p.padded_k, static_cast<uint64_t>(rows_left * p.padded_k));
+    const __amdgpu_buffer_rsrc_t srd_b = make_srd(p.b + n_base * p.row_bytes, static_cast<uint64_t>(cols_left * p.row_bytes));
+    const __amdgpu_buffer_rsrc_t srd_s = make_srd(static_cast<const unsigned char*>(p.scales) + n_base * p.kb * kScaleBytes,
+                                                  static_cast<uint64_t>(cols_left * p.kb) * kScaleBytes);
+    const __amdgpu_buffer_rsrc_t srd_z = make_srd(has_zp ? p.zp + n_base * p.zp_row : p.b, has_zp ? static_cast<uint64_t>(cols_left * p.zp_row) : 0);
+    const __amdgpu_buffer_rsrc_t srd_sa = make_srd(p.sa_t, static_cast<uint64_t>(p.kb * p.m) * 4);
+
+    // codes: thread -> (row t/4 + 64 i, piece t%4). weights: thread -> (column t/2, half t%2 of the step).
+    const uint32_t a_goff = static_cast<uint32_t>(t >> 2) * static_cast<uint32_t>(p.padded_k) + static_cast<uint32_t>((t & 3) * 16);
+    const uint32_t a_gstep = 64u * static_cast<uint32_t>(p.padded_k);
+    const uint32_t a_loff = static_cast<uint32_t>((t >> 2) * kPitch8 + (t & 3) * 16);
+    const int bcol = t >> 1, bhalf = t & 1;
+    const uint32_t b_goff = static_cast<uint32_t>(bcol) * static_cast<uint32_t>(p.row_bytes) + static_cast<uint32_t>(bhalf * 16);
+    const uint32_t b_loff = static_cast<uint32_t>(kTile * kPitch8 + bcol * kPitch8 + bhalf * 32);
+    const uint32_t s_goff = static_cast<uint32_t>(bcol) * static_cast<uint32_t>(p.kb) * kScaleBytes;
+    const uint32_t z_goff = static_cast<uint32_t>(bcol) * static_cast<uint32_t>(p.zp_row);
+    // activation scales: thread -> (slot t/128, row t%128)
+    const int sa_slot = t >> 7, sa_row = t & 127;
+    const uint32_t sa_goff = (sa_slot < kSlots && m_base + sa_row < p.m) ? static_cast<uint32_t>(m_base + sa_row) * 4u : kOutOfRange;
+    constexpr int kSaOff = 2 * kTile * kPitch8;                 // [kSlots][128] f32 activation scales of the step
+    constexpr int kSbOff = kSaOff + kSlots * kTile * 4;         // [kSlots][128] f32 weight scales of the step
+
+    // MFMA operand reads: lane (r = lane % 32, h = lane / 32) reads 16 consecutive codes of row r.
+    const uint32_t frag_off = static_cast<uint32_t>((lane & 31) * kPitch8 + (lane >> 5) * 16);
+
+    int16_t_v acc[TM][TN];
+    float y[TM][TN][16];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                acc[i][j][r] = 0;
+                y[i][j][r] = 0.f;
+            }
+
+    const int steps = static_cast<int>((p.padded_k + kStep - 1) / kStep);
+    constexpr int D = 4;
+    struct Regs {
+        uint4 a[2];
+        uint4 b;
+        uint32_t s, z, sa;
+    };
+    Regs regs[D];
+
+    auto block_of = [&](int kt, int half) -> uint32_t { return static_cast<uint32_t>((kt * kStep + half * 32) >> p.bs_log2); };
+    auto load_global = [&](Regs& r, int kt) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            uint32_t off = a_goff + static_cast<uint32_t>(i) * a_gstep;
+            if (ragged_k && static_cast<int64_t>(kt) * kStep + (t & 3) * 16 >= p.padded_k) off = kOutOfRange;   // else the next row's codes
+            r.a[i] = load16(srd_a, off, static_cast<uint32_t>(kt) * 64u);
+        }
+        r.b = load16(srd_b, b_goff, static_cast<uint32_t>(kt) * 32u);
+        const uint32_t blk = block_of(kt, bhalf);
+        if constexpr (SF32) r.s = __builtin_amdgcn_raw_buffer_load_b32(srd_s, static_cast<int>(s_goff + blk * 4u), 0, 0);
+        else r.s = __builtin_amdgcn_raw_buffer_load_b16(srd_s, static_cast<int>(s_goff + blk * 2u), 0, 0);
+        const uint32_t zbyte = has_zp ? static_cast<uint32_t>(__builtin_amdgcn_raw_buffer_load_b8(srd_z, static_cast<int>(z_goff + (blk >> 1)), 0, 0)) : 0x88u;
+        r.z = zbyte | ((blk & 1u) << 8);
+        r.sa = __builtin_amdgcn_raw_buffer_load_b32(srd_sa, static_cast<int>(sa_goff), static_cast<int>(block_of(kt, sa_slot) * static_cast<uint32_t>(p.m) * 4u), 0);
+    };
+    // Quarter `part` of a step's trip from registers into LDS buffer `buf`.
+    auto store_part = [&](const Regs& r, int buf, int part) {
+        unsigned char* base = smem + buf * kBufBytes;
+        if (part < 2) *reinterpret_cast<uint4*>(base + a_loff + part * 64 * kPitch8) = r.a[part];
+        const uint32_t w = part == 0 ? r.b.x : part == 1 ? r.b.y : part == 2 ? r.b.z : r.b.w;
+        const uint32_t zq = (r.z >> ((r.z >> 8) * 4u)) & 0xfu;
+        const uint32_t c4 = 0x80808080u - zq * 0x01010101u;
+        const uint32_t lo = ((w & 0x0f0f0f0fu) + c4) ^ 0x80808080u;            // elements 0,2,4,6 of the dword, minus zp
+        const uint32_t hi = (((w >> 4) & 0x0f0f0f0fu) + c4) ^ 0x80808080u;     // elements 1,3,5,7
+        *reinterpret_cast<uint2*>(base + b_loff + part * 8) = make_uint2(lo, hi);
+        if (part == 2 && bhalf < kSlots) {
+            const float sc = SF32 ? __uint_as_float(r.s) : (p.scales_bf16 ? __uint_as_float(r.s << 16) : f16_bits_to_f32(static_cast<uint16_t>(r.s)));
+            *reinterpret_cast<float*>(base + kSbOff + (bhalf * kTile + bcol) * 4) = sc;
+        }
+        if (part == 3 && sa_slot < kSlots) *reinterpret_cast<uint32_t*>(base + kSaOff + t * 4) = r.sa;
+    };
+    auto store_lds = [&](const Regs& r, int buf) {
+#pragma unroll
+        for (int part = 0; part < 4; ++part) store_part(r, buf, part);
+    };
+    // y += f32(acc) * (scale_a[row] * scale_b[column]) for the block in scale slot `slot` of buffer `buf`.
+    auto flush = [&](int buf, int slot) {
+        const unsigned char* base = smem + buf * kBufBytes;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const float sb = *reinterpret_cast<const float*>(base + kSbOff + (slot * kTile + wn * 64 + j * 32 + (lane & 31)) * 4);
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const float4 sa = *reinterpret_cast<const float4*>(base + kSaOff + (slot * kTile + wm * 64 + i * 32 + q * 8 + (lane >> 5) * 4) * 4);
+                    const float sav[4] = {sa.x, sa.y, sa.z, sa.w};
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        y[i][j][q * 4 + r] = fmaf(static_cast<float>(acc[i][j][q * 4 + r]), __fmul_rn(sav[r], sb), y[i][j][q * 4 + r]);
+                }
+            }
+        }
+    };
+    auto compute = [&](int buf, int kt, const Regs& next, bool store_next) {
+        const unsigned char* la = smem + buf * kBufBytes + wm * (64 * kPitch8) + frag_off;
+        const unsigned char* lb = smem + buf * kBufBytes + kTile * kPitch8 + wn * (64 * kPitch8) + frag_off;
+        // block size >= 128: the step opens / closes a block (wave-uniform)
+        const bool opens = NBS != 0 || ((kt * kStep) & ((1 << p.bs_log2) - 1)) == 0;
+        const bool closes = NBS != 0 || (((kt + 1) * kStep) & ((1 << p.bs_log2) - 1)) == 0;
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk) {
+            u32x4_t fa[TM], fb[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i) fa[i] = *reinterpret_cast<const u32x4_t*>(la + i * 32 * kPitch8 + kk * 32);
+#pragma unroll
+            for (int j = 0; j < TN; ++j) fb[j] = *reinterpret_cast<const u32x4_t*>(lb + j * 32 * kPitch8 + kk * 32);
+            const bool first = NBS == 2 ? true : (kk == 0 && opens);
+            const int16_t_v zero = {};
+            if (first) {
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(int4_t, fa[i]), __builtin_bit_cast(int4_t, fb[j]), zero, 0, 0, 0);
+            } else {
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(int4_t, fa[i]), __builtin_bit_cast(int4_t, fb[j]), acc[i][j], 0, 0, 0);
+            }
+            if (store_next) {
+                store_part(next, buf ^ 1, 2 * kk);
+                store_part(next, buf ^ 1, 2 * kk + 1);
+            }
+            if (NBS == 2) {
+                if (static_cast<int64_t>(kt) * 2 + kk < p.kb) flush(buf, kk);
+            } else if (kk == 1 && closes) {
+                flush(buf, 0);
+            }
+        }
+    };
+
+#pragma unroll
+    for (int s0 = 0; s0 < D - 1; ++s0) load_global(regs[s0], s0);
+    store_lds(regs[0], 0);
+    __syncthreads();
+    for (int kt0 = 0; kt0 < steps; kt0 += D) {
+#pragma unroll
+        for (int s0 = 0; s0 < D; ++s0) {
+            const int kt = kt0 + s0;
+            load_global(regs[(s0 + D - 1) % D], kt + D - 1);
+            if (kt < steps) {
+                compute(s0 & 1, kt, regs[(s0 + 1) % D], kt + 1 < steps);
+                __syncthreads();
+            }
+        }
+    }
+
+    // Epilogue. A 32x32 accumulator holds, in lane l, column l % 32 and rows 8 q + 4 (l / 32) + r (q, r = 0..3).
+    const int col_in_tile = lane & 31;
+    const int row_group = (lane >> 5) * 4;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const int64_t col = n_base + wn * 64 + j * 32 + col_in_tile;
+        if (col >= p.n) continue;
+        const float bias = p.bias ? load_as_f32(p.bias, p.bias_dtype, col) : 0.f;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int64_t row = m_base + wm * 64 + i * 32 + q * 8 + row_group + r;
+                    if (row < p.m) store_from_f32(p.y, p.y_dtype, row * p.n + col, y[i][j][q * 4 + r] + bias);
+                }
+            }
+        }
+    }
+}
+
+template <int NBS, bool SF32>
+static int launch_acc4_prefill(const Acc4PrefillParams& p, hipStream_t stream)
+{
+    const dim3 grid(static_cast<unsigned>((p.n + kTile - 1) / kTile), static_cast<unsigned>((p.m + kTile - 1) / kTile));
+    const size_t lds = 2 * (2 * kTile * kPitch8 + 2 * (NBS == 2 ? 2 : 1) * kTile * 4);
+    hipLaunchKernelGGL((acc4_prefill_kernel<NBS, SF32>), grid, dim3(256), lds, stream, p);
+    return static_cast<int>(hipGetLastError());
+}
+
+}  // namespace mnb
+
+extern "C" int rocm_acc4_mfma_eligible(const RocmMatMulNBitsArgs* a)
+{
+    if (a->m < 1 || a->n < 1 || a->block_size < 32) return 0;
+    const int64_t kb = (a->k + a->block_size - 1) / a->block_size;
+    const int64_t padded_k = kb * a->block_size;
+    if ((reinterpret_cast<uintptr_t>(a->b) & 15) != 0 || (reinterpret_cast<uintptr_t>(a->scales) & 3) != 0) return 0;
+    if (a->m <= 16) {
+        const bool bs_ok = a->block_size == 32 || a->block_size == 64 || a->block_size == 128;
+        return bs_ok && padded_k / 2 * 16 < 0x7fffffff && a->m * padded_k < 0x7ffffff0;
+    }
+    // prefill: 32-bit offsets inside one 128-row / 128-column window and inside the block-major scales
+    return padded_k / 2 * 128 < 0x7fffffff && padded_k * 128 < 0x7fffffff && kb * a->m * 4 < 0x7fffffff;
+}
+
+extern "C" int rocm_launch_acc4_mfma(const RocmMatMulNBitsArgs* a, const RocmAcc4Workspace* ws, int waves, rocm_stream_t stream)
+{
+    if (!rocm_acc4_mfma_eligible(a)) return -1;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (a->m > 16) {
+        mnb::Acc4PrefillParams q;
+        q.qa = ws->qa;
+        q.sa_t = ws->aux;
+        q.b = a->b;
+        q.scales = a->scales;
+        q.zp = a->zp;
+        q.bias = a->bias;
+        q.y = a->y;
+        q.m = a->m;
+        q.n = a->n;
+        q.kb = (a->k + a->block_size - 1) / a->block_size;
+        q.padded_k = q.kb * a->block_size;
+        q.row_bytes = q.padded_k / 2;
+        q.zp_row = (q.kb + 1) / 2;
+        q.bs_log2 = __builtin_ctz(static_cast<unsigned>(a->block_size));
+        q.scales_bf16 = a->scale_dtype == ROCM_DT_BF16;
+        q.bias_dtype = a->bias_dtype;
+        q.y_dtype = a->y_dtype;
+        const bool sf32 = a->scale_dtype == ROCM_DT_F32;
+        if (a->block_size == 32) return sf32 ? mnb::launch_acc4_prefill<2, true>(q, s) : mnb::launch_acc4_prefill<2, false>(q, s);
+        if (a->block_size == 64) return sf32 ? mnb::launch_acc4_prefill<1, true>(q, s) : mnb::launch_acc4_prefill<1, false>(q, s);
+        return sf32 ? mnb::launch_acc4_prefill<0, true>(q, s) : mnb::launch_acc4_prefill<0, false>(q, s);
+    }
+    mnb::Acc4DecodeParams p;
+    p.qa = ws->qa;
+    p.aq = ws->aq;
+    p.aux16 = ws->aux;
+    p.b = a->b;
+    p.scales = a->scales;
+    p.zp = a->zp;
+    p.bias = a->bias;
+    p.y = a->y;
+    p.m = a->m;
+    p.n = a->n;
+    p.kb = (a->k + a->block_size - 1) / a->block_size;
+    p.padded_k = p.kb * a->block_size;
+    p.row_bytes = p.padded_k / 2;
+    p.zp_row = (p.kb + 1) / 2;
+    p.tiles = static_cast<int>((p.padded_k + 127) / 128);
+    p.bias_dtype = a->bias_dtype;
+    p.y_dtype = a->y_dtype;
+    p.scales_bf16 = a->scale_dtype == ROCM_DT_BF16;
+
+    const int group_tiles = a->m <= 1 ? 4 : 2;
+    int w = waves;
+    if (w <= 0) {
+        const int64_t wgs = (a->n + 15) / 16;
+        const int want = static_cast<int>((8192 + wgs - 1) / wgs);
+        int by_work = p.tiles / group_tiles;
+        if (by_work < 1) by_work = 1;
+        w = want < by_work ? want : by_work;
+        if (w < 1) w = 1;
+    }
+    if (w > 8) w = 8;
+    int tpw = (p.tiles + w - 1) / w;
+    tpw = (tpw + group_tiles - 1) / group_tiles * group_tiles;
+    w = (p.tiles + tpw - 1) / tpw;
+    p.tiles_per_wave = tpw;
+
+    if (a->scale_dtype == ROCM_DT_F32) return mnb::launch_acc4_decode_bs<float>(p, a->block_size, w, s);
+    return mnb::launch_acc4_decode_bs<uint16_t>(p, a->block_size, w, s);
+}

@@ -20,14 +20,13 @@
 // flight. Activations travel with their tile in the most compact form (one 16-byte piece per lane
 // per four rows) and are turned into MFMA operand order through a small wave-private LDS buffer,
 // whose reads are counted separately from global loads and so never drain the prefetch queue.
-#include "common.hiph"
+#include "mfma_common.hiph"
 
 namespace mnb {
 
 typedef __attribute__((ext_vector_type(8))) _Float16 half8_t;
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float float4_t;
-typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
 
 struct DecodeParams {
     const uint16_t* a;
@@ -50,20 +49,7 @@ template <bool BF16> struct Magic;
 template <> struct Magic<false> { static constexpr uint32_t pos = 0x64006400u, neg = 0xE400E400u; };
 template <> struct Magic<true> { static constexpr uint32_t pos = 0x43004300u, neg = 0xC300C300u; };
 
-constexpr uint32_t kOutOfRange = 0x7ffffff0u;   // an offset beyond any range this kernel sets up: the load returns zeros
 constexpr int kRowPitch = 272;                   // bytes between activation rows in LDS: 256 + 16, so 16 rows hit 64 distinct banks
-
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_srd(const void* base, uint64_t bytes)
-{
-    const uint32_t range = bytes > 0x7fffffffull ? 0x7fffffffu : static_cast<uint32_t>(bytes);
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, static_cast<int>(range), 0x00020000);
-}
-
-__device__ __forceinline__ uint4 load16(__amdgpu_buffer_rsrc_t srd, uint32_t voffset, uint32_t soffset)
-{
-    const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(srd, static_cast<int>(voffset), static_cast<int>(soffset), 0);
-    return make_uint4(v.x, v.y, v.z, v.w);
-}
 
 template <bool BF16>
 __device__ __forceinline__ float4_t mfma16(const uint4& act, const uint4& wgt, float4_t acc)
@@ -92,30 +78,6 @@ __device__ __forceinline__ uint4 unpack8(uint32_t w, uint32_t mask, uint32_t mag
     r.w = and_or(__builtin_amdgcn_perm(w4, w, 0x0c070c03u), mask, magic);
     return r;
 }
-
-// 4x4 transpose of dwords across the four 16-lane groups: afterwards group g holds, in component d,
-// what group d held in component g.
-__device__ __forceinline__ void transpose_groups(uint4& v)
-{
-    auto s0 = __builtin_amdgcn_permlane32_swap(v.x, v.z, false, false);
-    auto s1 = __builtin_amdgcn_permlane32_swap(v.y, v.w, false, false);
-    auto t0 = __builtin_amdgcn_permlane16_swap(s0[0], s1[0], false, false);
-    auto t1 = __builtin_amdgcn_permlane16_swap(s0[1], s1[1], false, false);
-    v.x = t0[0];
-    v.y = t0[1];
-    v.z = t1[0];
-    v.w = t1[1];
-}
-
-template <typename ST> struct ScaleIo;
-template <> struct ScaleIo<float> {
-    static __device__ __forceinline__ uint32_t load(__amdgpu_buffer_rsrc_t srd, uint32_t v, uint32_t s) { return __builtin_amdgcn_raw_buffer_load_b32(srd, static_cast<int>(v), static_cast<int>(s), 0); }
-    static __device__ __forceinline__ float to_f32(uint32_t raw, bool) { return __uint_as_float(raw); }
-};
-template <> struct ScaleIo<uint16_t> {
-    static __device__ __forceinline__ uint32_t load(__amdgpu_buffer_rsrc_t srd, uint32_t v, uint32_t s) { return __builtin_amdgcn_raw_buffer_load_b16(srd, static_cast<int>(v), static_cast<int>(s), 0); }
-    static __device__ __forceinline__ float to_f32(uint32_t raw, bool bf16) { return bf16 ? __uint_as_float(raw << 16) : f16_bits_to_f32(static_cast<uint16_t>(raw)); }
-};
 
 // One group of U tiles held in registers: packed weights of CG column groups, the activations in compact
 // form, scales and zero points. NA / NS count the activation / scale loads of a group (see the kernel).
@@ -249,12 +211,6 @@ __global__ __launch_bounds__(512) void decode_mfma_kernel(DecodeParams p)
                 }
             }
         }
-    };
-    // LDS operations of one wave execute in issue order; the fences only keep the compiler from reordering them.
-    auto lds_order = [&]() {
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     };
     auto compute_tile = [&](const Grp& grp, int u, int parity) {
         // activations: compact registers -> LDS -> MFMA operand order

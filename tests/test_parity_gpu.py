@@ -347,6 +347,21 @@ ACC4_CASES = [
     (E.BF16, 128, True, 3, 77, 1024),
     (E.F16, 32, True, 20, 64, 256),
     (E.F32, 16, True, 2, 40, 80),
+    (E.F16, 64, True, 1, 333, 64 * 37),       # odd block count, ragged N, several waves per workgroup
+    (E.BF16, 32, True, 16, 48, 32 * 9),
+    (E.F32, 128, False, 2, 17, 128 * 3),
+    (E.F16, 64, True, 1, 64, 200),            # K ends inside a block
+    (E.F16, 32, False, 7, 130, 4096),
+    (E.F16, 128, True, 1, 512, 8192),
+    (E.BF16, 128, True, 9, 100, 128 * 5 + 64),
+    # M > 16: tiled int8 MFMA kernel
+    (E.F16, 64, True, 130, 200, 64 * 9),      # ragged M and N tiles
+    (E.F16, 32, True, 33, 64, 32 * 7),        # K ends in the middle of a 64-code step
+    (E.BF16, 128, False, 64, 128, 128 * 6),
+    (E.F32, 256, True, 40, 96, 256 * 3),
+    (E.F16, 64, True, 256, 256, 2048),
+    (E.F16, 32, False, 17, 130, 200),         # K ends inside a block
+    (E.F16, 16, True, 20, 64, 256),           # block size 16: not a matrix-core shape
 ]
 
 
@@ -359,7 +374,8 @@ def test_acc4_outputs(port, ref, a_dt, bs, zero_points, m, n, k, rounding):
         a = synth.make_activation(m, k, 80, a_dt)
         bias = synth.to_dtype(np.linspace(-1, 1, n).astype(np.float32), a_dt)
         y32, variant = run_op(provider, a, a_dt, b, s, a_dt, zp, n, k, bs, accuracy_level=4, bias=bias, bias_dtype=a_dt, y_dtype=E.F32)
-        assert variant.startswith("acc4")
+        on_matrix_cores = bs in (32, 64, 128) if m <= 16 else bs >= 32
+        assert variant == ("acc4_mfma_i8" if on_matrix_cores else "acc4_gemv_dot4")
         rnd = oracle.ROUND_HALF_EVEN if rounding == "mlas" else oracle.ROUND_HALF_AWAY
         af, sf, bf = synth.to_f32(a, a_dt), synth.to_f32(s, a_dt), synth.to_f32(bias, a_dt)
         want = port.matmul_acc4_f32(af, b, sf, zp, n, k, bs, rnd, bias=bf)
@@ -370,6 +386,23 @@ def test_acc4_outputs(port, ref, a_dt, bs, zero_points, m, n, k, rounding):
                 assert helpers.rel_l2(y32, y_ref) <= TOL_F32
         y, _ = run_op(provider, a, a_dt, b, s, a_dt, zp, n, k, bs, accuracy_level=4, bias=bias, bias_dtype=a_dt)
         assert np.array_equal(np.asarray(y).view(NPDT[a_dt] if a_dt != E.F32 else np.float32), np.asarray(port.narrow(y32, a_dt)))
+    finally:
+        provider.shutdown()
+
+
+@pytest.mark.parametrize("waves", [1, 3, 8])
+@pytest.mark.parametrize("s_dt", [E.F32, E.F16])
+def test_acc4_decode_wave_counts_agree(port, waves, s_dt):
+    a_dt, bs, n, k = E.F16, 64, 100, 64 * 50
+    provider = E.RocmExecutionProvider(0, {"decode_waves": str(waves)})
+    try:
+        b, s, zp = synth.make_weights(n, k, bs, 95, zero_points=True, scale_lo=0.002, scale_hi=0.01, scale_dtype=s_dt)
+        for m in (1, 6):
+            a = synth.make_activation(m, k, 95 + m, a_dt)
+            y32, variant = run_op(provider, a, a_dt, b, s, s_dt, zp, n, k, bs, accuracy_level=4, y_dtype=E.F32)
+            assert variant == "acc4_mfma_i8"
+            want = port.matmul_acc4_f32(synth.to_f32(a, a_dt), b, synth.to_f32(s, s_dt), zp, n, k, bs, oracle.ROUND_HALF_EVEN)
+            assert helpers.rel_l2(y32, want) <= TOL_F32
     finally:
         provider.shutdown()
 
