@@ -274,10 +274,10 @@ static int launch_acc4_decode_bs(const Acc4DecodeParams& p, int bs, int waves, h
 // Prefill (M > 16): 128 x 128 tiles of Y, K in steps of 64 codes, v_mfma_i32_32x32x32_i8.
 // ---------------------------------------------------------------------------------------------
 //
-// Per step a workgroup of four waves copies 128 x 64 activation codes to LDS and unpacks 128 x 64 weights into
+// Per step a workgroup of eight waves copies 128 x 64 activation codes to LDS and unpacks 128 x 64 weights into
 // signed int8 (q - zp) beside them: with c = 0x80 - zp in every byte, (q + c) ^ 0x80 is q - zp in two's
 // complement and no byte ever borrows from its neighbour. The zero point therefore costs two instructions per
-// four weights here instead of one per accumulator. Each wave owns a 64 x 64 sub-tile (2 x 2 MFMA tiles). When a
+// four weights here instead of one per accumulator. When a
 // block ends, every int32 accumulator is converted, scaled by scale_a[row] * scale_b[column] and added to the
 // f32 result: three VALU instructions per accumulator per block, which - not the matrix cores - bound this kernel.
 // Activation scales come block-major ([kb, M]) so that a step's 128 of them are one contiguous run.
@@ -303,12 +303,15 @@ constexpr int kPitch8 = 80;          // bytes per LDS row: 64 codes + 16 of padd
 
 // NBS: blocks per step - 2 (block size 32), 1 (block size 64) or 0 (block size >= 128: a block spans several steps).
 // SF32: scales stored as f32 (else 16 bits, f16 or bf16 by a run-time flag).
+// Eight waves, 4 (rows) x 2 (columns); each owns a 32 x 64 sub-tile: two MFMA tiles, 32 f32 results per lane. The
+// small per-wave state leaves room for four waves per SIMD, which is what overlaps one wave's flush arithmetic
+// with another's MFMAs.
 template <int NBS, bool SF32>
-__global__ __launch_bounds__(256) void acc4_prefill_kernel(Acc4PrefillParams p)
+__global__ __launch_bounds__(512) void acc4_prefill_kernel(Acc4PrefillParams p)
 {
     constexpr int kSlots = NBS == 2 ? 2 : 1;                   // scale slots per step
     constexpr int kBufBytes = 2 * kTile * kPitch8 + 2 * kSlots * kTile * 4;
-    constexpr int TM = 2, TN = 2;
+    constexpr int TN = 2;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
     const int t = threadIdx.x;
@@ -329,15 +332,14 @@ __global__ __launch_bounds__(256) void acc4_prefill_kernel(Acc4PrefillParams p)
     const __amdgpu_buffer_rsrc_t srd_z = make_srd(has_zp ? p.zp + n_base * p.zp_row : p.b, has_zp ? static_cast<uint64_t>(cols_left * p.zp_row) : 0);
     const __amdgpu_buffer_rsrc_t srd_sa = make_srd(p.sa_t, static_cast<uint64_t>(p.kb * p.m) * 4);
 
-    // codes: thread -> (row t/4 + 64 i, piece t%4). weights: thread -> (column t/2, half t%2 of the step).
-    const uint32_t a_goff = static_cast<uint32_t>(t >> 2) * static_cast<uint32_t>(p.padded_k) + static_cast<uint32_t>((t & 3) * 16);
-    const uint32_t a_gstep = 64u * static_cast<uint32_t>(p.padded_k);
-    const uint32_t a_loff = static_cast<uint32_t>((t >> 2) * kPitch8 + (t & 3) * 16);
-    const int bcol = t >> 1, bhalf = t & 1;
-    const uint32_t b_goff = static_cast<uint32_t>(bcol) * static_cast<uint32_t>(p.row_bytes) + static_cast<uint32_t>(bhalf * 16);
-    const uint32_t b_loff = static_cast<uint32_t>(kTile * kPitch8 + bcol * kPitch8 + bhalf * 32);
-    const uint32_t s_goff = static_cast<uint32_t>(bcol) * static_cast<uint32_t>(p.kb) * kScaleBytes;
-    const uint32_t z_goff = static_cast<uint32_t>(bcol) * static_cast<uint32_t>(p.zp_row);
+    // codes: thread -> (row t/4, 16-byte piece t%4). weights: thread -> (column t/4, 8-byte quarter t%4 of the step).
+    const int prow = t >> 2, quarter = t & 3;
+    const uint32_t a_goff = static_cast<uint32_t>(prow) * static_cast<uint32_t>(p.padded_k) + static_cast<uint32_t>(quarter * 16);
+    const uint32_t a_loff = static_cast<uint32_t>(prow * kPitch8 + quarter * 16);
+    const uint32_t b_goff = static_cast<uint32_t>(prow) * static_cast<uint32_t>(p.row_bytes) + static_cast<uint32_t>(quarter * 8);
+    const uint32_t b_loff = static_cast<uint32_t>(kTile * kPitch8 + prow * kPitch8 + quarter * 16);
+    const uint32_t s_goff = static_cast<uint32_t>(prow) * static_cast<uint32_t>(p.kb) * kScaleBytes;
+    const uint32_t z_goff = static_cast<uint32_t>(prow) * static_cast<uint32_t>(p.zp_row);
     // activation scales: thread -> (slot t/128, row t%128)
     const int sa_slot = t >> 7, sa_row = t & 127;
     const uint32_t sa_goff = (sa_slot < kSlots && m_base + sa_row < p.m) ? static_cast<uint32_t>(m_base + sa_row) * 4u : kOutOfRange;
@@ -347,125 +349,130 @@ __global__ __launch_bounds__(256) void acc4_prefill_kernel(Acc4PrefillParams p)
     // MFMA operand reads: lane (r = lane % 32, h = lane / 32) reads 16 consecutive codes of row r.
     const uint32_t frag_off = static_cast<uint32_t>((lane & 31) * kPitch8 + (lane >> 5) * 16);
 
-    int16_t_v acc[TM][TN];
-    float y[TM][TN][16];
+    int16_t_v acc[NBS == 0 ? TN : 1];   // integer accumulators that outlive a step (block size >= 128 only)
+    float y[TN][16];
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+    for (int j = 0; j < TN; ++j)
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                acc[i][j][r] = 0;
-                y[i][j][r] = 0.f;
-            }
+        for (int r = 0; r < 16; ++r) y[j][r] = 0.f;
 
     const int steps = static_cast<int>((p.padded_k + kStep - 1) / kStep);
+    // Global loads run D-1 steps ahead of the MFMAs, in D register sets.
     constexpr int D = 4;
     struct Regs {
-        uint4 a[2];
-        uint4 b;
+        uint4 a;
+        uint2 b;
         uint32_t s, z, sa;
     };
     Regs regs[D];
 
-    auto block_of = [&](int kt, int half) -> uint32_t { return static_cast<uint32_t>((kt * kStep + half * 32) >> p.bs_log2); };
+    auto block_of = [&](int kt, int offset) -> uint32_t { return static_cast<uint32_t>((kt * kStep + offset) >> p.bs_log2); };
     auto load_global = [&](Regs& r, int kt) {
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            uint32_t off = a_goff + static_cast<uint32_t>(i) * a_gstep;
-            if (ragged_k && static_cast<int64_t>(kt) * kStep + (t & 3) * 16 >= p.padded_k) off = kOutOfRange;   // else the next row's codes
-            r.a[i] = load16(srd_a, off, static_cast<uint32_t>(kt) * 64u);
-        }
-        r.b = load16(srd_b, b_goff, static_cast<uint32_t>(kt) * 32u);
-        const uint32_t blk = block_of(kt, bhalf);
+        uint32_t off = a_goff;
+        if (ragged_k && static_cast<int64_t>(kt) * kStep + quarter * 16 >= p.padded_k) off = kOutOfRange;   // else the next row's codes
+        r.a = load16(srd_a, off, static_cast<uint32_t>(kt) * 64u);
+        const auto w = __builtin_amdgcn_raw_buffer_load_b64(srd_b, static_cast<int>(b_goff), static_cast<int>(kt * 32), 0);
+        r.b = make_uint2(w[0], w[1]);
+        const uint32_t blk = block_of(kt, quarter * 16);
         if constexpr (SF32) r.s = __builtin_amdgcn_raw_buffer_load_b32(srd_s, static_cast<int>(s_goff + blk * 4u), 0, 0);
         else r.s = __builtin_amdgcn_raw_buffer_load_b16(srd_s, static_cast<int>(s_goff + blk * 2u), 0, 0);
         const uint32_t zbyte = has_zp ? static_cast<uint32_t>(__builtin_amdgcn_raw_buffer_load_b8(srd_z, static_cast<int>(z_goff + (blk >> 1)), 0, 0)) : 0x88u;
         r.z = zbyte | ((blk & 1u) << 8);
-        r.sa = __builtin_amdgcn_raw_buffer_load_b32(srd_sa, static_cast<int>(sa_goff), static_cast<int>(block_of(kt, sa_slot) * static_cast<uint32_t>(p.m) * 4u), 0);
+        r.sa = __builtin_amdgcn_raw_buffer_load_b32(srd_sa, static_cast<int>(sa_goff), static_cast<int>(block_of(kt, sa_slot * 32) * static_cast<uint32_t>(p.m) * 4u), 0);
     };
-    // Quarter `part` of a step's trip from registers into LDS buffer `buf`.
+    // Half `part` of a step's trip from registers into LDS buffer `buf`.
     auto store_part = [&](const Regs& r, int buf, int part) {
         unsigned char* base = smem + buf * kBufBytes;
-        if (part < 2) *reinterpret_cast<uint4*>(base + a_loff + part * 64 * kPitch8) = r.a[part];
-        const uint32_t w = part == 0 ? r.b.x : part == 1 ? r.b.y : part == 2 ? r.b.z : r.b.w;
+        const uint32_t w = part == 0 ? r.b.x : r.b.y;
         const uint32_t zq = (r.z >> ((r.z >> 8) * 4u)) & 0xfu;
         const uint32_t c4 = 0x80808080u - zq * 0x01010101u;
         const uint32_t lo = ((w & 0x0f0f0f0fu) + c4) ^ 0x80808080u;            // elements 0,2,4,6 of the dword, minus zp
         const uint32_t hi = (((w >> 4) & 0x0f0f0f0fu) + c4) ^ 0x80808080u;     // elements 1,3,5,7
         *reinterpret_cast<uint2*>(base + b_loff + part * 8) = make_uint2(lo, hi);
-        if (part == 2 && bhalf < kSlots) {
-            const float sc = SF32 ? __uint_as_float(r.s) : (p.scales_bf16 ? __uint_as_float(r.s << 16) : f16_bits_to_f32(static_cast<uint16_t>(r.s)));
-            *reinterpret_cast<float*>(base + kSbOff + (bhalf * kTile + bcol) * 4) = sc;
-        }
-        if (part == 3 && sa_slot < kSlots) *reinterpret_cast<uint32_t*>(base + kSaOff + t * 4) = r.sa;
-    };
-    auto store_lds = [&](const Regs& r, int buf) {
-#pragma unroll
-        for (int part = 0; part < 4; ++part) store_part(r, buf, part);
-    };
-    // y += f32(acc) * (scale_a[row] * scale_b[column]) for the block in scale slot `slot` of buffer `buf`.
-    auto flush = [&](int buf, int slot) {
-        const unsigned char* base = smem + buf * kBufBytes;
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            const float sb = *reinterpret_cast<const float*>(base + kSbOff + (slot * kTile + wn * 64 + j * 32 + (lane & 31)) * 4);
-#pragma unroll
-            for (int i = 0; i < TM; ++i) {
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const float4 sa = *reinterpret_cast<const float4*>(base + kSaOff + (slot * kTile + wm * 64 + i * 32 + q * 8 + (lane >> 5) * 4) * 4);
-                    const float sav[4] = {sa.x, sa.y, sa.z, sa.w};
-#pragma unroll
-                    for (int r = 0; r < 4; ++r)
-                        y[i][j][q * 4 + r] = fmaf(static_cast<float>(acc[i][j][q * 4 + r]), __fmul_rn(sav[r], sb), y[i][j][q * 4 + r]);
-                }
+        if (part == 0) {
+            *reinterpret_cast<uint4*>(base + a_loff) = r.a;
+        } else {
+            if ((quarter & 1) == 0 && (quarter >> 1) < kSlots) {
+                const float sc = SF32 ? __uint_as_float(r.s) : (p.scales_bf16 ? __uint_as_float(r.s << 16) : f16_bits_to_f32(static_cast<uint16_t>(r.s)));
+                *reinterpret_cast<float*>(base + kSbOff + ((quarter >> 1) * kTile + prow) * 4) = sc;
             }
+            if (sa_slot < kSlots) *reinterpret_cast<uint32_t*>(base + kSaOff + t * 4) = r.sa;
         }
+    };
+    // y[j] += f32(tile) * (scale_a[row] * scale_b[column]) for one 32x32 tile and the block in scale slot `slot`.
+    auto flush_tile = [&](const int16_t_v& tile, int buf, int slot, int j) {
+        const unsigned char* base = smem + buf * kBufBytes;
+        const float sb = *reinterpret_cast<const float*>(base + kSbOff + (slot * kTile + wn * 64 + j * 32 + (lane & 31)) * 4);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const float4 sa = *reinterpret_cast<const float4*>(base + kSaOff + (slot * kTile + wm * 32 + q * 8 + (lane >> 5) * 4) * 4);
+            const float sav[4] = {sa.x, sa.y, sa.z, sa.w};
+#pragma unroll
+            for (int r = 0; r < 4; ++r) y[j][q * 4 + r] = fmaf(static_cast<float>(tile[q * 4 + r]), __fmul_rn(sav[r], sb), y[j][q * 4 + r]);
+        }
+    };
+    auto mfma = [](const u32x4_t& a, const u32x4_t& b, const int16_t_v& c) {
+        return __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(int4_t, a), __builtin_bit_cast(int4_t, b), c, 0, 0, 0);
     };
     auto compute = [&](int buf, int kt, const Regs& next, bool store_next) {
-        const unsigned char* la = smem + buf * kBufBytes + wm * (64 * kPitch8) + frag_off;
+        const unsigned char* la = smem + buf * kBufBytes + wm * (32 * kPitch8) + frag_off;
         const unsigned char* lb = smem + buf * kBufBytes + kTile * kPitch8 + wn * (64 * kPitch8) + frag_off;
-        // block size >= 128: the step opens / closes a block (wave-uniform)
-        const bool opens = NBS != 0 || ((kt * kStep) & ((1 << p.bs_log2) - 1)) == 0;
-        const bool closes = NBS != 0 || (((kt + 1) * kStep) & ((1 << p.bs_log2) - 1)) == 0;
+        u32x4_t fa[2], fb[2][TN];
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk) {
-            u32x4_t fa[TM], fb[TN];
+            fa[kk] = *reinterpret_cast<const u32x4_t*>(la + kk * 32);
 #pragma unroll
-            for (int i = 0; i < TM; ++i) fa[i] = *reinterpret_cast<const u32x4_t*>(la + i * 32 * kPitch8 + kk * 32);
-#pragma unroll
-            for (int j = 0; j < TN; ++j) fb[j] = *reinterpret_cast<const u32x4_t*>(lb + j * 32 * kPitch8 + kk * 32);
-            const bool first = NBS == 2 ? true : (kk == 0 && opens);
-            const int16_t_v zero = {};
-            if (first) {
-#pragma unroll
-                for (int i = 0; i < TM; ++i)
-#pragma unroll
-                    for (int j = 0; j < TN; ++j)
-                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(int4_t, fa[i]), __builtin_bit_cast(int4_t, fb[j]), zero, 0, 0, 0);
-            } else {
-#pragma unroll
-                for (int i = 0; i < TM; ++i)
-#pragma unroll
-                    for (int j = 0; j < TN; ++j)
-                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(int4_t, fa[i]), __builtin_bit_cast(int4_t, fb[j]), acc[i][j], 0, 0, 0);
+            for (int j = 0; j < TN; ++j) fb[kk][j] = *reinterpret_cast<const u32x4_t*>(lb + j * 32 * kPitch8 + kk * 32);
+        }
+        const int16_t_v zero = {};
+        if constexpr (NBS == 1) {
+            // One block per step: the integer accumulators live only from the MFMAs to the flush.
+            int16_t_v t0 = mfma(fa[0], fb[0][0], zero);
+            int16_t_v t1 = mfma(fa[0], fb[0][1], zero);
+            t0 = mfma(fa[1], fb[1][0], t0);
+            t1 = mfma(fa[1], fb[1][1], t1);
+            if (store_next) store_part(next, buf ^ 1, 0);
+            flush_tile(t0, buf, 0, 0);
+            if (store_next) store_part(next, buf ^ 1, 1);
+            flush_tile(t1, buf, 0, 1);
+        } else if constexpr (NBS == 2) {
+            const bool second = static_cast<int64_t>(kt) * 2 + 1 < p.kb;   // the step's second block exists
+            const int16_t_v t0 = mfma(fa[0], fb[0][0], zero);
+            const int16_t_v t1 = mfma(fa[0], fb[0][1], zero);
+            const int16_t_v u0 = mfma(fa[1], fb[1][0], zero);
+            const int16_t_v u1 = mfma(fa[1], fb[1][1], zero);
+            if (store_next) store_part(next, buf ^ 1, 0);
+            flush_tile(t0, buf, 0, 0);
+            flush_tile(t1, buf, 0, 1);
+            if (store_next) store_part(next, buf ^ 1, 1);
+            if (second) {
+                flush_tile(u0, buf, 1, 0);
+                flush_tile(u1, buf, 1, 1);
             }
-            if (store_next) {
-                store_part(next, buf ^ 1, 2 * kk);
-                store_part(next, buf ^ 1, 2 * kk + 1);
+        } else {
+            // Block size >= 128: the step opens and / or closes a block (wave-uniform).
+            const bool opens = ((kt * kStep) & ((1 << p.bs_log2) - 1)) == 0;
+            const bool closes = (((kt + 1) * kStep) & ((1 << p.bs_log2) - 1)) == 0;
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                if (opens) acc[j] = mfma(fa[0], fb[0][j], zero);
+                else acc[j] = mfma(fa[0], fb[0][j], acc[j]);
+                acc[j] = mfma(fa[1], fb[1][j], acc[j]);
+                if (store_next) store_part(next, buf ^ 1, j);
             }
-            if (NBS == 2) {
-                if (static_cast<int64_t>(kt) * 2 + kk < p.kb) flush(buf, kk);
-            } else if (kk == 1 && closes) {
-                flush(buf, 0);
+            if (closes) {
+#pragma unroll
+                for (int j = 0; j < TN; ++j) flush_tile(acc[j], buf, 0, j);
             }
         }
     };
 
+    // Every load is issued unconditionally (past the end of K it reads in-range garbage or range-checked zeros that
+    // are never stored): with a fixed number of loads per step the compiler can wait for exactly the step it needs.
 #pragma unroll
     for (int s0 = 0; s0 < D - 1; ++s0) load_global(regs[s0], s0);
-    store_lds(regs[0], 0);
+    store_part(regs[0], 0, 0);
+    store_part(regs[0], 0, 1);
     __syncthreads();
     for (int kt0 = 0; kt0 < steps; kt0 += D) {
 #pragma unroll
@@ -488,14 +495,11 @@ __global__ __launch_bounds__(256) void acc4_prefill_kernel(Acc4PrefillParams p)
         if (col >= p.n) continue;
         const float bias = p.bias ? load_as_f32(p.bias, p.bias_dtype, col) : 0.f;
 #pragma unroll
-        for (int i = 0; i < TM; ++i) {
+        for (int q = 0; q < 4; ++q) {
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int64_t row = m_base + wm * 64 + i * 32 + q * 8 + row_group + r;
-                    if (row < p.m) store_from_f32(p.y, p.y_dtype, row * p.n + col, y[i][j][q * 4 + r] + bias);
-                }
+            for (int r = 0; r < 4; ++r) {
+                const int64_t row = m_base + wm * 32 + q * 8 + row_group + r;
+                if (row < p.m) store_from_f32(p.y, p.y_dtype, row * p.n + col, y[j][q * 4 + r] + bias);
             }
         }
     }
@@ -506,7 +510,7 @@ static int launch_acc4_prefill(const Acc4PrefillParams& p, hipStream_t stream)
 {
     const dim3 grid(static_cast<unsigned>((p.n + kTile - 1) / kTile), static_cast<unsigned>((p.m + kTile - 1) / kTile));
     const size_t lds = 2 * (2 * kTile * kPitch8 + 2 * (NBS == 2 ? 2 : 1) * kTile * 4);
-    hipLaunchKernelGGL((acc4_prefill_kernel<NBS, SF32>), grid, dim3(256), lds, stream, p);
+    hipLaunchKernelGGL((acc4_prefill_kernel<NBS, SF32>), grid, dim3(512), lds, stream, p);
     return static_cast<int>(hipGetLastError());
 }
 
