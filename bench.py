@@ -40,6 +40,11 @@ BS = 128
 A_DT = E.BF16
 
 
+# HBM bytes one gate/up launch (M=1, repacked weights) moves, from two rocprofv3 counter runs of `bench.py --only-roofline`:
+# FETCH_SIZE 35,293.85 KiB-units x 1.9997 (what the same counter reads for a 256 MiB copy) plus WRITE_SIZE 74.0 KiB.
+GATE_UP_HBM_BYTES_PER_LAUNCH = 72_346_700
+
+
 def _device_random_weights(ep, n, k, bs, seed, scale_lo, scale_hi, dtype, zero_points=True, reuse=None):
     """Packed nibbles, scales and zero points for one node, resident on the GPU. Random bytes ARE uniform
     nibbles; to keep set-up short the byte pattern of large tensors is generated once per shape and
@@ -248,9 +253,10 @@ def main():
     ms = time_graph(ep, g2, max(10, args.steps // 2), 3)
     launch_us = ms * 1e3 / len(gate_up)
     achieved = gate_up[0].bytes / (launch_us * 1e-6) / 1e9
-    roofline = {"bound": "hbm", "kernel": "decode_mfma_kernel<bf16, block 128> on gate_up 3584->37888, M=%d" % args.m,
+    roofline = {"bound": "hbm", "kernel": "%s<bf16, block 128> on gate_up 3584->37888, M=%d" % (gate_up[0].ops.kernel.last_variant(), args.m),
                 "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                "bytes_per_launch": gate_up[0].bytes, "us_per_launch": round(launch_us, 2), "traffic": None}
+                "bytes_per_launch": gate_up[0].bytes, "us_per_launch": round(launch_us, 2),
+                "traffic": GATE_UP_HBM_BYTES_PER_LAUNCH if args.m == 1 and gate_up[0].ops.kernel.last_variant() == "decode_mfma_packed" else None}
     g2.release()
 
     result = {
@@ -290,7 +296,8 @@ def roofline_only(ep, args):
         node = Node(ep, f"gate_up.{layer}", HIDDEN, 2 * INTER, BS, layer, A_DT, args.m, reuse=reuse)
         reuse = node.host_b if reuse is None else reuse
         nodes.append(node)
-    nodes[0].run(a)
+    for node in nodes:               # eager once: constant weights are repacked here, never inside a capture
+        node.run(a)
     ep.sync()
     graph = capture(ep, lambda: [n.run(a) for n in nodes])
     ms = time_graph(ep, graph, args.steps, args.warmup)
@@ -299,7 +306,7 @@ def roofline_only(ep, args):
     src, dst = ep.allocate(copy_bytes), ep.allocate(copy_bytes)
     ep.copy(dst, src, copy_bytes)
     ep.sync()
-    print(json.dumps({"kernel": "decode_mfma_kernel on gate_up 3584->37888", "m": args.m, "launches": len(nodes) * (args.steps + args.warmup) + 1,
+    print(json.dumps({"kernel": nodes[0].ops.kernel.last_variant() + " on gate_up 3584->37888", "m": args.m, "launches": len(nodes) * (args.steps + args.warmup) + 1,
                       "us_per_launch": round(us, 2), "bytes_per_launch": nodes[0].bytes, "achieved_gbs": round(nodes[0].bytes / us / 1e3, 1),
                       "copy_kernel_bytes_read": copy_bytes, "copy_kernel_bytes_written": copy_bytes}), flush=True)
 

@@ -17,6 +17,7 @@ HIP_SOURCES = [
     "kernels/dequant.hip",
     "kernels/gemv_generic.hip",
     "kernels/decode_mfma.hip",
+    "kernels/decode_packed.hip",
     "kernels/prefill_mfma.hip",
     "kernels/acc4.hip",
     "kernels/acc4_mfma.hip",

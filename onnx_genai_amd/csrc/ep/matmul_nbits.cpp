@@ -122,14 +122,18 @@ struct NxrtRocmMatMulNBits {
     std::string variant = "none";
     void* scratch = nullptr;             // kernel-owned workspace, grown on demand
     size_t scratch_bytes = 0;
+    void* packed = nullptr;              // constant B / scales / zero points in the decode kernel's streaming order
+    const void* packed_from[3] = {nullptr, nullptr, nullptr};   // the tensors `packed` was made from
+    int packed_scale_dtype = 0;
     NxrtKernelVtable vtable;
     uint32_t vt_a_dtype = 0, vt_scale_dtype = 0, vt_y_dtype = 0;
 
     ~NxrtRocmMatMulNBits()
     {
-        if (scratch && ep && ep->bind().code == NXRT_OK) {
+        if ((scratch || packed) && ep && ep->bind().code == NXRT_OK) {
             rocm_ffi_stream_sync(ep->stream);
-            rocm_ffi_free(scratch);
+            if (scratch) rocm_ffi_free(scratch);
+            if (packed) rocm_ffi_free(packed);
         }
     }
 };
@@ -150,6 +154,35 @@ Acc4Layout acc4_layout(const NxrtRocmMatMulNBits& kn, uint64_t m)
     return l;
 }
 uint64_t acc4_workspace_bytes(const NxrtRocmMatMulNBits& kn, uint64_t m) { return acc4_layout(kn, m).total; }
+
+// True when the call can run on the repacked copy of constant weights; makes that copy on first use (never while a
+// graph capture is open: a capture may neither allocate nor should it record the one-time repack). `rc` receives a
+// HIP error of the repack.
+bool use_packed(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& args, int& rc)
+{
+    rc = 0;
+    if (!kn.ep->prepack || !kn.constant_inputs[1] || !kn.constant_inputs[2] || (args.zp && !kn.constant_inputs[3])) return false;
+    if (!rocm_decode_packed_eligible(&args)) return false;
+    const bool current = kn.packed && kn.packed_from[0] == args.b && kn.packed_from[1] == args.scales && kn.packed_from[2] == args.zp &&
+                         kn.packed_scale_dtype == args.scale_dtype;
+    if (current) return true;
+    if (kn.ep->capturing) return false;
+    if (kn.packed) {
+        rocm_ffi_stream_sync(kn.ep->stream);
+        rocm_ffi_free(kn.packed);
+        kn.packed = nullptr;
+    }
+    if (rocm_ffi_malloc(&kn.packed, rocm_decode_packed_bytes(&args)) != 0) {
+        kn.packed = nullptr;
+        return false;                       // no memory for a second copy: stream the caller's tensors instead
+    }
+    rc = rocm_launch_pack_decode(&args, kn.packed, kn.ep->stream);
+    kn.packed_from[0] = args.b;
+    kn.packed_from[1] = args.scales;
+    kn.packed_from[2] = args.zp;
+    kn.packed_scale_dtype = args.scale_dtype;
+    return true;
+}
 
 NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, uint32_t n_in, NxrtRocmTensorView* out, uint32_t n_out,
                         void* workspace, uint64_t workspace_bytes)
@@ -288,6 +321,9 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
                 kn.variant = "acc4_gemv_dot4";
             }
         }
+    } else if (M <= 4 && use_packed(kn, args, rc)) {
+        if (rc == 0) rc = rocm_launch_decode_packed(&args, kn.packed, kn.ep->decode_waves, stream);
+        kn.variant = "decode_mfma_packed";
     } else if (M <= 16 && rocm_decode_mfma_eligible(&args)) {
         rc = rocm_launch_decode_mfma(&args, kn.ep->decode_waves, kn.ep->decode_col_groups, stream);
         kn.variant = "decode_mfma_splitk";

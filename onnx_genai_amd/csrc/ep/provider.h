@@ -18,6 +18,7 @@ struct NxrtRocmEp {
     int acc4_rounding = 0;                        // 0 = ties to even (MLAS), 1 = ties away (native)
     int decode_waves = 0;                         // 0 = chosen per shape
     int decode_col_groups = 0;
+    int prepack = 1;                              // repack constant weights for the decode kernel on first use
     std::mutex mu;
     std::unordered_map<void*, size_t> live;       // allocations handed out and not yet returned
     std::atomic<uint64_t> launches{0};

@@ -70,6 +70,13 @@ int rocm_launch_gemv_generic(const RocmMatMulNBitsArgs* args, rocm_stream_t stre
 int rocm_decode_mfma_eligible(const RocmMatMulNBitsArgs* args);
 int rocm_launch_decode_mfma(const RocmMatMulNBitsArgs* args, int waves, int col_groups, rocm_stream_t stream);
 
+/* Decode over constant weights repacked for streaming (M <= 4). `packed` holds rocm_decode_packed_bytes() bytes and is
+ * filled once by rocm_launch_pack_decode from args->b / scales / zp; rocm_launch_decode_packed then reads only it. */
+int rocm_decode_packed_eligible(const RocmMatMulNBitsArgs* args);
+uint64_t rocm_decode_packed_bytes(const RocmMatMulNBitsArgs* args);
+int rocm_launch_pack_decode(const RocmMatMulNBitsArgs* args, void* packed, rocm_stream_t stream);
+int rocm_launch_decode_packed(const RocmMatMulNBitsArgs* args, const void* packed, int waves, rocm_stream_t stream);
+
 /* Prefill (M > 16), f16/bf16 activations: B tiles dequantized into LDS, 32x32x16 MFMA. */
 int rocm_prefill_mfma_eligible(const RocmMatMulNBitsArgs* args);
 int rocm_launch_prefill_mfma(const RocmMatMulNBitsArgs* args, rocm_stream_t stream);

@@ -1,0 +1,383 @@
+// Decode path of MatMulNBits over weights repacked for streaming (M <= 4, f16/bf16 activations).
+//
+// When B, scales and zero points are constant initializers, the kernel object repacks them once into
+// the order in which the split-K MFMA kernel consumes them, so that every vector load of a wave is
+// one contiguous kilobyte and everything a group of four 128-element tiles needs lies in one chunk:
+//
+//   chunk(column group cg of 16 columns, tile group tg of 4 tiles) =
+//       4 x [lane 0..63] 16 bytes of weights      lane (c = lane % 16, g = lane / 16) of tile u at u*1024 + lane*16
+//       16 x record(column c)                     scales of the group's blocks, then one zero-point byte per block
+//
+// Dword j of a lane's 16 bytes holds the eight weights k = tile*128 + j*32 + g*8 + e (e = 0..7) of column c:
+// one MFMA therefore covers 32 consecutive k and never mixes two blocks, whatever the block size, and no
+// cross-lane transpose is needed. Inside the dword, element e sits at bit 4*(e/2) + 16*(e%2), so that
+// ((w >> 4i) & 0x000F000F) | magic is the pair (e = 2i, 2i+1) as two 16-bit floats - seven VALU
+// instructions per eight weights. The arithmetic is that of the unpacked decode kernel: magic-number
+// operands, a second MFMA with the constant -(magic + zp), one scale per block on the f32 accumulator.
+//
+// The copy costs one extra byte of device memory per byte of weights plus 2 to 6 % for the records; it is
+// read instead of the caller's tensors, which are not touched again.
+#include "mfma_common.hiph"
+
+namespace mnb {
+
+typedef __attribute__((ext_vector_type(8))) _Float16 half8p_t;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8p_t;
+typedef __attribute__((ext_vector_type(4))) float float4p_t;
+
+constexpr int kGroupTiles = 4;
+constexpr int kChunkWeights = kGroupTiles * 1024;
+constexpr int kRowPitchP = 272;   // bytes between activation rows in LDS: 256 + 16
+
+__host__ __device__ constexpr int packed_record_bytes(int bs, int scale_bytes)
+{
+    const int nb = kGroupTiles * 128 / bs;
+    return (nb * scale_bytes + nb + 15) / 16 * 16;
+}
+
+struct PackParams {
+    const uint8_t* b;
+    const void* scales;
+    const uint8_t* zp;
+    uint8_t* out;
+    int64_t n, kb, row_bytes, zp_row;
+    int bs_log2, scale_bytes;
+    int groups;             // tile groups per column group
+    int chunk_bytes, record;
+};
+
+// grid (tile group, column group), 256 threads: four dwords of weights per thread, then one record per thread < 16.
+__global__ __launch_bounds__(256) void pack_decode_kernel(PackParams p)
+{
+    const int t = threadIdx.x;
+    const int64_t tg = blockIdx.x, cg = blockIdx.y;
+    uint8_t* chunk = p.out + (cg * p.groups + tg) * static_cast<int64_t>(p.chunk_bytes);
+    const int64_t padded_k = p.kb << p.bs_log2;
+    const uint32_t* b32 = reinterpret_cast<const uint32_t*>(p.b);
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+        const int x = it * 256 + t;              // dword of the weight part: u*256 + lane*4 + j
+        const int u = x >> 8, lane = (x >> 2) & 63, j = x & 3;
+        const int64_t col = cg * 16 + (lane & 15);
+        const int64_t k = (tg * kGroupTiles + u) * 128 + j * 32 + (lane >> 4) * 8;
+        uint32_t out = 0;
+        if (col < p.n && k < padded_k) {
+            const uint32_t w = b32[(col * p.row_bytes + (k >> 1)) >> 2];   // eight weights, element e at bit 4e
+            uint32_t lo = w & 0x0f0f0f0fu, hi = (w >> 4) & 0x0f0f0f0fu;    // even / odd elements, one per byte
+            lo = (lo | (lo >> 4)) & 0x00ff00ffu;
+            lo = (lo | (lo >> 8)) & 0x0000ffffu;                            // e0 | e2 << 4 | e4 << 8 | e6 << 12
+            hi = (hi | (hi >> 4)) & 0x00ff00ffu;
+            hi = (hi | (hi >> 8)) & 0x0000ffffu;
+            out = lo | (hi << 16);
+        }
+        reinterpret_cast<uint32_t*>(chunk)[x] = out;
+    }
+    if (t < 16) {
+        const int nb = (kGroupTiles * 128) >> p.bs_log2;
+        uint8_t* rec = chunk + kChunkWeights + t * p.record;
+        const int64_t col = cg * 16 + t;
+        for (int i = 0; i < p.record; ++i) rec[i] = 0;
+        for (int bi = 0; bi < nb; ++bi) {
+            const int64_t blk = tg * nb + bi;
+            const bool live = col < p.n && blk < p.kb;
+            if (p.scale_bytes == 4) {
+                reinterpret_cast<uint32_t*>(rec)[bi] = live ? static_cast<const uint32_t*>(p.scales)[col * p.kb + blk] : 0u;
+            } else {
+                reinterpret_cast<uint16_t*>(rec)[bi] = live ? static_cast<const uint16_t*>(p.scales)[col * p.kb + blk] : static_cast<uint16_t>(0);
+            }
+            rec[nb * p.scale_bytes + bi] = static_cast<uint8_t>(live ? zero_point_of(p.zp ? p.zp + col * p.zp_row : nullptr, blk) : 8);
+        }
+    }
+}
+
+struct PackedParams {
+    const uint16_t* a;
+    const uint8_t* packed;
+    const void* bias;
+    void* y;
+    int64_t m, n, k;
+    int64_t cg_stride;      // bytes of one column group: groups * chunk_bytes
+    int groups;             // tile groups
+    int groups_per_wave;
+    int chunk_bytes;
+    int bias_dtype, y_dtype;
+    uint32_t nibble_mask;   // 0x000F000F
+    uint32_t magic;         // two 16-bit magic exponents; a kernel argument so that it stays in a scalar register
+};
+
+template <bool BF16>
+__device__ __forceinline__ float4p_t mfma16p(const uint4& act, const uint4& wgt, float4p_t acc)
+{
+    if constexpr (BF16) return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8p_t, act), __builtin_bit_cast(bf16x8p_t, wgt), acc, 0, 0, 0);
+    else return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8p_t, act), __builtin_bit_cast(half8p_t, wgt), acc, 0, 0, 0);
+}
+
+template <int NR, int NA>
+struct PackedGroup {
+    uint4 w[kGroupTiles];
+    uint4 r[NR];
+    uint4 a[NA];
+};
+
+// BF16: activation element type. BS: block size. MR: rows staged (1 or 4; M <= MR). ST: storage type of the scales.
+template <bool BF16, int BS, int MR, typename ST>
+__global__ __launch_bounds__(512) void decode_packed_kernel(PackedParams p)
+{
+    constexpr int U = kGroupTiles;
+    constexpr int NBT = 128 / BS;
+    constexpr int NB = U * NBT;
+    constexpr int R = packed_record_bytes(BS, static_cast<int>(sizeof(ST)));
+    constexpr int NR = R / 16;
+    constexpr int NA = MR == 1 ? 1 : U;
+    constexpr int kStageBytes = MR == 1 ? 1024 : MR * kRowPitchP;
+    constexpr uint32_t kMagicNeg = BF16 ? 0xC300C300u : 0xE400E400u;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int waves = blockDim.x >> 6;
+    const int c = lane & 15;
+    const int g = lane >> 4;
+    const int64_t n_base = static_cast<int64_t>(blockIdx.x) * 16;
+    const bool full_k = (p.k & 127) == 0;
+
+    const __amdgpu_buffer_rsrc_t srd_p = make_srd(p.packed + static_cast<int64_t>(blockIdx.x) * p.cg_stride, static_cast<uint64_t>(p.cg_stride));
+    const __amdgpu_buffer_rsrc_t srd_a = make_srd(p.a, static_cast<uint64_t>(p.m * p.k) * 2);
+
+    const uint32_t w_off = static_cast<uint32_t>(lane * 16);
+    const uint32_t r_off = static_cast<uint32_t>(kChunkWeights + c * R);
+    // compact activation load. MR = 1: piece c of tile g of the group. MR = 4: row g, piece c of one tile.
+    const uint32_t a_off = MR == 1 ? static_cast<uint32_t>(g * 256 + c * 16) : static_cast<uint32_t>(g) * static_cast<uint32_t>(p.k) * 2u + static_cast<uint32_t>(c * 16);
+    unsigned char* stage = smem + wave * (2 * kStageBytes);
+    const uint32_t st_write = MR == 1 ? static_cast<uint32_t>(lane * 16) : static_cast<uint32_t>(g * kRowPitchP + c * 16);
+    // operand of MFMA j: elements j*32 + g*8 .. +8 of the tile, of row c % MR
+    const uint32_t st_read = (MR == 1 ? 0u : static_cast<uint32_t>((c & (MR - 1)) * kRowPitchP)) + static_cast<uint32_t>(g * 16);
+    const uint32_t mask = __builtin_amdgcn_mov_dpp(p.nibble_mask, 0xE4, 0xf, 0xf, false), magic = p.magic;
+
+    float4p_t y = {0.f, 0.f, 0.f, 0.f};
+    float4p_t acc = {0.f, 0.f, 0.f, 0.f};
+
+    const int g_begin = wave * p.groups_per_wave;
+    const int g_end = min(g_begin + p.groups_per_wave, p.groups);
+
+    using Grp = PackedGroup<NR, NA>;
+    auto fetch_group = [&](Grp& grp, int gi) {
+        if (gi >= g_end) return;
+        const uint32_t soff = static_cast<uint32_t>(gi) * static_cast<uint32_t>(p.chunk_bytes);
+#pragma unroll
+        for (int u = 0; u < U; ++u) grp.w[u] = load16(srd_p, w_off + static_cast<uint32_t>(u * 1024), soff);
+#pragma unroll
+        for (int i = 0; i < NR; ++i) grp.r[i] = load16(srd_p, r_off + static_cast<uint32_t>(i * 16), soff);
+        const int t0 = gi * U;
+        if constexpr (MR == 1) {
+            uint32_t off = a_off;
+            if (!full_k && static_cast<int64_t>(t0 + g) * 128 + c * 8 + 8 > p.k) off = kOutOfRange;
+            grp.a[0] = load16(srd_a, off, static_cast<uint32_t>(t0) * 256u);
+        } else {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                uint32_t off = a_off;
+                if (!full_k && static_cast<int64_t>(t0 + u) * 128 + c * 8 + 8 > p.k) off = kOutOfRange;
+                if (static_cast<int64_t>(t0 + u) * 128 >= p.k) off = kOutOfRange;      // a padding tile of the last group
+                grp.a[u] = load16(srd_a, off, static_cast<uint32_t>(t0 + u) * 256u);
+            }
+        }
+    };
+    auto compute_tile = [&](const Grp& grp, int u, int parity) {
+        unsigned char* st = stage + (MR == 1 ? parity : (u & 1)) * kStageBytes;
+        if constexpr (MR != 1) {
+            *reinterpret_cast<uint4*>(st + st_write) = grp.a[u];
+            lds_order();
+        }
+        uint4 av[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) av[j] = *reinterpret_cast<const uint4*>(st + st_read + (MR == 1 ? u * 256 : 0) + j * 64);
+        const uint32_t wd[4] = {grp.w[u].x, grp.w[u].y, grp.w[u].z, grp.w[u].w};
+        uint32_t rr[NR * 4];
+#pragma unroll
+        for (int i = 0; i < NR; ++i) {
+            rr[4 * i] = grp.r[i].x;
+            rr[4 * i + 1] = grp.r[i].y;
+            rr[4 * i + 2] = grp.r[i].z;
+            rr[4 * i + 3] = grp.r[i].w;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int bi = u * NBT + (j * 32) / BS;                          // block of the group (compile-time)
+            const int zbyte = NB * static_cast<int>(sizeof(ST)) + bi;
+            const uint32_t z = (rr[zbyte / 4] >> ((zbyte % 4) * 8)) & 0xffu;
+            const uint32_t zpair = kMagicNeg | (z * 0x00010001u);
+            const uint4 zc = make_uint4(zpair, zpair, zpair, zpair);
+            const uint32_t w = wd[j];
+            uint4 op;
+            op.x = (w & mask) | magic;
+            op.y = ((w >> 4) & mask) | magic;
+            op.z = ((w >> 8) & mask) | magic;
+            op.w = ((w >> 12) & mask) | magic;
+            acc = mfma16p<BF16>(av[j], op, acc);
+            acc = mfma16p<BF16>(av[j], zc, acc);
+            if (((j + 1) * 32) % BS == 0 || j == 3) {
+                float sf;
+                if constexpr (sizeof(ST) == 4) {
+                    sf = __uint_as_float(rr[bi]);
+                } else {
+                    const uint32_t raw = (rr[bi / 2] >> ((bi % 2) * 16)) & 0xffffu;
+                    sf = BF16 ? __uint_as_float(raw << 16) : f16_bits_to_f32(static_cast<uint16_t>(raw));
+                }
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    y[r] = fmaf(sf, acc[r], y[r]);
+                    acc[r] = 0.f;
+                }
+            }
+        }
+    };
+    auto run_group = [&](const Grp& cur, Grp& next, int gi, int parity) {
+        fetch_group(next, gi + 1);
+        if constexpr (MR == 1) {
+            *reinterpret_cast<uint4*>(stage + parity * kStageBytes + st_write) = cur.a[0];
+            lds_order();
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) compute_tile(cur, u, parity);
+    };
+
+    Grp ga, gb;
+    fetch_group(ga, g_begin);
+    for (int gi = g_begin; gi < g_end; gi += 2) {
+        run_group(ga, gb, gi, 0);
+        if (gi + 1 < g_end) run_group(gb, ga, gi + 1, 1);
+    }
+
+    // ---- split-K reduction across the waves of this workgroup, in wave order ----
+    __syncthreads();
+    float* red = reinterpret_cast<float*>(smem);       // [waves][4][64]
+#pragma unroll
+    for (int r = 0; r < 4; ++r) red[(wave * 4 + r) * 64 + lane] = y[r];
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < 256; idx += blockDim.x) {
+        const int r = idx >> 6;
+        const int l = idx & 63;
+        const int row = 4 * (l >> 4) + r;
+        const int64_t col = n_base + (l & 15);
+        if (row < p.m && col < p.n) {
+            float total = 0.f;
+            for (int w = 0; w < waves; ++w) total += red[(w * 4 + r) * 64 + l];
+            if (p.bias) total += load_as_f32(p.bias, p.bias_dtype, col);
+            store_from_f32(p.y, p.y_dtype, static_cast<int64_t>(row) * p.n + col, total);
+        }
+    }
+}
+
+template <bool BF16, int BS, int MR, typename ST>
+static int launch_packed_cfg(const PackedParams& p, int waves, hipStream_t stream)
+{
+    const unsigned grid = static_cast<unsigned>((p.n + 15) / 16);
+    const size_t stage = static_cast<size_t>(waves) * 2 * (MR == 1 ? 1024 : MR * kRowPitchP);
+    const size_t red = static_cast<size_t>(waves) * 1024;
+    hipLaunchKernelGGL((decode_packed_kernel<BF16, BS, MR, ST>), dim3(grid), dim3(waves * 64), stage > red ? stage : red, stream, p);
+    return static_cast<int>(hipGetLastError());
+}
+
+template <bool BF16, typename ST>
+static int launch_packed_bs(const PackedParams& p, int bs, int waves, hipStream_t stream)
+{
+    if (p.m <= 1) {
+        switch (bs) {
+            case 32: return launch_packed_cfg<BF16, 32, 1, ST>(p, waves, stream);
+            case 64: return launch_packed_cfg<BF16, 64, 1, ST>(p, waves, stream);
+            default: return launch_packed_cfg<BF16, 128, 1, ST>(p, waves, stream);
+        }
+    }
+    switch (bs) {
+        case 32: return launch_packed_cfg<BF16, 32, 4, ST>(p, waves, stream);
+        case 64: return launch_packed_cfg<BF16, 64, 4, ST>(p, waves, stream);
+        default: return launch_packed_cfg<BF16, 128, 4, ST>(p, waves, stream);
+    }
+}
+
+static int packed_groups(const RocmMatMulNBitsArgs* a)
+{
+    const int64_t kb = (a->k + a->block_size - 1) / a->block_size;
+    const int64_t tiles = (kb * a->block_size + 127) / 128;
+    return static_cast<int>((tiles + kGroupTiles - 1) / kGroupTiles);
+}
+
+static int packed_chunk_bytes(const RocmMatMulNBitsArgs* a)
+{
+    return kChunkWeights + 16 * packed_record_bytes(a->block_size, a->scale_dtype == ROCM_DT_F32 ? 4 : 2);
+}
+
+}  // namespace mnb
+
+extern "C" int rocm_decode_packed_eligible(const RocmMatMulNBitsArgs* a)
+{
+    if (!rocm_decode_mfma_eligible(a) || a->m > 4) return 0;
+    return static_cast<int64_t>(mnb::packed_groups(a)) * mnb::packed_chunk_bytes(a) < 0x7fffffff;
+}
+
+extern "C" uint64_t rocm_decode_packed_bytes(const RocmMatMulNBitsArgs* a)
+{
+    const uint64_t col_groups = static_cast<uint64_t>((a->n + 15) / 16);
+    return col_groups * static_cast<uint64_t>(mnb::packed_groups(a)) * static_cast<uint64_t>(mnb::packed_chunk_bytes(a));
+}
+
+extern "C" int rocm_launch_pack_decode(const RocmMatMulNBitsArgs* a, void* packed, rocm_stream_t stream)
+{
+    mnb::PackParams p;
+    p.b = a->b;
+    p.scales = a->scales;
+    p.zp = a->zp;
+    p.out = static_cast<uint8_t*>(packed);
+    p.n = a->n;
+    p.kb = (a->k + a->block_size - 1) / a->block_size;
+    p.row_bytes = p.kb * a->block_size / 2;
+    p.zp_row = (p.kb + 1) / 2;
+    p.bs_log2 = __builtin_ctz(static_cast<unsigned>(a->block_size));
+    p.scale_bytes = a->scale_dtype == ROCM_DT_F32 ? 4 : 2;
+    p.groups = mnb::packed_groups(a);
+    p.chunk_bytes = mnb::packed_chunk_bytes(a);
+    p.record = mnb::packed_record_bytes(a->block_size, p.scale_bytes);
+    const dim3 grid(static_cast<unsigned>(p.groups), static_cast<unsigned>((a->n + 15) / 16));
+    hipLaunchKernelGGL(mnb::pack_decode_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream), p);
+    return static_cast<int>(hipGetLastError());
+}
+
+extern "C" int rocm_launch_decode_packed(const RocmMatMulNBitsArgs* a, const void* packed, int waves, rocm_stream_t stream)
+{
+    if (!rocm_decode_packed_eligible(a)) return -1;
+    mnb::PackedParams p;
+    p.a = static_cast<const uint16_t*>(a->a);
+    p.packed = static_cast<const uint8_t*>(packed);
+    p.bias = a->bias;
+    p.y = a->y;
+    p.m = a->m;
+    p.n = a->n;
+    p.k = a->k;
+    p.groups = mnb::packed_groups(a);
+    p.chunk_bytes = mnb::packed_chunk_bytes(a);
+    p.cg_stride = static_cast<int64_t>(p.groups) * p.chunk_bytes;
+    p.bias_dtype = a->bias_dtype;
+    p.y_dtype = a->y_dtype;
+    p.nibble_mask = 0x000F000Fu;
+    const bool bf16 = a->a_dtype == ROCM_DT_BF16;
+    p.magic = bf16 ? 0x43004300u : 0x64006400u;
+
+    int w = waves;
+    if (w <= 0) {
+        const int64_t wgs = (a->n + 15) / 16;
+        const int want = static_cast<int>((8192 + wgs - 1) / wgs);   // waves per workgroup to reach ~8k waves
+        w = want < p.groups ? want : p.groups;                       // at least one group per wave
+        if (w < 1) w = 1;
+    }
+    if (w > 8) w = 8;
+    if (w > p.groups) w = p.groups;
+    const int gpw = (p.groups + w - 1) / w;
+    w = (p.groups + gpw - 1) / gpw;
+    p.groups_per_wave = gpw;
+
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const bool f32_scales = a->scale_dtype == ROCM_DT_F32;
+    if (bf16) return f32_scales ? mnb::launch_packed_bs<true, float>(p, a->block_size, w, s) : mnb::launch_packed_bs<true, uint16_t>(p, a->block_size, w, s);
+    return f32_scales ? mnb::launch_packed_bs<false, float>(p, a->block_size, w, s) : mnb::launch_packed_bs<false, uint16_t>(p, a->block_size, w, s);
+}

@@ -39,3 +39,12 @@ def ep():
     assert info["arch"].startswith("gfx950"), info
     yield provider
     provider.shutdown()
+
+
+@pytest.fixture(scope="session")
+def ep_unpacked():
+    """A provider that never repacks constant weights: decode calls stream the caller's tensors as they are."""
+    from onnx_genai_amd.ep import RocmExecutionProvider
+    provider = RocmExecutionProvider(0, {"prepack": "0"})
+    yield provider
+    provider.shutdown()

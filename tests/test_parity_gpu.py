@@ -164,11 +164,16 @@ DECODE_CASES = [
     (E.F16, E.F16, 32, True, 9, 17, 72),        # K = 72: multiple of 8, not of the block size
     (E.BF16, E.BF16, 128, True, 2, 20, 200),    # partial last block
     (E.F16, E.F16, 64, True, 1, 1, 64),
+    (E.F16, E.F32, 64, True, 1, 100, 64 * 21),  # f32 scales, odd block count, tile groups padded
+    (E.BF16, E.F32, 32, True, 3, 50, 32 * 19),
+    (E.BF16, E.BF16, 64, False, 4, 70, 4096),
 ]
 
 
 @pytest.mark.parametrize("a_dt,s_dt,bs,zero_points,m,n,k", DECODE_CASES)
-def test_decode_matches_oracle(ep, port, a_dt, s_dt, bs, zero_points, m, n, k):
+@pytest.mark.parametrize("prepack", [True, False])
+def test_decode_matches_oracle(ep, ep_unpacked, port, prepack, a_dt, s_dt, bs, zero_points, m, n, k):
+    ep = ep if prepack else ep_unpacked
     b, s, zp = synth.make_weights(n, k, bs, 100 + n + k, zero_points=zero_points, scale_lo=0.002, scale_hi=0.01, scale_dtype=s_dt)
     a = synth.make_activation(m, k, n, a_dt)
     bias = synth.to_dtype(np.random.default_rng(n).standard_normal(n).astype(np.float32), a_dt)
@@ -176,7 +181,7 @@ def test_decode_matches_oracle(ep, port, a_dt, s_dt, bs, zero_points, m, n, k):
 
     # f32 output: the arithmetic itself, before any narrowing
     y32, variant = run_op(ep, a, a_dt, b, s, s_dt, zp, n, k, bs, bias=bias, bias_dtype=a_dt, y_dtype=E.F32)
-    assert variant == "decode_mfma_splitk"
+    assert variant == ("decode_mfma_packed" if prepack and m <= 4 else "decode_mfma_splitk")
     # The kernel carries each weight as (2^10 + q) in f16 or (2^7 + q) in bf16 and cancels the offset inside the
     # f32 accumulator, which costs 10 (7) of its 24 bits: a few 1e-5 on outputs that themselves cancel.
     assert helpers.rel_l2(y32, want64) <= 1e-4
@@ -204,6 +209,45 @@ def test_decode_launch_shapes_agree(port, waves, cg):
         assert helpers.rel_l2(y32, oracle_f64(port, a, a_dt, b, s, a_dt, zp, n, k, bs)) <= 2e-5
     finally:
         provider.shutdown()
+
+
+@pytest.mark.parametrize("waves", [1, 3, 8])
+def test_packed_decode_wave_counts_agree(port, waves):
+    provider = E.RocmExecutionProvider(0, {"decode_waves": waves})
+    try:
+        a_dt, bs, n, k = E.BF16, 128, 200, 3584
+        b, s, zp = synth.make_weights(n, k, bs, 78, zero_points=True, scale_lo=0.002, scale_hi=0.01, scale_dtype=a_dt)
+        for m in (1, 3):
+            a = synth.make_activation(m, k, 78 + m, a_dt)
+            y32, variant = run_op(provider, a, a_dt, b, s, a_dt, zp, n, k, bs, y_dtype=E.F32)
+            assert variant == "decode_mfma_packed"
+            assert helpers.rel_l2(y32, oracle_f64(port, a, a_dt, b, s, a_dt, zp, n, k, bs)) <= 2e-5
+    finally:
+        provider.shutdown()
+
+
+def test_packed_copy_follows_the_weights(ep, port):
+    """One kernel object, two different weight tensors in turn: the repacked copy is rebuilt when the pointers change."""
+    a_dt, bs, m, n, k = E.F16, 128, 1, 96, 1024
+    a = synth.make_activation(m, k, 5, a_dt)
+    ab, yb = ep.upload(a), ep.allocate(m * n * 4)
+    b1, s1, zp1 = synth.make_weights(n, k, bs, 31, zero_points=True, scale_lo=0.002, scale_hi=0.01, scale_dtype=a_dt)
+    first = E.DeviceOperands(ep, b1, s1, a_dt, zp1, n, k, bs)
+    b2, s2, zp2 = synth.make_weights(n, k, bs, 32, zero_points=True, scale_lo=0.002, scale_hi=0.01, scale_dtype=a_dt)
+    other = [ep.upload(b2), ep.upload(s2), ep.upload(zp2)]
+    kb = k // bs
+    first.kernel.execute(first.views(ab, a_dt, m), [E.TensorView(yb.ptr, E.F32, (m, n))])
+    y1 = ep.download(yb, (m, n), np.float32)
+    views2 = [E.TensorView(ab.ptr, a_dt, (m, k)), E.TensorView(other[0].ptr, E.U8, (n, kb, bs // 2)),
+              E.TensorView(other[1].ptr, a_dt, (n, kb)), E.TensorView(other[2].ptr, E.U8, (n, (kb + 1) // 2))]
+    first.kernel.execute(views2, [E.TensorView(yb.ptr, E.F32, (m, n))])
+    assert first.kernel.last_variant() == "decode_mfma_packed"
+    y2 = ep.download(yb, (m, n), np.float32)
+    assert helpers.rel_l2(y1, oracle_f64(port, a, a_dt, b1, s1, a_dt, zp1, n, k, bs)) <= 1e-4
+    assert helpers.rel_l2(y2, oracle_f64(port, a, a_dt, b2, s2, a_dt, zp2, n, k, bs)) <= 1e-4
+    for buf in other + [ab, yb]:
+        ep.deallocate(buf)
+    first.free()
 
 
 def test_decode_is_deterministic(ep):
