@@ -329,6 +329,7 @@ __global__ __launch_bounds__(512) void acc4_prefill_kernel(Acc4PrefillParams p)
     const __amdgpu_buffer_rsrc_t srd_b = make_srd(p.b + n_base * p.row_bytes, static_cast<uint64_t>(cols_left * p.row_bytes));
     const __amdgpu_buffer_rsrc_t srd_s = make_srd(static_cast<const unsigned char*>(p.scales) + n_base * p.kb * kScaleBytes,
                                                   static_cast<uint64_t>(cols_left * p.kb) * kScaleBytes);
+    const uint32_t zp_mask = has_zp ? 0xfu : 0u, zp_default = has_zp ? 0u : 8u;   // branch-free "8 when absent"
     const __amdgpu_buffer_rsrc_t srd_z = make_srd(has_zp ? p.zp + n_base * p.zp_row : p.b, has_zp ? static_cast<uint64_t>(cols_left * p.zp_row) : 0);
     const __amdgpu_buffer_rsrc_t srd_sa = make_srd(p.sa_t, static_cast<uint64_t>(p.kb * p.m) * 4);
 
@@ -362,7 +363,7 @@ __global__ __launch_bounds__(512) void acc4_prefill_kernel(Acc4PrefillParams p)
     struct Regs {
         uint4 a;
         uint2 b;
-        uint32_t s, z, sa;
+        uint32_t s, z, zsh, sa;
     };
     Regs regs[D];
 
@@ -376,15 +377,17 @@ __global__ __launch_bounds__(512) void acc4_prefill_kernel(Acc4PrefillParams p)
         const uint32_t blk = block_of(kt, quarter * 16);
         if constexpr (SF32) r.s = __builtin_amdgcn_raw_buffer_load_b32(srd_s, static_cast<int>(s_goff + blk * 4u), 0, 0);
         else r.s = __builtin_amdgcn_raw_buffer_load_b16(srd_s, static_cast<int>(s_goff + blk * 2u), 0, 0);
-        const uint32_t zbyte = has_zp ? static_cast<uint32_t>(__builtin_amdgcn_raw_buffer_load_b8(srd_z, static_cast<int>(z_goff + (blk >> 1)), 0, 0)) : 0x88u;
-        r.z = zbyte | ((blk & 1u) << 8);
+        // loaded even without zero points (the empty range then returns 0): a branch here would split the loop body
+        const uint32_t zraw = static_cast<uint32_t>(__builtin_amdgcn_raw_buffer_load_b8(srd_z, static_cast<int>(z_goff + (blk >> 1)), 0, 0));
+        r.z = zraw;                 // no arithmetic on a loaded value here: it would wait for the load at once
+        r.zsh = (blk & 1u) * 4u;
         r.sa = __builtin_amdgcn_raw_buffer_load_b32(srd_sa, static_cast<int>(sa_goff), static_cast<int>(block_of(kt, sa_slot * 32) * static_cast<uint32_t>(p.m) * 4u), 0);
     };
     // Half `part` of a step's trip from registers into LDS buffer `buf`.
     auto store_part = [&](const Regs& r, int buf, int part) {
         unsigned char* base = smem + buf * kBufBytes;
         const uint32_t w = part == 0 ? r.b.x : r.b.y;
-        const uint32_t zq = (r.z >> ((r.z >> 8) * 4u)) & 0xfu;
+        const uint32_t zq = ((r.z >> r.zsh) & zp_mask) | zp_default;
         const uint32_t c4 = 0x80808080u - zq * 0x01010101u;
         const uint32_t lo = ((w & 0x0f0f0f0fu) + c4) ^ 0x80808080u;            // elements 0,2,4,6 of the dword, minus zp
         const uint32_t hi = (((w >> 4) & 0x0f0f0f0fu) + c4) ^ 0x80808080u;     // elements 1,3,5,7
@@ -474,15 +477,24 @@ __global__ __launch_bounds__(512) void acc4_prefill_kernel(Acc4PrefillParams p)
     store_part(regs[0], 0, 0);
     store_part(regs[0], 0, 1);
     __syncthreads();
-    for (int kt0 = 0; kt0 < steps; kt0 += D) {
+    // Main loop: whole rounds of D steps with no branch on the step count inside, so that the wait before each
+    // step counts loads exactly and the newer ones stay in flight. The last round runs with the conditions.
+    int kt0 = 0;
+    for (; kt0 + D < steps; kt0 += D) {
 #pragma unroll
         for (int s0 = 0; s0 < D; ++s0) {
-            const int kt = kt0 + s0;
-            load_global(regs[(s0 + D - 1) % D], kt + D - 1);
-            if (kt < steps) {
-                compute(s0 & 1, kt, regs[(s0 + 1) % D], kt + 1 < steps);
-                __syncthreads();
-            }
+            load_global(regs[(s0 + D - 1) % D], kt0 + s0 + D - 1);
+            compute(s0 & 1, kt0 + s0, regs[(s0 + 1) % D], true);
+            __syncthreads();
+        }
+    }
+#pragma unroll
+    for (int s0 = 0; s0 < D; ++s0) {
+        const int kt = kt0 + s0;
+        load_global(regs[(s0 + D - 1) % D], kt + D - 1);
+        if (kt < steps) {
+            compute(s0 & 1, kt, regs[(s0 + 1) % D], kt + 1 < steps);
+            __syncthreads();
         }
     }
 

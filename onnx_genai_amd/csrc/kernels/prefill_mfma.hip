@@ -1,13 +1,14 @@
 // Prefill path of MatMulNBits (M > 16, f16/bf16 activations): Y[M,N] = A[M,K] . dequant(B)[N,K]^T on the matrix cores.
 //
-// A workgroup of four waves owns a BM x 128 tile of Y and walks K in steps of 64. Per step it
+// A workgroup of eight waves owns a BM x 128 tile of Y and walks K in steps of 64. Per step it
 //   * copies a BM x 64 tile of A from global memory to LDS (16 bytes per lane, rows padded to 144 bytes so that
 //     the 32 lanes of an MFMA operand read hit different banks);
-//   * reads 128 x 64 packed 4-bit weights (one 16-byte piece = 32 nibbles = one lane), dequantizes them in registers
+//   * reads 128 x 64 packed 4-bit weights (one 8-byte piece = 16 nibbles = one lane), dequantizes them in registers
 //     and writes them to LDS as 16-bit floats. f16 with f16 scales: (0x6400|q) is 1024+q, a packed subtract of 1024+zp
 //     is exact and one packed multiply by the scale rounds once - the tile is bit-identical to f16((q-zp)*scale).
 //     Otherwise (bf16, or f32 scales): (q-zp)*scale in f32, rounded to nearest even;
-//   * runs v_mfma_f32_32x32x16 on 2 x 2 waves, each owning a (BM/2) x 64 sub-tile, f32 accumulators.
+//   * runs v_mfma_f32_32x32x16 on 4 x 2 waves, each owning a (BM/4) x 64 sub-tile, f32 accumulators. Two waves share
+//     a SIMD, so one's LDS and global waits are covered by the other's MFMAs.
 // LDS is double buffered: the global loads of step t+1 are in flight while the MFMAs of step t run, and one barrier
 // per step separates the two buffers. Edges in M and N are handled by range-checked buffer loads and masked stores.
 #include <hip/hip_fp16.h>
@@ -93,13 +94,13 @@ __device__ __forceinline__ uint32_t finish_f32(uint32_t pair, float off, float s
 // BF16: element type. BM: rows of Y per workgroup (128 or 256). SF32: scales are stored as f32 (otherwise in the
 // activations' 16-bit type). f16 activations with f16 scales dequantize in packed f16, everything else in f32.
 template <bool BF16, int BM, bool SF32>
-__global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillParams p)
+__global__ __launch_bounds__(512) void prefill_mfma_kernel(PrefillParams p)
 {
     constexpr bool F32MATH = BF16 || SF32;
-    constexpr int WM = BM / 2;             // wave sub-tile rows
+    constexpr int WM = BM / 4;             // wave sub-tile rows
     constexpr int TM = WM / 32;            // 32x32 MFMA tiles per wave along M
     constexpr int TN = 2;                  // and along N (64 columns)
-    constexpr int A_LOADS = BM / 32;       // 16-byte pieces of A per lane per step
+    constexpr int A_LOADS = BM / 64;       // 16-byte pieces of A per lane per step
     constexpr uint32_t kMagic = BF16 ? 0x43004300u : 0x64006400u;
     constexpr float kMagicF = BF16 ? 128.0f : 1024.0f;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -109,7 +110,7 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillParams p)
     const int t = threadIdx.x;
     const int lane = t & 63;
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave >> 1, wn = wave & 1;      // 4 x 2 waves
     // Column blocks vary fastest: the workgroups running at one time share a few row blocks of A (each XCD's L2 then
     // holds them once) and sweep the small packed B.
     const int64_t m_base = static_cast<int64_t>(blockIdx.y) * BM;
@@ -122,15 +123,16 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillParams p)
     const __amdgpu_buffer_rsrc_t srd_s = make_srd_p(static_cast<const unsigned char*>(p.scales) + n_base * p.kb * kScaleBytes,
                                                     static_cast<uint64_t>(cols_left * p.kb) * kScaleBytes);
     const bool has_zp = p.zp != nullptr;
+    const uint32_t zp_mask = has_zp ? 0xfu : 0u, zp_default = has_zp ? 0u : 8u;   // branch-free "8 when absent"
     const __amdgpu_buffer_rsrc_t srd_z = make_srd_p(has_zp ? p.zp + n_base * p.zp_row : p.b, has_zp ? static_cast<uint64_t>(cols_left * p.zp_row) : 0);
 
-    // A: lane -> (row t/8 + 32 i, piece t%8). B: lane -> (column t/2, half t%2 of the 64-element step).
+    // A: lane -> (row t/8 + 64 i, piece t%8). B: lane -> (column t/4, quarter t%4 of the 64-element step).
     const uint32_t a_goff = static_cast<uint32_t>(t >> 3) * static_cast<uint32_t>(p.k) * 2u + static_cast<uint32_t>((t & 7) * 16);
-    const uint32_t a_gstep = 32u * static_cast<uint32_t>(p.k) * 2u;
+    const uint32_t a_gstep = 64u * static_cast<uint32_t>(p.k) * 2u;
     const uint32_t a_loff = static_cast<uint32_t>((t >> 3) * kPitch + (t & 7) * 16);
-    const int bcol = t >> 1, bhalf = t & 1;
-    const uint32_t b_goff = static_cast<uint32_t>(bcol) * static_cast<uint32_t>(p.row_bytes) + static_cast<uint32_t>(bhalf * 16);
-    const uint32_t b_loff = static_cast<uint32_t>(bcol * kPitch + bhalf * 64);
+    const int bcol = t >> 2, bquarter = t & 3;
+    const uint32_t b_goff = static_cast<uint32_t>(bcol) * static_cast<uint32_t>(p.row_bytes) + static_cast<uint32_t>(bquarter * 8);
+    const uint32_t b_loff = static_cast<uint32_t>(bcol * kPitch + bquarter * 32);
     const uint32_t s_goff = static_cast<uint32_t>(bcol) * static_cast<uint32_t>(p.kb) * kScaleBytes;
     const uint32_t z_goff = static_cast<uint32_t>(bcol) * static_cast<uint32_t>(p.zp_row);
 
@@ -151,37 +153,42 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillParams p)
     constexpr int D = 4;
     struct Regs {
         uint4 a[A_LOADS];
-        uint4 b;
+        uint2 b;
         uint32_t s;      // raw scale bits; converted when the step is dequantized, so that no load is waited for early
-        uint32_t z;      // raw zero-point byte and the nibble to take from it
+        uint32_t z;      // raw zero-point byte
+        uint32_t zsh;    // shift of the nibble to take from it
     };
     Regs regs[D];
 
     auto load_global = [&](Regs& r, int kt) {
 #pragma unroll
         for (int i = 0; i < A_LOADS; ++i) r.a[i] = load16_p(srd_a, a_goff + static_cast<uint32_t>(i) * a_gstep, static_cast<uint32_t>(kt) * 128u);
-        r.b = load16_p(srd_b, b_goff, static_cast<uint32_t>(kt) * 32u);
-        const uint32_t blk = static_cast<uint32_t>((kt * kBK + bhalf * 32) >> p.bs_log2);
+        const auto bw = __builtin_amdgcn_raw_buffer_load_b64(srd_b, static_cast<int>(b_goff), static_cast<int>(kt * 32), 0);
+        r.b = make_uint2(bw[0], bw[1]);
+        const uint32_t blk = static_cast<uint32_t>((kt * kBK + bquarter * 16) >> p.bs_log2);
         if constexpr (SF32) r.s = __builtin_amdgcn_raw_buffer_load_b32(srd_s, static_cast<int>(s_goff + blk * 4u), 0, 0);
         else r.s = __builtin_amdgcn_raw_buffer_load_b16(srd_s, static_cast<int>(s_goff + blk * 2u), 0, 0);
-        const uint32_t zbyte = has_zp ? static_cast<uint32_t>(__builtin_amdgcn_raw_buffer_load_b8(srd_z, static_cast<int>(z_goff + (blk >> 1)), 0, 0)) : 0x88u;
-        r.z = zbyte | ((blk & 1u) << 8);
+        // loaded even without zero points (the empty range then returns 0): a branch here would split the loop body
+        const uint32_t zraw = static_cast<uint32_t>(__builtin_amdgcn_raw_buffer_load_b8(srd_z, static_cast<int>(z_goff + (blk >> 1)), 0, 0));
+        r.z = zraw;                 // no arithmetic on a loaded value here: it would wait for the load at once
+        r.zsh = (blk & 1u) * 4u;
     };
-    // Quarter `part` (0..3) of one step's trip from registers to LDS: A pieces part, part+4, ... and packed dword `part`
-    // of B, dequantized. Four quarters make a step; they are issued between the MFMA batches of the step before, so
-    // that their VALU and LDS-write work runs while the matrix cores are busy.
+    // Quarter `part` (0..3) of one step's trip from registers to LDS: A pieces part, part+4, ... and, in quarters 0 and
+    // 2, one packed dword of B, dequantized. Four quarters make a step; they are issued between the MFMA batches of
+    // the step before, so that their VALU and LDS-write work runs while the matrix cores are busy.
     auto store_part = [&](const Regs& r, int buf, int part) {
         unsigned char* la = lds_a + buf * (BM * kPitch) + a_loff;
 #pragma unroll
-        for (int i = part; i < A_LOADS; i += 4) *reinterpret_cast<uint4*>(la + i * 32 * kPitch) = r.a[i];
+        for (int i = part; i < A_LOADS; i += 4) *reinterpret_cast<uint4*>(la + i * 64 * kPitch) = r.a[i];
+        if (part & 1) return;
         unsigned char* lb = lds_b + buf * (kBN * kPitch) + b_loff;
-        const uint32_t w = part == 0 ? r.b.x : part == 1 ? r.b.y : part == 2 ? r.b.z : r.b.w, w4 = w >> 4;
+        const uint32_t w = part == 0 ? r.b.x : r.b.y, w4 = w >> 4;
         uint32_t pr[4];
         pr[0] = magic_pair(w, w4, 0x0c040c00u, kMagic);
         pr[1] = magic_pair(w, w4, 0x0c050c01u, kMagic);
         pr[2] = magic_pair(w, w4, 0x0c060c02u, kMagic);
         pr[3] = magic_pair(w, w4, 0x0c070c03u, kMagic);
-        const uint32_t zq = (r.z >> ((r.z >> 8) * 4u)) & 0xfu;
+        const uint32_t zq = ((r.z >> r.zsh) & zp_mask) | zp_default;
         if constexpr (F32MATH) {
             const float off = kMagicF + static_cast<float>(zq);
             const float sc = SF32 ? __uint_as_float(r.s) : (BF16 ? __uint_as_float(r.s << 16) : f16_bits_to_f32(static_cast<uint16_t>(r.s)));
@@ -193,7 +200,7 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillParams p)
 #pragma unroll
             for (int i = 0; i < 4; ++i) pr[i] = finish_f16(pr[i], __builtin_bit_cast(half2_t, o2), __builtin_bit_cast(half2_t, s2));
         }
-        *reinterpret_cast<uint4*>(lb + part * 16) = make_uint4(pr[0], pr[1], pr[2], pr[3]);
+        *reinterpret_cast<uint4*>(lb + (part >> 1) * 16) = make_uint4(pr[0], pr[1], pr[2], pr[3]);
     };
     auto store_lds = [&](const Regs& r, int buf) {
 #pragma unroll
@@ -233,15 +240,25 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillParams p)
     for (int s0 = 0; s0 < D - 1; ++s0) load_global(regs[s0], s0);
     store_lds(regs[0], 0);
     __syncthreads();
-    for (int kt0 = 0; kt0 < steps; kt0 += D) {
+    // Main loop: whole rounds of D steps with no branch inside, so that the wait before each step counts loads
+    // exactly and the newer ones stay in flight (a branch would make the compiler drain them all). The last
+    // round, which holds the final step, runs with the conditions.
+    int kt0 = 0;
+    for (; kt0 + D < steps; kt0 += D) {
 #pragma unroll
         for (int s0 = 0; s0 < D; ++s0) {
-            const int kt = kt0 + s0;
-            load_global(regs[(s0 + D - 1) % D], kt + D - 1);
-            if (kt < steps) {
-                compute(s0 & 1, regs[(s0 + 1) % D], kt + 1 < steps);
-                __syncthreads();
-            }
+            load_global(regs[(s0 + D - 1) % D], kt0 + s0 + D - 1);
+            compute(s0 & 1, regs[(s0 + 1) % D], true);
+            __syncthreads();
+        }
+    }
+#pragma unroll
+    for (int s0 = 0; s0 < D; ++s0) {
+        const int kt = kt0 + s0;
+        load_global(regs[(s0 + D - 1) % D], kt + D - 1);
+        if (kt < steps) {
+            compute(s0 & 1, regs[(s0 + 1) % D], kt + 1 < steps);
+            __syncthreads();
         }
     }
 
@@ -277,7 +294,7 @@ static int launch_prefill(const PrefillParams& p, hipStream_t stream)
         const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
         if (e != hipSuccess) return static_cast<int>(e);
     }
-    hipLaunchKernelGGL(kernel, grid, dim3(256), lds, stream, p);
+    hipLaunchKernelGGL(kernel, grid, dim3(512), lds, stream, p);
     return static_cast<int>(hipGetLastError());
 }
 
