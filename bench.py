@@ -30,6 +30,7 @@ from onnx_genai_amd import synth  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA, published
+MFMA_I8_PEAK_TOPS = 5000.0     # MI355X dense int8 MFMA, published
 MFMA_I8_PEAK_TOPS = 5000.0
 
 LAYERS = 28
@@ -211,6 +212,8 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=20.0)
     ap.add_argument("--only-roofline", action="store_true",
                     help="run only the roofline leg (decode kernel on the gate_up shape) and one 256 MiB device copy: the command profiles are taken from")
+    ap.add_argument("--only-tables", action="store_true",
+                    help="run only the prefill and accuracy_level=4 tables, one JSON line per row (the command their profiles are taken from)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (no collectives exist on the MatMulNBits path); use --gpus 1")
@@ -219,6 +222,10 @@ def main():
     info = ep.device_info()
     if args.only_roofline:
         return roofline_only(ep, args)
+    if args.only_tables:
+        for row in prefill_table(ep) + acc4_table(ep):
+            print(json.dumps(row), flush=True)
+        return
     nodes, a_bufs = build_decode_stack(ep, args.m, args.layers)
     step_bytes = sum(n.bytes for n in nodes)
     step_flops = sum(n.flops for n in nodes)
@@ -374,19 +381,26 @@ def prefill_table(ep):
 
 
 def acc4_table(ep):
-    """accuracy_level=4 at 70B-class shapes (configs[4]): fp16, block 64, zero points; M=1 rows only here."""
+    """accuracy_level=4 at 70B-class shapes (configs[4]): fp16, block 64, zero points, M in {1, 256, 4096}. Each call is
+    the activation quantizer plus the int8 MFMA kernel. M=1 rows are priced against HBM, the others against int8 MFMA."""
     table = []
     for k, n in ((8192, 28672), (28672, 8192), (8192, 10240)):
-        for m in (1,):
+        for m in (1, 256, 4096):
             node = Node(ep, "acc4", k, n, 64, 9, E.F16, m, accuracy_level=4)
             a = ep.upload(synth.make_activation(m, k, 8, E.F16))
             node.run(a)
             ep.sync()
             graph = capture(ep, lambda: node.run(a))
-            ms = time_graph(ep, graph, 20, 2)
+            ms = time_graph(ep, graph, 20 if m == 1 else 3, 2 if m == 1 else 1)
             graph.release()
-            table.append({"k": k, "n": n, "m": m, "us": round(ms * 1e3, 1), "gbs": round(node.bytes / (ms * 1e-3) / 1e9, 1),
-                          "hbm_frac": round(node.bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "variant": node.ops.kernel.last_variant()})
+            row = {"k": k, "n": n, "m": m, "us": round(ms * 1e3, 1), "variant": node.ops.kernel.last_variant()}
+            if m == 1:
+                row["gbs"] = round(node.bytes / (ms * 1e-3) / 1e9, 1)
+                row["hbm_frac"] = round(node.bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+            else:
+                row["tops"] = round(node.flops / (ms * 1e-3) / 1e12, 1)
+                row["mfma_i8_frac"] = round(node.flops / (ms * 1e-3) / 1e12 / MFMA_I8_PEAK_TOPS, 4)
+            table.append(row)
             ep.deallocate(a)
             node.free(ep)
     return table
