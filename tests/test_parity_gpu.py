@@ -451,6 +451,48 @@ def test_acc4_decode_wave_counts_agree(port, waves, s_dt):
         provider.shutdown()
 
 
+def test_acc4_power_of_two_scaling_at_full_70b_shape(ep):
+    """Size-independent property at a full 70B-class shape: doubling A doubles every block scale and leaves the int8
+    codes alone, so Y doubles exactly (f32 output, no bias) - on the decode kernel and on the tiled kernel."""
+    a_dt, bs, n, k = E.F16, 64, 10240, 8192
+    b, s, zp = synth.make_weights(n, k, bs, 23, zero_points=True, scale_lo=0.002, scale_hi=0.01, scale_dtype=a_dt)
+    ops = E.DeviceOperands(ep, b, s, a_dt, zp, n, k, bs, accuracy_level=4)
+    for m in (1, 40):
+        a = np.random.default_rng(m).uniform(-1.0, 1.0, size=(m, k)).astype(np.float16)
+        ys = []
+        for scale in (1.0, 2.0):
+            ab, yb = ep.upload((a * np.float16(scale)).astype(np.float16)), ep.allocate(m * n * 4)
+            ops.run(ab, a_dt, m, yb, E.F32)
+            ys.append(ep.download(yb, (m, n), np.float32))
+            ep.deallocate(ab)
+            ep.deallocate(yb)
+        assert ops.kernel.last_variant() == "acc4_mfma_i8"
+        assert np.isfinite(ys[0]).all() and np.abs(ys[0]).max() > 0
+        assert np.array_equal(ys[1], 2.0 * ys[0])
+    ops.free()
+
+
+def test_prefill_linearity_at_full_8b_shape(ep):
+    """Size-independent property at a full Llama-3-8B MLP shape: with small-integer activations every product and
+    partial sum of A1 + A2 is the sum of those of A1 and A2 up to f32 rounding of the accumulation."""
+    a_dt, bs, m, n, k = E.F16, 32, 512, 14336, 4096
+    b, s, _ = synth.make_weights(n, k, bs, 29, zero_points=False, scale_lo=0.001, scale_hi=0.01, scale_dtype=a_dt)
+    ops = E.DeviceOperands(ep, b, s, a_dt, None, n, k, bs)
+    rng = np.random.default_rng(29)
+    a1 = rng.integers(-8, 9, size=(m, k)).astype(np.float16)
+    a2 = rng.integers(-8, 9, size=(m, k)).astype(np.float16)
+    ys = []
+    for a in (a1, a2, (a1 + a2).astype(np.float16)):
+        ab, yb = ep.upload(a), ep.allocate(m * n * 4)
+        ops.run(ab, a_dt, m, yb, E.F32)
+        ys.append(ep.download(yb, (m, n), np.float32).astype(np.float64))
+        ep.deallocate(ab)
+        ep.deallocate(yb)
+    assert ops.kernel.last_variant() == "prefill_mfma_lds"
+    assert helpers.rel_l2(ys[0] + ys[1], ys[2]) <= 1e-5
+    ops.free()
+
+
 def test_acc4_with_caller_workspace(ep, port):
     a_dt, bs, m, n, k = E.F16, 64, 4, 64, 512
     b, s, zp = synth.make_weights(n, k, bs, 91, zero_points=True, scale_lo=0.002, scale_hi=0.01, scale_dtype=a_dt)
