@@ -1,4 +1,4 @@
-// Decode path of MatMulNBits over weights repacked for streaming (M <= 4, f16/bf16 activations).
+// Decode path of MatMulNBits over weights repacked for streaming (f16/bf16 activations; M <= 4, or M <= 16 when N is large).
 //
 // When B, scales and zero points are constant initializers, the kernel object repacks them once into
 // the order in which the split-K MFMA kernel consumes them, so that every vector load of a wave is
@@ -296,6 +296,186 @@ static int launch_packed_bs(const PackedParams& p, int bs, int waves, hipStream_
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// The same stream for 5 <= M <= 16 and many columns: activations shared through LDS.
+// ---------------------------------------------------------------------------------------------
+//
+// With several rows the activations outweigh a column group's weights (16 rows x 128 k x 2 bytes against 16 columns
+// x 64 bytes per tile), and a kernel in which every wave fetches its own copy is bound by L2, not HBM. Here a
+// workgroup of eight waves owns eight column groups - one wave each, streaming the whole of K - and all eight read
+// the activations from one LDS copy, filled window by window (1024 k = two tile groups, double buffered: the next
+// window travels global -> registers while the current one is multiplied, and moves registers -> LDS just before the
+// barrier that ends the window). No split-K, so no reduction: a wave stores its 16 columns itself.
+
+constexpr int kWinK = 1024;                        // k per activation window: two tile groups
+constexpr int kWinPitch = kWinK * 2 + 16;          // bytes per LDS row: 16 rows start in 16 different bank quads
+constexpr int kWideWaves = 8;
+
+template <bool BF16, int BS, typename ST>
+__global__ __launch_bounds__(512) void decode_wide_kernel(PackedParams p)
+{
+    constexpr int U = kGroupTiles;
+    constexpr int NBT = 128 / BS;
+    constexpr int NB = U * NBT;
+    constexpr int R = packed_record_bytes(BS, static_cast<int>(sizeof(ST)));
+    constexpr int NR = R / 16;
+    constexpr int kBufBytes = 16 * kWinPitch;
+    constexpr uint32_t kMagicNeg = BF16 ? 0xC300C300u : 0xE400E400u;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];   // [2][16][kWinPitch]
+
+    const int t = threadIdx.x;
+    const int lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int c = lane & 15;
+    const int g = lane >> 4;
+    const int64_t col_groups = (p.n + 15) / 16;
+    const int64_t cgi = static_cast<int64_t>(blockIdx.x) * kWideWaves + wave;
+    const bool active = cgi < col_groups;                 // a wave beyond the last column group still helps with the windows
+    const int64_t n_base = cgi * 16;
+
+    const __amdgpu_buffer_rsrc_t srd_p = make_srd(p.packed + (active ? cgi : 0) * p.cg_stride, active ? static_cast<uint64_t>(p.cg_stride) : 0);
+    const __amdgpu_buffer_rsrc_t srd_a = make_srd(p.a, static_cast<uint64_t>(p.m * p.k) * 2);
+
+    const uint32_t w_off = static_cast<uint32_t>(lane * 16);
+    const uint32_t r_off = static_cast<uint32_t>(kChunkWeights + c * R);
+    // window fill: thread -> row t / 32, pieces t % 32 + 32 i (i < 4) of the row's 128 pieces
+    const int wrow = t >> 5, wpiece = t & 31;
+    const uint32_t win_goff = static_cast<uint32_t>(wrow) * static_cast<uint32_t>(p.k) * 2u + static_cast<uint32_t>(wpiece * 16);
+    const uint32_t win_loff = static_cast<uint32_t>(wrow * kWinPitch + wpiece * 16);
+    // operand of MFMA j of tile x of the window: row c, elements x*128 + j*32 + g*8 .. +8
+    const uint32_t frag_off = static_cast<uint32_t>(c * kWinPitch + g * 16);
+    const uint32_t mask = __builtin_amdgcn_mov_dpp(p.nibble_mask, 0xE4, 0xf, 0xf, false), magic = p.magic;
+
+    float4p_t y = {0.f, 0.f, 0.f, 0.f};
+    float4p_t acc = {0.f, 0.f, 0.f, 0.f};
+
+    struct Grp {
+        uint4 w[kGroupTiles];
+        uint4 r[NR];
+    };
+    auto fetch_group = [&](Grp& grp, int gi) {
+        if (gi >= p.groups) return;
+        const uint32_t soff = static_cast<uint32_t>(gi) * static_cast<uint32_t>(p.chunk_bytes);
+#pragma unroll
+        for (int u = 0; u < U; ++u) grp.w[u] = load16(srd_p, w_off + static_cast<uint32_t>(u * 1024), soff);
+#pragma unroll
+        for (int i = 0; i < NR; ++i) grp.r[i] = load16(srd_p, r_off + static_cast<uint32_t>(i * 16), soff);
+    };
+    uint4 wa[4];
+    auto load_window = [&](int win) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int64_t k0 = static_cast<int64_t>(win) * kWinK + (wpiece + 32 * i) * 8;
+            uint32_t off = win_goff + static_cast<uint32_t>(i * 512);
+            if (wrow >= p.m || k0 >= p.k) off = kOutOfRange;      // K is a multiple of 8: a piece is all inside or all outside
+            wa[i] = load16(srd_a, off, static_cast<uint32_t>(win) * (kWinK * 2u));
+        }
+    };
+    auto store_window = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) *reinterpret_cast<uint4*>(smem + buf * kBufBytes + win_loff + i * 512) = wa[i];
+    };
+    auto compute_group = [&](const Grp& grp, int buf, int half) {
+        uint32_t rr[NR * 4];
+#pragma unroll
+        for (int i = 0; i < NR; ++i) {
+            rr[4 * i] = grp.r[i].x;
+            rr[4 * i + 1] = grp.r[i].y;
+            rr[4 * i + 2] = grp.r[i].z;
+            rr[4 * i + 3] = grp.r[i].w;
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const unsigned char* fa = smem + buf * kBufBytes + frag_off + (half * U + u) * 256;
+            uint4 av[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) av[j] = *reinterpret_cast<const uint4*>(fa + j * 64);
+            const uint32_t wd[4] = {grp.w[u].x, grp.w[u].y, grp.w[u].z, grp.w[u].w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int bi = u * NBT + (j * 32) / BS;
+                const int zbyte = NB * static_cast<int>(sizeof(ST)) + bi;
+                const uint32_t z = (rr[zbyte / 4] >> ((zbyte % 4) * 8)) & 0xffu;
+                const uint32_t zpair = kMagicNeg | (z * 0x00010001u);
+                const uint4 zc = make_uint4(zpair, zpair, zpair, zpair);
+                const uint32_t w = wd[j];
+                uint4 op;
+                op.x = (w & mask) | magic;
+                op.y = ((w >> 4) & mask) | magic;
+                op.z = ((w >> 8) & mask) | magic;
+                op.w = ((w >> 12) & mask) | magic;
+                acc = mfma16p<BF16>(av[j], op, acc);
+                acc = mfma16p<BF16>(av[j], zc, acc);
+                if (((j + 1) * 32) % BS == 0 || j == 3) {
+                    float sf;
+                    if constexpr (sizeof(ST) == 4) {
+                        sf = __uint_as_float(rr[bi]);
+                    } else {
+                        const uint32_t raw = (rr[bi / 2] >> ((bi % 2) * 16)) & 0xffffu;
+                        sf = BF16 ? __uint_as_float(raw << 16) : f16_bits_to_f32(static_cast<uint16_t>(raw));
+                    }
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        y[r] = fmaf(sf, acc[r], y[r]);
+                        acc[r] = 0.f;
+                    }
+                }
+            }
+        }
+    };
+
+    const int windows = (p.groups + 1) / 2;
+    Grp ga, gb;
+    fetch_group(ga, 0);
+    load_window(0);
+    store_window(0);
+    __syncthreads();
+    for (int win = 0; win < windows; ++win) {
+        const int gi = win * 2;
+        const int buf = win & 1;
+        if (win + 1 < windows) load_window(win + 1);
+        fetch_group(gb, gi + 1);
+        compute_group(ga, buf, 0);
+        fetch_group(ga, gi + 2);
+        if (gi + 1 < p.groups) compute_group(gb, buf, 1);
+        if (win + 1 < windows) store_window(buf ^ 1);
+        __syncthreads();
+    }
+
+    if (active) {
+        const int64_t col = n_base + c;
+        if (col < p.n) {
+            const float bias = p.bias ? load_as_f32(p.bias, p.bias_dtype, col) : 0.f;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int row = 4 * g + r;
+                if (row < p.m) store_from_f32(p.y, p.y_dtype, static_cast<int64_t>(row) * p.n + col, y[r] + bias);
+            }
+        }
+    }
+}
+
+template <bool BF16, typename ST>
+static int launch_wide_bs(const PackedParams& p, int bs, hipStream_t stream)
+{
+    const int64_t col_groups = (p.n + 15) / 16;
+    const dim3 grid(static_cast<unsigned>((col_groups + kWideWaves - 1) / kWideWaves));
+    const size_t lds = 2 * 16 * kWinPitch;
+    auto go = [&](auto kernel) {
+        if (lds > 65536) {
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+            if (e != hipSuccess) return static_cast<int>(e);
+        }
+        hipLaunchKernelGGL(kernel, grid, dim3(kWideWaves * 64), lds, stream, p);
+        return static_cast<int>(hipGetLastError());
+    };
+    switch (bs) {
+        case 32: return go(decode_wide_kernel<BF16, 32, ST>);
+        case 64: return go(decode_wide_kernel<BF16, 64, ST>);
+        default: return go(decode_wide_kernel<BF16, 128, ST>);
+    }
+}
+
 static int packed_groups(const RocmMatMulNBitsArgs* a)
 {
     const int64_t kb = (a->k + a->block_size - 1) / a->block_size;
@@ -310,9 +490,13 @@ static int packed_chunk_bytes(const RocmMatMulNBitsArgs* a)
 
 }  // namespace mnb
 
+// Rows 5..16 only run from the repacked copy in the shared-activation kernel, which wants many column groups.
+static bool wide_shape(const RocmMatMulNBitsArgs* a) { return a->m >= 5 && a->n >= 16384; }
+
 extern "C" int rocm_decode_packed_eligible(const RocmMatMulNBitsArgs* a)
 {
-    if (!rocm_decode_mfma_eligible(a) || a->m > 4) return 0;
+    if (!rocm_decode_mfma_eligible(a)) return 0;
+    if (a->m > 4 && !wide_shape(a)) return 0;
     return static_cast<int64_t>(mnb::packed_groups(a)) * mnb::packed_chunk_bytes(a) < 0x7fffffff;
 }
 
@@ -363,6 +547,14 @@ extern "C" int rocm_launch_decode_packed(const RocmMatMulNBitsArgs* a, const voi
     const bool bf16 = a->a_dtype == ROCM_DT_BF16;
     p.magic = bf16 ? 0x43004300u : 0x64006400u;
 
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const bool f32_scales = a->scale_dtype == ROCM_DT_F32;
+    if (wide_shape(a)) {
+        p.groups_per_wave = p.groups;
+        if (bf16) return f32_scales ? mnb::launch_wide_bs<true, float>(p, a->block_size, s) : mnb::launch_wide_bs<true, uint16_t>(p, a->block_size, s);
+        return f32_scales ? mnb::launch_wide_bs<false, float>(p, a->block_size, s) : mnb::launch_wide_bs<false, uint16_t>(p, a->block_size, s);
+    }
+
     int w = waves;
     if (w <= 0) {
         const int64_t wgs = (a->n + 15) / 16;
@@ -376,8 +568,6 @@ extern "C" int rocm_launch_decode_packed(const RocmMatMulNBitsArgs* a, const voi
     w = (p.groups + gpw - 1) / gpw;
     p.groups_per_wave = gpw;
 
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    const bool f32_scales = a->scale_dtype == ROCM_DT_F32;
     if (bf16) return f32_scales ? mnb::launch_packed_bs<true, float>(p, a->block_size, w, s) : mnb::launch_packed_bs<true, uint16_t>(p, a->block_size, w, s);
     return f32_scales ? mnb::launch_packed_bs<false, float>(p, a->block_size, w, s) : mnb::launch_packed_bs<false, uint16_t>(p, a->block_size, w, s);
 }

@@ -167,6 +167,12 @@ DECODE_CASES = [
     (E.F16, E.F32, 64, True, 1, 100, 64 * 21),  # f32 scales, odd block count, tile groups padded
     (E.BF16, E.F32, 32, True, 3, 50, 32 * 19),
     (E.BF16, E.BF16, 64, False, 4, 70, 4096),
+    # many columns and several rows: activations shared through LDS, one wave per 16 columns
+    (E.BF16, E.BF16, 128, True, 16, 16400, 3584),
+    (E.F16, E.F16, 32, True, 5, 16384, 1000),
+    (E.F16, E.F32, 64, False, 6, 20000, 64 * 21),
+    (E.BF16, E.BF16, 128, True, 8, 37888, 3584),
+    (E.F16, E.F16, 128, True, 13, 16385, 2048 + 8),
 ]
 
 
@@ -181,7 +187,7 @@ def test_decode_matches_oracle(ep, ep_unpacked, port, prepack, a_dt, s_dt, bs, z
 
     # f32 output: the arithmetic itself, before any narrowing
     y32, variant = run_op(ep, a, a_dt, b, s, s_dt, zp, n, k, bs, bias=bias, bias_dtype=a_dt, y_dtype=E.F32)
-    assert variant == ("decode_mfma_packed" if prepack and m <= 4 else "decode_mfma_splitk")
+    assert variant == ("decode_mfma_packed" if prepack and (m <= 4 or n >= 16384) else "decode_mfma_splitk")   # m 2..4 at large n: the 4-row kernel
     # The kernel carries each weight as (2^10 + q) in f16 or (2^7 + q) in bf16 and cancels the offset inside the
     # f32 accumulator, which costs 10 (7) of its 24 bits: a few 1e-5 on outputs that themselves cancel.
     assert helpers.rel_l2(y32, want64) <= 1e-4
