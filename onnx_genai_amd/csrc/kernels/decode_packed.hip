@@ -120,10 +120,14 @@ struct PackedGroup {
 };
 
 // BF16: activation element type. BS: block size. MR: rows staged (1 or 4; M <= MR). ST: storage type of the scales.
-// The one-row, block-128, 16-bit-scale variant fits 96 registers without spilling, which buys a fifth wave per SIMD
-// (measured 3 % on the 3584 -> 37888 shape); the others keep the compiler's own choice.
-template <bool BF16, int BS, int MR, typename ST>
-__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu((BS == 128 && MR == 1 && sizeof(ST) == 2) ? 5 : 1))) void decode_packed_kernel(PackedParams p)
+// SETS: register sets of one group each. 2: the next group's loads are in flight while this one is multiplied - for
+// launches with few waves, where each wave must cover memory latency by itself. 1: no prefetch, 62 registers, eight
+// waves per SIMD - for launches with thousands of waves, where the other resident waves cover it better (measured on
+// 3584 -> 37888: 15.6 us against 17.0 us). With two sets the one-row, block-128, 16-bit-scale variant fits 96
+// registers without spilling (a fifth wave per SIMD); the other variants keep the compiler's own choice.
+template <bool BF16, int BS, int MR, typename ST, int SETS>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu((BS == 128 && MR == 1 && sizeof(ST) == 2) ? (SETS == 1 ? 8 : 5) : 1)))
+void decode_packed_kernel(PackedParams p)
 {
     constexpr int U = kGroupTiles;
     constexpr int NBT = 128 / BS;
@@ -244,11 +248,24 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu((BS == 128 
         for (int u = 0; u < U; ++u) compute_tile(cur, u, parity);
     };
 
-    Grp ga, gb;
-    fetch_group(ga, g_begin);
-    for (int gi = g_begin; gi < g_end; gi += 2) {
-        run_group(ga, gb, gi, 0);
-        if (gi + 1 < g_end) run_group(gb, ga, gi + 1, 1);
+    if constexpr (SETS == 2) {
+        Grp ga, gb;
+        fetch_group(ga, g_begin);
+        for (int gi = g_begin; gi < g_end; gi += 2) {
+            run_group(ga, gb, gi, 0);
+            if (gi + 1 < g_end) run_group(gb, ga, gi + 1, 1);
+        }
+    } else {
+        Grp ga;
+        for (int gi = g_begin; gi < g_end; ++gi) {
+            fetch_group(ga, gi);
+            if constexpr (MR == 1) {
+                *reinterpret_cast<uint4*>(stage + st_write) = ga.a[0];
+                lds_order();
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) compute_tile(ga, u, 0);
+        }
     }
 
     // ---- split-K reduction across the waves of this workgroup, in wave order ----
@@ -271,30 +288,30 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu((BS == 128 
     }
 }
 
-template <bool BF16, int BS, int MR, typename ST>
+template <bool BF16, int BS, int MR, typename ST, int SETS>
 static int launch_packed_cfg(const PackedParams& p, int waves, hipStream_t stream)
 {
     const unsigned grid = static_cast<unsigned>((p.n + 15) / 16);
     const size_t stage = static_cast<size_t>(waves) * 2 * (MR == 1 ? 1024 : MR * kRowPitchP);
     const size_t red = static_cast<size_t>(waves) * 1024;
-    hipLaunchKernelGGL((decode_packed_kernel<BF16, BS, MR, ST>), dim3(grid), dim3(waves * 64), stage > red ? stage : red, stream, p);
+    hipLaunchKernelGGL((decode_packed_kernel<BF16, BS, MR, ST, SETS>), dim3(grid), dim3(waves * 64), stage > red ? stage : red, stream, p);
     return static_cast<int>(hipGetLastError());
 }
 
-template <bool BF16, typename ST>
-static int launch_packed_bs(const PackedParams& p, int bs, int waves, hipStream_t stream)
+template <bool BF16, int BS, typename ST>
+static int launch_packed_mr(const PackedParams& p, int waves, bool single_set, hipStream_t stream)
 {
-    if (p.m <= 1) {
-        switch (bs) {
-            case 32: return launch_packed_cfg<BF16, 32, 1, ST>(p, waves, stream);
-            case 64: return launch_packed_cfg<BF16, 64, 1, ST>(p, waves, stream);
-            default: return launch_packed_cfg<BF16, 128, 1, ST>(p, waves, stream);
-        }
-    }
+    if (p.m <= 1) return single_set ? launch_packed_cfg<BF16, BS, 1, ST, 1>(p, waves, stream) : launch_packed_cfg<BF16, BS, 1, ST, 2>(p, waves, stream);
+    return launch_packed_cfg<BF16, BS, 4, ST, 2>(p, waves, stream);
+}
+
+template <bool BF16, typename ST>
+static int launch_packed_bs(const PackedParams& p, int bs, int waves, bool single_set, hipStream_t stream)
+{
     switch (bs) {
-        case 32: return launch_packed_cfg<BF16, 32, 4, ST>(p, waves, stream);
-        case 64: return launch_packed_cfg<BF16, 64, 4, ST>(p, waves, stream);
-        default: return launch_packed_cfg<BF16, 128, 4, ST>(p, waves, stream);
+        case 32: return launch_packed_mr<BF16, 32, ST>(p, waves, single_set, stream);
+        case 64: return launch_packed_mr<BF16, 64, ST>(p, waves, single_set, stream);
+        default: return launch_packed_mr<BF16, 128, ST>(p, waves, single_set, stream);
     }
 }
 
@@ -557,12 +574,22 @@ extern "C" int rocm_launch_decode_packed(const RocmMatMulNBitsArgs* a, const voi
         return f32_scales ? mnb::launch_wide_bs<false, float>(p, a->block_size, s) : mnb::launch_wide_bs<false, uint16_t>(p, a->block_size, s);
     }
 
+    // Waves per workgroup. Many column groups (thousands of waves even at four per group): short waves of at most two
+    // tile groups and no prefetch, so that eight of them fit a SIMD and cover each other's memory latency. Few column
+    // groups: enough waves per group to reach about 8k in flight, each prefetching its next group.
+    const int64_t wgs = (a->n + 15) / 16;
     int w = waves;
+    bool single_set = a->m <= 1 && wgs * 4 >= 6144;
     if (w <= 0) {
-        const int64_t wgs = (a->n + 15) / 16;
-        const int want = static_cast<int>((8192 + wgs - 1) / wgs);   // waves per workgroup to reach ~8k waves
-        w = want < p.groups ? want : p.groups;                       // at least one group per wave
+        if (single_set) {
+            w = (p.groups + 1) / 2;
+        } else {
+            const int want = static_cast<int>((8192 + wgs - 1) / wgs);
+            w = want < p.groups ? want : p.groups;               // at least one group per wave
+        }
         if (w < 1) w = 1;
+    } else {
+        single_set = a->m <= 1 && wgs * w >= 6144;
     }
     if (w > 8) w = 8;
     if (w > p.groups) w = p.groups;
@@ -570,6 +597,6 @@ extern "C" int rocm_launch_decode_packed(const RocmMatMulNBitsArgs* a, const voi
     w = (p.groups + gpw - 1) / gpw;
     p.groups_per_wave = gpw;
 
-    if (bf16) return f32_scales ? mnb::launch_packed_bs<true, float>(p, a->block_size, w, s) : mnb::launch_packed_bs<true, uint16_t>(p, a->block_size, w, s);
-    return f32_scales ? mnb::launch_packed_bs<false, float>(p, a->block_size, w, s) : mnb::launch_packed_bs<false, uint16_t>(p, a->block_size, w, s);
+    if (bf16) return f32_scales ? mnb::launch_packed_bs<true, float>(p, a->block_size, w, single_set, s) : mnb::launch_packed_bs<true, uint16_t>(p, a->block_size, w, single_set, s);
+    return f32_scales ? mnb::launch_packed_bs<false, float>(p, a->block_size, w, single_set, s) : mnb::launch_packed_bs<false, uint16_t>(p, a->block_size, w, single_set, s);
 }
