@@ -302,7 +302,7 @@ template <bool BF16, int BS, typename ST>
 static int launch_packed_mr(const PackedParams& p, int waves, bool single_set, hipStream_t stream)
 {
     if (p.m <= 1) return single_set ? launch_packed_cfg<BF16, BS, 1, ST, 1>(p, waves, stream) : launch_packed_cfg<BF16, BS, 1, ST, 2>(p, waves, stream);
-    return launch_packed_cfg<BF16, BS, 4, ST, 2>(p, waves, stream);
+    return single_set ? launch_packed_cfg<BF16, BS, 4, ST, 1>(p, waves, stream) : launch_packed_cfg<BF16, BS, 4, ST, 2>(p, waves, stream);
 }
 
 template <bool BF16, typename ST>
@@ -322,16 +322,18 @@ static int launch_packed_bs(const PackedParams& p, int bs, int waves, bool singl
 // With several rows the activations outweigh a column group's weights (16 rows x 128 k x 2 bytes against 16 columns
 // x 64 bytes per tile), and a kernel in which every wave fetches its own copy is bound by L2, not HBM. Here a
 // workgroup of eight waves owns eight column groups - one wave each, streaming the whole of K - and all eight read
-// the activations from one LDS copy, filled window by window (1024 k = two tile groups, double buffered: the next
+// the activations from one LDS copy, filled window by window (512 k = one tile group, double buffered: the next
 // window travels global -> registers while the current one is multiplied, and moves registers -> LDS just before the
-// barrier that ends the window). No split-K, so no reduction: a wave stores its 16 columns itself.
+// barrier that ends the window). No split-K, so no reduction: a wave stores its 16 columns itself. Weights are not
+// prefetched: the kernel is small enough (registers and 33 KB of LDS) for four workgroups per CU, and the other
+// resident waves cover a wave's memory latency better than a second register set does.
 
-constexpr int kWinK = 1024;                        // k per activation window: two tile groups
+constexpr int kWinK = 512;                         // k per activation window: one tile group
 constexpr int kWinPitch = kWinK * 2 + 16;          // bytes per LDS row: 16 rows start in 16 different bank quads
 constexpr int kWideWaves = 8;
 
 template <bool BF16, int BS, typename ST>
-__global__ __launch_bounds__(512) void decode_wide_kernel(PackedParams p)
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu((BS == 128 && sizeof(ST) == 2) ? 7 : 1))) void decode_wide_kernel(PackedParams p)
 {
     constexpr int U = kGroupTiles;
     constexpr int NBT = 128 / BS;
@@ -357,7 +359,7 @@ __global__ __launch_bounds__(512) void decode_wide_kernel(PackedParams p)
 
     const uint32_t w_off = static_cast<uint32_t>(lane * 16);
     const uint32_t r_off = static_cast<uint32_t>(kChunkWeights + c * R);
-    // window fill: thread -> row t / 32, pieces t % 32 + 32 i (i < 4) of the row's 128 pieces
+    // window fill: thread -> row t / 32, pieces t % 32 and t % 32 + 32 of the row's 64 pieces
     const int wrow = t >> 5, wpiece = t & 31;
     const uint32_t win_goff = static_cast<uint32_t>(wrow) * static_cast<uint32_t>(p.k) * 2u + static_cast<uint32_t>(wpiece * 16);
     const uint32_t win_loff = static_cast<uint32_t>(wrow * kWinPitch + wpiece * 16);
@@ -380,10 +382,10 @@ __global__ __launch_bounds__(512) void decode_wide_kernel(PackedParams p)
 #pragma unroll
         for (int i = 0; i < NR; ++i) grp.r[i] = load16(srd_p, r_off + static_cast<uint32_t>(i * 16), soff);
     };
-    uint4 wa[4];
+    uint4 wa[2];
     auto load_window = [&](int win) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < 2; ++i) {
             const int64_t k0 = static_cast<int64_t>(win) * kWinK + (wpiece + 32 * i) * 8;
             uint32_t off = win_goff + static_cast<uint32_t>(i * 512);
             if (wrow >= p.m || k0 >= p.k) off = kOutOfRange;      // K is a multiple of 8: a piece is all inside or all outside
@@ -392,9 +394,9 @@ __global__ __launch_bounds__(512) void decode_wide_kernel(PackedParams p)
     };
     auto store_window = [&](int buf) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) *reinterpret_cast<uint4*>(smem + buf * kBufBytes + win_loff + i * 512) = wa[i];
+        for (int i = 0; i < 2; ++i) *reinterpret_cast<uint4*>(smem + buf * kBufBytes + win_loff + i * 512) = wa[i];
     };
-    auto compute_group = [&](const Grp& grp, int buf, int half) {
+    auto compute_group = [&](const Grp& grp, int buf) {
         uint32_t rr[NR * 4];
 #pragma unroll
         for (int i = 0; i < NR; ++i) {
@@ -405,7 +407,7 @@ __global__ __launch_bounds__(512) void decode_wide_kernel(PackedParams p)
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const unsigned char* fa = smem + buf * kBufBytes + frag_off + (half * U + u) * 256;
+            const unsigned char* fa = smem + buf * kBufBytes + frag_off + u * 256;
             uint4 av[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) av[j] = *reinterpret_cast<const uint4*>(fa + j * 64);
@@ -443,21 +445,16 @@ __global__ __launch_bounds__(512) void decode_wide_kernel(PackedParams p)
         }
     };
 
-    const int windows = (p.groups + 1) / 2;
-    Grp ga, gb;
-    fetch_group(ga, 0);
+    Grp ga;
     load_window(0);
     store_window(0);
     __syncthreads();
-    for (int win = 0; win < windows; ++win) {
-        const int gi = win * 2;
-        const int buf = win & 1;
-        if (win + 1 < windows) load_window(win + 1);
-        fetch_group(gb, gi + 1);
-        compute_group(ga, buf, 0);
-        fetch_group(ga, gi + 2);
-        if (gi + 1 < p.groups) compute_group(gb, buf, 1);
-        if (win + 1 < windows) store_window(buf ^ 1);
+    for (int gi = 0; gi < p.groups; ++gi) {
+        const int buf = gi & 1;
+        if (gi + 1 < p.groups) load_window(gi + 1);
+        fetch_group(ga, gi);
+        compute_group(ga, buf);
+        if (gi + 1 < p.groups) store_window(buf ^ 1);
         __syncthreads();
     }
 
@@ -579,7 +576,7 @@ extern "C" int rocm_launch_decode_packed(const RocmMatMulNBitsArgs* a, const voi
     // groups: enough waves per group to reach about 8k in flight, each prefetching its next group.
     const int64_t wgs = (a->n + 15) / 16;
     int w = waves;
-    bool single_set = a->m <= 1 && wgs * 4 >= 6144;
+    bool single_set = wgs * 4 >= 6144;
     if (w <= 0) {
         if (single_set) {
             w = (p.groups + 1) / 2;
@@ -589,7 +586,7 @@ extern "C" int rocm_launch_decode_packed(const RocmMatMulNBitsArgs* a, const voi
         }
         if (w < 1) w = 1;
     } else {
-        single_set = a->m <= 1 && wgs * w >= 6144;
+        single_set = wgs * w >= 6144;
     }
     if (w > 8) w = 8;
     if (w > p.groups) w = p.groups;
