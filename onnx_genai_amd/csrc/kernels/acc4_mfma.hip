@@ -65,7 +65,9 @@ struct Acc4Group {
 // one load of codes (MR = 1) or two per tile (MR = 16), NS scale loads (lane group g fetches block 4i + g),
 // NZ zero-point loads (lane group g fetches the byte of blocks 8i + 2g and 8i + 2g + 1) and one load of
 // the activation-side pairs; scale and zero point reach the other lane groups by shuffle when a block ends.
-template <int BS, int MR, typename ST>
+// SETS: 2 = the next group's loads are in flight while this one is multiplied (few waves per launch); 1 = no prefetch,
+// fewer registers, more waves per SIMD (launches with thousands of waves, where occupancy hides latency better).
+template <int BS, int MR, typename ST, int SETS>
 __global__ __launch_bounds__(512) void acc4_decode_kernel(Acc4DecodeParams p)
 {
     constexpr bool kTranspose = BS < 128;
@@ -216,11 +218,27 @@ __global__ __launch_bounds__(512) void acc4_decode_kernel(Acc4DecodeParams p)
             if (t0 + u < t_end) compute_tile(cur, u, t0, parity);
     };
 
-    Grp ga, gb;
-    fetch_group(ga, t_begin);
-    for (int t0 = t_begin; t0 < t_end; t0 += 2 * U) {
-        run_group(ga, gb, t0, 0);
-        if (t0 + U < t_end) run_group(gb, ga, t0 + U, 1);
+    if constexpr (SETS == 2) {
+        Grp ga, gb;
+        fetch_group(ga, t_begin);
+        for (int t0 = t_begin; t0 < t_end; t0 += 2 * U) {
+            run_group(ga, gb, t0, 0);
+            if (t0 + U < t_end) run_group(gb, ga, t0 + U, 1);
+        }
+    } else {
+        Grp ga;
+        for (int t0 = t_begin; t0 < t_end; t0 += U) {
+            fetch_group(ga, t0);
+            if constexpr (MR == 1) {
+                *reinterpret_cast<uint4*>(stage + st_write) = ga.a[0];
+            } else {
+                *reinterpret_cast<uint4*>(aux_stage + lane * 16) = ga.x;
+            }
+            lds_order();
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (t0 + u < t_end) compute_tile(ga, u, t0, 0);
+        }
     }
 
     // ---- split-K reduction across the waves of this workgroup, in wave order ----
@@ -243,30 +261,30 @@ __global__ __launch_bounds__(512) void acc4_decode_kernel(Acc4DecodeParams p)
     }
 }
 
-template <int BS, int MR, typename ST>
+template <int BS, int MR, typename ST, int SETS>
 static int launch_acc4_decode(const Acc4DecodeParams& p, int waves, hipStream_t stream)
 {
     const unsigned grid = static_cast<unsigned>((p.n + 15) / 16);
     const size_t stage = static_cast<size_t>(waves) * (MR == 1 ? 2048 : 2 * 16 * kCodePitch + 2048);
     const size_t red = static_cast<size_t>(waves) * 1024;
-    hipLaunchKernelGGL((acc4_decode_kernel<BS, MR, ST>), dim3(grid), dim3(waves * 64), stage > red ? stage : red, stream, p);
+    hipLaunchKernelGGL((acc4_decode_kernel<BS, MR, ST, SETS>), dim3(grid), dim3(waves * 64), stage > red ? stage : red, stream, p);
     return static_cast<int>(hipGetLastError());
 }
 
-template <typename ST>
-static int launch_acc4_decode_bs(const Acc4DecodeParams& p, int bs, int waves, hipStream_t stream)
+template <int BS, typename ST>
+static int launch_acc4_decode_mr(const Acc4DecodeParams& p, int waves, bool single_set, hipStream_t stream)
 {
-    if (p.m <= 1) {
-        switch (bs) {
-            case 32: return launch_acc4_decode<32, 1, ST>(p, waves, stream);
-            case 64: return launch_acc4_decode<64, 1, ST>(p, waves, stream);
-            default: return launch_acc4_decode<128, 1, ST>(p, waves, stream);
-        }
-    }
+    if (p.m <= 1) return single_set ? launch_acc4_decode<BS, 1, ST, 1>(p, waves, stream) : launch_acc4_decode<BS, 1, ST, 2>(p, waves, stream);
+    return launch_acc4_decode<BS, 16, ST, 2>(p, waves, stream);
+}
+
+template <typename ST>
+static int launch_acc4_decode_bs(const Acc4DecodeParams& p, int bs, int waves, bool single_set, hipStream_t stream)
+{
     switch (bs) {
-        case 32: return launch_acc4_decode<32, 16, ST>(p, waves, stream);
-        case 64: return launch_acc4_decode<64, 16, ST>(p, waves, stream);
-        default: return launch_acc4_decode<128, 16, ST>(p, waves, stream);
+        case 32: return launch_acc4_decode_mr<32, ST>(p, waves, single_set, stream);
+        case 64: return launch_acc4_decode_mr<64, ST>(p, waves, single_set, stream);
+        default: return launch_acc4_decode_mr<128, ST>(p, waves, single_set, stream);
     }
 }
 
@@ -591,13 +609,14 @@ extern "C" int rocm_launch_acc4_mfma(const RocmMatMulNBitsArgs* a, const RocmAcc
     p.scales_bf16 = a->scale_dtype == ROCM_DT_BF16;
 
     const int group_tiles = a->m <= 1 ? 4 : 2;
+    const int64_t wgs = (a->n + 15) / 16;
     int w = waves;
     if (w <= 0) {
-        const int64_t wgs = (a->n + 15) / 16;
         const int want = static_cast<int>((8192 + wgs - 1) / wgs);
         int by_work = p.tiles / group_tiles;
         if (by_work < 1) by_work = 1;
         w = want < by_work ? want : by_work;
+        if (wgs * 4 >= 6144 && a->m <= 1) w = by_work;     // many column groups: short waves, no prefetch (see SETS)
         if (w < 1) w = 1;
     }
     if (w > 8) w = 8;
@@ -606,6 +625,7 @@ extern "C" int rocm_launch_acc4_mfma(const RocmMatMulNBitsArgs* a, const RocmAcc
     w = (p.tiles + tpw - 1) / tpw;
     p.tiles_per_wave = tpw;
 
-    if (a->scale_dtype == ROCM_DT_F32) return mnb::launch_acc4_decode_bs<float>(p, a->block_size, w, s);
-    return mnb::launch_acc4_decode_bs<uint16_t>(p, a->block_size, w, s);
+    const bool single_set = a->m <= 1 && wgs * w >= 6144;
+    if (a->scale_dtype == ROCM_DT_F32) return mnb::launch_acc4_decode_bs<float>(p, a->block_size, w, single_set, s);
+    return mnb::launch_acc4_decode_bs<uint16_t>(p, a->block_size, w, single_set, s);
 }
