@@ -162,7 +162,7 @@ bool use_packed(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& args, int& r
 {
     rc = 0;
     if (!kn.ep->prepack || !kn.constant_inputs[1] || !kn.constant_inputs[2] || (args.zp && !kn.constant_inputs[3])) return false;
-    if (!rocm_decode_packed_eligible(&args)) return false;
+    if (!(kn.accuracy_level == 4 ? rocm_acc4_packed_eligible(&args) : rocm_decode_packed_eligible(&args))) return false;
     const bool current = kn.packed && kn.packed_from[0] == args.b && kn.packed_from[1] == args.scales && kn.packed_from[2] == args.zp &&
                          kn.packed_scale_dtype == args.scale_dtype;
     if (current) return true;
@@ -311,9 +311,16 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
         w4.qa = reinterpret_cast<int8_t*>(ws);
         w4.aq = reinterpret_cast<float*>(ws + lay.codes);
         w4.aux = reinterpret_cast<float*>(ws + lay.codes + lay.pairs);
+        int pack_rc = 0;
+        const bool packed = M == 1 && use_packed(kn, args, pack_rc);
+        w4.code_order = packed ? 2 : 1;
         rc = rocm_launch_quantize_a_workspace(args.a, args.a_dtype, args.m, args.k, args.block_size, kn.ep->acc4_rounding, &w4, stream);
+        if (rc == 0 && pack_rc != 0) rc = pack_rc;
         if (rc == 0) {
-            if (rocm_acc4_mfma_eligible(&args)) {
+            if (packed) {
+                rc = rocm_launch_acc4_packed(&args, kn.packed, &w4, kn.ep->decode_waves, stream);
+                kn.variant = "acc4_mfma_i8_packed";
+            } else if (rocm_acc4_mfma_eligible(&args)) {
                 rc = rocm_launch_acc4_mfma(&args, &w4, kn.ep->decode_waves, stream);
                 kn.variant = "acc4_mfma_i8";
             } else {

@@ -89,12 +89,15 @@ int rocm_launch_quantize_a(const void* a, int a_dtype, int64_t m, int64_t k, int
 int rocm_launch_block_acc_i32(const int8_t* qa, const uint8_t* b, const uint8_t* zp,
                               int64_t m, int64_t n, int64_t k, int block_size, int32_t* acc, rocm_stream_t stream);
 /* Workspace of one accuracy_level 4 call (device memory, each part 256-byte aligned):
- * qa: int8 [M, kb*bs], inside every run of 8 the elements 0,2,4,6 then 1,3,5,7; aq: f32 [M, kb, 2] = (scale, sum of codes);
+ * qa: int8 [M, kb*bs], inside every run of 8 in the order `code_order` names (1: elements 0,2,4,6,1,3,5,7 - what the
+ * kernels over the caller's weight layout want; 2: 0,4,1,5,2,6,3,7 - what the repacked stream wants);
+ * aq: f32 [M, kb, 2] = (scale, sum of codes);
  * aux: for M <= 16, f32 [kb, 16, 2], the same pairs block-major; for M > 16, f32 [kb, M], the scales block-major. */
 typedef struct RocmAcc4Workspace {
   int8_t* qa;
   float* aq;
   float* aux;
+  int code_order;
 } RocmAcc4Workspace;
 int rocm_launch_quantize_a_workspace(const void* a, int a_dtype, int64_t m, int64_t k, int block_size, int rounding,
                                      const RocmAcc4Workspace* ws, rocm_stream_t stream);
@@ -104,6 +107,9 @@ int rocm_launch_acc4_gemv(const RocmMatMulNBitsArgs* args, const RocmAcc4Workspa
  * M > 16 with any block size >= 32 (tiled). */
 int rocm_acc4_mfma_eligible(const RocmMatMulNBitsArgs* args);
 int rocm_launch_acc4_mfma(const RocmMatMulNBitsArgs* args, const RocmAcc4Workspace* ws, int waves, rocm_stream_t stream);
+/* One row over the repacked copy of constant weights (the copy rocm_launch_pack_decode makes); code_order 2. */
+int rocm_acc4_packed_eligible(const RocmMatMulNBitsArgs* args);
+int rocm_launch_acc4_packed(const RocmMatMulNBitsArgs* args, const void* packed, const RocmAcc4Workspace* ws, int waves, rocm_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -37,8 +37,9 @@ __global__ __launch_bounds__(256) void quantize_a_kernel(
             r = fminf(fmaxf(r, -127.0f), 127.0f);
             code = static_cast<int>(r);
         }
-        // interleaved: inside every run of 8, elements 0,2,4,6 then 1,3,5,7
-        const int pos = interleave ? ((i & ~7) | ((i & 1) << 2) | ((i & 7) >> 1)) : i;
+        // inside every run of 8: as is (0), elements 0,2,4,6,1,3,5,7 (1), or 0,4,1,5,2,6,3,7 (2)
+        const int e = i & 7;
+        const int pos = (i & ~7) | (interleave == 1 ? (((e & 1) << 2) | (e >> 1)) : interleave == 2 ? (((e & 3) << 1) | (e >> 2)) : e);
         qa[(row * kb + blk) * bs + pos] = static_cast<int8_t>(code);
         sum += code;
     }
@@ -159,7 +160,7 @@ extern "C" int rocm_launch_quantize_a(const void* a, int a_dtype, int64_t m, int
 extern "C" int rocm_launch_quantize_a_workspace(const void* a, int a_dtype, int64_t m, int64_t k, int block_size, int rounding,
                                                 const RocmAcc4Workspace* ws, rocm_stream_t stream)
 {
-    return launch_quantize(a, a_dtype, m, k, block_size, rounding, 1, ws->qa, nullptr, nullptr, ws->aq, m <= 16 ? ws->aux : nullptr, m > 16 ? ws->aux : nullptr, stream);
+    return launch_quantize(a, a_dtype, m, k, block_size, rounding, ws->code_order, ws->qa, nullptr, nullptr, ws->aq, m <= 16 ? ws->aux : nullptr, m > 16 ? ws->aux : nullptr, stream);
 }
 
 extern "C" int rocm_launch_block_acc_i32(const int8_t* qa, const uint8_t* b, const uint8_t* zp, int64_t m, int64_t n, int64_t k,

@@ -492,6 +492,178 @@ static int launch_wide_bs(const PackedParams& p, int bs, hipStream_t stream)
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// accuracy_level = 4, one row, over the same repacked stream: v_mfma_i32_16x16x32_i8.
+// ---------------------------------------------------------------------------------------------
+//
+// `w & 0x0f0f0f0f` and `(w >> 4) & 0x0f0f0f0f` turn a repacked dword into the eight weights as unsigned bytes in the
+// order e0,e4,e1,e5 | e2,e6,e3,e7; the activation codes are stored in that same order inside every run of 8, so an
+// operand costs three instructions and no byte shuffles. Arithmetic as in the unpacked int8 kernel: exact integer
+// block sums, zero point through the code sums, one f32 scale-and-add per block.
+
+typedef __attribute__((ext_vector_type(4))) int int4p_t;
+
+struct Acc4PackedParams {
+    const int8_t* qa;       // [padded_k] codes of the one row, packed order
+    const float* aq;        // [kb, 2]: scale_a, f32(sum of codes)
+    const uint8_t* packed;
+    const void* bias;
+    void* y;
+    int64_t n, kb;
+    int64_t padded_k;
+    int64_t cg_stride;
+    int groups, groups_per_wave, chunk_bytes;
+    int bias_dtype, y_dtype;
+    int scales_bf16;
+};
+
+template <int NR>
+struct Acc4PackedGroup {
+    uint4 w[kGroupTiles];
+    uint4 r[NR];
+    uint4 a;      // 16 codes of the group (lanes 0..31)
+    uint2 x;      // (scale_a, code sum) of block `lane` of the group
+};
+
+template <int BS, typename ST, int SETS>
+__global__ __launch_bounds__(512) void acc4_packed_kernel(Acc4PackedParams p)
+{
+    constexpr int U = kGroupTiles;
+    constexpr int NBT = 128 / BS;
+    constexpr int NB = U * NBT;
+    constexpr int R = packed_record_bytes(BS, static_cast<int>(sizeof(ST)));
+    constexpr int NR = R / 16;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int waves = blockDim.x >> 6;
+    const int c = lane & 15;
+    const int g = lane >> 4;
+    const int64_t n_base = static_cast<int64_t>(blockIdx.x) * 16;
+    const bool bf16_scales = p.scales_bf16 != 0;
+
+    const __amdgpu_buffer_rsrc_t srd_p = make_srd(p.packed + static_cast<int64_t>(blockIdx.x) * p.cg_stride, static_cast<uint64_t>(p.cg_stride));
+    const __amdgpu_buffer_rsrc_t srd_a = make_srd(p.qa, static_cast<uint64_t>(p.padded_k));
+    const __amdgpu_buffer_rsrc_t srd_x = make_srd(p.aq, static_cast<uint64_t>(p.kb) * 8);
+
+    const uint32_t w_off = static_cast<uint32_t>(lane * 16);
+    const uint32_t r_off = static_cast<uint32_t>(kChunkWeights + c * R);
+    unsigned char* stage = smem + wave * (SETS * 512);
+    // operand of MFMA j of tile u: the 8 codes of elements u*128 + j*32 + g*8 .. +8 (only row 0 matters: every lane
+    // of a lane group reads the same 8 bytes)
+    const uint32_t st_read = static_cast<uint32_t>(g * 8);
+
+    float y = 0.f;
+    int4p_t acc = {0, 0, 0, 0};
+
+    const int g_begin = wave * p.groups_per_wave;
+    const int g_end = min(g_begin + p.groups_per_wave, p.groups);
+
+    using Grp = Acc4PackedGroup<NR>;
+    auto fetch_group = [&](Grp& grp, int gi) {
+        if (gi >= g_end) return;
+        const uint32_t soff = static_cast<uint32_t>(gi) * static_cast<uint32_t>(p.chunk_bytes);
+#pragma unroll
+        for (int u = 0; u < U; ++u) grp.w[u] = load16(srd_p, w_off + static_cast<uint32_t>(u * 1024), soff);
+#pragma unroll
+        for (int i = 0; i < NR; ++i) grp.r[i] = load16(srd_p, r_off + static_cast<uint32_t>(i * 16), soff);
+        grp.a = load16(srd_a, lane < 32 ? static_cast<uint32_t>(lane * 16) : kOutOfRange, static_cast<uint32_t>(gi) * 512u);   // the range ends the row at padded_k
+        const auto v = __builtin_amdgcn_raw_buffer_load_b64(srd_x, static_cast<int>(lane < NB ? lane * 8 : kOutOfRange), static_cast<int>(gi * NB * 8), 0);
+        grp.x = make_uint2(v[0], v[1]);
+    };
+    auto compute_group = [&](const Grp& grp, int gi, int slot) {
+        unsigned char* st = stage + slot * 512;
+        if (lane < 32) *reinterpret_cast<uint4*>(st + lane * 16) = grp.a;
+        lds_order();
+        uint32_t rr[NR * 4];
+#pragma unroll
+        for (int i = 0; i < NR; ++i) {
+            rr[4 * i] = grp.r[i].x;
+            rr[4 * i + 1] = grp.r[i].y;
+            rr[4 * i + 2] = grp.r[i].z;
+            rr[4 * i + 3] = grp.r[i].w;
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            long av[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) av[j] = *reinterpret_cast<const long*>(st + st_read + u * 128 + j * 32);
+            const uint32_t wd[4] = {grp.w[u].x, grp.w[u].y, grp.w[u].z, grp.w[u].w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const bool first = (j * 32) % BS == 0;
+                const bool last = ((j + 1) * 32) % BS == 0 || j == 3;
+                const uint64_t bw = static_cast<uint64_t>(wd[j] & 0x0f0f0f0fu) | (static_cast<uint64_t>((wd[j] >> 4) & 0x0f0f0f0fu) << 32);
+                const int4p_t zero = {0, 0, 0, 0};
+                acc = __builtin_amdgcn_mfma_i32_16x16x32_i8(av[j], static_cast<long>(bw), first ? zero : acc, 0, 0, 0);
+                if (last) {
+                    const int bi = u * NBT + (j * 32) / BS;
+                    if (static_cast<int64_t>(gi) * NB + bi < p.kb) {          // a block beyond K (wave-uniform)
+                        const int zbyte = NB * static_cast<int>(sizeof(ST)) + bi;
+                        const float zf = static_cast<float>((rr[zbyte / 4] >> ((zbyte % 4) * 8)) & 0xffu);
+                        float sb;
+                        if constexpr (sizeof(ST) == 4) {
+                            sb = __uint_as_float(rr[bi]);
+                        } else {
+                            const uint32_t raw = (rr[bi / 2] >> ((bi % 2) * 16)) & 0xffffu;
+                            sb = bf16_scales ? __uint_as_float(raw << 16) : f16_bits_to_f32(static_cast<uint16_t>(raw));
+                        }
+                        const float sa = __int_as_float(__builtin_amdgcn_readlane(static_cast<int>(grp.x.x), bi));
+                        const float qs = __int_as_float(__builtin_amdgcn_readlane(static_cast<int>(grp.x.y), bi));
+                        const float f = fmaf(-zf, qs, static_cast<float>(acc[0]));   // both terms are integers below 2^24: exact
+                        y = fmaf(f, __fmul_rn(sa, sb), y);
+                    }
+                }
+            }
+        }
+    };
+
+    if constexpr (SETS == 2) {
+        Grp ga, gb;
+        fetch_group(ga, g_begin);
+        for (int gi = g_begin; gi < g_end; gi += 2) {
+            fetch_group(gb, gi + 1);
+            compute_group(ga, gi, 0);
+            if (gi + 1 < g_end) {
+                fetch_group(ga, gi + 2);
+                compute_group(gb, gi + 1, 1);
+            }
+        }
+    } else {
+        Grp ga;
+        for (int gi = g_begin; gi < g_end; ++gi) {
+            fetch_group(ga, gi);
+            compute_group(ga, gi, 0);
+        }
+    }
+
+    // ---- split-K reduction across the waves of this workgroup, in wave order; row 0 lives in lanes 0..15 ----
+    __syncthreads();
+    float* red = reinterpret_cast<float*>(smem);       // [waves][16]
+    if (lane < 16) red[wave * 16 + lane] = y;
+    __syncthreads();
+    if (threadIdx.x < 16) {
+        const int64_t col = n_base + threadIdx.x;
+        if (col < p.n) {
+            float total = 0.f;
+            for (int w = 0; w < waves; ++w) total += red[w * 16 + threadIdx.x];
+            if (p.bias) total += load_as_f32(p.bias, p.bias_dtype, col);
+            store_from_f32(p.y, p.y_dtype, col, total);
+        }
+    }
+}
+
+template <int BS, typename ST>
+static int launch_acc4_packed(const Acc4PackedParams& p, int waves, bool single_set, hipStream_t stream)
+{
+    const unsigned grid = static_cast<unsigned>((p.n + 15) / 16);
+    const size_t lds = static_cast<size_t>(waves) * 1024;
+    if (single_set) hipLaunchKernelGGL((acc4_packed_kernel<BS, ST, 1>), dim3(grid), dim3(waves * 64), lds, stream, p);
+    else hipLaunchKernelGGL((acc4_packed_kernel<BS, ST, 2>), dim3(grid), dim3(waves * 64), lds, stream, p);
+    return static_cast<int>(hipGetLastError());
+}
+
 static int packed_groups(const RocmMatMulNBitsArgs* a)
 {
     const int64_t kb = (a->k + a->block_size - 1) / a->block_size;
@@ -596,4 +768,60 @@ extern "C" int rocm_launch_decode_packed(const RocmMatMulNBitsArgs* a, const voi
 
     if (bf16) return f32_scales ? mnb::launch_packed_bs<true, float>(p, a->block_size, w, single_set, s) : mnb::launch_packed_bs<true, uint16_t>(p, a->block_size, w, single_set, s);
     return f32_scales ? mnb::launch_packed_bs<false, float>(p, a->block_size, w, single_set, s) : mnb::launch_packed_bs<false, uint16_t>(p, a->block_size, w, single_set, s);
+}
+
+extern "C" int rocm_acc4_packed_eligible(const RocmMatMulNBitsArgs* a)
+{
+    const bool bs_ok = a->block_size == 32 || a->block_size == 64 || a->block_size == 128;
+    if (!(bs_ok && a->m == 1 && a->n >= 1)) return 0;
+    if ((reinterpret_cast<uintptr_t>(a->b) & 15) != 0 || (reinterpret_cast<uintptr_t>(a->scales) & 3) != 0) return 0;
+    return static_cast<int64_t>(mnb::packed_groups(a)) * mnb::packed_chunk_bytes(a) < 0x7fffffff;
+}
+
+extern "C" int rocm_launch_acc4_packed(const RocmMatMulNBitsArgs* a, const void* packed, const RocmAcc4Workspace* ws, int waves, rocm_stream_t stream)
+{
+    if (!rocm_acc4_packed_eligible(a)) return -1;
+    mnb::Acc4PackedParams p;
+    p.qa = ws->qa;
+    p.aq = ws->aq;
+    p.packed = static_cast<const uint8_t*>(packed);
+    p.bias = a->bias;
+    p.y = a->y;
+    p.n = a->n;
+    p.kb = (a->k + a->block_size - 1) / a->block_size;
+    p.padded_k = p.kb * a->block_size;
+    p.groups = mnb::packed_groups(a);
+    p.chunk_bytes = mnb::packed_chunk_bytes(a);
+    p.cg_stride = static_cast<int64_t>(p.groups) * p.chunk_bytes;
+    p.bias_dtype = a->bias_dtype;
+    p.y_dtype = a->y_dtype;
+    p.scales_bf16 = a->scale_dtype == ROCM_DT_BF16;
+
+    const int64_t wgs = (a->n + 15) / 16;
+    int w = waves;
+    bool single_set = wgs * 4 >= 6144;
+    if (w <= 0) {
+        if (single_set) {
+            w = (p.groups + 1) / 2;
+        } else {
+            const int want = static_cast<int>((8192 + wgs - 1) / wgs);
+            w = want < p.groups ? want : p.groups;
+        }
+        if (w < 1) w = 1;
+    } else {
+        single_set = wgs * w >= 6144;
+    }
+    if (w > 8) w = 8;
+    if (w > p.groups) w = p.groups;
+    const int gpw = (p.groups + w - 1) / w;
+    w = (p.groups + gpw - 1) / gpw;
+    p.groups_per_wave = gpw;
+
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const bool f32_scales = a->scale_dtype == ROCM_DT_F32;
+    switch (a->block_size) {
+        case 32: return f32_scales ? mnb::launch_acc4_packed<32, float>(p, w, single_set, s) : mnb::launch_acc4_packed<32, uint16_t>(p, w, single_set, s);
+        case 64: return f32_scales ? mnb::launch_acc4_packed<64, float>(p, w, single_set, s) : mnb::launch_acc4_packed<64, uint16_t>(p, w, single_set, s);
+        default: return f32_scales ? mnb::launch_acc4_packed<128, float>(p, w, single_set, s) : mnb::launch_acc4_packed<128, uint16_t>(p, w, single_set, s);
+    }
 }

@@ -416,16 +416,21 @@ ACC4_CASES = [
 
 
 @pytest.mark.parametrize("a_dt,bs,zero_points,m,n,k", ACC4_CASES)
-@pytest.mark.parametrize("rounding", ["mlas", "native"])
-def test_acc4_outputs(port, ref, a_dt, bs, zero_points, m, n, k, rounding):
-    provider = E.RocmExecutionProvider(0, {"acc4_rounding": rounding})
+@pytest.mark.parametrize("rounding,prepack", [("mlas", True), ("native", True), ("mlas", False)])
+def test_acc4_outputs(port, ref, a_dt, bs, zero_points, m, n, k, rounding, prepack):
+    if not prepack and m != 1:
+        pytest.skip("only one-row calls have a repacked path to turn off")
+    provider = E.RocmExecutionProvider(0, {"acc4_rounding": rounding, "prepack": "1" if prepack else "0"})
     try:
         b, s, zp = synth.make_weights(n, k, bs, 80 + n, zero_points=zero_points, scale_lo=0.002, scale_hi=0.01, scale_dtype=a_dt)
         a = synth.make_activation(m, k, 80, a_dt)
         bias = synth.to_dtype(np.linspace(-1, 1, n).astype(np.float32), a_dt)
         y32, variant = run_op(provider, a, a_dt, b, s, a_dt, zp, n, k, bs, accuracy_level=4, bias=bias, bias_dtype=a_dt, y_dtype=E.F32)
         on_matrix_cores = bs in (32, 64, 128) if m <= 16 else bs >= 32
-        assert variant == ("acc4_mfma_i8" if on_matrix_cores else "acc4_gemv_dot4")
+        expected = "acc4_mfma_i8" if on_matrix_cores else "acc4_gemv_dot4"
+        if prepack and m == 1 and on_matrix_cores:
+            expected = "acc4_mfma_i8_packed"                            # constant weights: the repacked stream
+        assert variant == expected
         rnd = oracle.ROUND_HALF_EVEN if rounding == "mlas" else oracle.ROUND_HALF_AWAY
         af, sf, bf = synth.to_f32(a, a_dt), synth.to_f32(s, a_dt), synth.to_f32(bias, a_dt)
         want = port.matmul_acc4_f32(af, b, sf, zp, n, k, bs, rnd, bias=bf)
@@ -442,15 +447,16 @@ def test_acc4_outputs(port, ref, a_dt, bs, zero_points, m, n, k, rounding):
 
 @pytest.mark.parametrize("waves", [1, 3, 8])
 @pytest.mark.parametrize("s_dt", [E.F32, E.F16])
-def test_acc4_decode_wave_counts_agree(port, waves, s_dt):
+@pytest.mark.parametrize("prepack", [True, False])
+def test_acc4_decode_wave_counts_agree(port, waves, s_dt, prepack):
     a_dt, bs, n, k = E.F16, 64, 100, 64 * 50
-    provider = E.RocmExecutionProvider(0, {"decode_waves": str(waves)})
+    provider = E.RocmExecutionProvider(0, {"decode_waves": str(waves), "prepack": "1" if prepack else "0"})
     try:
         b, s, zp = synth.make_weights(n, k, bs, 95, zero_points=True, scale_lo=0.002, scale_hi=0.01, scale_dtype=s_dt)
         for m in (1, 6):
             a = synth.make_activation(m, k, 95 + m, a_dt)
             y32, variant = run_op(provider, a, a_dt, b, s, s_dt, zp, n, k, bs, accuracy_level=4, y_dtype=E.F32)
-            assert variant == "acc4_mfma_i8"
+            assert variant == ("acc4_mfma_i8_packed" if prepack and m == 1 else "acc4_mfma_i8")
             want = port.matmul_acc4_f32(synth.to_f32(a, a_dt), b, synth.to_f32(s, s_dt), zp, n, k, bs, oracle.ROUND_HALF_EVEN)
             assert helpers.rel_l2(y32, want) <= TOL_F32
     finally:
@@ -472,7 +478,7 @@ def test_acc4_power_of_two_scaling_at_full_70b_shape(ep):
             ys.append(ep.download(yb, (m, n), np.float32))
             ep.deallocate(ab)
             ep.deallocate(yb)
-        assert ops.kernel.last_variant() == "acc4_mfma_i8"
+        assert ops.kernel.last_variant() == ("acc4_mfma_i8_packed" if m == 1 else "acc4_mfma_i8")
         assert np.isfinite(ys[0]).all() and np.abs(ys[0]).max() > 0
         assert np.array_equal(ys[1], 2.0 * ys[0])
     ops.free()
