@@ -22,17 +22,26 @@ __global__ __launch_bounds__(256) void quantize_a_kernel(
     const int64_t row = item / kb, blk = item - row * kb;
     const int64_t k0 = blk * bs;
     const int64_t valid = (k - k0 < bs) ? (k - k0) : bs;
+    // Block sizes up to 256 keep a lane's (at most four) elements in registers between the two passes.
+    constexpr int kHeld = 4;
+    float held[kHeld];
     float vmax = 0.0f;
-    for (int i = lane; i < valid; i += 64) vmax = fmaxf(vmax, fabsf(load_as_f32(a, a_dtype, row * k + k0 + i)));
+#pragma unroll
+    for (int j = 0; j < kHeld; ++j) {
+        const int i = lane + 64 * j;
+        held[j] = i < valid ? load_as_f32(a, a_dtype, row * k + k0 + i) : 0.0f;
+        vmax = fmaxf(vmax, fabsf(held[j]));
+    }
+    for (int i = lane + 64 * kHeld; i < valid; i += 64) vmax = fmaxf(vmax, fabsf(load_as_f32(a, a_dtype, row * k + k0 + i)));
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) vmax = fmaxf(vmax, __shfl_xor(vmax, off, 64));
     const float scale = __fdiv_rn(vmax, 127.0f);
     const float inv = vmax != 0.0f ? __fdiv_rn(127.0f, vmax) : 0.0f;
     int sum = 0;
-    for (int i = lane; i < bs; i += 64) {
+    auto emit = [&](int i, float value) {
         int code = 0;
         if (i < valid) {
-            const float scaled = __fmul_rn(load_as_f32(a, a_dtype, row * k + k0 + i), inv);
+            const float scaled = __fmul_rn(value, inv);
             float r = rounding == 1 ? roundf(scaled) : rintf(scaled);
             r = fminf(fmaxf(r, -127.0f), 127.0f);
             code = static_cast<int>(r);
@@ -42,7 +51,13 @@ __global__ __launch_bounds__(256) void quantize_a_kernel(
         const int pos = (i & ~7) | (interleave == 1 ? (((e & 1) << 2) | (e >> 1)) : interleave == 2 ? (((e & 3) << 1) | (e >> 2)) : e);
         qa[(row * kb + blk) * bs + pos] = static_cast<int8_t>(code);
         sum += code;
+    };
+#pragma unroll
+    for (int j = 0; j < kHeld; ++j) {
+        const int i = lane + 64 * j;
+        if (i < bs) emit(i, held[j]);
     }
+    for (int i = lane + 64 * kHeld; i < bs; i += 64) emit(i, i < valid ? load_as_f32(a, a_dtype, row * k + k0 + i) : 0.0f);
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
     if (lane == 0) {

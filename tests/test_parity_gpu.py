@@ -415,11 +415,13 @@ ACC4_CASES = [
 ]
 
 
-@pytest.mark.parametrize("a_dt,bs,zero_points,m,n,k", ACC4_CASES)
-@pytest.mark.parametrize("rounding,prepack", [("mlas", True), ("native", True), ("mlas", False)])
+# every case under both rounding rules; one-row cases once more with the repacked path turned off
+ACC4_RUNS = [case + (rounding, True) for case in ACC4_CASES for rounding in ("mlas", "native")] + \
+            [case + ("mlas", False) for case in ACC4_CASES if case[3] == 1]
+
+
+@pytest.mark.parametrize("a_dt,bs,zero_points,m,n,k,rounding,prepack", ACC4_RUNS)
 def test_acc4_outputs(port, ref, a_dt, bs, zero_points, m, n, k, rounding, prepack):
-    if not prepack and m != 1:
-        pytest.skip("only one-row calls have a repacked path to turn off")
     provider = E.RocmExecutionProvider(0, {"acc4_rounding": rounding, "prepack": "1" if prepack else "0"})
     try:
         b, s, zp = synth.make_weights(n, k, bs, 80 + n, zero_points=zero_points, scale_lo=0.002, scale_hi=0.01, scale_dtype=a_dt)
