@@ -335,7 +335,7 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
         rc = rocm_launch_decode_mfma(&args, kn.ep->decode_waves, kn.ep->decode_col_groups, stream);
         kn.variant = "decode_mfma_splitk";
     } else if (M > 16 && rocm_prefill_mfma_eligible(&args)) {
-        rc = rocm_launch_prefill_mfma(&args, stream);
+        rc = rocm_launch_prefill_mfma(&args, kn.ep->prefill_tile, stream);
         kn.variant = "prefill_mfma_lds";
     } else {
         rc = rocm_launch_gemv_generic(&args, stream);

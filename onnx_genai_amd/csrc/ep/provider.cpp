@@ -53,6 +53,7 @@ NxrtStatus nxrt_rocm_ep_create(uint32_t device_ordinal, const char* const* keys,
         if (const char* env = std::getenv("NXRT_ROCM_DECODE_WAVES")) ep->config.emplace("decode_waves", env);
         if (const char* env = std::getenv("NXRT_ROCM_DECODE_COL_GROUPS")) ep->config.emplace("decode_col_groups", env);
         if (const char* env = std::getenv("NXRT_ROCM_PREPACK")) ep->config.emplace("prepack", env);
+        if (const char* env = std::getenv("NXRT_ROCM_PREFILL_TILE")) ep->config.emplace("prefill_tile", env);
         auto it = ep->config.find("acc4_rounding");
         if (it != ep->config.end()) {
             if (it->second == "native") ep->acc4_rounding = 1;
@@ -65,6 +66,7 @@ NxrtStatus nxrt_rocm_ep_create(uint32_t device_ordinal, const char* const* keys,
         if ((it = ep->config.find("decode_waves")) != ep->config.end()) ep->decode_waves = parse_int(it->second, 0);
         if ((it = ep->config.find("decode_col_groups")) != ep->config.end()) ep->decode_col_groups = parse_int(it->second, 0);
         if ((it = ep->config.find("prepack")) != ep->config.end()) ep->prepack = parse_int(it->second, 1);
+        if ((it = ep->config.find("prefill_tile")) != ep->config.end()) ep->prefill_tile = parse_int(it->second, 0);
         NxrtStatus st = ep->bind();
         if (st.code == NXRT_OK) st = hip_status(rocm_ffi_stream_create(&ep->stream), "hipStreamCreate");
         if (st.code != NXRT_OK) {

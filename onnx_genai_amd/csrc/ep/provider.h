@@ -18,6 +18,7 @@ struct NxrtRocmEp {
     int acc4_rounding = 0;                        // 0 = ties to even (MLAS), 1 = ties away (native)
     int decode_waves = 0;                         // 0 = chosen per shape
     int decode_col_groups = 0;
+    int prefill_tile = 0;                         // 0 = chosen per shape; 1..3 force a tile (tests, tuning)
     int prepack = 1;                              // repack constant weights for the decode kernel on first use
     std::mutex mu;
     std::unordered_map<void*, size_t> live;       // allocations handed out and not yet returned

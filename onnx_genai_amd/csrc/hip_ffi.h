@@ -77,9 +77,10 @@ uint64_t rocm_decode_packed_bytes(const RocmMatMulNBitsArgs* args);
 int rocm_launch_pack_decode(const RocmMatMulNBitsArgs* args, void* packed, rocm_stream_t stream);
 int rocm_launch_decode_packed(const RocmMatMulNBitsArgs* args, const void* packed, int waves, rocm_stream_t stream);
 
-/* Prefill (M > 16), f16/bf16 activations: B tiles dequantized into LDS, 32x32x16 MFMA. */
+/* Prefill (M > 16), f16/bf16 activations: B tiles dequantized into LDS, 32x32x16 MFMA.
+ * tile_choice: 0 = by shape, 1 = 128 x 128, 2 = 256 x 128, 3 = 256 x 256 tiles of Y per workgroup. */
 int rocm_prefill_mfma_eligible(const RocmMatMulNBitsArgs* args);
-int rocm_launch_prefill_mfma(const RocmMatMulNBitsArgs* args, rocm_stream_t stream);
+int rocm_launch_prefill_mfma(const RocmMatMulNBitsArgs* args, int tile_choice, rocm_stream_t stream);
 
 /* accuracy_level 4. rounding: 0 = ties to even (MLAS rule), 1 = ties away (native Rust rule).
  * qa: int8 [M, kb*bs]; qscale: f32 [M, kb]; qsum: int32 [M, kb] (sum of codes per block). */

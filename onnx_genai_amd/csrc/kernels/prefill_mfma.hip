@@ -13,6 +13,8 @@
 // per step separates the two buffers. Edges in M and N are handled by range-checked buffer loads and masked stores.
 #include <hip/hip_fp16.h>
 
+#include <type_traits>
+
 #include "common.hiph"
 
 namespace mnb {
@@ -91,21 +93,25 @@ __device__ __forceinline__ uint32_t finish_f32(uint32_t pair, float off, float s
     else return static_cast<uint32_t>(f32_to_f16_bits(lo)) | (static_cast<uint32_t>(f32_to_f16_bits(hi)) << 16);
 }
 
-// BF16: element type. BM: rows of Y per workgroup (128 or 256). SF32: scales are stored as f32 (otherwise in the
-// activations' 16-bit type). f16 activations with f16 scales dequantize in packed f16, everything else in f32.
-template <bool BF16, int BM, bool SF32>
+// BF16: element type. BM x BN: tile of Y per workgroup (128 x 128, 256 x 128 or 256 x 256). SF32: scales are stored
+// as f32 (otherwise in the activations' 16-bit type). f16 activations with f16 scales dequantize in packed f16,
+// everything else in f32.
+template <bool BF16, int BM, int BN, bool SF32>
 __global__ __launch_bounds__(512) void prefill_mfma_kernel(PrefillParams p)
 {
     constexpr bool F32MATH = BF16 || SF32;
     constexpr int WM = BM / 4;             // wave sub-tile rows
+    constexpr int WN = BN / 2;             // and columns
     constexpr int TM = WM / 32;            // 32x32 MFMA tiles per wave along M
-    constexpr int TN = 2;                  // and along N (64 columns)
+    constexpr int TN = WN / 32;            // and along N
     constexpr int A_LOADS = BM / 64;       // 16-byte pieces of A per lane per step
+    constexpr int B_DW = BN / 64;          // packed dwords of B per lane per step (2 or 4)
+    constexpr int B_PIECES = 8 / B_DW;     // lanes that share one column's 32 bytes of a step
     constexpr uint32_t kMagic = BF16 ? 0x43004300u : 0x64006400u;
     constexpr float kMagicF = BF16 ? 128.0f : 1024.0f;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     unsigned char* lds_a = smem;                                   // [2][BM][kPitch]
-    unsigned char* lds_b = smem + 2 * BM * kPitch;                 // [2][kBN][kPitch]
+    unsigned char* lds_b = smem + 2 * BM * kPitch;                 // [2][BN][kPitch]
 
     const int t = threadIdx.x;
     const int lane = t & 63;
@@ -114,7 +120,7 @@ __global__ __launch_bounds__(512) void prefill_mfma_kernel(PrefillParams p)
     // Column blocks vary fastest: the workgroups running at one time share a few row blocks of A (each XCD's L2 then
     // holds them once) and sweep the small packed B.
     const int64_t m_base = static_cast<int64_t>(blockIdx.y) * BM;
-    const int64_t n_base = static_cast<int64_t>(blockIdx.x) * kBN;
+    const int64_t n_base = static_cast<int64_t>(blockIdx.x) * BN;
     const int64_t rows_left = p.m - m_base, cols_left = p.n - n_base;
 
     const __amdgpu_buffer_rsrc_t srd_a = make_srd_p(p.a + m_base * p.k, static_cast<uint64_t>(rows_left * p.k) * 2);
@@ -126,13 +132,13 @@ __global__ __launch_bounds__(512) void prefill_mfma_kernel(PrefillParams p)
     const uint32_t zp_mask = has_zp ? 0xfu : 0u, zp_default = has_zp ? 0u : 8u;   // branch-free "8 when absent"
     const __amdgpu_buffer_rsrc_t srd_z = make_srd_p(has_zp ? p.zp + n_base * p.zp_row : p.b, has_zp ? static_cast<uint64_t>(cols_left * p.zp_row) : 0);
 
-    // A: lane -> (row t/8 + 64 i, piece t%8). B: lane -> (column t/4, quarter t%4 of the 64-element step).
+    // A: lane -> (row t/8 + 64 i, piece t%8). B: lane -> (column t / B_PIECES, piece t % B_PIECES of the 64-element step).
     const uint32_t a_goff = static_cast<uint32_t>(t >> 3) * static_cast<uint32_t>(p.k) * 2u + static_cast<uint32_t>((t & 7) * 16);
     const uint32_t a_gstep = 64u * static_cast<uint32_t>(p.k) * 2u;
     const uint32_t a_loff = static_cast<uint32_t>((t >> 3) * kPitch + (t & 7) * 16);
-    const int bcol = t >> 2, bquarter = t & 3;
-    const uint32_t b_goff = static_cast<uint32_t>(bcol) * static_cast<uint32_t>(p.row_bytes) + static_cast<uint32_t>(bquarter * 8);
-    const uint32_t b_loff = static_cast<uint32_t>(bcol * kPitch + bquarter * 32);
+    const int bcol = t / B_PIECES, bpiece = t % B_PIECES;
+    const uint32_t b_goff = static_cast<uint32_t>(bcol) * static_cast<uint32_t>(p.row_bytes) + static_cast<uint32_t>(bpiece * B_DW * 4);
+    const uint32_t b_loff = static_cast<uint32_t>(bcol * kPitch + bpiece * B_DW * 16);
     const uint32_t s_goff = static_cast<uint32_t>(bcol) * static_cast<uint32_t>(p.kb) * kScaleBytes;
     const uint32_t z_goff = static_cast<uint32_t>(bcol) * static_cast<uint32_t>(p.zp_row);
 
@@ -150,10 +156,10 @@ __global__ __launch_bounds__(512) void prefill_mfma_kernel(PrefillParams p)
     const int steps = static_cast<int>(p.k / kBK);
     // Global loads run D-1 steps ahead of the MFMAs, in D register sets; step x lives in set x % D from its load
     // (issued while step x-D+1 is being multiplied) to its dequantize-and-store into LDS (while step x-1 is).
-    constexpr int D = 4;
+    constexpr int D = BN == 256 ? 3 : 4;   // the 256 x 256 tile has no registers left for a fourth set
     struct Regs {
         uint4 a[A_LOADS];
-        uint2 b;
+        uint32_t b[B_DW];
         uint32_t s;      // raw scale bits; converted when the step is dequantized, so that no load is waited for early
         uint32_t z;      // raw zero-point byte
         uint32_t zsh;    // shift of the nibble to take from it
@@ -163,9 +169,18 @@ __global__ __launch_bounds__(512) void prefill_mfma_kernel(PrefillParams p)
     auto load_global = [&](Regs& r, int kt) {
 #pragma unroll
         for (int i = 0; i < A_LOADS; ++i) r.a[i] = load16_p(srd_a, a_goff + static_cast<uint32_t>(i) * a_gstep, static_cast<uint32_t>(kt) * 128u);
-        const auto bw = __builtin_amdgcn_raw_buffer_load_b64(srd_b, static_cast<int>(b_goff), static_cast<int>(kt * 32), 0);
-        r.b = make_uint2(bw[0], bw[1]);
-        const uint32_t blk = static_cast<uint32_t>((kt * kBK + bquarter * 16) >> p.bs_log2);
+        if constexpr (B_DW == 2) {
+            const auto bw = __builtin_amdgcn_raw_buffer_load_b64(srd_b, static_cast<int>(b_goff), static_cast<int>(kt * 32), 0);
+            r.b[0] = bw[0];
+            r.b[1] = bw[1];
+        } else {
+            const uint4 bw = load16_p(srd_b, b_goff, static_cast<uint32_t>(kt) * 32u);
+            r.b[0] = bw.x;
+            r.b[1] = bw.y;
+            r.b[2] = bw.z;
+            r.b[3] = bw.w;
+        }
+        const uint32_t blk = static_cast<uint32_t>((kt * kBK + bpiece * B_DW * 8) >> p.bs_log2);
         if constexpr (SF32) r.s = __builtin_amdgcn_raw_buffer_load_b32(srd_s, static_cast<int>(s_goff + blk * 4u), 0, 0);
         else r.s = __builtin_amdgcn_raw_buffer_load_b16(srd_s, static_cast<int>(s_goff + blk * 2u), 0, 0);
         // loaded even without zero points (the empty range then returns 0): a branch here would split the loop body
@@ -173,16 +188,17 @@ __global__ __launch_bounds__(512) void prefill_mfma_kernel(PrefillParams p)
         r.z = zraw;                 // no arithmetic on a loaded value here: it would wait for the load at once
         r.zsh = (blk & 1u) * 4u;
     };
-    // Quarter `part` (0..3) of one step's trip from registers to LDS: A pieces part, part+4, ... and, in quarters 0 and
-    // 2, one packed dword of B, dequantized. Four quarters make a step; they are issued between the MFMA batches of
-    // the step before, so that their VALU and LDS-write work runs while the matrix cores are busy.
+    // Quarter `part` (0..3) of one step's trip from registers to LDS: A pieces part, part+4, ... and one packed dword of
+    // B, dequantized (with two dwords per lane: in quarters 0 and 2). Four quarters make a step; they are issued between
+    // the MFMA batches of the step before, so that their VALU and LDS-write work runs while the matrix cores are busy.
     auto store_part = [&](const Regs& r, int buf, int part) {
         unsigned char* la = lds_a + buf * (BM * kPitch) + a_loff;
 #pragma unroll
         for (int i = part; i < A_LOADS; i += 4) *reinterpret_cast<uint4*>(la + i * 64 * kPitch) = r.a[i];
-        if (part & 1) return;
-        unsigned char* lb = lds_b + buf * (kBN * kPitch) + b_loff;
-        const uint32_t w = part == 0 ? r.b.x : r.b.y, w4 = w >> 4;
+        if (B_DW == 2 && (part & 1)) return;
+        const int dw = B_DW == 2 ? (part >> 1) : part;
+        unsigned char* lb = lds_b + buf * (BN * kPitch) + b_loff;
+        const uint32_t w = r.b[dw], w4 = w >> 4;
         uint32_t pr[4];
         pr[0] = magic_pair(w, w4, 0x0c040c00u, kMagic);
         pr[1] = magic_pair(w, w4, 0x0c050c01u, kMagic);
@@ -200,7 +216,7 @@ __global__ __launch_bounds__(512) void prefill_mfma_kernel(PrefillParams p)
 #pragma unroll
             for (int i = 0; i < 4; ++i) pr[i] = finish_f16(pr[i], __builtin_bit_cast(half2_t, o2), __builtin_bit_cast(half2_t, s2));
         }
-        *reinterpret_cast<uint4*>(lb + (part >> 1) * 16) = make_uint4(pr[0], pr[1], pr[2], pr[3]);
+        *reinterpret_cast<uint4*>(lb + dw * 16) = make_uint4(pr[0], pr[1], pr[2], pr[3]);
     };
     auto store_lds = [&](const Regs& r, int buf) {
 #pragma unroll
@@ -210,7 +226,7 @@ __global__ __launch_bounds__(512) void prefill_mfma_kernel(PrefillParams p)
     // while these run, and (when asked) the following step moves from registers into the other buffer.
     auto compute = [&](int buf, const Regs& next, bool store_next) {
         const unsigned char* la = lds_a + buf * (BM * kPitch) + wm * (WM * kPitch) + frag_off;
-        const unsigned char* lb = lds_b + buf * (kBN * kPitch) + wn * (64 * kPitch) + frag_off;
+        const unsigned char* lb = lds_b + buf * (BN * kPitch) + wn * (WN * kPitch) + frag_off;
         uint4 fa[2][TM], fb[2][TN];
 #pragma unroll
         for (int i = 0; i < TM; ++i) fa[0][i] = *reinterpret_cast<const uint4*>(la + i * 32 * kPitch);
@@ -248,7 +264,7 @@ __global__ __launch_bounds__(512) void prefill_mfma_kernel(PrefillParams p)
 #pragma unroll
         for (int s0 = 0; s0 < D; ++s0) {
             load_global(regs[(s0 + D - 1) % D], kt0 + s0 + D - 1);
-            compute(s0 & 1, regs[(s0 + 1) % D], true);
+            compute((kt0 + s0) & 1, regs[(s0 + 1) % D], true);
             __syncthreads();
         }
     }
@@ -257,7 +273,7 @@ __global__ __launch_bounds__(512) void prefill_mfma_kernel(PrefillParams p)
         const int kt = kt0 + s0;
         load_global(regs[(s0 + D - 1) % D], kt + D - 1);
         if (kt < steps) {
-            compute(s0 & 1, regs[(s0 + 1) % D], kt + 1 < steps);
+            compute(kt & 1, regs[(s0 + 1) % D], kt + 1 < steps);
             __syncthreads();
         }
     }
@@ -267,7 +283,7 @@ __global__ __launch_bounds__(512) void prefill_mfma_kernel(PrefillParams p)
     const int row_group = (lane >> 5) * 4;
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
-        const int64_t col = n_base + wn * 64 + j * 32 + col_in_tile;
+        const int64_t col = n_base + wn * WN + j * 32 + col_in_tile;
         if (col >= p.n) continue;
         const float bias = p.bias ? load_as_f32(p.bias, p.bias_dtype, col) : 0.f;
 #pragma unroll
@@ -284,12 +300,12 @@ __global__ __launch_bounds__(512) void prefill_mfma_kernel(PrefillParams p)
     }
 }
 
-template <bool BF16, int BM, bool SF32>
+template <bool BF16, int BM, int BN, bool SF32>
 static int launch_prefill(const PrefillParams& p, hipStream_t stream)
 {
-    const dim3 grid(static_cast<unsigned>((p.n + kBN - 1) / kBN), static_cast<unsigned>((p.m + BM - 1) / BM));
-    const size_t lds = 2 * static_cast<size_t>(BM + kBN) * kPitch;
-    auto kernel = prefill_mfma_kernel<BF16, BM, SF32>;
+    const dim3 grid(static_cast<unsigned>((p.n + BN - 1) / BN), static_cast<unsigned>((p.m + BM - 1) / BM));
+    const size_t lds = 2 * static_cast<size_t>(BM + BN) * kPitch;
+    auto kernel = prefill_mfma_kernel<BF16, BM, BN, SF32>;
     if (lds > 65536) {
         const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
         if (e != hipSuccess) return static_cast<int>(e);
@@ -311,7 +327,7 @@ extern "C" int rocm_prefill_mfma_eligible(const RocmMatMulNBitsArgs* a)
     return (reinterpret_cast<uintptr_t>(a->a) & 15) == 0 && (reinterpret_cast<uintptr_t>(a->b) & 15) == 0;
 }
 
-extern "C" int rocm_launch_prefill_mfma(const RocmMatMulNBitsArgs* a, rocm_stream_t stream)
+extern "C" int rocm_launch_prefill_mfma(const RocmMatMulNBitsArgs* a, int tile_choice, rocm_stream_t stream)
 {
     if (!rocm_prefill_mfma_eligible(a)) return -1;
     mnb::PrefillParams p;
@@ -334,11 +350,20 @@ extern "C" int rocm_launch_prefill_mfma(const RocmMatMulNBitsArgs* a, rocm_strea
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool bf16 = a->a_dtype == ROCM_DT_BF16;
     const bool sf32 = a->scale_dtype == ROCM_DT_F32;
-    // 256-row tiles once there are enough of them to fill the chip; 128-row tiles otherwise.
-    const int64_t wg256 = ((a->m + 255) / 256) * ((a->n + 127) / 128);
-    const bool big = a->m >= 256 && wg256 >= 256;
-    if (bf16 && sf32) return big ? mnb::launch_prefill<true, 256, true>(p, s) : mnb::launch_prefill<true, 128, true>(p, s);
-    if (bf16) return big ? mnb::launch_prefill<true, 256, false>(p, s) : mnb::launch_prefill<true, 128, false>(p, s);
-    if (sf32) return big ? mnb::launch_prefill<false, 256, true>(p, s) : mnb::launch_prefill<false, 128, true>(p, s);
-    return big ? mnb::launch_prefill<false, 256, false>(p, s) : mnb::launch_prefill<false, 128, false>(p, s);
+    // The largest tile that still gives every CU a workgroup (256 x 256, then 256 x 128);
+    // 128 x 128 otherwise.
+    const int64_t wg_huge = ((a->m + 255) / 256) * ((a->n + 255) / 256);
+    const int64_t wg_big = ((a->m + 255) / 256) * ((a->n + 127) / 128);
+    int tile = (a->m >= 256 && wg_huge >= 256) ? 2 : (a->m >= 256 && wg_big >= 256) ? 1 : 0;
+    if (tile_choice >= 1 && tile_choice <= 3) tile = tile_choice - 1;      // 1: 128 x 128, 2: 256 x 128, 3: 256 x 256
+    auto go = [&](auto bf, auto sf) {
+        constexpr bool B = decltype(bf)::value, S = decltype(sf)::value;
+        if (tile == 2) return mnb::launch_prefill<B, 256, 256, S>(p, s);
+        if (tile == 1) return mnb::launch_prefill<B, 256, 128, S>(p, s);
+        return mnb::launch_prefill<B, 128, 128, S>(p, s);
+    };
+    if (bf16 && sf32) return go(std::true_type{}, std::true_type{});
+    if (bf16) return go(std::true_type{}, std::false_type{});
+    if (sf32) return go(std::false_type{}, std::true_type{});
+    return go(std::false_type{}, std::false_type{});
 }

@@ -309,6 +309,22 @@ def test_prefill_matches_oracle(ep, port, a_dt, s_dt, bs, zero_points, m, n, k):
     assert np.array_equal(np.asarray(y).view(np.uint16), np.asarray(port.narrow(y32, a_dt)).view(np.uint16))
 
 
+@pytest.mark.parametrize("tile", [1, 2, 3])
+@pytest.mark.parametrize("a_dt,s_dt,bs,zero_points", [(E.F16, E.F16, 32, True), (E.BF16, E.F32, 128, False), (E.BF16, E.BF16, 64, True)])
+def test_prefill_tile_shapes_agree(port, tile, a_dt, s_dt, bs, zero_points):
+    """Every workgroup tile (128 x 128, 256 x 128, 256 x 256) on a shape with ragged edges in M and N."""
+    m, n, k = 300, 520, 1024
+    provider = E.RocmExecutionProvider(0, {"prefill_tile": str(tile)})
+    try:
+        b, s, zp = synth.make_weights(n, k, bs, 41, zero_points=zero_points, scale_lo=0.002, scale_hi=0.01, scale_dtype=s_dt)
+        a = synth.make_activation(m, k, 41, a_dt)
+        y32, variant = run_op(provider, a, a_dt, b, s, s_dt, zp, n, k, bs, y_dtype=E.F32)
+        assert variant == "prefill_mfma_lds"
+        assert helpers.rel_l2(y32, oracle_f64(port, a, a_dt, b, s, s_dt, zp, n, k, bs)) <= TOL_HALF
+    finally:
+        provider.shutdown()
+
+
 @pytest.mark.parametrize("bs,zero_points", [(32, True), (64, False), (128, True)])
 def test_prefill_weight_tiles_are_f16_of_f32_dequant(ep, port, bs, zero_points):
     """One-hot activation rows read single weights back out of the GEMM: with f16 scales each must equal the f32
