@@ -78,7 +78,7 @@ int rocm_launch_pack_decode(const RocmMatMulNBitsArgs* args, void* packed, rocm_
 int rocm_launch_decode_packed(const RocmMatMulNBitsArgs* args, const void* packed, int waves, rocm_stream_t stream);
 
 /* Prefill (M > 16), f16/bf16 activations: B tiles dequantized into LDS, 32x32x16 MFMA.
- * tile_choice: 0 = by shape, 1 = 128 x 128, 2 = 256 x 128, 3 = 256 x 256 tiles of Y per workgroup. */
+ * tile_choice: 0 = by shape, 1 = 128 x 128, 2 = 256 x 128, 3 = 256 x 256, 4 = 128 x 64 tiles of Y per workgroup. */
 int rocm_prefill_mfma_eligible(const RocmMatMulNBitsArgs* args);
 int rocm_launch_prefill_mfma(const RocmMatMulNBitsArgs* args, int tile_choice, rocm_stream_t stream);
 

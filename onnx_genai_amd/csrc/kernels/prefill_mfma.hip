@@ -15,14 +15,13 @@
 
 #include <type_traits>
 
-#include "common.hiph"
+#include "mfma_common.hiph"
 
 namespace mnb {
 
 typedef __attribute__((ext_vector_type(8))) _Float16 half8_t;
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(16))) float float16_t;
-typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
 typedef __attribute__((ext_vector_type(2))) _Float16 half2_t;
 
 struct PrefillParams {
@@ -38,21 +37,8 @@ struct PrefillParams {
     int scale_dtype, bias_dtype, y_dtype;
 };
 
-constexpr int kBN = 128;
 constexpr int kBK = 64;
 constexpr int kPitch = 144;            // bytes per LDS row: 64 halfs + 8 of padding
-
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_srd_p(const void* base, uint64_t bytes)
-{
-    const uint32_t range = bytes > 0x7fffffffull ? 0x7fffffffu : static_cast<uint32_t>(bytes);
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, static_cast<int>(range), 0x00020000);
-}
-
-__device__ __forceinline__ uint4 load16_p(__amdgpu_buffer_rsrc_t srd, uint32_t voffset, uint32_t soffset)
-{
-    const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(srd, static_cast<int>(voffset), static_cast<int>(soffset), 0);
-    return make_uint4(v.x, v.y, v.z, v.w);
-}
 
 template <bool BF16>
 __device__ __forceinline__ float16_t mfma32(const uint4& a, const uint4& b, float16_t c)
@@ -93,7 +79,7 @@ __device__ __forceinline__ uint32_t finish_f32(uint32_t pair, float off, float s
     else return static_cast<uint32_t>(f32_to_f16_bits(lo)) | (static_cast<uint32_t>(f32_to_f16_bits(hi)) << 16);
 }
 
-// BF16: element type. BM x BN: tile of Y per workgroup (128 x 128, 256 x 128 or 256 x 256). SF32: scales are stored
+// BF16: element type. BM x BN: tile of Y per workgroup (128 x 64, 128 x 128, 256 x 128 or 256 x 256). SF32: scales are stored
 // as f32 (otherwise in the activations' 16-bit type). f16 activations with f16 scales dequantize in packed f16,
 // everything else in f32.
 template <bool BF16, int BM, int BN, bool SF32>
@@ -105,7 +91,7 @@ __global__ __launch_bounds__(512) void prefill_mfma_kernel(PrefillParams p)
     constexpr int TM = WM / 32;            // 32x32 MFMA tiles per wave along M
     constexpr int TN = WN / 32;            // and along N
     constexpr int A_LOADS = BM / 64;       // 16-byte pieces of A per lane per step
-    constexpr int B_DW = BN / 64;          // packed dwords of B per lane per step (2 or 4)
+    constexpr int B_DW = BN / 64;          // packed dwords of B per lane per step (1, 2 or 4)
     constexpr int B_PIECES = 8 / B_DW;     // lanes that share one column's 32 bytes of a step
     constexpr uint32_t kMagic = BF16 ? 0x43004300u : 0x64006400u;
     constexpr float kMagicF = BF16 ? 128.0f : 1024.0f;
@@ -123,14 +109,14 @@ __global__ __launch_bounds__(512) void prefill_mfma_kernel(PrefillParams p)
     const int64_t n_base = static_cast<int64_t>(blockIdx.x) * BN;
     const int64_t rows_left = p.m - m_base, cols_left = p.n - n_base;
 
-    const __amdgpu_buffer_rsrc_t srd_a = make_srd_p(p.a + m_base * p.k, static_cast<uint64_t>(rows_left * p.k) * 2);
-    const __amdgpu_buffer_rsrc_t srd_b = make_srd_p(p.b + n_base * p.row_bytes, static_cast<uint64_t>(cols_left * p.row_bytes));
+    const __amdgpu_buffer_rsrc_t srd_a = make_srd(p.a + m_base * p.k, static_cast<uint64_t>(rows_left * p.k) * 2);
+    const __amdgpu_buffer_rsrc_t srd_b = make_srd(p.b + n_base * p.row_bytes, static_cast<uint64_t>(cols_left * p.row_bytes));
     constexpr uint32_t kScaleBytes = SF32 ? 4 : 2;
-    const __amdgpu_buffer_rsrc_t srd_s = make_srd_p(static_cast<const unsigned char*>(p.scales) + n_base * p.kb * kScaleBytes,
+    const __amdgpu_buffer_rsrc_t srd_s = make_srd(static_cast<const unsigned char*>(p.scales) + n_base * p.kb * kScaleBytes,
                                                     static_cast<uint64_t>(cols_left * p.kb) * kScaleBytes);
     const bool has_zp = p.zp != nullptr;
     const uint32_t zp_mask = has_zp ? 0xfu : 0u, zp_default = has_zp ? 0u : 8u;   // branch-free "8 when absent"
-    const __amdgpu_buffer_rsrc_t srd_z = make_srd_p(has_zp ? p.zp + n_base * p.zp_row : p.b, has_zp ? static_cast<uint64_t>(cols_left * p.zp_row) : 0);
+    const __amdgpu_buffer_rsrc_t srd_z = make_srd(has_zp ? p.zp + n_base * p.zp_row : p.b, has_zp ? static_cast<uint64_t>(cols_left * p.zp_row) : 0);
 
     // A: lane -> (row t/8 + 64 i, piece t%8). B: lane -> (column t / B_PIECES, piece t % B_PIECES of the 64-element step).
     const uint32_t a_goff = static_cast<uint32_t>(t >> 3) * static_cast<uint32_t>(p.k) * 2u + static_cast<uint32_t>((t & 7) * 16);
@@ -168,13 +154,15 @@ __global__ __launch_bounds__(512) void prefill_mfma_kernel(PrefillParams p)
 
     auto load_global = [&](Regs& r, int kt) {
 #pragma unroll
-        for (int i = 0; i < A_LOADS; ++i) r.a[i] = load16_p(srd_a, a_goff + static_cast<uint32_t>(i) * a_gstep, static_cast<uint32_t>(kt) * 128u);
-        if constexpr (B_DW == 2) {
+        for (int i = 0; i < A_LOADS; ++i) r.a[i] = load16(srd_a, a_goff + static_cast<uint32_t>(i) * a_gstep, static_cast<uint32_t>(kt) * 128u);
+        if constexpr (B_DW == 1) {
+            r.b[0] = __builtin_amdgcn_raw_buffer_load_b32(srd_b, static_cast<int>(b_goff), static_cast<int>(kt * 32), 0);
+        } else if constexpr (B_DW == 2) {
             const auto bw = __builtin_amdgcn_raw_buffer_load_b64(srd_b, static_cast<int>(b_goff), static_cast<int>(kt * 32), 0);
             r.b[0] = bw[0];
             r.b[1] = bw[1];
         } else {
-            const uint4 bw = load16_p(srd_b, b_goff, static_cast<uint32_t>(kt) * 32u);
+            const uint4 bw = load16(srd_b, b_goff, static_cast<uint32_t>(kt) * 32u);
             r.b[0] = bw.x;
             r.b[1] = bw.y;
             r.b[2] = bw.z;
@@ -195,8 +183,8 @@ __global__ __launch_bounds__(512) void prefill_mfma_kernel(PrefillParams p)
         unsigned char* la = lds_a + buf * (BM * kPitch) + a_loff;
 #pragma unroll
         for (int i = part; i < A_LOADS; i += 4) *reinterpret_cast<uint4*>(la + i * 64 * kPitch) = r.a[i];
-        if (B_DW == 2 && (part & 1)) return;
-        const int dw = B_DW == 2 ? (part >> 1) : part;
+        if ((B_DW == 2 && (part & 1)) || (B_DW == 1 && part != 0)) return;
+        const int dw = B_DW == 4 ? part : (part >> 1);
         unsigned char* lb = lds_b + buf * (BN * kPitch) + b_loff;
         const uint32_t w = r.b[dw], w4 = w >> 4;
         uint32_t pr[4];
@@ -350,16 +338,17 @@ extern "C" int rocm_launch_prefill_mfma(const RocmMatMulNBitsArgs* a, int tile_c
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool bf16 = a->a_dtype == ROCM_DT_BF16;
     const bool sf32 = a->scale_dtype == ROCM_DT_F32;
-    // The largest tile that still gives every CU a workgroup (256 x 256, then 256 x 128);
-    // 128 x 128 otherwise.
+    // The largest tile that still gives every CU a workgroup: 256 x 256, then 256 x 128, 128 x 128, 128 x 64.
     const int64_t wg_huge = ((a->m + 255) / 256) * ((a->n + 255) / 256);
     const int64_t wg_big = ((a->m + 255) / 256) * ((a->n + 127) / 128);
-    int tile = (a->m >= 256 && wg_huge >= 256) ? 2 : (a->m >= 256 && wg_big >= 256) ? 1 : 0;
-    if (tile_choice >= 1 && tile_choice <= 3) tile = tile_choice - 1;      // 1: 128 x 128, 2: 256 x 128, 3: 256 x 256
+    const int64_t wg_small = ((a->m + 127) / 128) * ((a->n + 127) / 128);
+    int tile = (a->m >= 256 && wg_huge >= 256) ? 2 : (a->m >= 256 && wg_big >= 256) ? 1 : wg_small >= 256 ? 0 : 3;
+    if (tile_choice >= 1 && tile_choice <= 4) tile = tile_choice == 4 ? 3 : tile_choice - 1;   // 1: 128 x 128, 2: 256 x 128, 3: 256 x 256, 4: 128 x 64
     auto go = [&](auto bf, auto sf) {
         constexpr bool B = decltype(bf)::value, S = decltype(sf)::value;
         if (tile == 2) return mnb::launch_prefill<B, 256, 256, S>(p, s);
         if (tile == 1) return mnb::launch_prefill<B, 256, 128, S>(p, s);
+        if (tile == 3) return mnb::launch_prefill<B, 128, 64, S>(p, s);
         return mnb::launch_prefill<B, 128, 128, S>(p, s);
     };
     if (bf16 && sf32) return go(std::true_type{}, std::true_type{});

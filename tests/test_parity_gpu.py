@@ -309,10 +309,10 @@ def test_prefill_matches_oracle(ep, port, a_dt, s_dt, bs, zero_points, m, n, k):
     assert np.array_equal(np.asarray(y).view(np.uint16), np.asarray(port.narrow(y32, a_dt)).view(np.uint16))
 
 
-@pytest.mark.parametrize("tile", [1, 2, 3])
+@pytest.mark.parametrize("tile", [1, 2, 3, 4])
 @pytest.mark.parametrize("a_dt,s_dt,bs,zero_points", [(E.F16, E.F16, 32, True), (E.BF16, E.F32, 128, False), (E.BF16, E.BF16, 64, True)])
 def test_prefill_tile_shapes_agree(port, tile, a_dt, s_dt, bs, zero_points):
-    """Every workgroup tile (128 x 128, 256 x 128, 256 x 256) on a shape with ragged edges in M and N."""
+    """Every workgroup tile (128 x 128, 256 x 128, 256 x 256, 128 x 64) on a shape with ragged edges in M and N."""
     m, n, k = 300, 520, 1024
     provider = E.RocmExecutionProvider(0, {"prefill_tile": str(tile)})
     try:
