@@ -335,7 +335,28 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
         rc = rocm_launch_decode_mfma(&args, kn.ep->decode_waves, kn.ep->decode_col_groups, stream);
         kn.variant = "decode_mfma_splitk";
     } else if (M > 16 && rocm_prefill_mfma_eligible(&args)) {
-        rc = rocm_launch_prefill_mfma(&args, kn.ep->prefill_tile, stream);
+        // Small grids slice K and want scratch for the partial sums: the caller's workspace if it is large enough, else
+        // the kernel's own (grown outside a capture only; with too little the launcher slices less or not at all).
+        const uint64_t need = rocm_prefill_mfma_scratch_bytes(&args, kn.ep->prefill_tile);
+        void* scratch = workspace;
+        uint64_t scratch_bytes = workspace ? workspace_bytes : 0;
+        if (need > scratch_bytes) {
+            if (kn.scratch_bytes < need && !kn.ep->capturing) {
+                if (kn.scratch) {
+                    rocm_ffi_stream_sync(stream);
+                    rocm_ffi_free(kn.scratch);
+                    kn.scratch = nullptr;
+                    kn.scratch_bytes = 0;
+                }
+                if (rocm_ffi_malloc(&kn.scratch, need) == 0) kn.scratch_bytes = need;
+                else kn.scratch = nullptr;
+            }
+            if (kn.scratch_bytes > scratch_bytes) {
+                scratch = kn.scratch;
+                scratch_bytes = kn.scratch_bytes;
+            }
+        }
+        rc = rocm_launch_prefill_mfma(&args, kn.ep->prefill_tile, scratch, scratch_bytes, stream);
         kn.variant = "prefill_mfma_lds";
     } else {
         rc = rocm_launch_gemv_generic(&args, stream);
@@ -470,15 +491,36 @@ NxrtStatus nxrt_rocm_matmul_nbits_workspace_requirement(const NxrtRocmMatMulNBit
         if (!kernel || !out) return make_status(NXRT_INVALID_ARGUMENT, "MatMulNBits: null pointer in workspace_requirement");
         out->bytes = 0;
         out->alignment = 1;
-        if (kernel->accuracy_level != 4) return ok();
-        if (!inputs || n_inputs < 1 || inputs[0].ndim < 1 || !inputs[0].dims) return make_status(NXRT_INVALID_ARGUMENT, err("workspace_requirement needs the shape of A"));
+        if (!inputs || n_inputs < 1 || inputs[0].ndim < 1 || !inputs[0].dims) {
+            if (kernel->accuracy_level != 4) return ok();        // no shape, no slicing plan: the kernel manages without
+            return make_status(NXRT_INVALID_ARGUMENT, err("workspace_requirement needs the shape of A"));
+        }
         uint64_t m = 1;
         for (uint32_t i = 0; i + 1 < inputs[0].ndim; ++i) {
-            if (inputs[0].dims[i] < 0) return make_status(NXRT_INVALID_ARGUMENT, err("workspace_requirement needs static leading dimensions of A"));
+            if (inputs[0].dims[i] < 0) {
+                if (kernel->accuracy_level != 4) return ok();
+                return make_status(NXRT_INVALID_ARGUMENT, err("workspace_requirement needs static leading dimensions of A"));
+            }
             m *= static_cast<uint64_t>(inputs[0].dims[i]);
         }
-        out->bytes = acc4_workspace_bytes(*kernel, m);
-        out->alignment = 256;
+        if (kernel->accuracy_level == 4) {
+            out->bytes = acc4_workspace_bytes(*kernel, m);
+            out->alignment = 256;
+            return ok();
+        }
+        // float path: partial sums of a K-sliced prefill call (optional - without it the kernel allocates its own
+        // outside a capture, or does not slice)
+        RocmMatMulNBitsArgs probe;
+        std::memset(&probe, 0, sizeof(probe));
+        probe.a = probe.b = nullptr;
+        probe.a_dtype = probe.scale_dtype = static_cast<int>(inputs[0].dtype);
+        if (n_inputs > 2) probe.scale_dtype = static_cast<int>(inputs[2].dtype);
+        probe.m = static_cast<int64_t>(m);
+        probe.n = kernel->n;
+        probe.k = kernel->k;
+        probe.block_size = static_cast<int>(kernel->block_size);
+        out->bytes = m > 16 ? rocm_prefill_mfma_scratch_bytes(&probe, kernel->ep->prefill_tile) : 0;
+        out->alignment = out->bytes ? 256 : 1;
         return ok();
     });
 }

@@ -80,7 +80,11 @@ int rocm_launch_decode_packed(const RocmMatMulNBitsArgs* args, const void* packe
 /* Prefill (M > 16), f16/bf16 activations: B tiles dequantized into LDS, 32x32x16 MFMA.
  * tile_choice: 0 = by shape, 1 = 128 x 128, 2 = 256 x 128, 3 = 256 x 256, 4 = 128 x 64 tiles of Y per workgroup. */
 int rocm_prefill_mfma_eligible(const RocmMatMulNBitsArgs* args);
-int rocm_launch_prefill_mfma(const RocmMatMulNBitsArgs* args, int tile_choice, rocm_stream_t stream);
+/* Small grids with long K are cut into slices of K whose f32 partial sums land in `scratch` ([slices][M][N]) and are added up
+ * by a second kernel; rocm_prefill_mfma_scratch_bytes says how much the preferred plan wants (0 = no slicing). With less
+ * scratch the launcher uses fewer slices, with none it does not slice. */
+uint64_t rocm_prefill_mfma_scratch_bytes(const RocmMatMulNBitsArgs* args, int tile_choice);
+int rocm_launch_prefill_mfma(const RocmMatMulNBitsArgs* args, int tile_choice, void* scratch, uint64_t scratch_bytes, rocm_stream_t stream);
 
 /* accuracy_level 4. rounding: 0 = ties to even (MLAS rule), 1 = ties away (native Rust rule).
  * qa: int8 [M, kb*bs]; qscale: f32 [M, kb]; qsum: int32 [M, kb] (sum of codes per block). */

@@ -35,6 +35,8 @@ struct PrefillParams {
     int64_t row_bytes, zp_row;
     int bs_log2;
     int scale_dtype, bias_dtype, y_dtype;
+    int steps_per_split;    // K steps of 64 per workgroup along grid.z
+    float* partial;         // [splits][M][N] f32 partial sums when K is split (else NULL: the kernel writes Y itself)
 };
 
 constexpr int kBK = 64;
@@ -139,7 +141,10 @@ __global__ __launch_bounds__(512) void prefill_mfma_kernel(PrefillParams p)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    const int steps = static_cast<int>(p.k / kBK);
+    // K range of this workgroup: all of K, or one of grid.z slices whose f32 partial sums a second kernel adds up in
+    // slice order (small grids: long K, few tiles of Y).
+    const int kt_begin = static_cast<int>(blockIdx.z) * p.steps_per_split;
+    const int steps = min(kt_begin + p.steps_per_split, static_cast<int>(p.k / kBK));
     // Global loads run D-1 steps ahead of the MFMAs, in D register sets; step x lives in set x % D from its load
     // (issued while step x-D+1 is being multiplied) to its dequantize-and-store into LDS (while step x-1 is).
     constexpr int D = BN == 256 ? 3 : 4;   // the 256 x 256 tile has no registers left for a fourth set
@@ -241,13 +246,13 @@ __global__ __launch_bounds__(512) void prefill_mfma_kernel(PrefillParams p)
     // that are never stored): with a fixed number of loads per step the compiler can wait for exactly the step it
     // needs and leave the newer ones in flight.
 #pragma unroll
-    for (int s0 = 0; s0 < D - 1; ++s0) load_global(regs[s0], s0);
-    store_lds(regs[0], 0);
+    for (int s0 = 0; s0 < D - 1; ++s0) load_global(regs[s0], kt_begin + s0);
+    store_lds(regs[0], kt_begin & 1);
     __syncthreads();
     // Main loop: whole rounds of D steps with no branch inside, so that the wait before each step counts loads
     // exactly and the newer ones stay in flight (a branch would make the compiler drain them all). The last
     // round, which holds the final step, runs with the conditions.
-    int kt0 = 0;
+    int kt0 = kt_begin;
     for (; kt0 + D < steps; kt0 += D) {
 #pragma unroll
         for (int s0 = 0; s0 < D; ++s0) {
@@ -273,7 +278,8 @@ __global__ __launch_bounds__(512) void prefill_mfma_kernel(PrefillParams p)
     for (int j = 0; j < TN; ++j) {
         const int64_t col = n_base + wn * WN + j * 32 + col_in_tile;
         if (col >= p.n) continue;
-        const float bias = p.bias ? load_as_f32(p.bias, p.bias_dtype, col) : 0.f;
+        const float bias = (p.bias && !p.partial) ? load_as_f32(p.bias, p.bias_dtype, col) : 0.f;
+        float* part = p.partial ? p.partial + static_cast<int64_t>(blockIdx.z) * p.m * p.n : nullptr;
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
 #pragma unroll
@@ -281,17 +287,32 @@ __global__ __launch_bounds__(512) void prefill_mfma_kernel(PrefillParams p)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const int64_t row = m_base + wm * WM + i * 32 + q * 8 + row_group + r;
-                    if (row < p.m) store_from_f32(p.y, p.y_dtype, row * p.n + col, acc[i][j][q * 4 + r] + bias);
+                    if (row >= p.m) continue;
+                    if (part) part[row * p.n + col] = acc[i][j][q * 4 + r];
+                    else store_from_f32(p.y, p.y_dtype, row * p.n + col, acc[i][j][q * 4 + r] + bias);
                 }
             }
         }
     }
 }
 
-template <bool BF16, int BM, int BN, bool SF32>
-static int launch_prefill(const PrefillParams& p, hipStream_t stream)
+// Y = sum over slices of the partial sums, in slice order, plus bias; one thread per element.
+__global__ __launch_bounds__(256) void prefill_reduce_kernel(const float* __restrict__ partial, int splits, int64_t m, int64_t n,
+                                                             const void* __restrict__ bias, int bias_dtype, void* __restrict__ y, int y_dtype)
 {
-    const dim3 grid(static_cast<unsigned>((p.n + BN - 1) / BN), static_cast<unsigned>((p.m + BM - 1) / BM));
+    const int64_t total = m * n;
+    for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < total; i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+        float sum = 0.f;
+        for (int z = 0; z < splits; ++z) sum += partial[z * total + i];
+        if (bias) sum += load_as_f32(bias, bias_dtype, i % n);
+        store_from_f32(y, y_dtype, i, sum);
+    }
+}
+
+template <bool BF16, int BM, int BN, bool SF32>
+static int launch_prefill(const PrefillParams& p, int splits, hipStream_t stream)
+{
+    const dim3 grid(static_cast<unsigned>((p.n + BN - 1) / BN), static_cast<unsigned>((p.m + BM - 1) / BM), static_cast<unsigned>(splits));
     const size_t lds = 2 * static_cast<size_t>(BM + BN) * kPitch;
     auto kernel = prefill_mfma_kernel<BF16, BM, BN, SF32>;
     if (lds > 65536) {
@@ -315,7 +336,50 @@ extern "C" int rocm_prefill_mfma_eligible(const RocmMatMulNBitsArgs* a)
     return (reinterpret_cast<uintptr_t>(a->a) & 15) == 0 && (reinterpret_cast<uintptr_t>(a->b) & 15) == 0;
 }
 
-extern "C" int rocm_launch_prefill_mfma(const RocmMatMulNBitsArgs* a, int tile_choice, rocm_stream_t stream)
+namespace {
+
+struct PrefillPlan {
+    int tile;        // 0: 128 x 128, 1: 256 x 128, 2: 256 x 256, 3: 128 x 64
+    int splits;      // slices of K (1 = none)
+    int steps_per_split;
+};
+
+// The largest tile that still gives every CU a workgroup: 256 x 256, then 256 x 128, 128 x 128, 128 x 64. If even the
+// smallest leaves CUs idle and K is long, K is cut into slices (at least 8 steps each) until the grid covers the chip.
+PrefillPlan plan_prefill(const RocmMatMulNBitsArgs* a, int tile_choice, uint64_t scratch_bytes)
+{
+    const int64_t wg_huge = ((a->m + 255) / 256) * ((a->n + 255) / 256);
+    const int64_t wg_big = ((a->m + 255) / 256) * ((a->n + 127) / 128);
+    const int64_t wg_small = ((a->m + 127) / 128) * ((a->n + 127) / 128);
+    PrefillPlan plan;
+    plan.tile = (a->m >= 256 && wg_huge >= 256) ? 2 : (a->m >= 256 && wg_big >= 256) ? 1 : wg_small >= 256 ? 0 : 3;
+    if (tile_choice >= 1 && tile_choice <= 4) plan.tile = tile_choice == 4 ? 3 : tile_choice - 1;
+    const int steps = static_cast<int>(a->k / 64);
+    plan.splits = 1;
+    if (plan.tile == 3) {
+        const int64_t wgs = ((a->m + 127) / 128) * ((a->n + 63) / 64);
+        int want = static_cast<int>((384 + wgs - 1) / wgs);
+        if (want > steps / 8) want = steps / 8;
+        if (want > 16) want = 16;
+        const uint64_t per_split = static_cast<uint64_t>(a->m) * static_cast<uint64_t>(a->n) * 4;
+        while (want > 1 && static_cast<uint64_t>(want) * per_split > scratch_bytes) --want;   // never more than the scratch holds
+        if (want > 1) plan.splits = want;
+    }
+    plan.steps_per_split = (steps + plan.splits - 1) / plan.splits;
+    plan.splits = (steps + plan.steps_per_split - 1) / plan.steps_per_split;
+    return plan;
+}
+
+}  // namespace
+
+extern "C" uint64_t rocm_prefill_mfma_scratch_bytes(const RocmMatMulNBitsArgs* a, int tile_choice)
+{
+    if (!rocm_prefill_mfma_eligible(a)) return 0;
+    const PrefillPlan plan = plan_prefill(a, tile_choice, ~0ull);
+    return plan.splits > 1 ? static_cast<uint64_t>(plan.splits) * static_cast<uint64_t>(a->m) * static_cast<uint64_t>(a->n) * 4 : 0;
+}
+
+extern "C" int rocm_launch_prefill_mfma(const RocmMatMulNBitsArgs* a, int tile_choice, void* scratch, uint64_t scratch_bytes, rocm_stream_t stream)
 {
     if (!rocm_prefill_mfma_eligible(a)) return -1;
     mnb::PrefillParams p;
@@ -335,24 +399,28 @@ extern "C" int rocm_launch_prefill_mfma(const RocmMatMulNBitsArgs* a, int tile_c
     p.scale_dtype = a->scale_dtype;
     p.bias_dtype = a->bias_dtype;
     p.y_dtype = a->y_dtype;
+    const PrefillPlan plan = plan_prefill(a, tile_choice, scratch ? scratch_bytes : 0);
+    p.steps_per_split = plan.steps_per_split;
+    p.partial = plan.splits > 1 ? static_cast<float*>(scratch) : nullptr;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool bf16 = a->a_dtype == ROCM_DT_BF16;
     const bool sf32 = a->scale_dtype == ROCM_DT_F32;
-    // The largest tile that still gives every CU a workgroup: 256 x 256, then 256 x 128, 128 x 128, 128 x 64.
-    const int64_t wg_huge = ((a->m + 255) / 256) * ((a->n + 255) / 256);
-    const int64_t wg_big = ((a->m + 255) / 256) * ((a->n + 127) / 128);
-    const int64_t wg_small = ((a->m + 127) / 128) * ((a->n + 127) / 128);
-    int tile = (a->m >= 256 && wg_huge >= 256) ? 2 : (a->m >= 256 && wg_big >= 256) ? 1 : wg_small >= 256 ? 0 : 3;
-    if (tile_choice >= 1 && tile_choice <= 4) tile = tile_choice == 4 ? 3 : tile_choice - 1;   // 1: 128 x 128, 2: 256 x 128, 3: 256 x 256, 4: 128 x 64
     auto go = [&](auto bf, auto sf) {
         constexpr bool B = decltype(bf)::value, S = decltype(sf)::value;
-        if (tile == 2) return mnb::launch_prefill<B, 256, 256, S>(p, s);
-        if (tile == 1) return mnb::launch_prefill<B, 256, 128, S>(p, s);
-        if (tile == 3) return mnb::launch_prefill<B, 128, 64, S>(p, s);
-        return mnb::launch_prefill<B, 128, 128, S>(p, s);
+        if (plan.tile == 2) return mnb::launch_prefill<B, 256, 256, S>(p, plan.splits, s);
+        if (plan.tile == 1) return mnb::launch_prefill<B, 256, 128, S>(p, plan.splits, s);
+        if (plan.tile == 3) return mnb::launch_prefill<B, 128, 64, S>(p, plan.splits, s);
+        return mnb::launch_prefill<B, 128, 128, S>(p, plan.splits, s);
     };
-    if (bf16 && sf32) return go(std::true_type{}, std::true_type{});
-    if (bf16) return go(std::true_type{}, std::false_type{});
-    if (sf32) return go(std::false_type{}, std::true_type{});
-    return go(std::false_type{}, std::false_type{});
+    int rc;
+    if (bf16 && sf32) rc = go(std::true_type{}, std::true_type{});
+    else if (bf16) rc = go(std::true_type{}, std::false_type{});
+    else if (sf32) rc = go(std::false_type{}, std::true_type{});
+    else rc = go(std::false_type{}, std::false_type{});
+    if (rc != 0 || plan.splits == 1) return rc;
+    int64_t blocks = (a->m * a->n + 255) / 256;
+    if (blocks > 16384) blocks = 16384;
+    hipLaunchKernelGGL(mnb::prefill_reduce_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, static_cast<const float*>(scratch), plan.splits,
+                       a->m, a->n, a->bias, a->bias_dtype, a->y, a->y_dtype);
+    return static_cast<int>(hipGetLastError());
 }
