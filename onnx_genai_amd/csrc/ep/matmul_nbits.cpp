@@ -328,7 +328,7 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
                 kn.variant = "acc4_gemv_dot4";
             }
         }
-    } else if (M <= 16 && use_packed(kn, args, rc)) {
+    } else if (M <= 64 && use_packed(kn, args, rc)) {
         if (rc == 0) rc = rocm_launch_decode_packed(&args, kn.packed, kn.ep->decode_waves, stream);
         kn.variant = "decode_mfma_packed";
     } else if (M <= 16 && rocm_decode_mfma_eligible(&args)) {

@@ -1,4 +1,4 @@
-// Decode path of MatMulNBits over weights repacked for streaming (f16/bf16 activations; M <= 4, or M <= 16 when N is large).
+// Decode path of MatMulNBits over weights repacked for streaming (f16/bf16 activations; M <= 4, or M <= 64 when N is large).
 //
 // When B, scales and zero points are constant initializers, the kernel object repacks them once into
 // the order in which the split-K MFMA kernel consumes them, so that every vector load of a wave is
@@ -17,6 +17,8 @@
 //
 // The copy costs one extra byte of device memory per byte of weights plus 2 to 6 % for the records; it is
 // read instead of the caller's tensors, which are not touched again.
+#include <type_traits>
+
 #include "mfma_common.hiph"
 
 namespace mnb {
@@ -316,33 +318,42 @@ static int launch_packed_bs(const PackedParams& p, int bs, int waves, bool singl
 }
 
 // ---------------------------------------------------------------------------------------------
-// The same stream for 5 <= M <= 16 and many columns: activations shared through LDS.
+// The same stream for 5 <= M <= 64 and many columns: activations shared through LDS.
 // ---------------------------------------------------------------------------------------------
 //
 // With several rows the activations outweigh a column group's weights (16 rows x 128 k x 2 bytes against 16 columns
 // x 64 bytes per tile), and a kernel in which every wave fetches its own copy is bound by L2, not HBM. Here a
 // workgroup of eight waves owns eight column groups - one wave each, streaming the whole of K - and all eight read
-// the activations from one LDS copy, filled window by window (512 k = one tile group, double buffered: the next
-// window travels global -> registers while the current one is multiplied, and moves registers -> LDS just before the
-// barrier that ends the window). No split-K, so no reduction: a wave stores its 16 columns itself. Weights are not
-// prefetched: the kernel is small enough (registers and 33 KB of LDS) for four workgroups per CU, and the other
-// resident waves cover a wave's memory latency better than a second register set does.
+// the activations from one LDS copy, filled window by window (double buffered: the next window travels global ->
+// registers while the current one is multiplied, and moves registers -> LDS just before the barrier that ends the
+// window). No split-K, so no reduction: a wave stores its 16 columns itself. Weights are not prefetched: the kernel is
+// small enough for several workgroups per CU, and the other resident waves cover a wave's memory latency better than
+// a second register set does. Up to 64 rows ride on one pass over the weights: RB blocks of 16 rows, each with its own
+// accumulators, share every unpacked weight operand - up to that height the call still costs what streaming the
+// weights costs, which the tiled kernel cannot offer below a few hundred rows.
 
-constexpr int kWinK = 512;                         // k per activation window: one tile group
-constexpr int kWinPitch = kWinK * 2 + 16;          // bytes per LDS row: 16 rows start in 16 different bank quads
 constexpr int kWideWaves = 8;
 
-template <bool BF16, int BS, typename ST>
-__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu((BS == 128 && sizeof(ST) == 2) ? 7 : 1))) void decode_wide_kernel(PackedParams p)
+// RB: blocks of 16 rows (1, 2 or 4). A window is WT tiles of 128 k: a whole tile group for RB <= 2, half of one for
+// RB = 4, so that two buffers of RB * 16 rows stay within 66 KB.
+template <bool BF16, int BS, typename ST, int RB>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu((BS == 128 && sizeof(ST) == 2 && RB == 1) ? 6 : 1)))
+void decode_wide_kernel(PackedParams p)
 {
     constexpr int U = kGroupTiles;
     constexpr int NBT = 128 / BS;
     constexpr int NB = U * NBT;
     constexpr int R = packed_record_bytes(BS, static_cast<int>(sizeof(ST)));
     constexpr int NR = R / 16;
-    constexpr int kBufBytes = 16 * kWinPitch;
+    constexpr int WT = RB == 4 ? 2 : 4;                 // tiles per window
+    constexpr int kWindowsPerGroup = U / WT;
+    constexpr int kPitch = WT * 256 + 16;               // bytes per LDS row: consecutive rows start in different bank quads
+    constexpr int kRows = RB * 16;
+    constexpr int kBufBytes = kRows * kPitch;
+    constexpr int kPieces = WT * 16;                    // 16-byte pieces per row of a window
+    constexpr int NW = kRows * kPieces / 512;           // pieces per thread per window (2 or 4)
     constexpr uint32_t kMagicNeg = BF16 ? 0xC300C300u : 0xE400E400u;
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];   // [2][16][kWinPitch]
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];   // [2][kRows][kPitch]
 
     const int t = threadIdx.x;
     const int lane = t & 63;
@@ -359,44 +370,50 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu((BS == 128 
 
     const uint32_t w_off = static_cast<uint32_t>(lane * 16);
     const uint32_t r_off = static_cast<uint32_t>(kChunkWeights + c * R);
-    // window fill: thread -> row t / 32, pieces t % 32 and t % 32 + 32 of the row's 64 pieces
-    const int wrow = t >> 5, wpiece = t & 31;
-    const uint32_t win_goff = static_cast<uint32_t>(wrow) * static_cast<uint32_t>(p.k) * 2u + static_cast<uint32_t>(wpiece * 16);
-    const uint32_t win_loff = static_cast<uint32_t>(wrow * kWinPitch + wpiece * 16);
-    // operand of MFMA j of tile x of the window: row c, elements x*128 + j*32 + g*8 .. +8
-    const uint32_t frag_off = static_cast<uint32_t>(c * kWinPitch + g * 16);
+    // operand of MFMA j of tile x of the window, row block rb: row rb*16 + c, elements x*128 + j*32 + g*8 .. +8
+    const uint32_t frag_off = static_cast<uint32_t>(c * kPitch + g * 16);
     const uint32_t mask = __builtin_amdgcn_mov_dpp(p.nibble_mask, 0xE4, 0xf, 0xf, false), magic = p.magic;
 
-    float4p_t y = {0.f, 0.f, 0.f, 0.f};
-    float4p_t acc = {0.f, 0.f, 0.f, 0.f};
+    float4p_t y[RB], acc[RB];
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+        y[rb] = float4p_t{0.f, 0.f, 0.f, 0.f};
+        acc[rb] = float4p_t{0.f, 0.f, 0.f, 0.f};
+    }
 
     struct Grp {
         uint4 w[kGroupTiles];
         uint4 r[NR];
     };
     auto fetch_group = [&](Grp& grp, int gi) {
-        if (gi >= p.groups) return;
         const uint32_t soff = static_cast<uint32_t>(gi) * static_cast<uint32_t>(p.chunk_bytes);
 #pragma unroll
         for (int u = 0; u < U; ++u) grp.w[u] = load16(srd_p, w_off + static_cast<uint32_t>(u * 1024), soff);
 #pragma unroll
         for (int i = 0; i < NR; ++i) grp.r[i] = load16(srd_p, r_off + static_cast<uint32_t>(i * 16), soff);
     };
-    uint4 wa[2];
+    // window fill: piece q = t + 512 i of the window's kRows * kPieces pieces -> (row q / kPieces, piece q % kPieces)
+    uint4 wa[NW];
     auto load_window = [&](int win) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const int64_t k0 = static_cast<int64_t>(win) * kWinK + (wpiece + 32 * i) * 8;
-            uint32_t off = win_goff + static_cast<uint32_t>(i * 512);
-            if (wrow >= p.m || k0 >= p.k) off = kOutOfRange;      // K is a multiple of 8: a piece is all inside or all outside
-            wa[i] = load16(srd_a, off, static_cast<uint32_t>(win) * (kWinK * 2u));
+        for (int i = 0; i < NW; ++i) {
+            const int q = t + 512 * i;
+            const int row = q / kPieces, piece = q % kPieces;
+            const int64_t k0 = static_cast<int64_t>(win) * (WT * 128) + piece * 8;
+            uint32_t off = static_cast<uint32_t>(row) * static_cast<uint32_t>(p.k) * 2u + static_cast<uint32_t>(piece * 16);
+            if (row >= p.m || k0 >= p.k) off = kOutOfRange;       // K is a multiple of 8: a piece is all inside or all outside
+            wa[i] = load16(srd_a, off, static_cast<uint32_t>(win) * (WT * 256u));
         }
     };
     auto store_window = [&](int buf) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) *reinterpret_cast<uint4*>(smem + buf * kBufBytes + win_loff + i * 512) = wa[i];
+        for (int i = 0; i < NW; ++i) {
+            const int q = t + 512 * i;
+            *reinterpret_cast<uint4*>(smem + buf * kBufBytes + (q / kPieces) * kPitch + (q % kPieces) * 16) = wa[i];
+        }
     };
-    auto compute_group = [&](const Grp& grp, int buf) {
+    // tiles [first, first + WT) of the group against window buffer `buf`
+    auto compute_window = [&](const Grp& grp, int buf, int first) {
         uint32_t rr[NR * 4];
 #pragma unroll
         for (int i = 0; i < NR; ++i) {
@@ -406,11 +423,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu((BS == 128 
             rr[4 * i + 3] = grp.r[i].w;
         }
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const unsigned char* fa = smem + buf * kBufBytes + frag_off + u * 256;
-            uint4 av[4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) av[j] = *reinterpret_cast<const uint4*>(fa + j * 64);
+        for (int x = 0; x < WT; ++x) {
+            const int u = first + x;                               // tile of the group (compile-time after unrolling)
+            const unsigned char* fa = smem + buf * kBufBytes + frag_off + x * 256;
             const uint32_t wd[4] = {grp.w[u].x, grp.w[u].y, grp.w[u].z, grp.w[u].w};
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
@@ -425,37 +440,49 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu((BS == 128 
                 op.y = ((w >> 4) & mask) | magic;
                 op.z = ((w >> 8) & mask) | magic;
                 op.w = ((w >> 12) & mask) | magic;
-                acc = mfma16p<BF16>(av[j], op, acc);
-                acc = mfma16p<BF16>(av[j], zc, acc);
-                if (((j + 1) * 32) % BS == 0 || j == 3) {
-                    float sf;
+                const bool last = ((j + 1) * 32) % BS == 0 || j == 3;
+                float sf = 0.f;
+                if (last) {
                     if constexpr (sizeof(ST) == 4) {
                         sf = __uint_as_float(rr[bi]);
                     } else {
                         const uint32_t raw = (rr[bi / 2] >> ((bi % 2) * 16)) & 0xffffu;
                         sf = BF16 ? __uint_as_float(raw << 16) : f16_bits_to_f32(static_cast<uint16_t>(raw));
                     }
+                }
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        y[r] = fmaf(sf, acc[r], y[r]);
-                        acc[r] = 0.f;
+                for (int rb = 0; rb < RB; ++rb) {
+                    const uint4 av = *reinterpret_cast<const uint4*>(fa + rb * 16 * kPitch + j * 64);
+                    acc[rb] = mfma16p<BF16>(av, op, acc[rb]);
+                    acc[rb] = mfma16p<BF16>(av, zc, acc[rb]);
+                    if (last) {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            y[rb][r] = fmaf(sf, acc[rb][r], y[rb][r]);
+                            acc[rb][r] = 0.f;
+                        }
                     }
                 }
             }
         }
     };
 
+    const int windows = p.groups * kWindowsPerGroup;
     Grp ga;
     load_window(0);
     store_window(0);
     __syncthreads();
     for (int gi = 0; gi < p.groups; ++gi) {
-        const int buf = gi & 1;
-        if (gi + 1 < p.groups) load_window(gi + 1);
         fetch_group(ga, gi);
-        compute_group(ga, buf);
-        if (gi + 1 < p.groups) store_window(buf ^ 1);
-        __syncthreads();
+#pragma unroll
+        for (int h = 0; h < kWindowsPerGroup; ++h) {
+            const int win = gi * kWindowsPerGroup + h;
+            const int buf = win & 1;
+            if (win + 1 < windows) load_window(win + 1);
+            compute_window(ga, buf, h * WT);
+            if (win + 1 < windows) store_window(buf ^ 1);
+            __syncthreads();
+        }
     }
 
     if (active) {
@@ -463,9 +490,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu((BS == 128 
         if (col < p.n) {
             const float bias = p.bias ? load_as_f32(p.bias, p.bias_dtype, col) : 0.f;
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int row = 4 * g + r;
-                if (row < p.m) store_from_f32(p.y, p.y_dtype, static_cast<int64_t>(row) * p.n + col, y[r] + bias);
+            for (int rb = 0; rb < RB; ++rb) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int row = rb * 16 + 4 * g + r;
+                    if (row < p.m) store_from_f32(p.y, p.y_dtype, static_cast<int64_t>(row) * p.n + col, y[rb][r] + bias);
+                }
             }
         }
     }
@@ -476,8 +506,7 @@ static int launch_wide_bs(const PackedParams& p, int bs, hipStream_t stream)
 {
     const int64_t col_groups = (p.n + 15) / 16;
     const dim3 grid(static_cast<unsigned>((col_groups + kWideWaves - 1) / kWideWaves));
-    const size_t lds = 2 * 16 * kWinPitch;
-    auto go = [&](auto kernel) {
+    auto go = [&](auto kernel, size_t lds) {
         if (lds > 65536) {
             const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
             if (e != hipSuccess) return static_cast<int>(e);
@@ -485,10 +514,17 @@ static int launch_wide_bs(const PackedParams& p, int bs, hipStream_t stream)
         hipLaunchKernelGGL(kernel, grid, dim3(kWideWaves * 64), lds, stream, p);
         return static_cast<int>(hipGetLastError());
     };
+    auto by_rows = [&](auto bs_tag) {
+        constexpr int BS = decltype(bs_tag)::value;
+        if (p.m <= 16) return go(decode_wide_kernel<BF16, BS, ST, 1>, 2 * 16 * (4 * 256 + 16));
+        if (p.m <= 32) return go(decode_wide_kernel<BF16, BS, ST, 2>, 2 * 32 * (4 * 256 + 16));
+        if constexpr (BS == 32) return -1;
+        else return go(decode_wide_kernel<BF16, BS, ST, 4>, 2 * 64 * (2 * 256 + 16));
+    };
     switch (bs) {
-        case 32: return go(decode_wide_kernel<BF16, 32, ST>);
-        case 64: return go(decode_wide_kernel<BF16, 64, ST>);
-        default: return go(decode_wide_kernel<BF16, 128, ST>);
+        case 32: return by_rows(std::integral_constant<int, 32>{});
+        case 64: return by_rows(std::integral_constant<int, 64>{});
+        default: return by_rows(std::integral_constant<int, 128>{});
     }
 }
 
@@ -678,12 +714,16 @@ static int packed_chunk_bytes(const RocmMatMulNBitsArgs* a)
 
 }  // namespace mnb
 
-// Rows 5..16 only run from the repacked copy in the shared-activation kernel, which wants many column groups.
-static bool wide_shape(const RocmMatMulNBitsArgs* a) { return a->m >= 5 && a->n >= 16384; }
+// Rows 5..64 only run from the repacked copy in the shared-activation kernel, which wants many column groups.
+// (block size 32 stops at 32 rows: four row blocks of it do not fit the register file)
+static bool wide_shape(const RocmMatMulNBitsArgs* a) { return a->m >= 5 && a->m <= (a->block_size == 32 ? 32 : 64) && a->n >= 16384; }
 
 extern "C" int rocm_decode_packed_eligible(const RocmMatMulNBitsArgs* a)
 {
-    if (!rocm_decode_mfma_eligible(a)) return 0;
+    RocmMatMulNBitsArgs base = *a;
+    if (base.m > 16) base.m = 16;                         // the shared-activation kernel takes up to 64 rows
+    if (!rocm_decode_mfma_eligible(&base)) return 0;
+    if (a->m * a->k * 2 >= 0x7ffffff0) return 0;
     if (a->m > 4 && !wide_shape(a)) return 0;
     return static_cast<int64_t>(mnb::packed_groups(a)) * mnb::packed_chunk_bytes(a) < 0x7fffffff;
 }
