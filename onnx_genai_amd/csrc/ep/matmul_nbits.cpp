@@ -184,6 +184,35 @@ bool use_packed(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& args, int& r
     return true;
 }
 
+// 17..32 rows as two blocks of at most 16 through the decode kernels. The tiled kernel needs a few hundred rows to
+// pay for itself; below that a call costs what streaming the weights costs, and two streams are still cheaper than
+// one under-filled tiled launch (measured at the 7B shapes: 19.8 against 22.6 us, 38 against 55 us; three are not). Returns false (nothing launched) when the decode kernels do not take the shape.
+bool decode_in_row_blocks(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& args, int& rc)
+{
+    rc = 0;
+    RocmMatMulNBitsArgs probe = args;
+    probe.m = 16;
+    if (!rocm_decode_mfma_eligible(&probe)) return false;
+    const size_t a_elem = 2;                                            // eligibility means f16 / bf16 activations
+    const size_t y_elem = args.y_dtype == ROCM_DT_F32 ? 4 : 2;
+    bool all_packed = true;
+    for (int64_t row0 = 0; row0 < args.m && rc == 0; row0 += 16) {
+        RocmMatMulNBitsArgs part = args;
+        part.m = args.m - row0 < 16 ? args.m - row0 : 16;
+        part.a = static_cast<const uint8_t*>(args.a) + static_cast<size_t>(row0) * static_cast<size_t>(args.k) * a_elem;
+        part.y = static_cast<uint8_t*>(args.y) + static_cast<size_t>(row0) * static_cast<size_t>(args.n) * y_elem;
+        int pack_rc = 0;
+        if (use_packed(kn, part, pack_rc)) {
+            rc = pack_rc != 0 ? pack_rc : rocm_launch_decode_packed(&part, kn.packed, kn.ep->decode_waves, kn.ep->stream);
+        } else {
+            all_packed = false;
+            rc = rocm_launch_decode_mfma(&part, kn.ep->decode_waves, kn.ep->decode_col_groups, kn.ep->stream);
+        }
+    }
+    kn.variant = all_packed ? "decode_mfma_packed" : "decode_mfma_splitk";
+    return true;
+}
+
 NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, uint32_t n_in, NxrtRocmTensorView* out, uint32_t n_out,
                         void* workspace, uint64_t workspace_bytes)
 {
@@ -334,6 +363,8 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
     } else if (M <= 16 && rocm_decode_mfma_eligible(&args)) {
         rc = rocm_launch_decode_mfma(&args, kn.ep->decode_waves, kn.ep->decode_col_groups, stream);
         kn.variant = "decode_mfma_splitk";
+    } else if (M <= 32 && decode_in_row_blocks(kn, args, rc)) {
+        // done: a few passes of the streaming kernels beat one pass of the tiled kernel at these heights
     } else if (M > 16 && rocm_prefill_mfma_eligible(&args)) {
         // Small grids slice K and want scratch for the partial sums: the caller's workspace if it is large enough, else
         // the kernel's own (grown outside a capture only; with too little the launcher slices less or not at all).

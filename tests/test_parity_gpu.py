@@ -194,7 +194,8 @@ def test_decode_matches_oracle(ep, ep_unpacked, port, prepack, a_dt, s_dt, bs, z
     if m <= 16:
         assert variant == ("decode_mfma_packed" if prepack and (m <= 4 or n >= 16384) else "decode_mfma_splitk")   # m 2..4 at large n: the 4-row kernel
     else:
-        assert variant == ("decode_mfma_packed" if prepack else "prefill_mfma_lds" if k % 64 == 0 else "gemv_generic_f32")
+        unpacked = "decode_mfma_splitk" if m <= 32 else "prefill_mfma_lds" if k % 64 == 0 else "gemv_generic_f32"   # m <= 32: two row blocks
+        assert variant == ("decode_mfma_packed" if prepack else unpacked)
     # The kernel carries each weight as (2^10 + q) in f16 or (2^7 + q) in bf16 and cancels the offset inside the
     # f32 accumulator, which costs 10 (7) of its 24 bits: a few 1e-5 on outputs that themselves cancel.
     # (The tiled kernel, which serves these row counts when nothing is repacked, rounds weights to 16 bits in LDS.)
@@ -238,6 +239,23 @@ def test_packed_decode_wave_counts_agree(port, waves):
             assert helpers.rel_l2(y32, oracle_f64(port, a, a_dt, b, s, a_dt, zp, n, k, bs)) <= 2e-5
     finally:
         provider.shutdown()
+
+
+@pytest.mark.parametrize("prepack", [True, False])
+@pytest.mark.parametrize("m", [17, 25, 32])
+def test_row_blocks_through_the_decode_kernels(ep, ep_unpacked, port, prepack, m):
+    """17..32 rows at a shape without many columns: a block of 16 rows and a remainder through the decode kernels."""
+    ep = ep if prepack else ep_unpacked
+    a_dt, bs, n, k = E.BF16, 128, 300, 1024
+    b, s, zp = synth.make_weights(n, k, bs, 55, zero_points=True, scale_lo=0.002, scale_hi=0.01, scale_dtype=a_dt)
+    a = synth.make_activation(m, k, 55 + m, a_dt)
+    bias = synth.to_dtype(np.linspace(-2, 2, n).astype(np.float32), a_dt)
+    y32, variant = run_op(ep, a, a_dt, b, s, a_dt, zp, n, k, bs, bias=bias, bias_dtype=a_dt, y_dtype=E.F32)
+    # with the repacked copy, blocks of more than 4 rows still stream the caller's layout at this width
+    assert variant == "decode_mfma_splitk"
+    assert helpers.rel_l2(y32, oracle_f64(port, a, a_dt, b, s, a_dt, zp, n, k, bs, bias, a_dt)) <= 1e-4
+    y, _ = run_op(ep, a, a_dt, b, s, a_dt, zp, n, k, bs, bias=bias, bias_dtype=a_dt)
+    assert np.array_equal(np.asarray(y).view(np.uint16), np.asarray(port.narrow(y32, a_dt)).view(np.uint16))
 
 
 def test_packed_copy_follows_the_weights(ep, port):
@@ -300,6 +318,8 @@ PREFILL_CASES = [
     (E.BF16, E.BF16, 128, True, 257, 384, 3584),
     (E.BF16, E.BF16, 32, False, 33, 100, 128),
     (E.BF16, E.F32, 64, True, 1030, 128, 512),
+    (E.F16, E.F16, 64, True, 49, 128, 64),
+    (E.BF16, E.BF16, 32, False, 60, 100, 128),
 ]
 
 
@@ -310,7 +330,7 @@ def test_prefill_matches_oracle(ep, port, a_dt, s_dt, bs, zero_points, m, n, k):
     bias = synth.to_dtype(np.random.default_rng(n).standard_normal(n).astype(np.float32), a_dt)
     want64 = oracle_f64(port, a, a_dt, b, s, s_dt, zp, n, k, bs, bias, a_dt)
     y32, variant = run_op(ep, a, a_dt, b, s, s_dt, zp, n, k, bs, bias=bias, bias_dtype=a_dt, y_dtype=E.F32)
-    assert variant == "prefill_mfma_lds"
+    assert variant == "prefill_mfma_lds" if m > 32 else variant.startswith("decode_mfma")    # up to 32 rows: row blocks through the decode kernels
     assert helpers.rel_l2(y32, want64) <= TOL_HALF
     y, _ = run_op(ep, a, a_dt, b, s, s_dt, zp, n, k, bs, bias=bias, bias_dtype=a_dt)
     assert helpers.rel_l2(synth.to_f32(y, a_dt), want64) <= TOL_HALF
