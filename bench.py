@@ -123,6 +123,45 @@ def build_decode_stack(ep, m, layers):
     return nodes, a_bufs
 
 
+def small_model_step(ep):
+    """configs[1]: the decode step of a Qwen2.5-0.5B-architecture stack (24 layers of q, k, v, o, gate, up, down plus
+    lm_head; fp16, M=1, block 32, zero points), replayed as one HIP graph. Reported beside the headline workload."""
+    hidden, inter, vocab, layers, kv = 896, 4864, 151936, 24, 128
+    shapes = [("q", hidden, hidden), ("k", hidden, kv), ("v", hidden, kv), ("o", hidden, hidden),
+              ("gate", hidden, inter), ("up", hidden, inter), ("down", inter, hidden)]
+    a_bufs = {k: ep.upload(synth.make_activation(1, k, 6, E.F16)) for k in (hidden, inter)}
+    nodes, reuse = [], {}
+    for layer in range(layers):
+        for name, k, n in shapes:
+            node = Node(ep, f"{name}.{layer}", k, n, 32, 7000 + 10 * layer + len(nodes), E.F16, 1, reuse=reuse.get((k, n)))
+            reuse.setdefault((k, n), node.host_b)
+            node.host_b = None
+            nodes.append(node)
+    nodes.append(Node(ep, "lm_head", hidden, vocab, 32, 98, E.F16, 1))
+    nodes[-1].host_b = None
+
+    def one_step():
+        for node in nodes:
+            node.run(a_bufs[node.k])
+
+    one_step()
+    ep.sync()
+    graph = capture(ep, one_step)
+    ms = time_graph(ep, graph, 20, 3)
+    graph.release()
+    step_bytes = sum(n.bytes for n in nodes)
+    out = {"workload": "Qwen2.5-0.5B decode-step MatMulNBits sweep (configs[1]): 24 layers x (q, k, v, o, gate, up, down) + lm_head, M=1, fp16, "
+                       "block_size 32, zero points; %d calls per step" % len(nodes),
+           "ms_per_step": round(ms, 4), "bytes_per_step": step_bytes, "gbs": round(step_bytes / (ms * 1e-3) / 1e9, 1),
+           "hbm_frac": round(step_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "us_per_call": round(ms * 1e3 / len(nodes), 2),
+           "kernel_variants": sorted({n.ops.kernel.last_variant() for n in nodes})}
+    for node in nodes:
+        node.free(ep)
+    for buf in a_bufs.values():
+        ep.deallocate(buf)
+    return out
+
+
 def cpu_baseline(seconds_budget=20.0, threads=None):
     """The reference's CPU path (vendored MLAS through its plain-C shim, oracle/_ref) on this host, on a bounded
     sample of the workload: the gate/up projection (3584 -> 37888), bf16 activations widened to f32 before and
@@ -288,6 +327,7 @@ def main():
     if not args.no_sweep:
         result["prefill"] = prefill_table(ep)
         result["acc4"] = acc4_table(ep)
+        result["small_model_step"] = small_model_step(ep)
     ep.shutdown()
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(args.cpu_seconds)
