@@ -2,6 +2,7 @@
 // Attribute parsing, input validation and their messages follow the reference's CPU kernel
 // (crates/onnx-runtime-ep-cpu/src/kernels/matmul_nbits.rs:1410-1600, helpers at :10254-10378);
 // the contiguity rule follows its CUDA sibling (crates/onnx-runtime-ep-cuda/src/kernels/matmul_nbits.rs:7089-7106).
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -125,6 +126,7 @@ struct NxrtRocmMatMulNBits {
     void* packed = nullptr;              // constant B / scales / zero points in the decode kernel's streaming order
     const void* packed_from[3] = {nullptr, nullptr, nullptr};   // the tensors `packed` was made from
     int packed_scale_dtype = 0;
+    std::mutex mu;                       // one execute at a time per kernel object: scratch, repacked copy and variant are per-object state
     NxrtKernelVtable vtable;
     uint32_t vt_a_dtype = 0, vt_scale_dtype = 0, vt_y_dtype = 0;
 
@@ -216,6 +218,7 @@ bool decode_in_row_blocks(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& ar
 NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, uint32_t n_in, NxrtRocmTensorView* out, uint32_t n_out,
                         void* workspace, uint64_t workspace_bytes)
 {
+    std::lock_guard<std::mutex> lock(kn.mu);
     // kernels/mod.rs:1898-1919 (check_arity)
     if (n_in < 3 || n_in > 6) return make_status(NXRT_INVALID_ARGUMENT, "MatMulNBits: expected 3..=6 inputs, got " + std::to_string(n_in));
     if (n_out < 1) return make_status(NXRT_INVALID_ARGUMENT, "MatMulNBits: expected at least 1 output(s), got " + std::to_string(n_out));

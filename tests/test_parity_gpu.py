@@ -661,6 +661,43 @@ def test_kernel_vtable_execute(ep, port):
     ops.free()
 
 
+def test_concurrent_execute_on_one_kernel(ep, port):
+    """Two host threads drive the same kernel object (the plugin contract asks for thread-safe vtables): every call
+    must see consistent per-object state (repacked copy, scratch) and produce its own result."""
+    import threading
+    a_dt, bs, n, k = E.F16, 64, 160, 1024
+    b, s, zp = synth.make_weights(n, k, bs, 71, zero_points=True, scale_lo=0.002, scale_hi=0.01, scale_dtype=a_dt)
+    ops = E.DeviceOperands(ep, b, s, a_dt, zp, n, k, bs, accuracy_level=4)
+    jobs = []
+    for i, m in enumerate((1, 3, 20, 1, 40, 2)):
+        a = synth.make_activation(m, k, 700 + i, a_dt)
+        jobs.append((m, a, ep.upload(a), ep.allocate(m * n * 4)))
+    errors = []
+
+    def work(part):
+        try:
+            for _ in range(10):
+                for m, _, ab, yb in part:
+                    ops.run(ab, a_dt, m, yb, E.F32)
+        except Exception as exc:                                   # noqa: BLE001 - reported below
+            errors.append(exc)
+
+    threads = [threading.Thread(target=work, args=(jobs[i::2],)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    ep.sync()
+    assert not errors, errors
+    for m, a, ab, yb in jobs:
+        got = ep.download(yb, (m, n), np.float32)
+        want = port.matmul_acc4_f32(synth.to_f32(a, a_dt), b, synth.to_f32(s, a_dt), zp, n, k, bs, oracle.ROUND_HALF_EVEN)
+        assert helpers.rel_l2(got, want) <= TOL_F32
+        ep.deallocate(ab)
+        ep.deallocate(yb)
+    ops.free()
+
+
 def test_launch_counter_proves_native_path(ep):
     before = ep.kernel_launch_count()
     test_low_nibble_before_high_nibble(ep)
