@@ -661,6 +661,41 @@ def test_kernel_vtable_execute(ep, port):
     ops.free()
 
 
+def _random_cases(count, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for _ in range(count):
+        bs = int(rng.choice([16, 32, 64, 128, 256]))
+        a_dt = int(rng.choice([E.F32, E.F16, E.BF16]))
+        s_dt = a_dt if rng.random() < 0.7 else E.F32
+        m = int(rng.choice([1, 2, 3, 4, 5, 8, 13, 16, 17, 24, 32, 33, 50, 64, 65, 130, 300]))
+        n = int(rng.integers(1, 700)) if rng.random() < 0.8 else int(rng.integers(16384, 17000))
+        blocks = int(rng.integers(1, 40))
+        k = blocks * bs - (int(rng.integers(0, bs // 8)) * 8 if rng.random() < 0.3 else 0)
+        acc = 4 if rng.random() < 0.35 else 0
+        cases.append((a_dt, s_dt, bs, bool(rng.random() < 0.6), m, n, max(k, 8), acc, bool(rng.random() < 0.5)))
+    return cases
+
+
+@pytest.mark.parametrize("a_dt,s_dt,bs,zero_points,m,n,k,acc,with_bias", _random_cases(60, 20260101))
+def test_random_shapes_against_oracle(ep, port, a_dt, s_dt, bs, zero_points, m, n, k, acc, with_bias):
+    """Seeded random shapes over every dispatch path (whatever kernel the shape lands on) against the CPU oracle."""
+    b, s, zp = synth.make_weights(n, k, bs, 900 + n + k, zero_points=zero_points, scale_lo=0.002, scale_hi=0.01, scale_dtype=s_dt)
+    a = synth.make_activation(m, k, 900 + m, a_dt)
+    bias = synth.to_dtype(np.random.default_rng(n).standard_normal(n).astype(np.float32), a_dt) if with_bias else None
+    y32, variant = run_op(ep, a, a_dt, b, s, s_dt, zp, n, k, bs, accuracy_level=acc, bias=bias, bias_dtype=a_dt, y_dtype=E.F32)
+    af, sf = synth.to_f32(a, a_dt), synth.to_f32(s, s_dt)
+    bf = None if bias is None else synth.to_f32(bias, a_dt)
+    if acc == 4:
+        want = port.matmul_acc4_f32(af, b, sf, zp, n, k, bs, oracle.ROUND_HALF_EVEN, bias=bf)
+        assert variant.startswith("acc4_")
+        assert helpers.rel_l2(y32, want) <= TOL_F32, variant
+    else:
+        want = port.matmul_f64(af, b, sf, zp, n, k, bs, bias=bf)
+        tol = TOL_F32 if a_dt == E.F32 else TOL_HALF
+        assert helpers.rel_l2(y32, want) <= tol, variant
+
+
 def test_concurrent_execute_on_one_kernel(ep, port):
     """Two host threads drive the same kernel object (the plugin contract asks for thread-safe vtables): every call
     must see consistent per-object state (repacked copy, scratch) and produce its own result."""
