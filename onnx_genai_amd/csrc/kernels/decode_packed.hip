@@ -128,7 +128,8 @@ struct PackedGroup {
 // 3584 -> 37888: 15.6 us against 17.0 us). With two sets the one-row, block-128, 16-bit-scale variant fits 96
 // registers without spilling (a fifth wave per SIMD); the other variants keep the compiler's own choice.
 template <bool BF16, int BS, int MR, typename ST, int SETS>
-__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu((BS == 128 && MR == 1 && sizeof(ST) == 2) ? (SETS == 1 ? 8 : 5) : 1)))
+__global__ __launch_bounds__((BS == 128 && sizeof(ST) == 2) ? 1024 : 512)   // block 128, 16-bit scales: up to 16 waves split a long K
+__attribute__((amdgpu_waves_per_eu((BS == 128 && MR == 1 && sizeof(ST) == 2) ? (SETS == 1 ? 8 : 5) : 1)))
 void decode_packed_kernel(PackedParams p)
 {
     constexpr int U = kGroupTiles;
@@ -800,7 +801,8 @@ extern "C" int rocm_launch_decode_packed(const RocmMatMulNBitsArgs* a, const voi
     } else {
         single_set = wgs * w >= 6144;
     }
-    if (w > 8) w = 8;
+    const int w_max = (a->block_size == 128 && !f32_scales) ? 16 : 8;      // see the kernel's launch bounds
+    if (w > w_max) w = w_max;
     if (w > p.groups) w = p.groups;
     const int gpw = (p.groups + w - 1) / w;
     w = (p.groups + gpw - 1) / gpw;
