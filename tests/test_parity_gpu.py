@@ -6,6 +6,8 @@ Bars (from the parity contract of this build):
   * outputs, f32 activations ................... rel-L2 <= 1e-5
   * outputs, f16/bf16 activations .............. rel-L2 <= 5e-3
 """
+import os
+
 import numpy as np
 import pytest
 
@@ -731,6 +733,18 @@ def test_concurrent_execute_on_one_kernel(ep, port):
         ep.deallocate(ab)
         ep.deallocate(yb)
     ops.free()
+
+
+def test_plain_c_host_roundtrip():
+    """tests/harness/nxrt_roundtrip.c: a host in plain C loads the library the way the reference's loader does, runs
+    MatMulNBits through the plugin allocator and the kernel mirror, and checks the result itself."""
+    import subprocess
+    here = os.path.dirname(os.path.abspath(__file__))
+    exe = os.path.join(here, "harness", "nxrt_roundtrip")
+    assert os.path.exists(exe), "tests/harness/nxrt_roundtrip is built by __graft_entry__.build()"
+    run = subprocess.run([exe, E.LIB_PATH], capture_output=True, text=True, timeout=100)
+    assert run.returncode == 0, run.stdout + run.stderr
+    assert "roundtrip ok" in run.stdout and "accuracy_level 4" in run.stdout
 
 
 def test_launch_counter_proves_native_path(ep):
