@@ -215,6 +215,26 @@ bool decode_in_row_blocks(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& ar
     return true;
 }
 
+// f32 activations: passes of up to four rows through the f32 streaming kernel. Returns false (nothing launched) when
+// that kernel does not take the shape.
+bool f32_in_row_blocks(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& args, int& rc)
+{
+    rc = 0;
+    RocmMatMulNBitsArgs probe = args;
+    probe.m = 1;
+    if (!rocm_gemv_f32_eligible(&probe)) return false;
+    const size_t y_elem = args.y_dtype == ROCM_DT_F32 ? 4 : 2;
+    for (int64_t row0 = 0; row0 < args.m && rc == 0; row0 += 4) {
+        RocmMatMulNBitsArgs part = args;
+        part.m = args.m - row0 < 4 ? args.m - row0 : 4;
+        part.a = static_cast<const uint8_t*>(args.a) + static_cast<size_t>(row0) * static_cast<size_t>(args.k) * 4;
+        part.y = static_cast<uint8_t*>(args.y) + static_cast<size_t>(row0) * static_cast<size_t>(args.n) * y_elem;
+        rc = rocm_launch_gemv_f32(&part, kn.ep->stream);
+    }
+    kn.variant = "gemv_f32_valu";
+    return true;
+}
+
 NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, uint32_t n_in, NxrtRocmTensorView* out, uint32_t n_out,
                         void* workspace, uint64_t workspace_bytes)
 {
@@ -392,6 +412,8 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
         }
         rc = rocm_launch_prefill_mfma(&args, kn.ep->prefill_tile, scratch, scratch_bytes, stream);
         kn.variant = "prefill_mfma_lds";
+    } else if (M <= 64 && f32_in_row_blocks(kn, args, rc)) {
+        // done: f32 activations stay in f32 arithmetic end to end
     } else {
         rc = rocm_launch_gemv_generic(&args, stream);
         kn.variant = "gemv_generic_f32";

@@ -64,6 +64,9 @@ int rocm_launch_dequant_f32(const uint8_t* b, const void* scales, int scale_dtyp
 
 /* Any dtype mix, any K, any block size: f32 math, one wave per output column. */
 int rocm_launch_gemv_generic(const RocmMatMulNBitsArgs* args, rocm_stream_t stream);
+/* f32 activations, M <= 4, block size >= 32, K % 4 == 0, A and B 16-byte aligned: f32 FMA streaming kernel */
+int rocm_gemv_f32_eligible(const RocmMatMulNBitsArgs* args);
+int rocm_launch_gemv_f32(const RocmMatMulNBitsArgs* args, rocm_stream_t stream);
 
 /* Decode (M <= 16), f16/bf16 activations: split-K MFMA GEMV. Returns -1 when the shape is not eligible.
  * waves/col_groups = 0 lets the launcher choose. */

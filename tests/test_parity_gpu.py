@@ -104,14 +104,14 @@ def test_accuracy_envelope_against_f64(ep, port):
 
 
 # ---------------------------------------------------------------------------------------------
-# f32 activations (generic kernel): rel-L2 <= 1e-5
+# f32 activations (f32 FMA streaming kernel; the scalar catch-all below block size 32 or odd K): rel-L2 <= 1e-5
 # ---------------------------------------------------------------------------------------------
 def test_config1_qwen_mlp_shape_f32(ep, port, ref):
     m, k, n, bs = 1, 896, 4864, 32
     b, s, _ = synth.make_weights(n, k, bs, 1, zero_points=False, scale_lo=0.005, scale_hi=0.02, scale_dtype=E.F32)
     a = synth.make_activation(m, k, 1, E.F32, dist="uniform")
     y, variant = run_op(ep, a, E.F32, b, s, E.F32, None, n, k, bs)
-    assert variant == "gemv_generic_f32"
+    assert variant == "gemv_f32_valu"
     want = port.matmul_f64(a, b, s, None, n, k, bs)
     assert helpers.rel_l2(y, want) <= TOL_F32
     y_ref = ref.matmul(a, b, s, None, n, k, bs, ref.COMP_FP32)
@@ -142,6 +142,34 @@ def test_ragged_k_f32(ep, port, k, bs):
     a = synth.make_activation(m, k, 3, E.F32)
     y, _ = run_op(ep, a, E.F32, b, s, E.F32, zp, n, k, bs)
     assert helpers.rel_l2(y, port.matmul_f64(a, b, s, zp, n, k, bs)) <= TOL_F32
+
+
+F32_CASES = [
+    # s_dt, bs, zp, m, n, k      (K windows of 2048, steps of 512: whole, ragged and multi-window spans)
+    (E.F32, 32, True, 1, 896, 896),
+    (E.F32, 32, False, 2, 33, 4096),
+    (E.F32, 64, True, 3, 100, 4100),
+    (E.F32, 128, True, 4, 257, 8192),
+    (E.F16, 128, True, 1, 64, 18944),
+    (E.BF16, 64, False, 5, 31, 1000),
+    (E.F32, 32, True, 9, 65, 516),
+    (E.F32, 256, True, 1, 40, 3584),
+    (E.F32, 128, True, 64, 32, 640),
+    (E.F32, 32, True, 65, 16, 512),       # beyond 64 rows: the catch-all
+    (E.F32, 16, True, 1, 48, 512),        # block size 16: the catch-all
+    (E.F32, 32, True, 1, 48, 130),        # K % 4 != 0: the catch-all
+]
+
+
+@pytest.mark.parametrize("s_dt,bs,zero_points,m,n,k", F32_CASES)
+def test_f32_activations_match_oracle(ep, port, s_dt, bs, zero_points, m, n, k):
+    b, s, zp = synth.make_weights(n, k, bs, 7 + n + k, zero_points=zero_points, scale_lo=0.002, scale_hi=0.01, scale_dtype=s_dt)
+    a = synth.make_activation(m, k, n, E.F32)
+    bias = np.random.default_rng(n).standard_normal(n).astype(np.float32)
+    y, variant = run_op(ep, a, E.F32, b, s, s_dt, zp, n, k, bs, bias=bias)
+    assert variant == ("gemv_f32_valu" if m <= 64 and bs >= 32 and k % 4 == 0 else "gemv_generic_f32")
+    want = oracle_f64(port, a, E.F32, b, s, s_dt, zp, n, k, bs, bias, E.F32)
+    assert helpers.rel_l2(y, want) <= TOL_F32
 
 
 # ---------------------------------------------------------------------------------------------
