@@ -18,6 +18,7 @@ namespace mnb {
 
 typedef __attribute__((ext_vector_type(4))) int int4_t;
 typedef __attribute__((ext_vector_type(16))) int int16_t_v;
+typedef __attribute__((ext_vector_type(32))) float float32_v;
 
 __device__ __forceinline__ long pack64(uint32_t lo, uint32_t hi)
 {
@@ -420,17 +421,22 @@ __global__ __launch_bounds__(512) void acc4_prefill_kernel(Acc4PrefillParams p)
             if (sa_slot < kSlots) *reinterpret_cast<uint32_t*>(base + kSaOff + t * 4) = r.sa;
         }
     };
-    // y[j] += f32(tile) * (scale_a[row] * scale_b[column]) for one 32x32 tile and the block in scale slot `slot`.
-    auto flush_tile = [&](const int16_t_v& tile, int buf, int slot, int j) {
+    // The products scale_a[row] * scale_b[column] of the wave's two 32x32 tiles for the block in scale slot `slot`,
+    // as one outer-product MFMA (two blocks of 32x32x1: lanes 0..31 carry tile 0's columns, lanes 32..63 tile 1's; both
+    // halves carry the wave's 32 rows). Its result has the accumulators' layout, tile j in components 16 j .. 16 j + 15.
+    // The matrix cores are mostly idle in this kernel and the vector ALUs are not: this takes one multiply per
+    // accumulator and block off them.
+    auto scale_tiles = [&](int buf, int slot) -> float32_v {
         const unsigned char* base = smem + buf * kBufBytes;
-        const float sb = *reinterpret_cast<const float*>(base + kSbOff + (slot * kTile + wn * 64 + j * 32 + (lane & 31)) * 4);
+        const float sa = *reinterpret_cast<const float*>(base + kSaOff + (slot * kTile + wm * 32 + (lane & 31)) * 4);
+        const float sb = *reinterpret_cast<const float*>(base + kSbOff + (slot * kTile + wn * 64 + lane) * 4);
+        const float32_v zero = {};
+        return __builtin_amdgcn_mfma_f32_32x32x1f32(sa, sb, zero, 0, 0, 0);
+    };
+    // y[j] += f32(tile) * (scale_a[row] * scale_b[column]) for 32x32 tile j.
+    auto flush_tile = [&](const int16_t_v& tile, const float32_v& sc, int j) {
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const float4 sa = *reinterpret_cast<const float4*>(base + kSaOff + (slot * kTile + wm * 32 + q * 8 + (lane >> 5) * 4) * 4);
-            const float sav[4] = {sa.x, sa.y, sa.z, sa.w};
-#pragma unroll
-            for (int r = 0; r < 4; ++r) y[j][q * 4 + r] = fmaf(static_cast<float>(tile[q * 4 + r]), __fmul_rn(sav[r], sb), y[j][q * 4 + r]);
-        }
+        for (int i = 0; i < 16; ++i) y[j][i] = fmaf(static_cast<float>(tile[i]), sc[j * 16 + i], y[j][i]);
     };
     auto mfma = [](const u32x4_t& a, const u32x4_t& b, const int16_t_v& c) {
         return __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(int4_t, a), __builtin_bit_cast(int4_t, b), c, 0, 0, 0);
@@ -452,23 +458,26 @@ __global__ __launch_bounds__(512) void acc4_prefill_kernel(Acc4PrefillParams p)
             int16_t_v t1 = mfma(fa[0], fb[0][1], zero);
             t0 = mfma(fa[1], fb[1][0], t0);
             t1 = mfma(fa[1], fb[1][1], t1);
+            const float32_v sc = scale_tiles(buf, 0);
             if (store_next) store_part(next, buf ^ 1, 0);
-            flush_tile(t0, buf, 0, 0);
+            flush_tile(t0, sc, 0);
             if (store_next) store_part(next, buf ^ 1, 1);
-            flush_tile(t1, buf, 0, 1);
+            flush_tile(t1, sc, 1);
         } else if constexpr (NBS == 2) {
             const bool second = static_cast<int64_t>(kt) * 2 + 1 < p.kb;   // the step's second block exists
             const int16_t_v t0 = mfma(fa[0], fb[0][0], zero);
             const int16_t_v t1 = mfma(fa[0], fb[0][1], zero);
             const int16_t_v u0 = mfma(fa[1], fb[1][0], zero);
             const int16_t_v u1 = mfma(fa[1], fb[1][1], zero);
+            const float32_v sc0 = scale_tiles(buf, 0);
+            const float32_v sc1 = scale_tiles(buf, 1);
             if (store_next) store_part(next, buf ^ 1, 0);
-            flush_tile(t0, buf, 0, 0);
-            flush_tile(t1, buf, 0, 1);
+            flush_tile(t0, sc0, 0);
+            flush_tile(t1, sc0, 1);
             if (store_next) store_part(next, buf ^ 1, 1);
             if (second) {
-                flush_tile(u0, buf, 1, 0);
-                flush_tile(u1, buf, 1, 1);
+                flush_tile(u0, sc1, 0);
+                flush_tile(u1, sc1, 1);
             }
         } else {
             // Block size >= 128: the step opens and / or closes a block (wave-uniform).
@@ -482,8 +491,9 @@ __global__ __launch_bounds__(512) void acc4_prefill_kernel(Acc4PrefillParams p)
                 if (store_next) store_part(next, buf ^ 1, j);
             }
             if (closes) {
+                const float32_v sc = scale_tiles(buf, 0);
 #pragma unroll
-                for (int j = 0; j < TN; ++j) flush_tile(acc[j], buf, 0, j);
+                for (int j = 0; j < TN; ++j) flush_tile(acc[j], sc, j);
             }
         }
     };
