@@ -58,11 +58,17 @@ NxrtStatus nxrt_rocm_ep_create(uint32_t device_ordinal, const char* const* keys,
         if (it != ep->config.end()) {
             if (it->second == "native") ep->acc4_rounding = 1;
             else if (it->second == "mlas") ep->acc4_rounding = 0;
+            else if (it->second == "auto") ep->acc4_rounding = 2;
             else {
                 delete ep;
-                return make_status(NXRT_INVALID_ARGUMENT, "RocmExecutionProvider: acc4_rounding must be 'mlas' or 'native'");
+                return make_status(NXRT_INVALID_ARGUMENT, "RocmExecutionProvider: acc4_rounding must be 'mlas', 'native' or 'auto'");
             }
         }
+        // 'auto' follows the CPU provider's route (matmul_nbits.rs:640-660): fewer rows than the crossover take the native
+        // rule, the rest the MLAS rule. The crossover is host-dependent there (twice the decode threads), so it is a
+        // setting here, read from the same environment variable when the config does not give it.
+        if (const char* env = std::getenv("NXRT_SQNBIT_DECODE_MIN")) ep->config.emplace("acc4_native_below", env);
+        if ((it = ep->config.find("acc4_native_below")) != ep->config.end()) ep->acc4_native_below = parse_int(it->second, 0);
         if ((it = ep->config.find("decode_waves")) != ep->config.end()) ep->decode_waves = parse_int(it->second, 0);
         if ((it = ep->config.find("decode_col_groups")) != ep->config.end()) ep->decode_col_groups = parse_int(it->second, 0);
         if ((it = ep->config.find("prepack")) != ep->config.end()) ep->prepack = parse_int(it->second, 1);

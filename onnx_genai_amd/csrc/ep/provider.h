@@ -15,7 +15,8 @@ struct NxrtRocmEp {
     rocm_stream_t stream = nullptr;
     std::string name = "RocmExecutionProvider";
     std::map<std::string, std::string> config;   // EpConfig: a string map
-    int acc4_rounding = 0;                        // 0 = ties to even (MLAS), 1 = ties away (native)
+    int acc4_rounding = 0;                        // 0 = ties to even (MLAS), 1 = ties away (native), 2 = by row count
+    int acc4_native_below = 0;                    // with 2: calls with fewer rows than this round the native way
     int decode_waves = 0;                         // 0 = chosen per shape
     int decode_col_groups = 0;
     int prefill_tile = 0;                         // 0 = chosen per shape; 1..3 force a tile (tests, tuning)

@@ -521,6 +521,22 @@ def test_acc4_outputs(port, ref, a_dt, bs, zero_points, m, n, k, rounding, prepa
         provider.shutdown()
 
 
+@pytest.mark.parametrize("m,rule", [(2, oracle.ROUND_HALF_AWAY), (4, oracle.ROUND_HALF_EVEN), (40, oracle.ROUND_HALF_EVEN)])
+def test_acc4_rounding_route_follows_row_count(port, m, rule):
+    """acc4_rounding = auto: fewer rows than the crossover round the native way, the rest the MLAS way
+    (matmul_nbits.rs:640-660, where the crossover is NXRT_SQNBIT_DECODE_MIN or twice the decode threads)."""
+    bs, n, k = 64, 48, 64 * 6
+    provider = E.RocmExecutionProvider(0, {"acc4_rounding": "auto", "acc4_native_below": "4"})
+    try:
+        b, s, zp = synth.make_weights(n, k, bs, 91, zero_points=True, scale_lo=0.002, scale_hi=0.01, scale_dtype=E.F32)
+        a = _tie_heavy_activation(m, k, bs, 92, E.F32)
+        y, _ = run_op(provider, a, E.F32, b, s, E.F32, zp, n, k, bs, accuracy_level=4)
+        assert helpers.rel_l2(y, port.matmul_acc4_f32(a, b, s, zp, n, k, bs, rule)) <= TOL_F32
+        assert helpers.rel_l2(y, port.matmul_acc4_f32(a, b, s, zp, n, k, bs, 1 - rule)) > 10 * TOL_F32   # the other rule is told apart
+    finally:
+        provider.shutdown()
+
+
 @pytest.mark.parametrize("waves", [1, 3, 8])
 @pytest.mark.parametrize("s_dt", [E.F32, E.F16])
 @pytest.mark.parametrize("prepack", [True, False])
