@@ -366,7 +366,7 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
         int pack_rc = 0;
         const bool packed = M == 1 && use_packed(kn, args, pack_rc);
         w4.code_order = packed ? 2 : 1;
-        const int rounding = kn.ep->acc4_rounding == 2 ? (M < kn.ep->acc4_native_below ? 1 : 0) : kn.ep->acc4_rounding;   // matmul_nbits.rs:640-660
+        const int rounding = kn.ep->acc4_rounding == 2 ? (static_cast<int64_t>(M) < static_cast<int64_t>(kn.ep->acc4_native_below) ? 1 : 0) : kn.ep->acc4_rounding;   // matmul_nbits.rs:640-660
         rc = rocm_launch_quantize_a_workspace(args.a, args.a_dtype, args.m, args.k, args.block_size, rounding, &w4, stream);
         if (rc == 0 && pack_rc != 0) rc = pack_rc;
         if (rc == 0) {
