@@ -26,6 +26,7 @@ namespace mnb {
 typedef __attribute__((ext_vector_type(8))) _Float16 half8p_t;
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8p_t;
 typedef __attribute__((ext_vector_type(4))) float float4p_t;
+typedef __attribute__((ext_vector_type(2))) _Float16 half2p_t;
 
 constexpr int kGroupTiles = 4;
 constexpr int kChunkWeights = kGroupTiles * 1024;
@@ -121,6 +122,45 @@ struct PackedGroup {
     uint4 a[NA];
 };
 
+// v + (v of the lane a DPP control selects): quad_perm [1,0,3,2] = 0xB1, [2,3,0,1] = 0x4E, row_half_mirror = 0x141,
+// row_mirror = 0x140 - applied in that order they leave the sum over 4, 8, 16 lanes in every lane of the run.
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v)
+{
+    return v + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+
+// Sum of the 8 activations of one 16-byte piece, in f32.
+template <bool BF16>
+__device__ __forceinline__ float sum_piece(const uint4& v)
+{
+    const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        if constexpr (BF16) {
+            s += __uint_as_float(d[i] << 16);
+            s += __uint_as_float(d[i] & 0xffff0000u);
+        } else {
+            const half2p_t h = __builtin_bit_cast(half2p_t, d[i]);
+            s += static_cast<float>(h.x);
+            s += static_cast<float>(h.y);
+        }
+    }
+    return s;
+}
+
+// Sum over the BS / 8 consecutive lanes that hold one block's pieces; every lane of the run receives it.
+template <int BS>
+__device__ __forceinline__ float block_sum(float s)
+{
+    s = dpp_add<0xB1>(s);
+    s = dpp_add<0x4E>(s);
+    if constexpr (BS >= 64) s = dpp_add<0x141>(s);
+    if constexpr (BS >= 128) s = dpp_add<0x140>(s);
+    return s;
+}
+
 // BF16: activation element type. BS: block size. MR: rows staged (1 or 4; M <= MR). ST: storage type of the scales.
 // SETS: register sets of one group each. 2: the next group's loads are in flight while this one is multiplied - for
 // launches with few waves, where each wave must cover memory latency by itself. 1: no prefetch, 62 registers, eight
@@ -139,7 +179,16 @@ void decode_packed_kernel(PackedParams p)
     constexpr int NR = R / 16;
     constexpr int NA = MR == 1 ? 1 : U;
     constexpr int kStageBytes = MR == 1 ? 1024 : MR * kRowPitchP;
+    constexpr float kMagicF = BF16 ? 128.0f : 1024.0f;
     constexpr uint32_t kMagicNeg = BF16 ? 0xC300C300u : 0xE400E400u;
+    // How the magic offset and the zero point leave the accumulator. Launches of many short waves (one row, no
+    // prefetch) are bound by what a wave computes per byte: there they leave through the block's activation sum,
+    // y += scale * (acc - (magic + zp) * sum a), one FMA per block. Elsewhere a second MFMA per 32 elements against
+    // -(magic + zp) does it: more matrix-core work, but nothing between a wave's loads and its first MFMA, which is
+    // what the few-wave launches are sensitive to (measured: 3584 -> 37888 16.4 against 17.0 us and 3584 -> 152064 54.5
+    // against 59 us with the sums; 18944 -> 3584 12.2 against 11.4 us, so not there).
+    constexpr bool SUMS = MR == 1 && SETS == 1;
+    constexpr int kBlockLanes = BS / 8;         // lanes whose 16-byte pieces make up one block
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
     const int lane = threadIdx.x & 63;
@@ -192,7 +241,8 @@ void decode_packed_kernel(PackedParams p)
             }
         }
     };
-    auto compute_tile = [&](const Grp& grp, int u, int parity) {
+    // `asum` (with SUMS): this lane's block sum of the group's tile lane / 16 (one load covers the group's four tiles).
+    auto compute_tile = [&](const Grp& grp, int u, int parity, float asum) {
         unsigned char* st = stage + (MR == 1 ? parity : (u & 1)) * kStageBytes;
         if constexpr (MR != 1) {
             *reinterpret_cast<uint4*>(st + st_write) = grp.a[u];
@@ -214,9 +264,6 @@ void decode_packed_kernel(PackedParams p)
         for (int j = 0; j < 4; ++j) {
             const int bi = u * NBT + (j * 32) / BS;                          // block of the group (compile-time)
             const int zbyte = NB * static_cast<int>(sizeof(ST)) + bi;
-            const uint32_t z = (rr[zbyte / 4] >> ((zbyte % 4) * 8)) & 0xffu;
-            const uint32_t zpair = kMagicNeg | (z * 0x00010001u);
-            const uint4 zc = make_uint4(zpair, zpair, zpair, zpair);
             const uint32_t w = wd[j];
             uint4 op;
             op.x = (w & mask) | magic;
@@ -224,7 +271,11 @@ void decode_packed_kernel(PackedParams p)
             op.z = ((w >> 8) & mask) | magic;
             op.w = ((w >> 12) & mask) | magic;
             acc = mfma16p<BF16>(av[j], op, acc);
-            acc = mfma16p<BF16>(av[j], zc, acc);
+            const uint32_t z = (rr[zbyte / 4] >> ((zbyte % 4) * 8)) & 0xffu;
+            if constexpr (!SUMS) {
+                const uint32_t zpair = kMagicNeg | (z * 0x00010001u);
+                acc = mfma16p<BF16>(av[j], make_uint4(zpair, zpair, zpair, zpair), acc);
+            }
             if (((j + 1) * 32) % BS == 0 || j == 3) {
                 float sf;
                 if constexpr (sizeof(ST) == 4) {
@@ -233,10 +284,22 @@ void decode_packed_kernel(PackedParams p)
                     const uint32_t raw = (rr[bi / 2] >> ((bi % 2) * 16)) & 0xffffu;
                     sf = BF16 ? __uint_as_float(raw << 16) : f16_bits_to_f32(static_cast<uint16_t>(raw));
                 }
+                if constexpr (SUMS) {
+                    // the block's pieces sit in lanes first .. first + kBlockLanes - 1 of lane group u; any of them has the sum
+                    const int first = u * 16 + ((j * 32) / BS) % NBT * kBlockLanes;
+                    const float sa = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(asum), first));
+                    const float off = kMagicF + static_cast<float>(z);
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    y[r] = fmaf(sf, acc[r], y[r]);
-                    acc[r] = 0.f;
+                    for (int r = 0; r < 4; ++r) {
+                        y[r] = fmaf(sf, fmaf(-off, sa, acc[r]), y[r]);      // the product is not rounded on its own
+                        acc[r] = 0.f;
+                    }
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        y[r] = fmaf(sf, acc[r], y[r]);
+                        acc[r] = 0.f;
+                    }
                 }
             }
         }
@@ -248,7 +311,7 @@ void decode_packed_kernel(PackedParams p)
             lds_order();
         }
 #pragma unroll
-        for (int u = 0; u < U; ++u) compute_tile(cur, u, parity);
+        for (int u = 0; u < U; ++u) compute_tile(cur, u, parity, 0.f);
     };
 
     if constexpr (SETS == 2) {
@@ -262,12 +325,14 @@ void decode_packed_kernel(PackedParams p)
         Grp ga;
         for (int gi = g_begin; gi < g_end; ++gi) {
             fetch_group(ga, gi);
+            float asum = 0.f;
             if constexpr (MR == 1) {
                 *reinterpret_cast<uint4*>(stage + st_write) = ga.a[0];
                 lds_order();
+                if constexpr (SUMS) asum = block_sum<BS>(sum_piece<BF16>(ga.a[0]));
             }
 #pragma unroll
-            for (int u = 0; u < U; ++u) compute_tile(ga, u, 0);
+            for (int u = 0; u < U; ++u) compute_tile(ga, u, 0, asum);
         }
     }
 
