@@ -403,7 +403,7 @@ constexpr int kWideWaves = 8;
 // RB: blocks of 16 rows (1, 2 or 4). A window is WT tiles of 128 k: a whole tile group for RB <= 2, half of one for
 // RB = 4, so that two buffers of RB * 16 rows stay within 66 KB.
 template <bool BF16, int BS, typename ST, int RB>
-__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu((BS == 128 && sizeof(ST) == 2 && RB == 1) ? 6 : 1)))
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu((BS == 128 && sizeof(ST) == 2 && RB == 1) ? 5 : 1)))
 void decode_wide_kernel(PackedParams p)
 {
     constexpr int U = kGroupTiles;
@@ -418,8 +418,14 @@ void decode_wide_kernel(PackedParams p)
     constexpr int kBufBytes = kRows * kPitch;
     constexpr int kPieces = WT * 16;                    // 16-byte pieces per row of a window
     constexpr int NW = kRows * kPieces / 512;           // pieces per thread per window (2 or 4)
-    constexpr uint32_t kMagicNeg = BF16 ? 0xC300C300u : 0xE400E400u;
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];   // [2][kRows][kPitch]
+    constexpr float kMagicF = BF16 ? 128.0f : 1024.0f;
+    constexpr int kBlockLanes = BS / 8;                 // consecutive threads whose pieces make up one block of a row
+    constexpr int kWinBlocks = WT * NBT;                // blocks per window
+    constexpr int kSumBytes = kWinBlocks * kRows * 4;
+    // [2][kRows][kPitch] activations, then [2][kWinBlocks][kRows] f32 sums of each row over each block of the window:
+    // the magic offset and the zero point leave the accumulators through them, y += scale * (acc - (magic + zp) * sum a)
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    float* lds_sums = reinterpret_cast<float*>(smem + 2 * kBufBytes);
 
     const int t = threadIdx.x;
     const int lane = t & 63;
@@ -475,7 +481,10 @@ void decode_wide_kernel(PackedParams p)
 #pragma unroll
         for (int i = 0; i < NW; ++i) {
             const int q = t + 512 * i;
-            *reinterpret_cast<uint4*>(smem + buf * kBufBytes + (q / kPieces) * kPitch + (q % kPieces) * 16) = wa[i];
+            const int row = q / kPieces, piece = q % kPieces;
+            *reinterpret_cast<uint4*>(smem + buf * kBufBytes + row * kPitch + piece * 16) = wa[i];
+            const float sum = block_sum<BS>(sum_piece<BF16>(wa[i]));      // a block's pieces sit in consecutive lanes
+            if (piece % kBlockLanes == 0) lds_sums[(buf * kWinBlocks + piece / kBlockLanes) * kRows + row] = sum;
         }
     };
     // tiles [first, first + WT) of the group against window buffer `buf`
@@ -497,9 +506,6 @@ void decode_wide_kernel(PackedParams p)
             for (int j = 0; j < 4; ++j) {
                 const int bi = u * NBT + (j * 32) / BS;
                 const int zbyte = NB * static_cast<int>(sizeof(ST)) + bi;
-                const uint32_t z = (rr[zbyte / 4] >> ((zbyte % 4) * 8)) & 0xffu;
-                const uint32_t zpair = kMagicNeg | (z * 0x00010001u);
-                const uint4 zc = make_uint4(zpair, zpair, zpair, zpair);
                 const uint32_t w = wd[j];
                 uint4 op;
                 op.x = (w & mask) | magic;
@@ -507,7 +513,7 @@ void decode_wide_kernel(PackedParams p)
                 op.z = ((w >> 8) & mask) | magic;
                 op.w = ((w >> 12) & mask) | magic;
                 const bool last = ((j + 1) * 32) % BS == 0 || j == 3;
-                float sf = 0.f;
+                float sf = 0.f, off = 0.f;
                 if (last) {
                     if constexpr (sizeof(ST) == 4) {
                         sf = __uint_as_float(rr[bi]);
@@ -515,16 +521,20 @@ void decode_wide_kernel(PackedParams p)
                         const uint32_t raw = (rr[bi / 2] >> ((bi % 2) * 16)) & 0xffffu;
                         sf = BF16 ? __uint_as_float(raw << 16) : f16_bits_to_f32(static_cast<uint16_t>(raw));
                     }
+                    off = kMagicF + static_cast<float>((rr[zbyte / 4] >> ((zbyte % 4) * 8)) & 0xffu);
                 }
+                const int wb = x * NBT + (j * 32) / BS;                // block of the window
 #pragma unroll
                 for (int rb = 0; rb < RB; ++rb) {
                     const uint4 av = *reinterpret_cast<const uint4*>(fa + rb * 16 * kPitch + j * 64);
                     acc[rb] = mfma16p<BF16>(av, op, acc[rb]);
-                    acc[rb] = mfma16p<BF16>(av, zc, acc[rb]);
                     if (last) {
+                        // this lane's accumulator rows are rows rb * 16 + 4 g + r of the window
+                        const float4 sa = *reinterpret_cast<const float4*>(lds_sums + (buf * kWinBlocks + wb) * kRows + rb * 16 + 4 * g);
+                        const float sav[4] = {sa.x, sa.y, sa.z, sa.w};
 #pragma unroll
                         for (int r = 0; r < 4; ++r) {
-                            y[rb][r] = fmaf(sf, acc[rb][r], y[rb][r]);
+                            y[rb][r] = fmaf(sf, fmaf(-off, sav[r], acc[rb][r]), y[rb][r]);
                             acc[rb][r] = 0.f;
                         }
                     }
@@ -582,10 +592,12 @@ static int launch_wide_bs(const PackedParams& p, int bs, hipStream_t stream)
     };
     auto by_rows = [&](auto bs_tag) {
         constexpr int BS = decltype(bs_tag)::value;
-        if (p.m <= 16) return go(decode_wide_kernel<BF16, BS, ST, 1>, 2 * 16 * (4 * 256 + 16));
-        if (p.m <= 32) return go(decode_wide_kernel<BF16, BS, ST, 2>, 2 * 32 * (4 * 256 + 16));
+        // two window buffers of rows x (tiles x 256 + 16) bytes, then two tables of (blocks per window) x rows f32 sums
+        constexpr int NBT = 128 / BS;
+        if (p.m <= 16) return go(decode_wide_kernel<BF16, BS, ST, 1>, 2 * 16 * (4 * 256 + 16) + 2 * 4 * NBT * 16 * 4);
+        if (p.m <= 32) return go(decode_wide_kernel<BF16, BS, ST, 2>, 2 * 32 * (4 * 256 + 16) + 2 * 4 * NBT * 32 * 4);
         if constexpr (BS == 32) return -1;
-        else return go(decode_wide_kernel<BF16, BS, ST, 4>, 2 * 64 * (2 * 256 + 16));
+        else return go(decode_wide_kernel<BF16, BS, ST, 4>, 2 * 64 * (2 * 256 + 16) + 2 * 2 * NBT * 64 * 4);
     };
     switch (bs) {
         case 32: return by_rows(std::integral_constant<int, 32>{});
