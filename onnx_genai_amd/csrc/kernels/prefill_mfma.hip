@@ -37,6 +37,9 @@ struct PrefillParams {
     int scale_dtype, bias_dtype, y_dtype;
     int steps_per_split;    // K steps of 64 per workgroup along grid.z
     float* partial;         // [splits][M][N] f32 partial sums when K is split (else NULL: the kernel writes Y itself)
+    // 0x000F000F and the two 16-bit magic exponents, as arguments rather than literals: the mask is moved to a vector
+    // register and the magic stays in a scalar one, which is what lets (x & mask) | magic be one v_and_or_b32
+    uint32_t nibble_mask, magic;
 };
 
 constexpr int kBK = 64;
@@ -50,9 +53,9 @@ __device__ __forceinline__ float16_t mfma32(const uint4& a, const uint4& b, floa
 }
 
 // Two nibbles (elements 2i, 2i+1 of a packed dword) as a pair of 16-bit floats carrying magic + q.
-__device__ __forceinline__ uint32_t magic_pair(uint32_t w, uint32_t w4, uint32_t sel, uint32_t magic)
+__device__ __forceinline__ uint32_t magic_pair(uint32_t w, uint32_t w4, uint32_t sel, uint32_t mask, uint32_t magic)
 {
-    return (__builtin_amdgcn_perm(w4, w, sel) & 0x000F000Fu) | magic;
+    return (__builtin_amdgcn_perm(w4, w, sel) & mask) | magic;
 }
 
 // f16, f16 scale: exact subtract, one rounding multiply.
@@ -95,8 +98,8 @@ __global__ __launch_bounds__(512) void prefill_mfma_kernel(PrefillParams p)
     constexpr int A_LOADS = BM / 64;       // 16-byte pieces of A per lane per step
     constexpr int B_DW = BN / 64;          // packed dwords of B per lane per step (1, 2 or 4)
     constexpr int B_PIECES = 8 / B_DW;     // lanes that share one column's 32 bytes of a step
-    constexpr uint32_t kMagic = BF16 ? 0x43004300u : 0x64006400u;
     constexpr float kMagicF = BF16 ? 128.0f : 1024.0f;
+    const uint32_t nib_mask = __builtin_amdgcn_mov_dpp(p.nibble_mask, 0xE4, 0xf, 0xf, false);
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     unsigned char* lds_a = smem;                                   // [2][BM][kPitch]
     unsigned char* lds_b = smem + 2 * BM * kPitch;                 // [2][BN][kPitch]
@@ -193,10 +196,10 @@ __global__ __launch_bounds__(512) void prefill_mfma_kernel(PrefillParams p)
         unsigned char* lb = lds_b + buf * (BN * kPitch) + b_loff;
         const uint32_t w = r.b[dw], w4 = w >> 4;
         uint32_t pr[4];
-        pr[0] = magic_pair(w, w4, 0x0c040c00u, kMagic);
-        pr[1] = magic_pair(w, w4, 0x0c050c01u, kMagic);
-        pr[2] = magic_pair(w, w4, 0x0c060c02u, kMagic);
-        pr[3] = magic_pair(w, w4, 0x0c070c03u, kMagic);
+        pr[0] = magic_pair(w, w4, 0x0c040c00u, nib_mask, p.magic);
+        pr[1] = magic_pair(w, w4, 0x0c050c01u, nib_mask, p.magic);
+        pr[2] = magic_pair(w, w4, 0x0c060c02u, nib_mask, p.magic);
+        pr[3] = magic_pair(w, w4, 0x0c070c03u, nib_mask, p.magic);
         const uint32_t zq = ((r.z >> r.zsh) & zp_mask) | zp_default;
         if constexpr (F32MATH) {
             const float off = kMagicF + static_cast<float>(zq);
@@ -399,6 +402,8 @@ extern "C" int rocm_launch_prefill_mfma(const RocmMatMulNBitsArgs* a, int tile_c
     p.scale_dtype = a->scale_dtype;
     p.bias_dtype = a->bias_dtype;
     p.y_dtype = a->y_dtype;
+    p.nibble_mask = 0x000F000Fu;
+    p.magic = a->a_dtype == ROCM_DT_BF16 ? 0x43004300u : 0x64006400u;
     const PrefillPlan plan = plan_prefill(a, tile_choice, scratch ? scratch_bytes : 0);
     p.steps_per_split = plan.steps_per_split;
     p.partial = plan.splits > 1 ? static_cast<float*>(scratch) : nullptr;
