@@ -65,23 +65,30 @@ __device__ __forceinline__ uint32_t finish_f16(uint32_t pair, half2_t neg_off, h
     return __builtin_bit_cast(uint32_t, v);
 }
 
-// (q - zp) * scale in f32 for both halves of a magic pair (bf16 magic 0x4300 or f16 magic 0x6400), rounded to 16 bits.
+// Eight weights of one packed dword as (q - zp) * scale, computed in f32 and rounded once to the 16-bit type (nearest
+// even), in element order. `shift` is (16 - zp) in every byte: the bytes q + 16 - zp (1..31, no borrow between them)
+// convert to f32 with one instruction each, and t * scale - 16 * scale in one FMA is exactly (q - zp) * scale rounded
+// once, because 16 * scale is exact.
+typedef __attribute__((ext_vector_type(2))) float float2_t;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
 template <bool BF16>
-__device__ __forceinline__ uint32_t finish_f32(uint32_t pair, float off, float scale)
+__device__ __forceinline__ uint4 dequant_dword_f32(uint32_t w, uint32_t shift, float scale, float neg16_scale)
 {
-    float lo, hi;
-    if constexpr (BF16) {
-        lo = __uint_as_float(pair << 16);
-        hi = __uint_as_float(pair & 0xffff0000u);
-    } else {
-        const half2_t h = __builtin_bit_cast(half2_t, pair);
-        lo = static_cast<float>(h.x);
-        hi = static_cast<float>(h.y);
+    uint32_t even = (w & 0x0f0f0f0fu) + shift;            // elements 0, 2, 4, 6, one per byte
+    uint32_t odd = ((w >> 4) & 0x0f0f0f0fu) + shift;      // elements 1, 3, 5, 7
+    asm volatile("" : "+v"(even), "+v"(odd));             // keep the bytes whole: one byte-to-float convert each
+    uint32_t out[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float lo = fmaf(static_cast<float>((even >> (8 * i)) & 0xffu), scale, neg16_scale);
+        const float hi = fmaf(static_cast<float>((odd >> (8 * i)) & 0xffu), scale, neg16_scale);
+        if constexpr (BF16) {
+            out[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(float2_t{lo, hi}, bf16x2_t));   // v_cvt_pk_bf16_f32
+        } else {
+            out[i] = static_cast<uint32_t>(f32_to_f16_bits(lo)) | (static_cast<uint32_t>(f32_to_f16_bits(hi)) << 16);
+        }
     }
-    lo = __fmul_rn(lo - off, scale);
-    hi = __fmul_rn(hi - off, scale);
-    if constexpr (BF16) return static_cast<uint32_t>(f32_to_bf16_bits(lo)) | (static_cast<uint32_t>(f32_to_bf16_bits(hi)) << 16);
-    else return static_cast<uint32_t>(f32_to_f16_bits(lo)) | (static_cast<uint32_t>(f32_to_f16_bits(hi)) << 16);
+    return make_uint4(out[0], out[1], out[2], out[3]);
 }
 
 // BF16: element type. BM x BN: tile of Y per workgroup (128 x 64, 128 x 128, 256 x 128 or 256 x 256). SF32: scales are stored
@@ -98,7 +105,6 @@ __global__ __launch_bounds__(512) void prefill_mfma_kernel(PrefillParams p)
     constexpr int A_LOADS = BM / 64;       // 16-byte pieces of A per lane per step
     constexpr int B_DW = BN / 64;          // packed dwords of B per lane per step (1, 2 or 4)
     constexpr int B_PIECES = 8 / B_DW;     // lanes that share one column's 32 bytes of a step
-    constexpr float kMagicF = BF16 ? 128.0f : 1024.0f;
     const uint32_t nib_mask = __builtin_amdgcn_mov_dpp(p.nibble_mask, 0xE4, 0xf, 0xf, false);
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     unsigned char* lds_a = smem;                                   // [2][BM][kPitch]
@@ -194,25 +200,24 @@ __global__ __launch_bounds__(512) void prefill_mfma_kernel(PrefillParams p)
         if ((B_DW == 2 && (part & 1)) || (B_DW == 1 && part != 0)) return;
         const int dw = B_DW == 4 ? part : (part >> 1);
         unsigned char* lb = lds_b + buf * (BN * kPitch) + b_loff;
-        const uint32_t w = r.b[dw], w4 = w >> 4;
-        uint32_t pr[4];
-        pr[0] = magic_pair(w, w4, 0x0c040c00u, nib_mask, p.magic);
-        pr[1] = magic_pair(w, w4, 0x0c050c01u, nib_mask, p.magic);
-        pr[2] = magic_pair(w, w4, 0x0c060c02u, nib_mask, p.magic);
-        pr[3] = magic_pair(w, w4, 0x0c070c03u, nib_mask, p.magic);
+        const uint32_t w = r.b[dw];
         const uint32_t zq = ((r.z >> r.zsh) & zp_mask) | zp_default;
         if constexpr (F32MATH) {
-            const float off = kMagicF + static_cast<float>(zq);
             const float sc = SF32 ? __uint_as_float(r.s) : (BF16 ? __uint_as_float(r.s << 16) : f16_bits_to_f32(static_cast<uint16_t>(r.s)));
-#pragma unroll
-            for (int i = 0; i < 4; ++i) pr[i] = finish_f32<BF16>(pr[i], off, sc);
+            *reinterpret_cast<uint4*>(lb + dw * 16) = dequant_dword_f32<BF16>(w, (16u - zq) * 0x01010101u, sc, -16.0f * sc);
         } else {
+            const uint32_t w4 = w >> 4;
+            uint32_t pr[4];
+            pr[0] = magic_pair(w, w4, 0x0c040c00u, nib_mask, p.magic);
+            pr[1] = magic_pair(w, w4, 0x0c050c01u, nib_mask, p.magic);
+            pr[2] = magic_pair(w, w4, 0x0c060c02u, nib_mask, p.magic);
+            pr[3] = magic_pair(w, w4, 0x0c070c03u, nib_mask, p.magic);
             const uint32_t o2 = 0xE400E400u | (zq * 0x00010001u);   // -(1024 + zp) twice, exact in f16
             const uint32_t s2 = r.s * 0x00010001u;                  // the f16 scale twice
 #pragma unroll
             for (int i = 0; i < 4; ++i) pr[i] = finish_f16(pr[i], __builtin_bit_cast(half2_t, o2), __builtin_bit_cast(half2_t, s2));
+            *reinterpret_cast<uint4*>(lb + dw * 16) = make_uint4(pr[0], pr[1], pr[2], pr[3]);
         }
-        *reinterpret_cast<uint4*>(lb + dw * 16) = make_uint4(pr[0], pr[1], pr[2], pr[3]);
     };
     auto store_lds = [&](const Regs& r, int buf) {
 #pragma unroll
