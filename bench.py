@@ -262,7 +262,7 @@ def main():
     if args.only_roofline:
         return roofline_only(ep, args)
     if args.only_tables:
-        for row in prefill_table(ep) + acc4_table(ep):
+        for row in prefill_table(ep) + prefill_7b_table(ep) + acc4_table(ep):
             print(json.dumps(row), flush=True)
         return
     nodes, a_bufs = build_decode_stack(ep, args.m, args.layers)
@@ -326,6 +326,7 @@ def main():
         ep.deallocate(buf)
     if not args.no_sweep:
         result["prefill"] = prefill_table(ep)
+        result["prefill_7b_bf16"] = prefill_7b_table(ep)
         result["acc4"] = acc4_table(ep)
         result["small_model_step"] = small_model_step(ep)
     ep.shutdown()
@@ -394,13 +395,13 @@ def sweep(ep, nodes, a_bufs, args):
     return table
 
 
-def prefill_table(ep):
-    """Prefill GEMM at Llama-3-8B MLP shapes (configs[3]): fp16, block 32, no zero points."""
+def prefill_table(ep, shapes=((4096, 14336), (14336, 4096)), rows=(512, 2048, 8192), dtype=E.F16, bs=32, zero_points=False):
+    """Prefill GEMM. Defaults: Llama-3-8B MLP shapes (configs[3]): fp16, block 32, no zero points."""
     table = []
-    for k, n in ((4096, 14336), (14336, 4096)):
-        for m in (512, 2048, 8192):
-            node = Node(ep, "prefill", k, n, 32, 7, E.F16, m, zero_points=False, scale_range=(0.001, 0.01))
-            a = ep.upload(synth.make_activation(m, k, 8, E.F16))
+    for k, n in shapes:
+        for m in rows:
+            node = Node(ep, "prefill", k, n, bs, 7, dtype, m, zero_points=zero_points, scale_range=(0.001, 0.01))
+            a = ep.upload(synth.make_activation(m, k, 8, dtype))
             node.run(a)
             ep.sync()
             variant = node.ops.kernel.last_variant()
@@ -418,6 +419,11 @@ def prefill_table(ep):
             ep.deallocate(a)
             node.free(ep)
     return table
+
+
+def prefill_7b_table(ep):
+    """The same kernel at the Qwen2.5-7B shapes of the decode sweep: bf16, block 128, zero points, M = 4096."""
+    return prefill_table(ep, shapes=((3584, 37888), (18944, 3584)), rows=(4096,), dtype=E.BF16, bs=128, zero_points=True)
 
 
 def acc4_table(ep):
