@@ -339,6 +339,16 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
     rocm_stream_t stream = kn.ep->stream;
     int rc = 0;
     if (kn.accuracy_level == 4) {
+        const int rounding = kn.ep->acc4_rounding == 2 ? (static_cast<int64_t>(M) < static_cast<int64_t>(kn.ep->acc4_native_below) ? 1 : 0) : kn.ep->acc4_rounding;   // matmul_nbits.rs:640-660
+        int pack_rc = 0;
+        const bool packed = M == 1 && use_packed(kn, args, pack_rc);
+        if (packed && rocm_acc4_packed_fuses_quantizer(&args)) {
+            // one f16 / bf16 row over the repacked stream: the kernel quantizes the row itself, no workspace and no second launch
+            rc = pack_rc != 0 ? pack_rc : rocm_launch_acc4_packed(&args, kn.packed, nullptr, rounding, kn.ep->decode_waves, stream);
+            kn.variant = "acc4_mfma_i8_packed";
+            kn.ep->launches.fetch_add(1);
+            return hip_status(rc, "MatMulNBits: kernel launch");
+        }
         const uint64_t need = acc4_workspace_bytes(kn, M);
         uint8_t* ws = static_cast<uint8_t*>(workspace);
         if (!ws || workspace_bytes < need) {
@@ -363,15 +373,12 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
         w4.qa = reinterpret_cast<int8_t*>(ws);
         w4.aq = reinterpret_cast<float*>(ws + lay.codes);
         w4.aux = reinterpret_cast<float*>(ws + lay.codes + lay.pairs);
-        int pack_rc = 0;
-        const bool packed = M == 1 && use_packed(kn, args, pack_rc);
         w4.code_order = packed ? 2 : 1;
-        const int rounding = kn.ep->acc4_rounding == 2 ? (static_cast<int64_t>(M) < static_cast<int64_t>(kn.ep->acc4_native_below) ? 1 : 0) : kn.ep->acc4_rounding;   // matmul_nbits.rs:640-660
         rc = rocm_launch_quantize_a_workspace(args.a, args.a_dtype, args.m, args.k, args.block_size, rounding, &w4, stream);
         if (rc == 0 && pack_rc != 0) rc = pack_rc;
         if (rc == 0) {
             if (packed) {
-                rc = rocm_launch_acc4_packed(&args, kn.packed, &w4, kn.ep->decode_waves, stream);
+                rc = rocm_launch_acc4_packed(&args, kn.packed, &w4, rounding, kn.ep->decode_waves, stream);
                 kn.variant = "acc4_mfma_i8_packed";
             } else if (rocm_acc4_mfma_eligible(&args)) {
                 rc = rocm_launch_acc4_mfma(&args, &w4, kn.ep->decode_waves, stream);

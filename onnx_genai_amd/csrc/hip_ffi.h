@@ -117,7 +117,10 @@ int rocm_acc4_mfma_eligible(const RocmMatMulNBitsArgs* args);
 int rocm_launch_acc4_mfma(const RocmMatMulNBitsArgs* args, const RocmAcc4Workspace* ws, int waves, rocm_stream_t stream);
 /* One row over the repacked copy of constant weights (the copy rocm_launch_pack_decode makes); code_order 2. */
 int rocm_acc4_packed_eligible(const RocmMatMulNBitsArgs* args);
-int rocm_launch_acc4_packed(const RocmMatMulNBitsArgs* args, const void* packed, const RocmAcc4Workspace* ws, int waves, rocm_stream_t stream);
+/* `ws` = NULL: the kernel quantizes the row itself (rocm_acc4_packed_fuses_quantizer() must hold: f16 / bf16 row,
+ * K % 8 == 0, 16-byte aligned) with the given rounding rule; otherwise codes and pairs come from the workspace. */
+int rocm_acc4_packed_fuses_quantizer(const RocmMatMulNBitsArgs* args);
+int rocm_launch_acc4_packed(const RocmMatMulNBitsArgs* args, const void* packed, const RocmAcc4Workspace* ws, int rounding, int waves, rocm_stream_t stream);
 
 #ifdef __cplusplus
 }

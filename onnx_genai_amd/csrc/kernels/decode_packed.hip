@@ -130,6 +130,17 @@ __device__ __forceinline__ float dpp_add(float v)
     return v + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
 }
 
+template <int CTRL>
+__device__ __forceinline__ float dpp_max(float v)
+{
+    return fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false)));
+}
+template <int CTRL>
+__device__ __forceinline__ int dpp_addi(int v)
+{
+    return v + __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, false);
+}
+
 // Sum of the 8 activations of one 16-byte piece, in f32.
 template <bool BF16>
 __device__ __forceinline__ float sum_piece(const uint4& v)
@@ -620,6 +631,9 @@ typedef __attribute__((ext_vector_type(4))) int int4p_t;
 struct Acc4PackedParams {
     const int8_t* qa;       // [padded_k] codes of the one row, packed order
     const float* aq;        // [kb, 2]: scale_a, f32(sum of codes)
+    const void* a;          // FUSE: the one row itself, f16 or bf16 [k]; every wave quantizes the groups it multiplies
+    int64_t k;
+    int rounding;           // FUSE: 0 = ties to even, 1 = ties away from zero
     const uint8_t* packed;
     const void* bias;
     void* y;
@@ -639,7 +653,12 @@ struct Acc4PackedGroup {
     uint2 x;      // (scale_a, code sum) of block `lane` of the group
 };
 
-template <int BS, typename ST, int SETS>
+// FUSE: 0 = codes and (scale, sum) pairs come from the workspace a quantizer kernel filled; 1 / 2 = the row arrives as
+// f16 / bf16 and each wave quantizes the 512 activations of a group itself, with the arithmetic of quantize_a_kernel
+// (one correctly rounded divide each for scale and inverse, one multiply and one rounding per element) - a lane holds
+// 8 consecutive activations, a block is BS / 8 consecutive lanes. That is redundant across workgroups but saves the
+// separate launch, which at one row costs about as much as a fifth of this kernel.
+template <int BS, typename ST, int SETS, int FUSE>
 __global__ __launch_bounds__(512) void acc4_packed_kernel(Acc4PackedParams p)
 {
     constexpr int U = kGroupTiles;
@@ -658,8 +677,9 @@ __global__ __launch_bounds__(512) void acc4_packed_kernel(Acc4PackedParams p)
     const bool bf16_scales = p.scales_bf16 != 0;
 
     const __amdgpu_buffer_rsrc_t srd_p = make_srd(p.packed + static_cast<int64_t>(blockIdx.x) * p.cg_stride, static_cast<uint64_t>(p.cg_stride));
-    const __amdgpu_buffer_rsrc_t srd_a = make_srd(p.qa, static_cast<uint64_t>(p.padded_k));
-    const __amdgpu_buffer_rsrc_t srd_x = make_srd(p.aq, static_cast<uint64_t>(p.kb) * 8);
+    const __amdgpu_buffer_rsrc_t srd_a = FUSE ? make_srd(p.a, static_cast<uint64_t>(p.k) * 2) : make_srd(p.qa, static_cast<uint64_t>(p.padded_k));
+    const __amdgpu_buffer_rsrc_t srd_x = make_srd(p.aq, FUSE ? 0 : static_cast<uint64_t>(p.kb) * 8);
+    constexpr int kBlockLanes = BS / 8;
 
     const uint32_t w_off = static_cast<uint32_t>(lane * 16);
     const uint32_t r_off = static_cast<uint32_t>(kChunkWeights + c * R);
@@ -682,13 +702,61 @@ __global__ __launch_bounds__(512) void acc4_packed_kernel(Acc4PackedParams p)
         for (int u = 0; u < U; ++u) grp.w[u] = load16(srd_p, w_off + static_cast<uint32_t>(u * 1024), soff);
 #pragma unroll
         for (int i = 0; i < NR; ++i) grp.r[i] = load16(srd_p, r_off + static_cast<uint32_t>(i * 16), soff);
-        grp.a = load16(srd_a, lane < 32 ? static_cast<uint32_t>(lane * 16) : kOutOfRange, static_cast<uint32_t>(gi) * 512u);   // the range ends the row at padded_k
-        const auto v = __builtin_amdgcn_raw_buffer_load_b64(srd_x, static_cast<int>(lane < NB ? lane * 8 : kOutOfRange), static_cast<int>(gi * NB * 8), 0);
-        grp.x = make_uint2(v[0], v[1]);
+        if constexpr (FUSE) {
+            grp.a = load16(srd_a, static_cast<uint32_t>(lane * 16), static_cast<uint32_t>(gi) * 1024u);   // 8 activations; K % 8 == 0 and the range ends the row
+        } else {
+            grp.a = load16(srd_a, lane < 32 ? static_cast<uint32_t>(lane * 16) : kOutOfRange, static_cast<uint32_t>(gi) * 512u);   // the range ends the row at padded_k
+            const auto v = __builtin_amdgcn_raw_buffer_load_b64(srd_x, static_cast<int>(lane < NB ? lane * 8 : kOutOfRange), static_cast<int>(gi * NB * 8), 0);
+            grp.x = make_uint2(v[0], v[1]);
+        }
     };
     auto compute_group = [&](const Grp& grp, int gi, int slot) {
         unsigned char* st = stage + slot * 512;
-        if (lane < 32) *reinterpret_cast<uint4*>(st + lane * 16) = grp.a;
+        float sa_lane = 0.f, qs_lane = 0.f;          // FUSE: scale and f32(code sum) of the block this lane's activations lie in
+        if constexpr (FUSE) {
+            const uint32_t d[4] = {grp.a.x, grp.a.y, grp.a.z, grp.a.w};
+            float v[8];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if constexpr (FUSE == 2) {
+                    v[2 * i] = __uint_as_float(d[i] << 16);
+                    v[2 * i + 1] = __uint_as_float(d[i] & 0xffff0000u);
+                } else {
+                    const half2p_t h = __builtin_bit_cast(half2p_t, d[i]);
+                    v[2 * i] = static_cast<float>(h.x);
+                    v[2 * i + 1] = static_cast<float>(h.y);
+                }
+            }
+            float vmax = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) vmax = fmaxf(vmax, fabsf(v[i]));
+            vmax = dpp_max<0xB1>(vmax);
+            vmax = dpp_max<0x4E>(vmax);
+            if constexpr (BS >= 64) vmax = dpp_max<0x141>(vmax);
+            if constexpr (BS >= 128) vmax = dpp_max<0x140>(vmax);
+            sa_lane = __fdiv_rn(vmax, 127.0f);
+            const float inv = vmax != 0.0f ? __fdiv_rn(127.0f, vmax) : 0.0f;
+            int q[8], sum = 0;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float scaled = __fmul_rn(v[i], inv);
+                float r = p.rounding == 1 ? roundf(scaled) : rintf(scaled);
+                r = fminf(fmaxf(r, -127.0f), 127.0f);
+                q[i] = static_cast<int>(r);
+                sum += q[i];
+            }
+            sum = dpp_addi<0xB1>(sum);
+            sum = dpp_addi<0x4E>(sum);
+            if constexpr (BS >= 64) sum = dpp_addi<0x141>(sum);
+            if constexpr (BS >= 128) sum = dpp_addi<0x140>(sum);
+            qs_lane = static_cast<float>(sum);                     // |sum| <= 127 * BS: exact
+            // the byte order the repacked weights unpack to: elements 0,4,1,5 | 2,6,3,7
+            const uint32_t lo = (q[0] & 0xff) | ((q[4] & 0xff) << 8) | ((q[1] & 0xff) << 16) | (static_cast<uint32_t>(q[5]) << 24);
+            const uint32_t hi = (q[2] & 0xff) | ((q[6] & 0xff) << 8) | ((q[3] & 0xff) << 16) | (static_cast<uint32_t>(q[7]) << 24);
+            *reinterpret_cast<uint2*>(st + lane * 8) = make_uint2(lo, hi);
+        } else {
+            if (lane < 32) *reinterpret_cast<uint4*>(st + lane * 16) = grp.a;
+        }
         lds_order();
         uint32_t rr[NR * 4];
 #pragma unroll
@@ -723,8 +791,9 @@ __global__ __launch_bounds__(512) void acc4_packed_kernel(Acc4PackedParams p)
                             const uint32_t raw = (rr[bi / 2] >> ((bi % 2) * 16)) & 0xffffu;
                             sb = bf16_scales ? __uint_as_float(raw << 16) : f16_bits_to_f32(static_cast<uint16_t>(raw));
                         }
-                        const float sa = __int_as_float(__builtin_amdgcn_readlane(static_cast<int>(grp.x.x), bi));
-                        const float qs = __int_as_float(__builtin_amdgcn_readlane(static_cast<int>(grp.x.y), bi));
+                        const int src = FUSE ? bi * kBlockLanes : bi;         // a lane of the block, or the lane that loaded its pair
+                        const float sa = __int_as_float(__builtin_amdgcn_readlane(FUSE ? __float_as_int(sa_lane) : static_cast<int>(grp.x.x), src));
+                        const float qs = __int_as_float(__builtin_amdgcn_readlane(FUSE ? __float_as_int(qs_lane) : static_cast<int>(grp.x.y), src));
                         const float f = fmaf(-zf, qs, static_cast<float>(acc[0]));   // both terms are integers below 2^24: exact
                         y = fmaf(f, __fmul_rn(sa, sb), y);
                     }
@@ -769,12 +838,18 @@ __global__ __launch_bounds__(512) void acc4_packed_kernel(Acc4PackedParams p)
 }
 
 template <int BS, typename ST>
-static int launch_acc4_packed(const Acc4PackedParams& p, int waves, bool single_set, hipStream_t stream)
+static int launch_acc4_packed(const Acc4PackedParams& p, int waves, bool single_set, int fuse, hipStream_t stream)
 {
     const unsigned grid = static_cast<unsigned>((p.n + 15) / 16);
     const size_t lds = static_cast<size_t>(waves) * 1024;
-    if (single_set) hipLaunchKernelGGL((acc4_packed_kernel<BS, ST, 1>), dim3(grid), dim3(waves * 64), lds, stream, p);
-    else hipLaunchKernelGGL((acc4_packed_kernel<BS, ST, 2>), dim3(grid), dim3(waves * 64), lds, stream, p);
+    auto go = [&](auto fuse) {
+        constexpr int F = decltype(fuse)::value;
+        if (single_set) hipLaunchKernelGGL((acc4_packed_kernel<BS, ST, 1, F>), dim3(grid), dim3(waves * 64), lds, stream, p);
+        else hipLaunchKernelGGL((acc4_packed_kernel<BS, ST, 2, F>), dim3(grid), dim3(waves * 64), lds, stream, p);
+    };
+    if (fuse == 1) go(std::integral_constant<int, 1>{});
+    else if (fuse == 2) go(std::integral_constant<int, 2>{});
+    else go(std::integral_constant<int, 0>{});
     return static_cast<int>(hipGetLastError());
 }
 
@@ -897,12 +972,23 @@ extern "C" int rocm_acc4_packed_eligible(const RocmMatMulNBitsArgs* a)
     return static_cast<int64_t>(mnb::packed_groups(a)) * mnb::packed_chunk_bytes(a) < 0x7fffffff;
 }
 
-extern "C" int rocm_launch_acc4_packed(const RocmMatMulNBitsArgs* a, const void* packed, const RocmAcc4Workspace* ws, int waves, rocm_stream_t stream)
+extern "C" int rocm_acc4_packed_fuses_quantizer(const RocmMatMulNBitsArgs* a)
+{
+    return rocm_acc4_packed_eligible(a) && (a->a_dtype == ROCM_DT_F16 || a->a_dtype == ROCM_DT_BF16) && a->k % 8 == 0 &&
+           (reinterpret_cast<uintptr_t>(a->a) & 15) == 0;
+}
+
+extern "C" int rocm_launch_acc4_packed(const RocmMatMulNBitsArgs* a, const void* packed, const RocmAcc4Workspace* ws, int rounding, int waves, rocm_stream_t stream)
 {
     if (!rocm_acc4_packed_eligible(a)) return -1;
+    const int fuse = ws ? 0 : (a->a_dtype == ROCM_DT_BF16 ? 2 : 1);
+    if (!ws && !rocm_acc4_packed_fuses_quantizer(a)) return -1;
     mnb::Acc4PackedParams p;
-    p.qa = ws->qa;
-    p.aq = ws->aq;
+    p.qa = ws ? ws->qa : nullptr;
+    p.aq = ws ? ws->aq : nullptr;
+    p.a = a->a;
+    p.k = a->k;
+    p.rounding = rounding;
     p.packed = static_cast<const uint8_t*>(packed);
     p.bias = a->bias;
     p.y = a->y;
@@ -939,8 +1025,8 @@ extern "C" int rocm_launch_acc4_packed(const RocmMatMulNBitsArgs* a, const void*
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool f32_scales = a->scale_dtype == ROCM_DT_F32;
     switch (a->block_size) {
-        case 32: return f32_scales ? mnb::launch_acc4_packed<32, float>(p, w, single_set, s) : mnb::launch_acc4_packed<32, uint16_t>(p, w, single_set, s);
-        case 64: return f32_scales ? mnb::launch_acc4_packed<64, float>(p, w, single_set, s) : mnb::launch_acc4_packed<64, uint16_t>(p, w, single_set, s);
-        default: return f32_scales ? mnb::launch_acc4_packed<128, float>(p, w, single_set, s) : mnb::launch_acc4_packed<128, uint16_t>(p, w, single_set, s);
+        case 32: return f32_scales ? mnb::launch_acc4_packed<32, float>(p, w, single_set, fuse, s) : mnb::launch_acc4_packed<32, uint16_t>(p, w, single_set, fuse, s);
+        case 64: return f32_scales ? mnb::launch_acc4_packed<64, float>(p, w, single_set, fuse, s) : mnb::launch_acc4_packed<64, uint16_t>(p, w, single_set, fuse, s);
+        default: return f32_scales ? mnb::launch_acc4_packed<128, float>(p, w, single_set, fuse, s) : mnb::launch_acc4_packed<128, uint16_t>(p, w, single_set, fuse, s);
     }
 }
