@@ -352,26 +352,45 @@ struct PrefillPlan {
     int steps_per_split;
 };
 
-// The largest tile that still gives every CU a workgroup: 256 x 256, then 256 x 128, 128 x 128, 128 x 64. If even the
-// smallest leaves CUs idle and K is long, K is cut into slices (at least 8 steps each) until the grid covers the chip.
+// The largest tile that still gives every CU a workgroup: 256 x 256, then 256 x 128, 128 x 128. If 128 x 128 tiles leave
+// CUs idle, K is cut into slices over grid.z (measured at M = 512: 18944 -> 3584 113 us against 134 us with 128 x 64
+// tiles in slices; 14336 -> 4096 106 against 111 us); shapes too short for that take 128 x 64 tiles, sliced if they can be.
 PrefillPlan plan_prefill(const RocmMatMulNBitsArgs* a, int tile_choice, uint64_t scratch_bytes)
 {
-    const int64_t wg_huge = ((a->m + 255) / 256) * ((a->n + 255) / 256);
-    const int64_t wg_big = ((a->m + 255) / 256) * ((a->n + 127) / 128);
-    const int64_t wg_small = ((a->m + 127) / 128) * ((a->n + 127) / 128);
-    PrefillPlan plan;
-    plan.tile = (a->m >= 256 && wg_huge >= 256) ? 2 : (a->m >= 256 && wg_big >= 256) ? 1 : wg_small >= 256 ? 0 : 3;
-    if (tile_choice >= 1 && tile_choice <= 4) plan.tile = tile_choice == 4 ? 3 : tile_choice - 1;
     const int steps = static_cast<int>(a->k / 64);
-    plan.splits = 1;
-    if (plan.tile == 3) {
-        const int64_t wgs = ((a->m + 127) / 128) * ((a->n + 63) / 64);
+    const uint64_t per_split = static_cast<uint64_t>(a->m) * static_cast<uint64_t>(a->n) * 4;
+    auto workgroups = [&](int tile) {
+        const int bm = (tile == 1 || tile == 2) ? 256 : 128;
+        const int bn = tile == 2 ? 256 : tile == 3 ? 64 : 128;
+        return ((a->m + bm - 1) / bm) * ((a->n + bn - 1) / bn);
+    };
+    // slices of K that bring a short grid to about 1.5 workgroups per CU: at least 8 steps each, at most 16, and never
+    // more than the scratch holds
+    auto slices = [&](int tile) {
+        const int64_t wgs = workgroups(tile);
         int want = static_cast<int>((384 + wgs - 1) / wgs);
         if (want > steps / 8) want = steps / 8;
         if (want > 16) want = 16;
-        const uint64_t per_split = static_cast<uint64_t>(a->m) * static_cast<uint64_t>(a->n) * 4;
-        while (want > 1 && static_cast<uint64_t>(want) * per_split > scratch_bytes) --want;   // never more than the scratch holds
-        if (want > 1) plan.splits = want;
+        while (want > 1 && static_cast<uint64_t>(want) * per_split > scratch_bytes) --want;
+        return want < 1 ? 1 : want;
+    };
+    PrefillPlan plan;
+    plan.splits = 1;
+    if (tile_choice >= 1 && tile_choice <= 4) {
+        plan.tile = tile_choice == 4 ? 3 : tile_choice - 1;
+        plan.splits = slices(plan.tile);
+    } else if (a->m >= 256 && workgroups(2) >= 256) {
+        plan.tile = 2;
+    } else if (a->m >= 256 && workgroups(1) >= 256) {
+        plan.tile = 1;
+    } else if (workgroups(0) >= 256) {
+        plan.tile = 0;
+    } else if (a->m >= 512 && workgroups(0) * slices(0) >= 256) {
+        plan.tile = 0;                       // few tiles of Y but a long K: 128 x 128 tiles over slices of K (below 512 rows 128 x 64 is ahead)
+        plan.splits = slices(0);
+    } else {
+        plan.tile = 3;
+        plan.splits = slices(3);
     }
     plan.steps_per_split = (steps + plan.splits - 1) / plan.splits;
     plan.splits = (steps + plan.steps_per_split - 1) / plan.steps_per_split;
