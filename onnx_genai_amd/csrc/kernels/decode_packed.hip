@@ -413,8 +413,12 @@ constexpr int kWideWaves = 8;
 
 // RB: blocks of 16 rows (1, 2 or 4). A window is WT tiles of 128 k: a whole tile group for RB <= 2, half of one for
 // RB = 4, so that two buffers of RB * 16 rows stay within 66 KB.
-template <bool BF16, int BS, typename ST, int RB>
-__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu((BS == 128 && sizeof(ST) == 2 && RB == 1) ? 5 : 1)))
+// SUMS: offset and zero point leave through the block activation sums (one FMA per accumulator and block) instead of a
+// second MFMA per 32 elements. Fewer matrix-core cycles, but 95 registers instead of 80 at 16 rows: launches with
+// several workgroups per CU run better with the sixth wave per SIMD (3584 -> 152064 at 16 rows: 59 against 64 us), the
+// others with the sums (3584 -> 37888: 22.9 against 24.5 us).
+template <bool BF16, int BS, typename ST, int RB, bool SUMS>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu((BS == 128 && sizeof(ST) == 2 && RB == 1) ? (SUMS ? 5 : 6) : 1)))
 void decode_wide_kernel(PackedParams p)
 {
     constexpr int U = kGroupTiles;
@@ -430,6 +434,7 @@ void decode_wide_kernel(PackedParams p)
     constexpr int kPieces = WT * 16;                    // 16-byte pieces per row of a window
     constexpr int NW = kRows * kPieces / 512;           // pieces per thread per window (2 or 4)
     constexpr float kMagicF = BF16 ? 128.0f : 1024.0f;
+    constexpr uint32_t kMagicNeg = BF16 ? 0xC300C300u : 0xE400E400u;
     constexpr int kBlockLanes = BS / 8;                 // consecutive threads whose pieces make up one block of a row
     constexpr int kWinBlocks = WT * NBT;                // blocks per window
     constexpr int kSumBytes = kWinBlocks * kRows * 4;
@@ -494,8 +499,10 @@ void decode_wide_kernel(PackedParams p)
             const int q = t + 512 * i;
             const int row = q / kPieces, piece = q % kPieces;
             *reinterpret_cast<uint4*>(smem + buf * kBufBytes + row * kPitch + piece * 16) = wa[i];
-            const float sum = block_sum<BS>(sum_piece<BF16>(wa[i]));      // a block's pieces sit in consecutive lanes
-            if (piece % kBlockLanes == 0) lds_sums[(buf * kWinBlocks + piece / kBlockLanes) * kRows + row] = sum;
+            if constexpr (SUMS) {
+                const float sum = block_sum<BS>(sum_piece<BF16>(wa[i]));      // a block's pieces sit in consecutive lanes
+                if (piece % kBlockLanes == 0) lds_sums[(buf * kWinBlocks + piece / kBlockLanes) * kRows + row] = sum;
+            }
         }
     };
     // tiles [first, first + WT) of the group against window buffer `buf`
@@ -532,20 +539,29 @@ void decode_wide_kernel(PackedParams p)
                         const uint32_t raw = (rr[bi / 2] >> ((bi % 2) * 16)) & 0xffffu;
                         sf = BF16 ? __uint_as_float(raw << 16) : f16_bits_to_f32(static_cast<uint16_t>(raw));
                     }
-                    off = kMagicF + static_cast<float>((rr[zbyte / 4] >> ((zbyte % 4) * 8)) & 0xffu);
+                    if constexpr (SUMS) off = kMagicF + static_cast<float>((rr[zbyte / 4] >> ((zbyte % 4) * 8)) & 0xffu);
                 }
+                const uint32_t zpair = kMagicNeg | (((rr[zbyte / 4] >> ((zbyte % 4) * 8)) & 0xffu) * 0x00010001u);
+                const uint4 zc = make_uint4(zpair, zpair, zpair, zpair);       // used without SUMS only
                 const int wb = x * NBT + (j * 32) / BS;                // block of the window
 #pragma unroll
                 for (int rb = 0; rb < RB; ++rb) {
                     const uint4 av = *reinterpret_cast<const uint4*>(fa + rb * 16 * kPitch + j * 64);
                     acc[rb] = mfma16p<BF16>(av, op, acc[rb]);
+                    if constexpr (!SUMS) acc[rb] = mfma16p<BF16>(av, zc, acc[rb]);
                     if (last) {
-                        // this lane's accumulator rows are rows rb * 16 + 4 g + r of the window
-                        const float4 sa = *reinterpret_cast<const float4*>(lds_sums + (buf * kWinBlocks + wb) * kRows + rb * 16 + 4 * g);
-                        const float sav[4] = {sa.x, sa.y, sa.z, sa.w};
+                        float sav[4] = {0.f, 0.f, 0.f, 0.f};
+                        if constexpr (SUMS) {
+                            // this lane's accumulator rows are rows rb * 16 + 4 g + r of the window
+                            const float4 sa = *reinterpret_cast<const float4*>(lds_sums + (buf * kWinBlocks + wb) * kRows + rb * 16 + 4 * g);
+                            sav[0] = sa.x;
+                            sav[1] = sa.y;
+                            sav[2] = sa.z;
+                            sav[3] = sa.w;
+                        }
 #pragma unroll
                         for (int r = 0; r < 4; ++r) {
-                            y[rb][r] = fmaf(sf, fmaf(-off, sav[r], acc[rb][r]), y[rb][r]);
+                            y[rb][r] = fmaf(sf, SUMS ? fmaf(-off, sav[r], acc[rb][r]) : acc[rb][r], y[rb][r]);
                             acc[rb][r] = 0.f;
                         }
                     }
@@ -605,10 +621,13 @@ static int launch_wide_bs(const PackedParams& p, int bs, hipStream_t stream)
         constexpr int BS = decltype(bs_tag)::value;
         // two window buffers of rows x (tiles x 256 + 16) bytes, then two tables of (blocks per window) x rows f32 sums
         constexpr int NBT = 128 / BS;
-        if (p.m <= 16) return go(decode_wide_kernel<BF16, BS, ST, 1>, 2 * 16 * (4 * 256 + 16) + 2 * 4 * NBT * 16 * 4);
-        if (p.m <= 32) return go(decode_wide_kernel<BF16, BS, ST, 2>, 2 * 32 * (4 * 256 + 16) + 2 * 4 * NBT * 32 * 4);
+        if (p.m <= 16) {
+            if (grid.x >= 768) return go(decode_wide_kernel<BF16, BS, ST, 1, false>, 2 * 16 * (4 * 256 + 16));      // three or more workgroups per CU
+            return go(decode_wide_kernel<BF16, BS, ST, 1, true>, 2 * 16 * (4 * 256 + 16) + 2 * 4 * NBT * 16 * 4);
+        }
+        if (p.m <= 32) return go(decode_wide_kernel<BF16, BS, ST, 2, true>, 2 * 32 * (4 * 256 + 16) + 2 * 4 * NBT * 32 * 4);
         if constexpr (BS == 32) return -1;
-        else return go(decode_wide_kernel<BF16, BS, ST, 4>, 2 * 64 * (2 * 256 + 16) + 2 * 2 * NBT * 64 * 4);
+        else return go(decode_wide_kernel<BF16, BS, ST, 4, true>, 2 * 64 * (2 * 256 + 16) + 2 * 2 * NBT * 64 * 4);
     };
     switch (bs) {
         case 32: return by_rows(std::integral_constant<int, 32>{});
