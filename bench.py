@@ -365,19 +365,25 @@ def sweep(ep, nodes, a_bufs, args):
     by_shape = {}
     for n in nodes:
         by_shape.setdefault(n.name.split(".")[0], []).append(n)
+    # A shape with one buffer in the stack (lm_head) gets two more over distinct device memory for this table: replaying
+    # one 290 MB buffer would let the 256 MB last-level cache serve part of it.
+    extra = []
+    for shape, group in by_shape.items():
+        while len(group) < 3:
+            first = group[0]
+            clone = Node(ep, "%s.copy%d" % (shape, len(group)), first.k, first.n, BS, 7000 + len(group), A_DT, first.m)
+            clone.host_b = None
+            group.append(clone)
+            extra.append(clone)
     for m in (1, 4, 8, 16):
         a_m = {k: ep.upload(synth.make_activation(m, k, 6, A_DT)) for k in (HIDDEN, INTER)}
         for shape, group in by_shape.items():
-            group = list(group)
-            if shape == "lm_head":
-                pass
             saved = [(g.m, g.y) for g in group]
-            ys = []
             for g in group:
                 g.m = m
                 g.y = ep.allocate(m * g.n * 2)
-                ys.append(g.y)
-            group[0].run(a_m[group[0].k])
+            for g in group:
+                g.run(a_m[g.k])                    # first call of a kernel object: repacks its weights (never under capture)
             ep.sync()
             graph = capture(ep, lambda: [g.run(a_m[g.k]) for g in group])
             ms = time_graph(ep, graph, 20, 3)
@@ -392,6 +398,8 @@ def sweep(ep, nodes, a_bufs, args):
                 g.m, g.y = m0, y0
         for buf in a_m.values():
             ep.deallocate(buf)
+    for clone in extra:
+        clone.free(ep)
     return table
 
 
