@@ -31,8 +31,12 @@ typedef struct NxrtRocmMatMulNBits NxrtRocmMatMulNBits;   /* one kernel = one Ma
 /* ---- ExecutionProvider (crates/onnx-runtime-ep-api/src/provider.rs:708-1600) ------------------ */
 
 /* initialize(&EpConfig) — provider.rs:93 (string map). keys/values: n_config NUL-terminated pairs.
- * Known keys: "acc4_rounding" = "mlas" (ties to even, default) | "native" (ties away);
- *             "decode_waves", "decode_col_groups" = launch overrides for the decode GEMV. */
+ * Known keys: "acc4_rounding" = "mlas" (ties to even, default) | "native" (ties away) | "auto" (native below
+ *             "acc4_native_below" rows, else mlas: the CPU provider's route, matmul_nbits.rs:640-660);
+ *             "prepack" = "1" (default: constant weights are copied once into the decode kernels' streaming order) | "0";
+ *             "decode_waves", "decode_col_groups", "prefill_tile" = launch overrides (tests, tuning).
+ * The same settings are read from NXRT_ROCM_ACC4_ROUNDING, NXRT_SQNBIT_DECODE_MIN, NXRT_ROCM_PREPACK,
+ * NXRT_ROCM_DECODE_WAVES, NXRT_ROCM_DECODE_COL_GROUPS, NXRT_ROCM_PREFILL_TILE when the map does not give them. */
 NxrtStatus nxrt_rocm_ep_create(uint32_t device_ordinal, const char* const* config_keys,
                                const char* const* config_values, uint32_t n_config, NxrtRocmEp** out_ep);
 /* shutdown + drop. Frees the stream and every buffer the provider still owns. */
