@@ -480,6 +480,9 @@ ACC4_CASES = [
     (E.F16, 32, False, 7, 130, 4096),
     (E.F16, 128, True, 1, 512, 8192),
     (E.BF16, 128, True, 9, 100, 128 * 5 + 64),
+    (E.BF16, 32, True, 1, 100, 32 * 11),      # one bf16 row: quantized inside the kernel, blocks of 4 lanes
+    (E.BF16, 128, False, 1, 64, 1024),
+    (E.F16, 32, False, 1, 48, 4100),          # K % 8 != 0: the separate quantizer serves the row
     # M > 16: tiled int8 MFMA kernel
     (E.F16, 64, True, 130, 200, 64 * 9),      # ragged M and N tiles
     (E.F16, 32, True, 33, 64, 32 * 7),        # K ends in the middle of a 64-code step
