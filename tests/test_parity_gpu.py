@@ -290,6 +290,70 @@ def test_row_blocks_through_the_decode_kernels(ep, ep_unpacked, port, prepack, m
     assert np.array_equal(np.asarray(y).view(np.uint16), np.asarray(port.narrow(y32, a_dt)).view(np.uint16))
 
 
+GRAPH_CASES = [
+    # a_dt, bs, accuracy_level, m, n, k, what runs
+    (E.BF16, 128, 0, 1, 300, 3584),        # one-row decode over the repacked stream
+    (E.BF16, 128, 0, 8, 16400, 1024),      # shared-activation decode
+    (E.F16, 32, 0, 40, 200, 1024),         # tiled kernel
+    (E.F16, 64, 0, 100, 130, 4096),        # tiled kernel over slices of K: partial sums in the kernel's own scratch + reduce
+    (E.F32, 32, 0, 3, 100, 1000),          # f32 activations
+    (E.F16, 64, 4, 1, 160, 1024),          # accuracy_level 4, one row: quantized inside the kernel, no workspace
+    (E.F16, 64, 4, 5, 96, 512),            # accuracy_level 4 with the caller's workspace: quantizer + int8 MFMA
+    (E.F16, 64, 4, 130, 200, 576),
+]
+
+
+@pytest.mark.parametrize("a_dt,bs,acc,m,n,k", GRAPH_CASES)
+def test_graph_replays_match_eager(ep, a_dt, bs, acc, m, n, k):
+    """A call recorded into a HIP graph gives, on every replay, bit for bit what the eager call gave - with other eager
+    work and synchronisations between the replays, and after the input has changed."""
+    s_dt = a_dt
+    b, s, zp = synth.make_weights(n, k, bs, 61 + n, zero_points=True, scale_lo=0.002, scale_hi=0.01, scale_dtype=s_dt)
+    ops = E.DeviceOperands(ep, b, s, s_dt, zp, n, k, bs, accuracy_level=acc, rows=m, a_dtype=a_dt)
+    y_dt = a_dt
+    elem = 4 if y_dt == E.F32 else 2
+    np_y = np.float32 if y_dt == E.F32 else np.uint16
+    inputs = [synth.make_activation(m, k, 70 + i, a_dt) for i in range(3)]
+    ab, yb = ep.upload(inputs[0]), ep.allocate(m * n * elem)
+    scratch_y = ep.allocate(m * n * elem)
+    workspace = None
+    if acc == 4:
+        need, _ = ops.kernel.workspace_requirement([((m, k), a_dt)])
+        workspace = ep.allocate(need)
+    out = [E.TensorView(yb.ptr, y_dt, (m, n), device_index=ep.device_index)]
+    other = [E.TensorView(scratch_y.ptr, y_dt, (m, n), device_index=ep.device_index)]
+
+    def run(target):
+        ops.kernel.execute(ops.views(ab, a_dt, m), target, workspace=workspace)
+
+    eager = []
+    for a in inputs:                                   # eager results for each input (the first call also repacks / allocates)
+        ep.copy_from_host(ab, a)
+        run(out)
+        eager.append(ep.download(yb, (m, n), np_y).copy())
+    ep.sync()
+    ep.capture_begin()
+    try:
+        run(out)
+    finally:
+        graph = ep.capture_end()
+    try:
+        for i, a in enumerate(inputs):
+            ep.copy_from_host(ab, a)
+            run(other)                                 # eager work of the same kernel object between replays
+            ep.sync()
+            ep.copy_from_host(yb, np.full(m * n * elem, 0xFF, np.uint8))     # a replay must overwrite all of Y
+            graph.replay()
+            got = ep.download(yb, (m, n), np_y)
+            assert np.array_equal(got.view(np.uint8), eager[i].view(np.uint8)), "replay %d differs from the eager result" % i
+    finally:
+        graph.release()
+        for buf in (ab, yb, scratch_y, workspace):
+            if buf is not None:
+                ep.deallocate(buf)
+        ops.free()
+
+
 def test_packed_copy_follows_the_weights(ep, port):
     """One kernel object, two different weight tensors in turn: the repacked copy is rebuilt when the pointers change."""
     a_dt, bs, m, n, k = E.F16, 128, 1, 96, 1024
