@@ -199,6 +199,8 @@ void decode_packed_kernel(PackedParams p)
     // what the few-wave launches are sensitive to (measured: 3584 -> 37888 16.4 against 17.0 us and 3584 -> 152064 54.5
     // against 59 us with the sums; 18944 -> 3584 12.2 against 11.4 us, so not there).
     constexpr bool SUMS = MR == 1 && SETS == 1;
+    // With one row staged every accumulator row is a copy of row 0: only component 0 is scaled and reduced.
+    constexpr int kRowsKept = MR == 1 ? 1 : 4;
     constexpr int kBlockLanes = BS / 8;         // lanes whose 16-byte pieces make up one block
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
@@ -302,13 +304,13 @@ void decode_packed_kernel(PackedParams p)
                     const float off = kMagicF + static_cast<float>(z);
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
-                        y[r] = fmaf(sf, fmaf(-off, sa, acc[r]), y[r]);      // the product is not rounded on its own
+                        if (r < kRowsKept) y[r] = fmaf(sf, fmaf(-off, sa, acc[r]), y[r]);      // the product is not rounded on its own
                         acc[r] = 0.f;
                     }
                 } else {
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
-                        y[r] = fmaf(sf, acc[r], y[r]);
+                        if (r < kRowsKept) y[r] = fmaf(sf, acc[r], y[r]);
                         acc[r] = 0.f;
                     }
                 }
@@ -351,9 +353,9 @@ void decode_packed_kernel(PackedParams p)
     __syncthreads();
     float* red = reinterpret_cast<float*>(smem);       // [waves][4][64]
 #pragma unroll
-    for (int r = 0; r < 4; ++r) red[(wave * 4 + r) * 64 + lane] = y[r];
+    for (int r = 0; r < kRowsKept; ++r) red[(wave * 4 + r) * 64 + lane] = y[r];
     __syncthreads();
-    for (int idx = threadIdx.x; idx < 256; idx += blockDim.x) {
+    for (int idx = threadIdx.x; idx < kRowsKept * 64; idx += blockDim.x) {
         const int r = idx >> 6;
         const int l = idx & 63;
         const int row = 4 * (l >> 4) + r;
