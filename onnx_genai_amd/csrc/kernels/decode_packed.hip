@@ -758,14 +758,18 @@ __global__ __launch_bounds__(512) void acc4_packed_kernel(Acc4PackedParams p)
             sa_lane = __fdiv_rn(vmax, 127.0f);
             const float inv = vmax != 0.0f ? __fdiv_rn(127.0f, vmax) : 0.0f;
             int q[8], sum = 0;
+            auto round_all = [&](auto away) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const float scaled = __fmul_rn(v[i], inv);
-                float r = p.rounding == 1 ? roundf(scaled) : rintf(scaled);
-                r = fminf(fmaxf(r, -127.0f), 127.0f);
-                q[i] = static_cast<int>(r);
-                sum += q[i];
-            }
+                for (int i = 0; i < 8; ++i) {
+                    const float scaled = __fmul_rn(v[i], inv);
+                    float r = decltype(away)::value ? roundf(scaled) : rintf(scaled);
+                    r = fminf(fmaxf(r, -127.0f), 127.0f);
+                    q[i] = static_cast<int>(r);
+                    sum += q[i];
+                }
+            };
+            if (p.rounding == 1) round_all(std::true_type{});      // wave-uniform: one branch per group, not one select per element
+            else round_all(std::false_type{});
             sum = dpp_addi<0xB1>(sum);
             sum = dpp_addi<0x4E>(sum);
             if constexpr (BS >= 64) sum = dpp_addi<0x141>(sum);
@@ -802,22 +806,21 @@ __global__ __launch_bounds__(512) void acc4_packed_kernel(Acc4PackedParams p)
                 acc = __builtin_amdgcn_mfma_i32_16x16x32_i8(av[j], static_cast<long>(bw), first ? zero : acc, 0, 0, 0);
                 if (last) {
                     const int bi = u * NBT + (j * 32) / BS;
-                    if (static_cast<int64_t>(gi) * NB + bi < p.kb) {          // a block beyond K (wave-uniform)
-                        const int zbyte = NB * static_cast<int>(sizeof(ST)) + bi;
-                        const float zf = static_cast<float>((rr[zbyte / 4] >> ((zbyte % 4) * 8)) & 0xffu);
-                        float sb;
-                        if constexpr (sizeof(ST) == 4) {
-                            sb = __uint_as_float(rr[bi]);
-                        } else {
-                            const uint32_t raw = (rr[bi / 2] >> ((bi % 2) * 16)) & 0xffffu;
-                            sb = bf16_scales ? __uint_as_float(raw << 16) : f16_bits_to_f32(static_cast<uint16_t>(raw));
-                        }
-                        const int src = FUSE ? bi * kBlockLanes : bi;         // a lane of the block, or the lane that loaded its pair
-                        const float sa = __int_as_float(__builtin_amdgcn_readlane(FUSE ? __float_as_int(sa_lane) : static_cast<int>(grp.x.x), src));
-                        const float qs = __int_as_float(__builtin_amdgcn_readlane(FUSE ? __float_as_int(qs_lane) : static_cast<int>(grp.x.y), src));
-                        const float f = fmaf(-zf, qs, static_cast<float>(acc[0]));   // both terms are integers below 2^24: exact
-                        y = fmaf(f, __fmul_rn(sa, sb), y);
+                    // (a block beyond K needs no guard: its repacked scale is 0 and its codes and sums are 0)
+                    const int zbyte = NB * static_cast<int>(sizeof(ST)) + bi;
+                    const float zf = static_cast<float>((rr[zbyte / 4] >> ((zbyte % 4) * 8)) & 0xffu);
+                    float sb;
+                    if constexpr (sizeof(ST) == 4) {
+                        sb = __uint_as_float(rr[bi]);
+                    } else {
+                        const uint32_t raw = (rr[bi / 2] >> ((bi % 2) * 16)) & 0xffffu;
+                        sb = bf16_scales ? __uint_as_float(raw << 16) : f16_bits_to_f32(static_cast<uint16_t>(raw));
                     }
+                    const int src = FUSE ? bi * kBlockLanes : bi;         // a lane of the block, or the lane that loaded its pair
+                    const float sa = __int_as_float(__builtin_amdgcn_readlane(FUSE ? __float_as_int(sa_lane) : static_cast<int>(grp.x.x), src));
+                    const float qs = __int_as_float(__builtin_amdgcn_readlane(FUSE ? __float_as_int(qs_lane) : static_cast<int>(grp.x.y), src));
+                    const float f = fmaf(-zf, qs, static_cast<float>(acc[0]));   // both terms are integers below 2^24: exact
+                    y = fmaf(f, __fmul_rn(sa, sb), y);
                 }
             }
         }
