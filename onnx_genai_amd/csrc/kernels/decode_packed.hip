@@ -210,7 +210,6 @@ void decode_packed_kernel(PackedParams p)
     const int c = lane & 15;
     const int g = lane >> 4;
     const int64_t n_base = static_cast<int64_t>(blockIdx.x) * 16;
-    const bool full_k = (p.k & 127) == 0;
 
     const __amdgpu_buffer_rsrc_t srd_p = make_srd(p.packed + static_cast<int64_t>(blockIdx.x) * p.cg_stride, static_cast<uint64_t>(p.cg_stride));
     const __amdgpu_buffer_rsrc_t srd_a = make_srd(p.a, static_cast<uint64_t>(p.m * p.k) * 2);
@@ -232,27 +231,31 @@ void decode_packed_kernel(PackedParams p)
     const int g_end = min(g_begin + p.groups_per_wave, p.groups);
 
     using Grp = PackedGroup<NR, NA>;
+    // No branch in here: a group past the wave's last one (the prefetch of the final iteration) gets every offset out of
+    // range, which fetches nothing and returns zeros - weights 0, scale 0, activations 0: a group that adds nothing.
+    // With a branch instead, the compiler waits for all loads in flight at the next use, the prefetch included.
     auto fetch_group = [&](Grp& grp, int gi) {
-        if (gi >= g_end) return;
+        const uint32_t oor = gi < g_end ? 0u : kOutOfRange;        // or-ed in: any offset with these bits is out of range
         const uint32_t soff = static_cast<uint32_t>(gi) * static_cast<uint32_t>(p.chunk_bytes);
-#pragma unroll
-        for (int u = 0; u < U; ++u) grp.w[u] = load16(srd_p, w_off + static_cast<uint32_t>(u * 1024), soff);
-#pragma unroll
-        for (int i = 0; i < NR; ++i) grp.r[i] = load16(srd_p, r_off + static_cast<uint32_t>(i * 16), soff);
         const int t0 = gi * U;
-        if constexpr (MR == 1) {
-            uint32_t off = a_off;
-            if (!full_k && static_cast<int64_t>(t0 + g) * 128 + c * 8 + 8 > p.k) off = kOutOfRange;
-            grp.a[0] = load16(srd_a, off, static_cast<uint32_t>(t0) * 256u);
-        } else {
+        // every offset first, then the loads back to back: vector arithmetic between two loads can land in a register
+        // that an outstanding load still owns, and then waits for it
+        uint32_t a_voff[NA];
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                uint32_t off = a_off;
-                if (!full_k && static_cast<int64_t>(t0 + u) * 128 + c * 8 + 8 > p.k) off = kOutOfRange;
-                if (static_cast<int64_t>(t0 + u) * 128 >= p.k) off = kOutOfRange;      // a padding tile of the last group
-                grp.a[u] = load16(srd_a, off, static_cast<uint32_t>(t0 + u) * 256u);
-            }
+        for (int u = 0; u < NA; ++u) {
+            const int tile = MR == 1 ? t0 + g : t0 + u;
+            const bool beyond = static_cast<int64_t>(tile) * 128 + c * 8 + 8 > p.k;        // K is a multiple of 8: a piece is all in or all out
+            a_voff[u] = (beyond ? kOutOfRange : a_off) | oor;
         }
+        const uint32_t w_voff = w_off | oor, r_voff = r_off | oor;
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < U; ++u) grp.w[u] = load16(srd_p, w_voff + static_cast<uint32_t>(u * 1024), soff);
+#pragma unroll
+        for (int i = 0; i < NR; ++i) grp.r[i] = load16(srd_p, r_voff + static_cast<uint32_t>(i * 16), soff);
+#pragma unroll
+        for (int u = 0; u < NA; ++u) grp.a[u] = load16(srd_a, a_voff[u], static_cast<uint32_t>(MR == 1 ? t0 : t0 + u) * 256u);
+        __builtin_amdgcn_sched_barrier(0);
     };
     // `asum` (with SUMS): this lane's block sum of the group's tile lane / 16 (one load covers the group's four tiles).
     auto compute_tile = [&](const Grp& grp, int u, int parity, float asum) {
@@ -273,6 +276,10 @@ void decode_packed_kernel(PackedParams p)
             rr[4 * i + 2] = grp.r[i].z;
             rr[4 * i + 3] = grp.r[i].w;
         }
+        // Every dword of the record counts as used here, also the padding at its end: a destination register of a load
+        // that the compiler knows to be dead is handed out again at once, and writing it waits for the load in flight.
+#pragma unroll
+        for (int i = 0; i < NR * 4; ++i) asm volatile("" : : "v"(rr[i]));
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int bi = u * NBT + (j * 32) / BS;                          // block of the group (compile-time)
@@ -317,8 +324,11 @@ void decode_packed_kernel(PackedParams p)
             }
         }
     };
-    auto run_group = [&](const Grp& cur, Grp& next, int gi, int parity) {
-        fetch_group(next, gi + 1);
+    auto run_group = [&](const Grp& cur, Grp& next, int gi, int parity, bool prefetch) {
+        // Nothing of this group moves up into the previous one: its activation piece is the newest load in flight
+        // there, and staging it early would wait for every load, the prefetch included.
+        __builtin_amdgcn_sched_barrier(0);
+        if (prefetch) fetch_group(next, gi + 1);
         if constexpr (MR == 1) {
             *reinterpret_cast<uint4*>(stage + parity * kStageBytes + st_write) = cur.a[0];
             lds_order();
@@ -330,10 +340,13 @@ void decode_packed_kernel(PackedParams p)
     if constexpr (SETS == 2) {
         Grp ga, gb;
         fetch_group(ga, g_begin);
-        for (int gi = g_begin; gi < g_end; gi += 2) {
-            run_group(ga, gb, gi, 0);
-            if (gi + 1 < g_end) run_group(gb, ga, gi + 1, 1);
+        int gi = g_begin;
+        for (; gi + 1 < g_end; gi += 2) {                      // whole pairs, no branch inside: every wait counts loads exactly
+            run_group(ga, gb, gi, 0, true);
+            run_group(gb, ga, gi + 1, 1, true);                // past the end this prefetch fetches nothing
         }
+        if (gi < g_end) run_group(ga, gb, gi, 0, false);       // an odd group out
+
     } else {
         Grp ga;
         for (int gi = g_begin; gi < g_end; ++gi) {
@@ -716,18 +729,20 @@ __global__ __launch_bounds__(512) void acc4_packed_kernel(Acc4PackedParams p)
     const int g_end = min(g_begin + p.groups_per_wave, p.groups);
 
     using Grp = Acc4PackedGroup<NR>;
+    // No branch in here (a branch would make the compiler wait for every load in flight, the prefetch included): a group
+    // past the wave's last one gets every offset out of range, fetches nothing and reads as zeros - it adds nothing.
     auto fetch_group = [&](Grp& grp, int gi) {
-        if (gi >= g_end) return;
+        const uint32_t oor = gi < g_end ? 0u : kOutOfRange;        // or-ed in: any offset with these bits is out of range
         const uint32_t soff = static_cast<uint32_t>(gi) * static_cast<uint32_t>(p.chunk_bytes);
 #pragma unroll
-        for (int u = 0; u < U; ++u) grp.w[u] = load16(srd_p, w_off + static_cast<uint32_t>(u * 1024), soff);
+        for (int u = 0; u < U; ++u) grp.w[u] = load16(srd_p, (w_off + static_cast<uint32_t>(u * 1024)) | oor, soff);
 #pragma unroll
-        for (int i = 0; i < NR; ++i) grp.r[i] = load16(srd_p, r_off + static_cast<uint32_t>(i * 16), soff);
+        for (int i = 0; i < NR; ++i) grp.r[i] = load16(srd_p, (r_off + static_cast<uint32_t>(i * 16)) | oor, soff);
         if constexpr (FUSE) {
-            grp.a = load16(srd_a, static_cast<uint32_t>(lane * 16), static_cast<uint32_t>(gi) * 1024u);   // 8 activations; K % 8 == 0 and the range ends the row
+            grp.a = load16(srd_a, static_cast<uint32_t>(lane * 16) | oor, static_cast<uint32_t>(gi) * 1024u);   // 8 activations; K % 8 == 0 and the range ends the row
         } else {
-            grp.a = load16(srd_a, lane < 32 ? static_cast<uint32_t>(lane * 16) : kOutOfRange, static_cast<uint32_t>(gi) * 512u);   // the range ends the row at padded_k
-            const auto v = __builtin_amdgcn_raw_buffer_load_b64(srd_x, static_cast<int>(lane < NB ? lane * 8 : kOutOfRange), static_cast<int>(gi * NB * 8), 0);
+            grp.a = load16(srd_a, (lane < 32 ? static_cast<uint32_t>(lane * 16) : kOutOfRange) | oor, static_cast<uint32_t>(gi) * 512u);   // the range ends the row at padded_k
+            const auto v = __builtin_amdgcn_raw_buffer_load_b64(srd_x, static_cast<int>((lane < NB ? static_cast<uint32_t>(lane * 8) : kOutOfRange) | oor), static_cast<int>(gi * NB * 8), 0);
             grp.x = make_uint2(v[0], v[1]);
         }
     };
@@ -791,6 +806,10 @@ __global__ __launch_bounds__(512) void acc4_packed_kernel(Acc4PackedParams p)
             rr[4 * i + 2] = grp.r[i].z;
             rr[4 * i + 3] = grp.r[i].w;
         }
+        // every dword of the record counts as used, also its padding: a load destination known to be dead is handed out
+        // again at once, and writing it waits for the load in flight
+#pragma unroll
+        for (int i = 0; i < NR * 4; ++i) asm volatile("" : : "v"(rr[i]));
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             long av[4];
@@ -829,14 +848,19 @@ __global__ __launch_bounds__(512) void acc4_packed_kernel(Acc4PackedParams p)
     if constexpr (SETS == 2) {
         Grp ga, gb;
         fetch_group(ga, g_begin);
-        for (int gi = g_begin; gi < g_end; gi += 2) {
+        int gi = g_begin;
+        for (; gi + 1 < g_end; gi += 2) {                      // whole pairs, no branch inside: every wait counts loads exactly
+            __builtin_amdgcn_sched_barrier(0);                 // nothing of a group moves up into the one before it
             fetch_group(gb, gi + 1);
+            __builtin_amdgcn_sched_barrier(0);
             compute_group(ga, gi, 0);
-            if (gi + 1 < g_end) {
-                fetch_group(ga, gi + 2);
-                compute_group(gb, gi + 1, 1);
-            }
+            __builtin_amdgcn_sched_barrier(0);
+            fetch_group(ga, gi + 2);                           // past the end this fetches nothing
+            __builtin_amdgcn_sched_barrier(0);
+            compute_group(gb, gi + 1, 1);
         }
+        if (gi < g_end) compute_group(ga, gi, 0);              // an odd group out
+
     } else {
         Grp ga;
         for (int gi = g_begin; gi < g_end; ++gi) {
