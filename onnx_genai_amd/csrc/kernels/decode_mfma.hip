@@ -81,12 +81,12 @@ __device__ __forceinline__ uint4 unpack8(uint32_t w, uint32_t mask, uint32_t mag
 
 // One group of U tiles held in registers: packed weights of CG column groups, the activations in compact
 // form, scales and zero points. NA / NS count the activation / scale loads of a group (see the kernel).
-template <int U, int CG, int NA, int NS>
+template <int U, int CG, int NA, int NS, typename SRaw>
 struct Group {
     uint4 w[U][CG];
     uint4 a[NA];
-    uint32_t s[NS][CG];
-    uint32_t z[NS][CG];
+    SRaw s[NS][CG];             // as loaded; widened where used, so that nothing waits for the load before that
+    unsigned char z[NS][CG];
 };
 
 // BF16: activation element type. BS: block size (32, 64, 128). CG: 16-column groups per workgroup.
@@ -120,7 +120,6 @@ __global__ __launch_bounds__(512) void decode_mfma_kernel(DecodeParams p)
     const int64_t n_base = static_cast<int64_t>(blockIdx.x) * (16 * CG);
     const int64_t cols_left = p.n - n_base;
     const bool has_zp = p.zp != nullptr;
-    const bool full_k = (p.k & 127) == 0;
 
     const __amdgpu_buffer_rsrc_t srd_b = make_srd(p.b + n_base * p.row_bytes, static_cast<uint64_t>(cols_left * p.row_bytes));
     const __amdgpu_buffer_rsrc_t srd_s = make_srd(static_cast<const ST*>(p.scales) + n_base * p.kb, static_cast<uint64_t>(cols_left * p.kb) * sizeof(ST));
@@ -162,55 +161,61 @@ __global__ __launch_bounds__(512) void decode_mfma_kernel(DecodeParams p)
     const int t_begin = wave * p.tiles_per_wave;
     const int t_end = min(t_begin + p.tiles_per_wave, p.tiles);
 
-    using Grp = Group<U, CG, NA, NS>;
+    using Grp = Group<U, CG, NA, NS, typename ScaleIo<ST>::raw_t>;
+    const uint32_t zp_mask = has_zp ? 0xfu : 0u, zp_default = has_zp ? 0u : 8u;     // branch-free "8 when absent"
+    // No branch in here: a tile past the wave's range gets every offset out of range, which fetches nothing and returns
+    // zeros - weights 0, scale 0, activations 0, a tile that adds nothing. With branches around the loads the compiler
+    // waits for every load in flight at the next use, the prefetch included. All offsets first, then the loads back
+    // to back.
     auto fetch_group = [&](Grp& grp, int t0) {
-        if (t0 >= t_end) return;
+        uint32_t tile_oor[U];
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            if (t0 + u < t_end) {
-#pragma unroll
-                for (int cg = 0; cg < CG; ++cg) grp.w[u][cg] = load16(srd_b, b_off[cg], static_cast<uint32_t>(t0 + u) * 64u);
-            }
-        }
+        for (int u = 0; u < U; ++u) tile_oor[u] = t0 + u < t_end ? 0u : kOutOfRange;       // or-ed in: out of range
+        uint32_t a_voff[NA];
         if constexpr (kGroupA) {
-            uint32_t off = a_off;
-            if (g >= U || t0 + g >= t_end || (!full_k && static_cast<int64_t>(t0 + g) * 128 + c * 8 + 8 > p.k)) off = kOutOfRange;
-            grp.a[0] = load16(srd_a, off, static_cast<uint32_t>(t0) * 256u);
+            const bool out = g >= U || t0 + g >= t_end || static_cast<int64_t>(t0 + g) * 128 + c * 8 + 8 > p.k;
+            a_voff[0] = out ? kOutOfRange : a_off;
         } else {
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                if (t0 + u < t_end) {
+                const bool out = static_cast<int64_t>(t0 + u) * 128 + c * 8 + 8 > p.k || (MR < 4 && g >= MR);
 #pragma unroll
-                    for (int i = 0; i < AR; ++i) {
-                        uint32_t off = a_off + static_cast<uint32_t>(i) * a_row_step;
-                        if (!full_k && static_cast<int64_t>(t0 + u) * 128 + c * 8 + 8 > p.k) off = kOutOfRange;
-                        if (MR < 4 && g >= MR) off = kOutOfRange;
-                        grp.a[u * AR + i] = load16(srd_a, off, static_cast<uint32_t>(t0 + u) * 256u);
-                    }
-                }
+                for (int i = 0; i < AR; ++i) a_voff[u * AR + i] = (out ? kOutOfRange : a_off + static_cast<uint32_t>(i) * a_row_step) | tile_oor[u];
             }
+        }
+        const uint32_t group_oor = (g < U && t0 + g < t_end) ? 0u : kOutOfRange;           // per-group scales: lane group g fetches tile t0 + g's
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int cg = 0; cg < CG; ++cg) grp.w[u][cg] = load16(srd_b, b_off[cg] | tile_oor[u], static_cast<uint32_t>(t0 + u) * 64u);
+        if constexpr (kGroupA) {
+            grp.a[0] = load16(srd_a, a_voff[0], static_cast<uint32_t>(t0) * 256u);
+        } else {
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int i = 0; i < AR; ++i) grp.a[u * AR + i] = load16(srd_a, a_voff[u * AR + i], static_cast<uint32_t>(t0 + u) * 256u);
         }
         if constexpr (kGroupS) {
             // lane group g fetches scale and zero point of tile t0 + g (t0 is even, so the nibble is g & 1)
-            const bool mine = g < U && t0 + g < t_end;
 #pragma unroll
             for (int cg = 0; cg < CG; ++cg) {
-                grp.s[0][cg] = ScaleIo<ST>::load(srd_s, mine ? s_off[cg] : kOutOfRange, static_cast<uint32_t>(t0) * static_cast<uint32_t>(sizeof(ST)));
-                grp.z[0][cg] = has_zp ? static_cast<uint32_t>(__builtin_amdgcn_raw_buffer_load_b8(srd_z, static_cast<int>(mine ? z_off[cg] : kOutOfRange), static_cast<int>(t0 >> 1), 0)) : 0x88u;
+                grp.s[0][cg] = ScaleIo<ST>::load_raw(srd_s, s_off[cg] | group_oor, static_cast<uint32_t>(t0) * static_cast<uint32_t>(sizeof(ST)));
+                grp.z[0][cg] = __builtin_amdgcn_raw_buffer_load_b8(srd_z, static_cast<int>(z_off[cg] | group_oor), static_cast<int>(t0 >> 1), 0);
             }
         } else {
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                if (t0 + u < t_end) {
-                    const uint32_t blk0 = static_cast<uint32_t>(t0 + u) * kBlocksPerTile;
+                const uint32_t blk0 = static_cast<uint32_t>(t0 + u) * kBlocksPerTile;
 #pragma unroll
-                    for (int cg = 0; cg < CG; ++cg) {
-                        grp.s[u][cg] = ScaleIo<ST>::load(srd_s, s_off[cg], blk0 * static_cast<uint32_t>(sizeof(ST)));
-                        grp.z[u][cg] = has_zp ? static_cast<uint32_t>(__builtin_amdgcn_raw_buffer_load_b8(srd_z, static_cast<int>(z_off[cg]), static_cast<int>(blk0 >> 1), 0)) : 0x88u;
-                    }
+                for (int cg = 0; cg < CG; ++cg) {
+                    grp.s[u][cg] = ScaleIo<ST>::load_raw(srd_s, s_off[cg] | tile_oor[u], blk0 * static_cast<uint32_t>(sizeof(ST)));
+                    grp.z[u][cg] = __builtin_amdgcn_raw_buffer_load_b8(srd_z, static_cast<int>(z_off[cg] | tile_oor[u]), static_cast<int>(blk0 >> 1), 0);
                 }
             }
         }
+        __builtin_amdgcn_sched_barrier(0);
     };
     auto compute_tile = [&](const Grp& grp, int u, int parity) {
         // activations: compact registers -> LDS -> MFMA operand order
@@ -230,8 +235,8 @@ __global__ __launch_bounds__(512) void decode_mfma_kernel(DecodeParams p)
             if constexpr (kTranspose) transpose_groups(w);
             const uint32_t wd[4] = {w.x, w.y, w.z, w.w};
             // scale and zero-point nibble this lane fetched: of its own block (BS < 128) or of tile g (BS = 128)
-            const uint32_t z_lane = (grp.z[kGroupS ? 0 : u][cg] >> ((lane_blk & 1u) * 4u)) & 0xfu;
-            const uint32_t s_lane = grp.s[kGroupS ? 0 : u][cg];
+            const uint32_t z_lane = (((static_cast<uint32_t>(grp.z[kGroupS ? 0 : u][cg]) >> ((lane_blk & 1u) * 4u)) & 0xfu) & zp_mask) | zp_default;
+            const uint32_t s_lane = static_cast<uint32_t>(grp.s[kGroupS ? 0 : u][cg]);
             uint32_t z_tile = z_lane, s_tile = s_lane;
             if constexpr (kGroupS) {
                 z_tile = __shfl(z_lane, c + 16 * u, kWave);
@@ -260,23 +265,26 @@ __global__ __launch_bounds__(512) void decode_mfma_kernel(DecodeParams p)
             }
         }
     };
-    auto run_group = [&](const Grp& cur, Grp& next, int t0, int parity) {
-        fetch_group(next, t0 + U);
+    auto run_group = [&](const Grp& cur, Grp& next, int t0, int parity, bool prefetch) {
+        // nothing of this group moves up into the previous one (its loads are the newest in flight there)
+        __builtin_amdgcn_sched_barrier(0);
+        if (prefetch) fetch_group(next, t0 + U);
         if constexpr (kGroupA) {
             *reinterpret_cast<uint4*>(stage + parity * kStageBytes + st_write) = cur.a[0];
             lds_order();
         }
 #pragma unroll
-        for (int u = 0; u < U; ++u)
-            if (t0 + u < t_end) compute_tile(cur, u, parity);
+        for (int u = 0; u < U; ++u) compute_tile(cur, u, parity);        // a tile past the range is all zeros
     };
 
     Grp ga, gb;
     fetch_group(ga, t_begin);
-    for (int t0 = t_begin; t0 < t_end; t0 += 2 * U) {
-        run_group(ga, gb, t0, 0);
-        if (t0 + U < t_end) run_group(gb, ga, t0 + U, 1);
+    int t0 = t_begin;
+    for (; t0 + U < t_end; t0 += 2 * U) {                  // whole pairs of groups, no branch inside: every wait counts loads exactly
+        run_group(ga, gb, t0, 0, true);
+        run_group(gb, ga, t0 + U, 1, true);                // past the end this prefetch fetches nothing
     }
+    if (t0 < t_end) run_group(ga, gb, t0, 0, false);       // an odd group out
 
     // ---- split-K reduction across the waves of this workgroup, in wave order ----
     __syncthreads();                                   // every wave is done with its staging tiles
