@@ -402,7 +402,9 @@ __global__ __launch_bounds__(512) void acc4_prefill_kernel(Acc4PrefillParams p)
         const uint32_t zraw = static_cast<uint32_t>(__builtin_amdgcn_raw_buffer_load_b8(srd_z, static_cast<int>(z_goff + (blk >> 1)), 0, 0));
         r.z = zraw;                 // no arithmetic on a loaded value here: it would wait for the load at once
         r.zsh = (blk & 1u) * 4u;
-        r.sa = __builtin_amdgcn_raw_buffer_load_b32(srd_sa, static_cast<int>(sa_goff), static_cast<int>(block_of(kt, sa_slot * 32) * static_cast<uint32_t>(p.m) * 4u), 0);
+        // the block depends on the thread's slot, so it travels in the vector offset: as a scalar offset the compiler
+        // would loop over its distinct values (an out-of-range sa_goff stays out of range: kb * m * 4 < 2^31)
+        r.sa = __builtin_amdgcn_raw_buffer_load_b32(srd_sa, static_cast<int>(sa_goff + block_of(kt, sa_slot * 32) * static_cast<uint32_t>(p.m) * 4u), 0, 0);
     };
     // Half `part` of a step's trip from registers into LDS buffer `buf`.
     auto store_part = [&](const Regs& r, int buf, int part) {
