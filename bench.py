@@ -403,34 +403,47 @@ def sweep(ep, nodes, a_bufs, args):
     return table
 
 
+def prefill_routes(ep):
+    """The three ways a tall 16-bit call can run, each as its own provider: the hand-written tiled kernel only; the
+    default dispatch (from 1024 rows: weights expanded into one shared 16-bit buffer per call, then the library GEMM);
+    constant weights keeping a resident 16-bit copy (the call is the library GEMM alone)."""
+    return [("tiled", E.RocmExecutionProvider(0, {"dense_gemm_min_rows": "0"}), True), ("default", ep, False),
+            ("resident", E.RocmExecutionProvider(0, {"dense_weights": "resident"}), True)]
+
+
 def prefill_table(ep, shapes=((4096, 14336), (14336, 4096)), rows=(512, 2048, 8192), dtype=E.F16, bs=32, zero_points=False):
-    """Prefill GEMM. Defaults: Llama-3-8B MLP shapes (configs[3]): fp16, block 32, no zero points."""
+    """Prefill GEMM. Defaults: Llama-3-8B MLP shapes (configs[3]): fp16, block 32, no zero points. One row per route
+    that runs a different kernel sequence for the shape."""
     table = []
+    routes = prefill_routes(ep)
     for k, n in shapes:
         for m in rows:
-            node = Node(ep, "prefill", k, n, bs, 7, dtype, m, zero_points=zero_points, scale_range=(0.001, 0.01))
-            a = ep.upload(synth.make_activation(m, k, 8, dtype))
-            node.run(a)
-            ep.sync()
-            variant = node.ops.kernel.last_variant()
-            if not variant.startswith("prefill") and m > 512:      # the catch-all kernel is not a prefill path: one row of the table is enough
-                ep.deallocate(a)
-                node.free(ep)
-                continue
-            reps = 10 if variant.startswith("prefill") else 1
-            graph = capture(ep, lambda: node.run(a))
-            ms = time_graph(ep, graph, reps, 1)
-            graph.release()
-            tflops = node.flops / (ms * 1e-3) / 1e12
-            table.append({"k": k, "n": n, "m": m, "us": round(ms * 1e3, 1), "tflops": round(tflops, 1),
-                          "mfma_frac": round(tflops / MFMA_F16_PEAK_TFLOPS, 4), "variant": variant})
-            ep.deallocate(a)
-            node.free(ep)
+            seen = set()
+            for route, provider, _ in routes:
+                node = Node(provider, "prefill", k, n, bs, 7, dtype, m, zero_points=zero_points, scale_range=(0.001, 0.01))
+                a = provider.upload(synth.make_activation(m, k, 8, dtype))
+                node.run(a)
+                provider.sync()
+                variant = node.ops.kernel.last_variant()
+                tall = variant.startswith("prefill") or variant.startswith("dense")
+                if variant not in seen and (tall or m <= 512):   # the catch-all kernel is not a prefill path: one row of the table is enough
+                    seen.add(variant)
+                    graph = capture(provider, lambda: node.run(a))
+                    ms = time_graph(provider, graph, 10 if tall else 1, 1)
+                    graph.release()
+                    tflops = node.flops / (ms * 1e-3) / 1e12
+                    table.append({"k": k, "n": n, "m": m, "route": route, "us": round(ms * 1e3, 1), "tflops": round(tflops, 1),
+                                  "mfma_frac": round(tflops / MFMA_F16_PEAK_TFLOPS, 4), "variant": variant})
+                provider.deallocate(a)
+                node.free(provider)
+    for _, provider, owned in routes:
+        if owned:
+            provider.shutdown()
     return table
 
 
 def prefill_7b_table(ep):
-    """The same kernel at the Qwen2.5-7B shapes of the decode sweep: bf16, block 128, zero points, M = 4096."""
+    """The same routes at the Qwen2.5-7B shapes of the decode sweep: bf16, block 128, zero points, M = 4096."""
     return prefill_table(ep, shapes=((3584, 37888), (18944, 3584)), rows=(4096,), dtype=E.BF16, bs=128, zero_points=True)
 
 

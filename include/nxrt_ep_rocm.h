@@ -34,9 +34,17 @@ typedef struct NxrtRocmMatMulNBits NxrtRocmMatMulNBits;   /* one kernel = one Ma
  * Known keys: "acc4_rounding" = "mlas" (ties to even, default) | "native" (ties away) | "auto" (native below
  *             "acc4_native_below" rows, else mlas: the CPU provider's route, matmul_nbits.rs:640-660);
  *             "prepack" = "1" (default: constant weights are copied once into the decode kernels' streaming order) | "0";
+ *             "dense_gemm_min_rows" = rows from which a 16-bit call expands the weights to a dense [N, K] matrix and runs
+ *             the library GEMM ("0" = never; default 1024, or 256 with resident copies; the CUDA provider's
+ *             dequantize + cuBLASLt route, onnx-runtime-ep-cuda/src/kernels/matmul_nbits.rs:6176-6222);
+ *             "dense_gemm_max_mb" = largest dense copy of one weight (default 1024, as matmul_nbits.rs:6212);
+ *             "dense_weights" = "transient" (default: one buffer per provider, refilled by every such call) |
+ *             "resident" (a constant weight keeps its dense copy: 2 bytes per weight of HBM for a call that is the
+ *             GEMM alone);
  *             "decode_waves", "decode_col_groups", "prefill_tile" = launch overrides (tests, tuning).
  * The same settings are read from NXRT_ROCM_ACC4_ROUNDING, NXRT_SQNBIT_DECODE_MIN, NXRT_ROCM_PREPACK,
- * NXRT_ROCM_DECODE_WAVES, NXRT_ROCM_DECODE_COL_GROUPS, NXRT_ROCM_PREFILL_TILE when the map does not give them. */
+ * NXRT_ROCM_DENSE_GEMM_MIN_ROWS, NXRT_ROCM_DENSE_GEMM_MAX_MB, NXRT_ROCM_DENSE_WEIGHTS, NXRT_ROCM_DECODE_WAVES,
+ * NXRT_ROCM_DECODE_COL_GROUPS, NXRT_ROCM_PREFILL_TILE when the map does not give them. */
 NxrtStatus nxrt_rocm_ep_create(uint32_t device_ordinal, const char* const* config_keys,
                                const char* const* config_values, uint32_t n_config, NxrtRocmEp** out_ep);
 /* shutdown + drop. Frees the stream and every buffer the provider still owns. */

@@ -20,6 +20,7 @@ HIP_SOURCES = [
     "kernels/decode_mfma.hip",
     "kernels/decode_packed.hip",
     "kernels/prefill_mfma.hip",
+    "kernels/dense_gemm.hip",
     "kernels/acc4.hip",
     "kernels/acc4_mfma.hip",
 ]
@@ -53,7 +54,7 @@ def build(force: bool = True) -> str:
         jobs.append(["g++", *HOST_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj])
     with ThreadPoolExecutor(max_workers=8) as pool:
         list(pool.map(_run, jobs))
-    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs, "-Wl,-z,defs", "-Wl,--exclude-libs,ALL"])
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs, "-L/opt/rocm/lib", "-lhipblaslt", "-Wl,-z,defs", "-Wl,--exclude-libs,ALL"])
     return LIB
 
 

@@ -126,16 +126,20 @@ struct NxrtRocmMatMulNBits {
     void* packed = nullptr;              // constant B / scales / zero points in the decode kernel's streaming order
     const void* packed_from[3] = {nullptr, nullptr, nullptr};   // the tensors `packed` was made from
     int packed_scale_dtype = 0;
+    void* dense = nullptr;               // constant weights expanded to the activations' 16-bit type, [N, K] (dense_weights = resident)
+    const void* dense_from[3] = {nullptr, nullptr, nullptr};
+    int dense_dtype = 0, dense_scale_dtype = 0;
     std::mutex mu;                       // one execute at a time per kernel object: scratch, repacked copy and variant are per-object state
     NxrtKernelVtable vtable;
     uint32_t vt_a_dtype = 0, vt_scale_dtype = 0, vt_y_dtype = 0;
 
     ~NxrtRocmMatMulNBits()
     {
-        if ((scratch || packed) && ep && ep->bind().code == NXRT_OK) {
+        if ((scratch || packed || dense) && ep && ep->bind().code == NXRT_OK) {
             rocm_ffi_stream_sync(ep->stream);
             if (scratch) rocm_ffi_free(scratch);
             if (packed) rocm_ffi_free(packed);
+            if (dense) rocm_ffi_free(dense);
         }
     }
 };
@@ -183,6 +187,79 @@ bool use_packed(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& args, int& r
     kn.packed_from[1] = args.scales;
     kn.packed_from[2] = args.zp;
     kn.packed_scale_dtype = args.scale_dtype;
+    return true;
+}
+
+// Tall 16-bit calls: expand the weights to a dense [N, K] matrix of the activations' type and run the library GEMM (the
+// CUDA provider's route for M >= 8, onnx-runtime-ep-cuda/src/kernels/matmul_nbits.rs:6176-6222). Returns false with
+// nothing launched when the route does not apply or is not ready (then the tiled kernel takes the call): too few rows,
+// another dtype mix, a dense copy beyond the configured size, no library kernel for the shape, or a first use while a
+// graph capture is open (nothing may allocate then).
+bool dense_route(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& args, int& rc)
+{
+    rc = 0;
+    NxrtRocmEp& ep = *kn.ep;
+    if (ep.dense_gemm_min_rows <= 0 || args.m < ep.dense_gemm_min_rows) return false;
+    if ((args.a_dtype != ROCM_DT_F16 && args.a_dtype != ROCM_DT_BF16) || args.y_dtype != args.a_dtype || (args.k & 7) != 0) return false;
+    if ((reinterpret_cast<uintptr_t>(args.a) & 15) != 0 || (reinterpret_cast<uintptr_t>(args.y) & 15) != 0 || (reinterpret_cast<uintptr_t>(args.b) & 3) != 0) return false;
+    const uint64_t need = static_cast<uint64_t>(args.n) * static_cast<uint64_t>(args.k) * 2;
+    if (need > ep.dense_gemm_max_bytes) return false;
+    const int bias_dtype = args.bias ? args.bias_dtype : -1;
+
+    std::lock_guard<std::mutex> lock(ep.dense_mu);
+    if (!ep.dense) {
+        if (ep.capturing || rocm_dense_gemm_create(&ep.dense) != 0) {
+            ep.dense = nullptr;
+            return false;
+        }
+    }
+    if (!rocm_dense_gemm_ready(ep.dense, args.m, args.n, args.k, args.a_dtype, bias_dtype, ep.capturing ? 0 : 1)) return false;
+
+    const bool constant = kn.constant_inputs[1] && kn.constant_inputs[2] && (!args.zp || kn.constant_inputs[3]);
+    const void* w16 = nullptr;
+    if (ep.dense_resident && constant) {
+        const bool current = kn.dense && kn.dense_from[0] == args.b && kn.dense_from[1] == args.scales && kn.dense_from[2] == args.zp &&
+                             kn.dense_dtype == args.a_dtype && kn.dense_scale_dtype == args.scale_dtype;
+        if (!current) {
+            if (ep.capturing) return false;
+            if (kn.dense) {
+                rocm_ffi_stream_sync(ep.stream);
+                rocm_ffi_free(kn.dense);
+                kn.dense = nullptr;
+            }
+            if (rocm_ffi_malloc(&kn.dense, need) != 0) {
+                kn.dense = nullptr;
+                return false;                   // no memory for a dense copy: the tiled kernel reads the packed weights
+            }
+            rc = rocm_launch_dequant_16(args.b, args.scales, args.scale_dtype, args.zp, args.n, args.k, args.block_size, args.a_dtype, kn.dense, ep.stream);
+            kn.dense_from[0] = args.b;
+            kn.dense_from[1] = args.scales;
+            kn.dense_from[2] = args.zp;
+            kn.dense_dtype = args.a_dtype;
+            kn.dense_scale_dtype = args.scale_dtype;
+        }
+        w16 = kn.dense;
+        kn.variant = "dense_resident_blaslt";
+    } else {
+        if (ep.dense_scratch_bytes < need) {
+            if (ep.capturing) return false;
+            if (ep.dense_scratch) {
+                rocm_ffi_stream_sync(ep.stream);
+                rocm_ffi_free(ep.dense_scratch);
+                ep.dense_scratch = nullptr;
+                ep.dense_scratch_bytes = 0;
+            }
+            if (rocm_ffi_malloc(&ep.dense_scratch, need) != 0) {
+                ep.dense_scratch = nullptr;
+                return false;
+            }
+            ep.dense_scratch_bytes = need;
+        }
+        rc = rocm_launch_dequant_16(args.b, args.scales, args.scale_dtype, args.zp, args.n, args.k, args.block_size, args.a_dtype, ep.dense_scratch, ep.stream);
+        w16 = ep.dense_scratch;
+        kn.variant = "dense_transient_blaslt";
+    }
+    if (rc == 0) rc = rocm_dense_gemm_run(ep.dense, w16, args.a, args.y, args.bias, args.bias_dtype, args.m, args.n, args.k, args.a_dtype, ep.stream);
     return true;
 }
 
@@ -396,6 +473,8 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
         kn.variant = "decode_mfma_splitk";
     } else if (M <= 32 && decode_in_row_blocks(kn, args, rc)) {
         // done: a few passes of the streaming kernels beat one pass of the tiled kernel at these heights
+    } else if (dense_route(kn, args, rc)) {
+        // done: weights expanded to 16 bits, then the library GEMM
     } else if (M > 16 && rocm_prefill_mfma_eligible(&args)) {
         // Small grids slice K and want scratch for the partial sums: the caller's workspace if it is large enough, else
         // the kernel's own (grown outside a capture only; with too little the launcher slices less or not at all).

@@ -21,6 +21,13 @@ struct NxrtRocmEp {
     int decode_col_groups = 0;
     int prefill_tile = 0;                         // 0 = chosen per shape; 1..3 force a tile (tests, tuning)
     int prepack = 1;                              // repack constant weights for the decode kernel on first use
+    int dense_gemm_min_rows = 0;                  // calls with at least this many rows expand the weights and run the library GEMM; 0 = never
+    uint64_t dense_gemm_max_bytes = 1ull << 30;   // largest dense copy of one weight that route makes
+    int dense_resident = 0;                       // 1: a constant weight keeps its dense copy (made once); 0: one shared buffer, refilled per call
+    RocmDenseGemm* dense = nullptr;               // library handle + its workspace, made on first use
+    void* dense_scratch = nullptr;                // the shared buffer of dense_resident = 0
+    uint64_t dense_scratch_bytes = 0;
+    std::mutex dense_mu;                          // expansion and GEMM of one call are enqueued back to back under it
     std::mutex mu;
     std::unordered_map<void*, size_t> live;       // allocations handed out and not yet returned
     std::atomic<uint64_t> launches{0};

@@ -31,6 +31,7 @@ inline NxrtStatus ok() { return make_status(NXRT_OK); }
 inline NxrtStatus hip_status(int err, const char* what)
 {
     if (err == 0) return ok();
+    if (err >= 10000) return make_status(NXRT_DEVICE_ERROR, std::string(what) + ": hipBLASLt status " + std::to_string(err - 10000));
     const uint32_t code = err == 2 /* hipErrorOutOfMemory */ ? NXRT_OUT_OF_MEMORY : NXRT_DEVICE_ERROR;
     return make_status(code, std::string(what) + ": " + rocm_ffi_error_string(err));
 }

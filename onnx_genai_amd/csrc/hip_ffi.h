@@ -62,6 +62,22 @@ typedef struct RocmMatMulNBitsArgs {
 int rocm_launch_dequant_f32(const uint8_t* b, const void* scales, int scale_dtype, const uint8_t* zp,
                             int64_t n, int64_t k, int block_size, float* out_nk, rocm_stream_t stream);
 
+/* w[n,k] = (q - zp) * scale, computed in f32 and rounded once (nearest even) to out_dtype (f16 or bf16), [N, K].
+ * K % 8 == 0 and out_nk 16-byte aligned. */
+int rocm_launch_dequant_16(const uint8_t* b, const void* scales, int scale_dtype, const uint8_t* zp,
+                           int64_t n, int64_t k, int block_size, int out_dtype, void* out_nk, rocm_stream_t stream);
+
+/* The library GEMM (hipBLASLt) behind the dense prefill route: Y[M,N] = A[M,K] * W[N,K]^T (+ bias[N]); A, W, Y of one
+ * 16-bit type, f32 accumulation. create / destroy allocate and free (never inside a graph capture); ready looks a shape
+ * up once (may_plan = 0 only consults earlier lookups) and returns 1 when a kernel is on hand; run enqueues it and
+ * returns 0, a HIP error code, or 10000 + the library's status. */
+typedef struct RocmDenseGemm RocmDenseGemm;
+int rocm_dense_gemm_create(RocmDenseGemm** out);
+void rocm_dense_gemm_destroy(RocmDenseGemm* g);
+int rocm_dense_gemm_ready(RocmDenseGemm* g, int64_t m, int64_t n, int64_t k, int dtype, int bias_dtype, int may_plan);
+int rocm_dense_gemm_run(RocmDenseGemm* g, const void* w_nk, const void* a, void* y, const void* bias, int bias_dtype,
+                        int64_t m, int64_t n, int64_t k, int dtype, rocm_stream_t stream);
+
 /* Any dtype mix, any K, any block size: f32 math, one wave per output column. */
 int rocm_launch_gemv_generic(const RocmMatMulNBitsArgs* args, rocm_stream_t stream);
 /* f32 activations, M <= 4, block size >= 32, K % 4 == 0, A and B 16-byte aligned: f32 FMA streaming kernel */

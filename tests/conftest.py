@@ -48,3 +48,12 @@ def ep_unpacked():
     provider = RocmExecutionProvider(0, {"prepack": "0"})
     yield provider
     provider.shutdown()
+
+
+@pytest.fixture(scope="session")
+def ep_tiled():
+    """A provider whose tall 16-bit calls stay on the hand-written tiled kernel (no dense copy, no library GEMM)."""
+    from onnx_genai_amd.ep import RocmExecutionProvider
+    provider = RocmExecutionProvider(0, {"dense_gemm_min_rows": "0"})
+    yield provider
+    provider.shutdown()

@@ -300,6 +300,7 @@ GRAPH_CASES = [
     (E.F16, 64, 4, 1, 160, 1024),          # accuracy_level 4, one row: quantized inside the kernel, no workspace
     (E.F16, 64, 4, 5, 96, 512),            # accuracy_level 4 with the caller's workspace: quantizer + int8 MFMA
     (E.F16, 64, 4, 130, 200, 576),
+    (E.BF16, 128, 0, 1024, 136, 512),      # tall call: weights expanded to 16 bits + the library GEMM
 ]
 
 
@@ -420,7 +421,8 @@ PREFILL_CASES = [
 
 
 @pytest.mark.parametrize("a_dt,s_dt,bs,zero_points,m,n,k", PREFILL_CASES)
-def test_prefill_matches_oracle(ep, port, a_dt, s_dt, bs, zero_points, m, n, k):
+def test_prefill_matches_oracle(ep_tiled, port, a_dt, s_dt, bs, zero_points, m, n, k):
+    ep = ep_tiled
     b, s, zp = synth.make_weights(n, k, bs, 200 + n + k, zero_points=zero_points, scale_lo=0.001, scale_hi=0.01, scale_dtype=s_dt)
     a = synth.make_activation(m, k, n, a_dt)
     bias = synth.to_dtype(np.random.default_rng(n).standard_normal(n).astype(np.float32), a_dt)
@@ -463,6 +465,102 @@ def test_prefill_weight_tiles_are_f16_of_f32_dequant(ep, port, bs, zero_points):
     w = port.dequantize_nk(b, synth.to_f32(s, E.F16), zp, n, k, bs)            # f32 [N, K], bit-exact reference definition
     want = port.narrow(np.ascontiguousarray(w[:, ks].T), oracle.F16)
     assert np.array_equal(y.view(np.uint16), want.view(np.uint16))
+
+
+# ---------------------------------------------------------------------------------------------
+# dense route: weights expanded to 16 bits, then the library GEMM (tall calls)
+# ---------------------------------------------------------------------------------------------
+DENSE_CASES = [
+    # a_dt, s_dt, bs, zp, m, n, k, bias dtype (None = no bias)
+    (E.F16, E.F16, 32, False, 200, 256, 512, E.F16),
+    (E.F16, E.F32, 64, True, 96, 120, 256, None),
+    (E.F16, E.F16, 128, True, 1030, 136, 1024, E.F32),
+    (E.BF16, E.BF16, 128, True, 130, 384, 3584, E.F32),
+    (E.BF16, E.BF16, 32, False, 64, 100, 128, E.BF16),
+    (E.BF16, E.F32, 16, True, 257, 72, 136, None),
+]
+
+
+@pytest.mark.parametrize("mode", ["transient", "resident"])
+@pytest.mark.parametrize("a_dt,s_dt,bs,zero_points,m,n,k,bias_dt", DENSE_CASES)
+def test_dense_route_matches_oracle(port, mode, a_dt, s_dt, bs, zero_points, m, n, k, bias_dt):
+    provider = E.RocmExecutionProvider(0, {"dense_gemm_min_rows": "64", "dense_weights": mode})
+    try:
+        b, s, zp = synth.make_weights(n, k, bs, 500 + n + k, zero_points=zero_points, scale_lo=0.001, scale_hi=0.01, scale_dtype=s_dt)
+        a = synth.make_activation(m, k, n, a_dt)
+        bias = None if bias_dt is None else synth.to_dtype(np.random.default_rng(n).standard_normal(n).astype(np.float32), bias_dt)
+        want64 = oracle_f64(port, a, a_dt, b, s, s_dt, zp, n, k, bs, bias, bias_dt if bias_dt is not None else E.F32)
+        y, variant = run_op(provider, a, a_dt, b, s, s_dt, zp, n, k, bs, bias=bias, bias_dtype=bias_dt if bias_dt is not None else E.F32)
+        assert variant == "dense_%s_blaslt" % mode
+        assert helpers.rel_l2(synth.to_f32(y, a_dt), want64) <= TOL_HALF
+    finally:
+        provider.shutdown()
+
+
+@pytest.mark.parametrize("a_dt,s_dt", [(E.F16, E.F16), (E.BF16, E.BF16), (E.BF16, E.F32)])
+@pytest.mark.parametrize("bs,zero_points", [(32, True), (128, False)])
+def test_dense_weights_are_the_f32_dequant_rounded_once(port, a_dt, s_dt, bs, zero_points):
+    """One-hot activation rows read single weights back out of the library GEMM: each must equal the f32 dequantized
+    weight rounded once to the 16-bit type, bit for bit (a product by 1 and sums with zeros are exact)."""
+    m, n, k = 64, 256, 256
+    provider = E.RocmExecutionProvider(0, {"dense_gemm_min_rows": "64"})
+    try:
+        b, s, zp = synth.make_weights(n, k, bs, 300 + bs, zero_points=zero_points, scale_lo=0.001, scale_hi=0.01, scale_dtype=s_dt)
+        ks = (np.arange(m) * 37) % k
+        a32 = np.zeros((m, k), np.float32)
+        a32[np.arange(m), ks] = 1.0
+        y, variant = run_op(provider, synth.to_dtype(a32, a_dt), a_dt, b, s, s_dt, zp, n, k, bs)
+        assert variant == "dense_transient_blaslt"
+        w = port.dequantize_nk(b, synth.to_f32(s, s_dt), zp, n, k, bs)            # f32 [N, K], bit-exact reference definition
+        want = port.narrow(np.ascontiguousarray(w[:, ks].T), oracle.F16 if a_dt == E.F16 else oracle.BF16)
+        assert np.array_equal(np.asarray(y).view(np.uint16), np.asarray(want).view(np.uint16))
+    finally:
+        provider.shutdown()
+
+
+def test_dense_route_declines_what_it_cannot_take(port):
+    """f32 outputs, short calls and weights beyond the configured size stay on the hand-written kernels; so does a first
+    use while a graph capture is open (the route may not allocate then), and the captured call still gives the result."""
+    a_dt, bs, m, n, k = E.F16, 32, 128, 128, 256
+    b, s, zp = synth.make_weights(n, k, bs, 77, zero_points=True, scale_lo=0.002, scale_hi=0.01, scale_dtype=a_dt)
+    a = synth.make_activation(m, k, 77, a_dt)
+    want = oracle_f64(port, a, a_dt, b, s, a_dt, zp, n, k, bs)
+    provider = E.RocmExecutionProvider(0, {"dense_gemm_min_rows": "64"})
+    small = E.RocmExecutionProvider(0, {"dense_gemm_min_rows": "64", "dense_gemm_max_mb": "0"})
+    try:
+        y32, variant = run_op(provider, a, a_dt, b, s, a_dt, zp, n, k, bs, y_dtype=E.F32)
+        assert variant == "prefill_mfma_lds" and helpers.rel_l2(y32, want) <= TOL_HALF
+        _, variant = run_op(provider, a[:48], a_dt, b, s, a_dt, zp, n, k, bs)
+        assert variant == "prefill_mfma_lds"
+        _, variant = run_op(small, a, a_dt, b, s, a_dt, zp, n, k, bs)
+        assert variant == "prefill_mfma_lds"
+        # first use inside a capture
+        fresh = E.RocmExecutionProvider(0, {"dense_gemm_min_rows": "64"})
+        try:
+            ops = E.DeviceOperands(fresh, b, s, a_dt, zp, n, k, bs)
+            ab, yb = fresh.upload(a), fresh.allocate(m * n * 2)
+            fresh.sync()
+            fresh.capture_begin()
+            try:
+                ops.run(ab, a_dt, m, yb)
+            finally:
+                graph = fresh.capture_end()
+            assert ops.kernel.last_variant() == "prefill_mfma_lds"
+            graph.replay()
+            got = fresh.download(yb, (m, n), np.float16)
+            assert helpers.rel_l2(got.astype(np.float32), want) <= TOL_HALF
+            graph.release()
+            ops.run(ab, a_dt, m, yb)                     # outside the capture the route sets itself up
+            assert ops.kernel.last_variant() == "dense_transient_blaslt"
+            assert helpers.rel_l2(fresh.download(yb, (m, n), np.float16).astype(np.float32), want) <= TOL_HALF
+            fresh.deallocate(ab)
+            fresh.deallocate(yb)
+            ops.free()
+        finally:
+            fresh.shutdown()
+    finally:
+        provider.shutdown()
+        small.shutdown()
 
 
 # ---------------------------------------------------------------------------------------------
