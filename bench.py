@@ -42,8 +42,8 @@ A_DT = E.BF16
 
 
 # HBM bytes one gate/up launch (M=1, repacked weights) moves, from two rocprofv3 counter runs of `bench.py --only-roofline`:
-# FETCH_SIZE 35,284.0 KiB-units x 1.9997 (what the same counter reads for a 256 MiB copy) plus WRITE_SIZE 74.0 KiB.
-GATE_UP_HBM_BYTES_PER_LAUNCH = 72_327_400
+# FETCH_SIZE 35,282.4 KiB-units x 1.9997 (what the same counter reads for a 256 MiB copy) plus WRITE_SIZE 74.0 KiB.
+GATE_UP_HBM_BYTES_PER_LAUNCH = 72_324_100
 
 
 def _device_random_weights(ep, n, k, bs, seed, scale_lo, scale_hi, dtype, zero_points=True, reuse=None):

@@ -325,7 +325,7 @@ constexpr int kPitch8 = 80;          // bytes per LDS row: 64 codes + 16 of padd
 // Eight waves, 4 (rows) x 2 (columns); each owns a 32 x 64 sub-tile: two MFMA tiles, 32 f32 results per lane. The
 // small per-wave state leaves room for four waves per SIMD, which is what overlaps one wave's flush arithmetic
 // with another's MFMAs.
-template <int NBS, bool SF32>
+template <int NBS, bool SF32, int D>
 __global__ __launch_bounds__(512) void acc4_prefill_kernel(Acc4PrefillParams p)
 {
     constexpr int kSlots = NBS == 2 ? 2 : 1;                   // scale slots per step
@@ -377,10 +377,10 @@ __global__ __launch_bounds__(512) void acc4_prefill_kernel(Acc4PrefillParams p)
         for (int r = 0; r < 16; ++r) y[j][r] = 0.f;
 
     const int steps = static_cast<int>((p.padded_k + kStep - 1) / kStep);
-    // Global loads run D-1 steps ahead of the MFMAs, in D register sets. Block size 64 and up: two sets keep the kernel
-    // within 128 registers, so that two workgroups share a CU (measured +2 to +8 %); block size 32, whose steps hold two
-    // flushes, does better with four sets and one workgroup per CU.
-    constexpr int D = NBS == 2 ? 4 : 2;
+    // Global loads run D-1 steps ahead of the MFMAs, in D register sets (D = 2 or 4; the launcher chooses). Two sets
+    // keep the kernel within 128 registers, so that two workgroups share a CU: better on grids that fill the GPU twice
+    // over (measured +2 to +8 %). A grid with at most one workgroup per CU gains nothing from that and runs its lone
+    // workgroup 30 % faster with four sets in flight; so does block size 32, whose steps hold two flushes.
     struct Regs {
         uint4 a;
         uint2 b;
@@ -402,9 +402,14 @@ __global__ __launch_bounds__(512) void acc4_prefill_kernel(Acc4PrefillParams p)
         const uint32_t zraw = static_cast<uint32_t>(__builtin_amdgcn_raw_buffer_load_b8(srd_z, static_cast<int>(z_goff + (blk >> 1)), 0, 0));
         r.z = zraw;                 // no arithmetic on a loaded value here: it would wait for the load at once
         r.zsh = (blk & 1u) * 4u;
-        // the block depends on the thread's slot, so it travels in the vector offset: as a scalar offset the compiler
-        // would loop over its distinct values (an out-of-range sa_goff stays out of range: kb * m * 4 < 2^31)
-        r.sa = __builtin_amdgcn_raw_buffer_load_b32(srd_sa, static_cast<int>(sa_goff + block_of(kt, sa_slot * 32) * static_cast<uint32_t>(p.m) * 4u), 0, 0);
+        // The block depends on the thread's slot, so it belongs in the vector offset (an out-of-range sa_goff stays out
+        // of range: kb * m * 4 < 2^31): as a scalar offset the compiler loops over its distinct values. With one block
+        // per step that loop is kept on purpose: it splits the step into two scheduling regions, and the schedule the
+        // compiler finds for the whole step in one region needs 203 registers instead of 126 with two register sets
+        // (one workgroup per CU instead of two, 20 % slower) and spills with four.
+        const uint32_t sa_block = block_of(kt, sa_slot * 32) * static_cast<uint32_t>(p.m) * 4u;
+        if constexpr (NBS == 1) r.sa = __builtin_amdgcn_raw_buffer_load_b32(srd_sa, static_cast<int>(sa_goff), static_cast<int>(sa_block), 0);
+        else r.sa = __builtin_amdgcn_raw_buffer_load_b32(srd_sa, static_cast<int>(sa_goff + sa_block), 0, 0);
     };
     // Half `part` of a step's trip from registers into LDS buffer `buf`.
     auto store_part = [&](const Regs& r, int buf, int part) {
@@ -554,7 +559,9 @@ static int launch_acc4_prefill(const Acc4PrefillParams& p, hipStream_t stream)
 {
     const dim3 grid(static_cast<unsigned>((p.n + kTile - 1) / kTile), static_cast<unsigned>((p.m + kTile - 1) / kTile));
     const size_t lds = 2 * (2 * kTile * kPitch8 + 2 * (NBS == 2 ? 2 : 1) * kTile * 4);
-    hipLaunchKernelGGL((acc4_prefill_kernel<NBS, SF32>), grid, dim3(512), lds, stream, p);
+    const bool deep = NBS == 2 || static_cast<uint64_t>(grid.x) * grid.y <= 256;    // at most one workgroup per CU anyway
+    if (deep) hipLaunchKernelGGL((acc4_prefill_kernel<NBS, SF32, 4>), grid, dim3(512), lds, stream, p);
+    else hipLaunchKernelGGL((acc4_prefill_kernel<NBS, SF32, NBS == 2 ? 4 : 2>), grid, dim3(512), lds, stream, p);
     return static_cast<int>(hipGetLastError());
 }
 
