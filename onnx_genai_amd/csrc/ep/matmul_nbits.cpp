@@ -148,7 +148,8 @@ namespace {
 
 // Scratch of accuracy_level=4 for M rows: int8 codes, (scale, code sum) pairs, and a block-major copy of the
 // pairs (M <= 16) or of the scales (M > 16) for the matrix-core kernels.
-struct Acc4Layout { uint64_t codes, pairs, aux, total; };
+// Last comes room for the f32 partial sums of a tiled call that cuts K into slices (small grids only).
+struct Acc4Layout { uint64_t codes, pairs, aux, partial, total; };
 Acc4Layout acc4_layout(const NxrtRocmMatMulNBits& kn, uint64_t m)
 {
     const uint64_t kb = (kn.k + kn.block_size - 1) / kn.block_size;
@@ -156,7 +157,14 @@ Acc4Layout acc4_layout(const NxrtRocmMatMulNBits& kn, uint64_t m)
     l.codes = (m * kb * kn.block_size + 255) / 256 * 256;
     l.pairs = (m * kb * 8 + 255) / 256 * 256;
     l.aux = (kb * (m > 32 ? m : 32) * 4 + 255) / 256 * 256;
-    l.total = l.codes + l.pairs + l.aux;
+    RocmMatMulNBitsArgs probe;
+    std::memset(&probe, 0, sizeof(probe));
+    probe.m = static_cast<int64_t>(m);
+    probe.n = kn.n;
+    probe.k = kn.k;
+    probe.block_size = static_cast<int>(kn.block_size);
+    l.partial = (rocm_acc4_mfma_scratch_bytes(&probe) + 255) / 256 * 256;
+    l.total = l.codes + l.pairs + l.aux + l.partial;
     return l;
 }
 uint64_t acc4_workspace_bytes(const NxrtRocmMatMulNBits& kn, uint64_t m) { return acc4_layout(kn, m).total; }
@@ -451,6 +459,8 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
         w4.aq = reinterpret_cast<float*>(ws + lay.codes);
         w4.aux = reinterpret_cast<float*>(ws + lay.codes + lay.pairs);
         w4.code_order = packed ? 2 : 1;
+        w4.partial = lay.partial ? reinterpret_cast<float*>(ws + lay.codes + lay.pairs + lay.aux) : nullptr;
+        w4.partial_bytes = lay.partial;
         rc = rocm_launch_quantize_a_workspace(args.a, args.a_dtype, args.m, args.k, args.block_size, rounding, &w4, stream);
         if (rc == 0 && pack_rc != 0) rc = pack_rc;
         if (rc == 0) {

@@ -103,6 +103,9 @@ int rocm_prefill_mfma_eligible(const RocmMatMulNBitsArgs* args);
  * by a second kernel; rocm_prefill_mfma_scratch_bytes says how much the preferred plan wants (0 = no slicing). With less
  * scratch the launcher uses fewer slices, with none it does not slice. */
 uint64_t rocm_prefill_mfma_scratch_bytes(const RocmMatMulNBitsArgs* args, int tile_choice);
+/* Y = sum over `slices` of partial[slice][M][N] (f32), in slice order, + bias. */
+int rocm_launch_slice_reduce(const float* partial, int slices, int64_t m, int64_t n, const void* bias, int bias_dtype, void* y, int y_dtype,
+                             rocm_stream_t stream);
 int rocm_launch_prefill_mfma(const RocmMatMulNBitsArgs* args, int tile_choice, void* scratch, uint64_t scratch_bytes, rocm_stream_t stream);
 
 /* accuracy_level 4. rounding: 0 = ties to even (MLAS rule), 1 = ties away (native Rust rule).
@@ -122,6 +125,8 @@ typedef struct RocmAcc4Workspace {
   float* aq;
   float* aux;
   int code_order;
+  float* partial;          /* M > 16: room for the f32 partial sums of K slices (rocm_acc4_mfma_scratch_bytes), or NULL */
+  uint64_t partial_bytes;
 } RocmAcc4Workspace;
 int rocm_launch_quantize_a_workspace(const void* a, int a_dtype, int64_t m, int64_t k, int block_size, int rounding,
                                      const RocmAcc4Workspace* ws, rocm_stream_t stream);
@@ -130,6 +135,9 @@ int rocm_launch_acc4_gemv(const RocmMatMulNBitsArgs* args, const RocmAcc4Workspa
 /* The same on the int8 matrix cores: M <= 16 with block size 32/64/128 (split-K; waves = 0 lets the launcher choose),
  * M > 16 with any block size >= 32 (tiled). */
 int rocm_acc4_mfma_eligible(const RocmMatMulNBitsArgs* args);
+/* Bytes of partial sums the tiled kernel wants when it cuts K into slices (small grids); 0 when it does not. With less
+ * it uses fewer slices or none. */
+uint64_t rocm_acc4_mfma_scratch_bytes(const RocmMatMulNBitsArgs* args);
 int rocm_launch_acc4_mfma(const RocmMatMulNBitsArgs* args, const RocmAcc4Workspace* ws, int waves, rocm_stream_t stream);
 /* One row over the repacked copy of constant weights (the copy rocm_launch_pack_decode makes); code_order 2. */
 int rocm_acc4_packed_eligible(const RocmMatMulNBitsArgs* args);

@@ -314,6 +314,8 @@ struct Acc4PrefillParams {
     int bs_log2;
     int scales_bf16;
     int bias_dtype, y_dtype;
+    int steps_per_slice;    // K steps per grid.z slice (a whole number of blocks); all steps when there is one slice
+    float* partial;         // [slices, M, N] f32 partial sums when K is cut into slices, else NULL
 };
 
 constexpr int kTile = 128;           // rows and columns of Y per workgroup
@@ -376,7 +378,10 @@ __global__ __launch_bounds__(512) void acc4_prefill_kernel(Acc4PrefillParams p)
 #pragma unroll
         for (int r = 0; r < 16; ++r) y[j][r] = 0.f;
 
-    const int steps = static_cast<int>((p.padded_k + kStep - 1) / kStep);
+    // K range of this workgroup: all of K, or one of grid.z slices whose f32 partial sums a second kernel adds in slice
+    // order (small grids: few tiles of Y, long K). `kt` below counts steps from the slice's first.
+    const int kt_base = static_cast<int>(blockIdx.z) * p.steps_per_slice;
+    const int steps = min(static_cast<int>((p.padded_k + kStep - 1) / kStep) - kt_base, p.steps_per_slice);
     // Global loads run D-1 steps ahead of the MFMAs, in D register sets (D = 2 or 4; the launcher chooses). Two sets
     // keep the kernel within 128 registers, so that two workgroups share a CU: better on grids that fill the GPU twice
     // over (measured +2 to +8 %). A grid with at most one workgroup per CU gains nothing from that and runs its lone
@@ -389,7 +394,8 @@ __global__ __launch_bounds__(512) void acc4_prefill_kernel(Acc4PrefillParams p)
     Regs regs[D];
 
     auto block_of = [&](int kt, int offset) -> uint32_t { return static_cast<uint32_t>((kt * kStep + offset) >> p.bs_log2); };
-    auto load_global = [&](Regs& r, int kt) {
+    auto load_global = [&](Regs& r, int kt_in_slice) {
+        const int kt = kt_base + kt_in_slice;
         uint32_t off = a_goff;
         if (ragged_k && static_cast<int64_t>(kt) * kStep + quarter * 16 >= p.padded_k) off = kOutOfRange;   // else the next row's codes
         r.a = load16(srd_a, off, static_cast<uint32_t>(kt) * 64u);
@@ -450,7 +456,8 @@ __global__ __launch_bounds__(512) void acc4_prefill_kernel(Acc4PrefillParams p)
     auto mfma = [](const u32x4_t& a, const u32x4_t& b, const int16_t_v& c) {
         return __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(int4_t, a), __builtin_bit_cast(int4_t, b), c, 0, 0, 0);
     };
-    auto compute = [&](int buf, int kt, const Regs& next, bool store_next) {
+    auto compute = [&](int buf, int kt_in_slice, const Regs& next, bool store_next) {
+        const int kt = kt_base + kt_in_slice;
         const unsigned char* la = smem + buf * kBufBytes + wm * (32 * kPitch8) + frag_off;
         const unsigned char* lb = smem + buf * kBufBytes + kTile * kPitch8 + wn * (64 * kPitch8) + frag_off;
         u32x4_t fa[2], fb[2][TN];
@@ -542,24 +549,49 @@ __global__ __launch_bounds__(512) void acc4_prefill_kernel(Acc4PrefillParams p)
     for (int j = 0; j < TN; ++j) {
         const int64_t col = n_base + wn * 64 + j * 32 + col_in_tile;
         if (col >= p.n) continue;
-        const float bias = p.bias ? load_as_f32(p.bias, p.bias_dtype, col) : 0.f;
+        const float bias = (p.bias && !p.partial) ? load_as_f32(p.bias, p.bias_dtype, col) : 0.f;
+        float* part = p.partial ? p.partial + static_cast<int64_t>(blockIdx.z) * p.m * p.n : nullptr;
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int64_t row = m_base + wm * 32 + q * 8 + row_group + r;
-                if (row < p.m) store_from_f32(p.y, p.y_dtype, row * p.n + col, y[j][q * 4 + r] + bias);
+                if (row >= p.m) continue;
+                if (part) part[row * p.n + col] = y[j][q * 4 + r];
+                else store_from_f32(p.y, p.y_dtype, row * p.n + col, y[j][q * 4 + r] + bias);
             }
         }
     }
 }
 
-template <int NBS, bool SF32>
-static int launch_acc4_prefill(const Acc4PrefillParams& p, hipStream_t stream)
+// Slices of K for a grid that leaves CUs idle. Two workgroups of the two-set variant share a CU, so up to 512 run at
+// once: slices bring the grid to at most that, with at least 8 steps each, a whole number of blocks per slice, at most 8.
+static int acc4_prefill_slices(int64_t m, int64_t n, int64_t padded_k, int block_size)
 {
-    const dim3 grid(static_cast<unsigned>((p.n + kTile - 1) / kTile), static_cast<unsigned>((p.m + kTile - 1) / kTile));
+    const int64_t tiles = ((n + kTile - 1) / kTile) * ((m + kTile - 1) / kTile);
+    const int64_t steps = (padded_k + kStep - 1) / kStep;
+    if (block_size < 64 || tiles > 170) return 1;          // block size 32 keeps four register sets: one workgroup per CU
+    int64_t want = 512 / tiles;
+    if (want > 8) want = 8;
+    if (want > steps / 8) want = steps / 8;
+    return want < 2 ? 1 : static_cast<int>(want);
+}
+
+static int acc4_steps_per_slice(int64_t padded_k, int block_size, int slices)
+{
+    const int64_t steps = (padded_k + kStep - 1) / kStep;
+    const int64_t unit = block_size > kStep ? block_size / kStep : 1;            // steps per block
+    int64_t per = (steps + slices - 1) / slices;
+    per = (per + unit - 1) / unit * unit;
+    return static_cast<int>(per);
+}
+
+template <int NBS, bool SF32>
+static int launch_acc4_prefill(const Acc4PrefillParams& p, int slices, hipStream_t stream)
+{
+    const dim3 grid(static_cast<unsigned>((p.n + kTile - 1) / kTile), static_cast<unsigned>((p.m + kTile - 1) / kTile), static_cast<unsigned>(slices));
     const size_t lds = 2 * (2 * kTile * kPitch8 + 2 * (NBS == 2 ? 2 : 1) * kTile * 4);
-    const bool deep = NBS == 2 || static_cast<uint64_t>(grid.x) * grid.y <= 256;    // at most one workgroup per CU anyway
+    const bool deep = NBS == 2 || static_cast<uint64_t>(grid.x) * grid.y * grid.z <= 256;    // at most one workgroup per CU anyway
     if (deep) hipLaunchKernelGGL((acc4_prefill_kernel<NBS, SF32, 4>), grid, dim3(512), lds, stream, p);
     else hipLaunchKernelGGL((acc4_prefill_kernel<NBS, SF32, NBS == 2 ? 4 : 2>), grid, dim3(512), lds, stream, p);
     return static_cast<int>(hipGetLastError());
@@ -579,6 +611,14 @@ extern "C" int rocm_acc4_mfma_eligible(const RocmMatMulNBitsArgs* a)
     }
     // prefill: 32-bit offsets inside one 128-row / 128-column window and inside the block-major scales
     return padded_k / 2 * 128 < 0x7fffffff && padded_k * 128 < 0x7fffffff && kb * a->m * 4 < 0x7fffffff;
+}
+
+extern "C" uint64_t rocm_acc4_mfma_scratch_bytes(const RocmMatMulNBitsArgs* a)
+{
+    if (a->m <= 16 || a->block_size < 32) return 0;
+    const int64_t padded_k = (a->k + a->block_size - 1) / a->block_size * a->block_size;
+    const int slices = mnb::acc4_prefill_slices(a->m, a->n, padded_k, a->block_size);
+    return slices > 1 ? static_cast<uint64_t>(slices) * static_cast<uint64_t>(a->m) * static_cast<uint64_t>(a->n) * 4 : 0;
 }
 
 extern "C" int rocm_launch_acc4_mfma(const RocmMatMulNBitsArgs* a, const RocmAcc4Workspace* ws, int waves, rocm_stream_t stream)
@@ -605,9 +645,21 @@ extern "C" int rocm_launch_acc4_mfma(const RocmMatMulNBitsArgs* a, const RocmAcc
         q.bias_dtype = a->bias_dtype;
         q.y_dtype = a->y_dtype;
         const bool sf32 = a->scale_dtype == ROCM_DT_F32;
-        if (a->block_size == 32) return sf32 ? mnb::launch_acc4_prefill<2, true>(q, s) : mnb::launch_acc4_prefill<2, false>(q, s);
-        if (a->block_size == 64) return sf32 ? mnb::launch_acc4_prefill<1, true>(q, s) : mnb::launch_acc4_prefill<1, false>(q, s);
-        return sf32 ? mnb::launch_acc4_prefill<0, true>(q, s) : mnb::launch_acc4_prefill<0, false>(q, s);
+        // slices of K when the grid is small and the workspace has room for their partial sums
+        int slices = mnb::acc4_prefill_slices(a->m, a->n, q.padded_k, a->block_size);
+        const uint64_t per_slice = static_cast<uint64_t>(a->m) * static_cast<uint64_t>(a->n) * 4;
+        if (!ws->partial || ws->partial_bytes < 2 * per_slice) slices = 1;
+        else if (ws->partial_bytes < slices * per_slice) slices = static_cast<int>(ws->partial_bytes / per_slice);
+        const int64_t steps = (q.padded_k + mnb::kStep - 1) / mnb::kStep;
+        q.steps_per_slice = mnb::acc4_steps_per_slice(q.padded_k, a->block_size, slices);
+        slices = static_cast<int>((steps + q.steps_per_slice - 1) / q.steps_per_slice);          // no empty slice after rounding to blocks
+        q.partial = slices > 1 ? ws->partial : nullptr;
+        int rc;
+        if (a->block_size == 32) rc = sf32 ? mnb::launch_acc4_prefill<2, true>(q, slices, s) : mnb::launch_acc4_prefill<2, false>(q, slices, s);
+        else if (a->block_size == 64) rc = sf32 ? mnb::launch_acc4_prefill<1, true>(q, slices, s) : mnb::launch_acc4_prefill<1, false>(q, slices, s);
+        else rc = sf32 ? mnb::launch_acc4_prefill<0, true>(q, slices, s) : mnb::launch_acc4_prefill<0, false>(q, slices, s);
+        if (rc != 0 || slices == 1) return rc;
+        return rocm_launch_slice_reduce(ws->partial, slices, a->m, a->n, a->bias, a->bias_dtype, a->y, a->y_dtype, stream);
     }
     mnb::Acc4DecodeParams p;
     p.qa = ws->qa;

@@ -447,9 +447,15 @@ extern "C" int rocm_launch_prefill_mfma(const RocmMatMulNBitsArgs* a, int tile_c
     else if (sf32) rc = go(std::false_type{}, std::true_type{});
     else rc = go(std::false_type{}, std::false_type{});
     if (rc != 0 || plan.splits == 1) return rc;
-    int64_t blocks = (a->m * a->n + 255) / 256;
+    return rocm_launch_slice_reduce(static_cast<const float*>(scratch), plan.splits, a->m, a->n, a->bias, a->bias_dtype, a->y, a->y_dtype, stream);
+}
+
+extern "C" int rocm_launch_slice_reduce(const float* partial, int slices, int64_t m, int64_t n, const void* bias, int bias_dtype, void* y, int y_dtype,
+                                        rocm_stream_t stream)
+{
+    int64_t blocks = (m * n + 255) / 256;
     if (blocks > 16384) blocks = 16384;
-    hipLaunchKernelGGL(mnb::prefill_reduce_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, static_cast<const float*>(scratch), plan.splits,
-                       a->m, a->n, a->bias, a->bias_dtype, a->y, a->y_dtype);
+    hipLaunchKernelGGL(mnb::prefill_reduce_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, static_cast<hipStream_t>(stream), partial, slices, m, n,
+                       bias, bias_dtype, y, y_dtype);
     return static_cast<int>(hipGetLastError());
 }

@@ -300,6 +300,7 @@ GRAPH_CASES = [
     (E.F16, 64, 4, 1, 160, 1024),          # accuracy_level 4, one row: quantized inside the kernel, no workspace
     (E.F16, 64, 4, 5, 96, 512),            # accuracy_level 4 with the caller's workspace: quantizer + int8 MFMA
     (E.F16, 64, 4, 130, 200, 576),
+    (E.F16, 64, 4, 130, 200, 2048),        # the same over slices of K: partial sums in the workspace + reduce
     (E.BF16, 128, 0, 1024, 136, 512),      # tall call: weights expanded to 16 bits + the library GEMM
 ]
 
@@ -650,7 +651,10 @@ ACC4_CASES = [
     (E.F16, 32, True, 33, 64, 32 * 7),        # K ends in the middle of a 64-code step
     (E.BF16, 128, False, 64, 128, 128 * 6),
     (E.F32, 256, True, 40, 96, 256 * 3),
-    (E.F16, 64, True, 256, 256, 2048),
+    (E.F16, 64, True, 256, 256, 2048),        # few tiles of Y, long K: K in four slices + reduce
+    (E.BF16, 128, True, 130, 200, 128 * 20),  # five slices of whole blocks (two steps per block)
+    (E.F16, 256, False, 64, 130, 256 * 9),    # slices rounded up to whole blocks of four steps
+    (E.F16, 64, True, 40, 96, 64 * 17),       # two unequal slices
     (E.F16, 32, False, 17, 130, 200),         # K ends inside a block
     (E.F16, 16, True, 20, 64, 256),           # block size 16: not a matrix-core shape
 ]
