@@ -123,6 +123,7 @@ struct NxrtRocmMatMulNBits {
     std::string variant = "none";
     void* scratch = nullptr;             // kernel-owned workspace, grown on demand
     size_t scratch_bytes = 0;
+    std::vector<void*> retired;          // outgrown workspaces: kept until the kernel dies, since a HIP graph recorded earlier may still name them
     void* packed = nullptr;              // constant B / scales / zero points in the decode kernel's streaming order
     const void* packed_from[3] = {nullptr, nullptr, nullptr};   // the tensors `packed` was made from
     int packed_scale_dtype = 0;
@@ -135,8 +136,9 @@ struct NxrtRocmMatMulNBits {
 
     ~NxrtRocmMatMulNBits()
     {
-        if ((scratch || packed || dense) && ep && ep->bind().code == NXRT_OK) {
+        if ((scratch || packed || dense || !retired.empty()) && ep && ep->bind().code == NXRT_OK) {
             rocm_ffi_stream_sync(ep->stream);
+            for (void* old : retired) rocm_ffi_free(old);
             if (scratch) rocm_ffi_free(scratch);
             if (packed) rocm_ffi_free(packed);
             if (dense) rocm_ffi_free(dense);
@@ -168,6 +170,19 @@ Acc4Layout acc4_layout(const NxrtRocmMatMulNBits& kn, uint64_t m)
     return l;
 }
 uint64_t acc4_workspace_bytes(const NxrtRocmMatMulNBits& kn, uint64_t m) { return acc4_layout(kn, m).total; }
+
+// Replaces an owned device buffer by a larger one. The old buffer is not freed but retired: a HIP graph recorded while
+// it was current would otherwise write through a dangling pointer on its next replay. Returns the HIP error code.
+int grow_buffer(void*& buf, size_t& bytes, uint64_t need, std::vector<void*>& retired)
+{
+    void* fresh = nullptr;
+    const int e = rocm_ffi_malloc(&fresh, need);
+    if (e != 0) return e;
+    if (buf) retired.push_back(buf);
+    buf = fresh;
+    bytes = static_cast<size_t>(need);
+    return 0;
+}
 
 // True when the call can run on the repacked copy of constant weights; makes that copy on first use (never while a
 // graph capture is open: a capture may neither allocate nor should it record the one-time repack). `rc` receives a
@@ -251,17 +266,7 @@ bool dense_route(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& args, int& 
     } else {
         if (ep.dense_scratch_bytes < need) {
             if (ep.capturing) return false;
-            if (ep.dense_scratch) {
-                rocm_ffi_stream_sync(ep.stream);
-                rocm_ffi_free(ep.dense_scratch);
-                ep.dense_scratch = nullptr;
-                ep.dense_scratch_bytes = 0;
-            }
-            if (rocm_ffi_malloc(&ep.dense_scratch, need) != 0) {
-                ep.dense_scratch = nullptr;
-                return false;
-            }
-            ep.dense_scratch_bytes = need;
+            if (grow_buffer(ep.dense_scratch, ep.dense_scratch_bytes, need, ep.dense_retired) != 0) return false;
         }
         rc = rocm_launch_dequant_16(args.b, args.scales, args.scale_dtype, args.zp, args.n, args.k, args.block_size, args.a_dtype, ep.dense_scratch, ep.stream);
         w16 = ep.dense_scratch;
@@ -441,15 +446,8 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
                 if (kn.ep->capturing)
                     return make_status(NXRT_INVALID_ARGUMENT, err("accuracy_level=4 under graph capture needs a caller workspace of " + std::to_string(need) +
                                                                   " bytes (see workspace_requirement); the kernel may not allocate while a capture is open"));
-                if (kn.scratch) {
-                    rocm_ffi_stream_sync(stream);
-                    rocm_ffi_free(kn.scratch);
-                    kn.scratch = nullptr;
-                    kn.scratch_bytes = 0;
-                }
-                const int e = rocm_ffi_malloc(&kn.scratch, need);
+                const int e = grow_buffer(kn.scratch, kn.scratch_bytes, need, kn.retired);
                 if (e != 0) return hip_status(e, "MatMulNBits: workspace hipMalloc");
-                kn.scratch_bytes = need;
             }
             ws = static_cast<uint8_t*>(kn.scratch);
         }
@@ -492,16 +490,7 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
         void* scratch = workspace;
         uint64_t scratch_bytes = workspace ? workspace_bytes : 0;
         if (need > scratch_bytes) {
-            if (kn.scratch_bytes < need && !kn.ep->capturing) {
-                if (kn.scratch) {
-                    rocm_ffi_stream_sync(stream);
-                    rocm_ffi_free(kn.scratch);
-                    kn.scratch = nullptr;
-                    kn.scratch_bytes = 0;
-                }
-                if (rocm_ffi_malloc(&kn.scratch, need) == 0) kn.scratch_bytes = need;
-                else kn.scratch = nullptr;
-            }
+            if (kn.scratch_bytes < need && !kn.ep->capturing) (void)grow_buffer(kn.scratch, kn.scratch_bytes, need, kn.retired);   // on failure: slice less
             if (kn.scratch_bytes > scratch_bytes) {
                 scratch = kn.scratch;
                 scratch_bytes = kn.scratch_bytes;

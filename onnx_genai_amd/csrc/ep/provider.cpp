@@ -18,6 +18,7 @@ NxrtRocmEp::~NxrtRocmEp()
         if (stream) rocm_ffi_stream_sync(stream);
         for (auto& kv : live) rocm_ffi_free(kv.first);
         if (dense_scratch) rocm_ffi_free(dense_scratch);
+        for (void* old : dense_retired) rocm_ffi_free(old);
         if (dense) rocm_dense_gemm_destroy(dense);
         if (stream) rocm_ffi_stream_destroy(stream);
     }

@@ -7,6 +7,7 @@
 #include <mutex>
 #include <string>
 #include <unordered_map>
+#include <vector>
 
 #include "status.h"
 
@@ -26,7 +27,8 @@ struct NxrtRocmEp {
     int dense_resident = 0;                       // 1: a constant weight keeps its dense copy (made once); 0: one shared buffer, refilled per call
     RocmDenseGemm* dense = nullptr;               // library handle + its workspace, made on first use
     void* dense_scratch = nullptr;                // the shared buffer of dense_resident = 0
-    uint64_t dense_scratch_bytes = 0;
+    size_t dense_scratch_bytes = 0;
+    std::vector<void*> dense_retired;             // outgrown shared buffers, kept for graphs recorded while they were current
     std::mutex dense_mu;                          // expansion and GEMM of one call are enqueued back to back under it
     std::mutex mu;
     std::unordered_map<void*, size_t> live;       // allocations handed out and not yet returned

@@ -356,6 +356,37 @@ def test_graph_replays_match_eager(ep, a_dt, bs, acc, m, n, k):
         ops.free()
 
 
+def test_graph_survives_a_later_larger_call(ep_tiled):
+    """A graph recorded while the kernel's own scratch had one size still replays correctly after a later, taller call made
+    the kernel grow that scratch (the outgrown buffer stays allocated for the graphs that name it)."""
+    ep = ep_tiled
+    a_dt, bs, n, k = E.F16, 64, 130, 4096                      # few tiles of Y, long K: K in slices, partial sums in scratch
+    b, s, zp = synth.make_weights(n, k, bs, 63, zero_points=True, scale_lo=0.002, scale_hi=0.01, scale_dtype=a_dt)
+    ops = E.DeviceOperands(ep, b, s, a_dt, zp, n, k, bs)
+    small, tall = 100, 400
+    a1 = ep.upload(synth.make_activation(small, k, 64, a_dt))
+    a2 = ep.upload(synth.make_activation(tall, k, 65, a_dt))
+    y1, y2 = ep.allocate(small * n * 2), ep.allocate(tall * n * 2)
+    try:
+        ops.run(a1, a_dt, small, y1)
+        eager = ep.download(y1, (small, n), np.uint16).copy()
+        ep.capture_begin()
+        try:
+            ops.run(a1, a_dt, small, y1)
+        finally:
+            graph = ep.capture_end()
+        ops.run(a2, a_dt, tall, y2)                              # needs more scratch than the recorded call had
+        ep.sync()
+        ep.copy_from_host(y1, np.full(small * n * 2, 0xFF, np.uint8))
+        graph.replay()
+        assert np.array_equal(ep.download(y1, (small, n), np.uint16), eager)
+        graph.release()
+    finally:
+        for buf in (a1, a2, y1, y2):
+            ep.deallocate(buf)
+        ops.free()
+
+
 def test_packed_copy_follows_the_weights(ep, port):
     """One kernel object, two different weight tensors in turn: the repacked copy is rebuilt when the pointers change."""
     a_dt, bs, m, n, k = E.F16, 128, 1, 96, 1024
