@@ -432,10 +432,14 @@ constexpr int kWideWaves = 8;
 // second MFMA per 32 elements. Fewer matrix-core cycles, but 95 registers instead of 80 at 16 rows: launches with
 // several workgroups per CU run better with the sixth wave per SIMD (3584 -> 152064 at 16 rows: 59 against 64 us), the
 // others with the sums (3584 -> 37888: 22.9 against 24.5 us).
-template <bool BF16, int BS, typename ST, int RB, bool SUMS>
-__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu((BS == 128 && sizeof(ST) == 2 && RB == 1) ? (SUMS ? 5 : 6) : 1)))
+// PF (with DEEP only): the next group's weights travel while the current one is multiplied (a second register set):
+// for grids with fewer workgroups than CUs, where no other workgroup covers a wave's memory latency.
+// DEEP: the activation windows travel two ahead instead of one (a second set of window registers; RB <= 2).
+template <bool BF16, int BS, typename ST, int RB, bool SUMS, bool PF, bool DEEP>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu((BS == 128 && sizeof(ST) == 2 && RB == 1) ? (PF ? (SUMS ? 3 : 4) : SUMS ? (DEEP ? 4 : 5) : (DEEP ? 5 : 6)) : 1)))
 void decode_wide_kernel(PackedParams p)
 {
+    static_assert(DEEP || !PF, "weights ahead only together with deep windows");
     constexpr int U = kGroupTiles;
     constexpr int NBT = 128 / BS;
     constexpr int NB = U * NBT;
@@ -488,6 +492,7 @@ void decode_wide_kernel(PackedParams p)
         uint4 w[kGroupTiles];
         uint4 r[NR];
     };
+    // a group past the last lies beyond the column group's range: the loads return zeros and touch no memory
     auto fetch_group = [&](Grp& grp, int gi) {
         const uint32_t soff = static_cast<uint32_t>(gi) * static_cast<uint32_t>(p.chunk_bytes);
 #pragma unroll
@@ -497,7 +502,8 @@ void decode_wide_kernel(PackedParams p)
     };
     // window fill: piece q = t + 512 i of the window's kRows * kPieces pieces -> (row q / kPieces, piece q % kPieces)
     uint4 wa[NW];
-    auto load_window = [&](int win) {
+    uint4 wb[DEEP ? NW : 1];                               // DEEP: the second set of window registers
+    auto load_window_into = [&](uint4* dst, int win) {
 #pragma unroll
         for (int i = 0; i < NW; ++i) {
             const int q = t + 512 * i;
@@ -505,21 +511,23 @@ void decode_wide_kernel(PackedParams p)
             const int64_t k0 = static_cast<int64_t>(win) * (WT * 128) + piece * 8;
             uint32_t off = static_cast<uint32_t>(row) * static_cast<uint32_t>(p.k) * 2u + static_cast<uint32_t>(piece * 16);
             if (row >= p.m || k0 >= p.k) off = kOutOfRange;       // K is a multiple of 8: a piece is all inside or all outside
-            wa[i] = load16(srd_a, off, static_cast<uint32_t>(win) * (WT * 256u));
+            dst[i] = load16(srd_a, off, static_cast<uint32_t>(win) * (WT * 256u));
         }
     };
-    auto store_window = [&](int buf) {
+    auto load_window = [&](int win) { load_window_into(wa, win); };
+    auto store_window_from = [&](const uint4* src, int buf) {
 #pragma unroll
         for (int i = 0; i < NW; ++i) {
             const int q = t + 512 * i;
             const int row = q / kPieces, piece = q % kPieces;
-            *reinterpret_cast<uint4*>(smem + buf * kBufBytes + row * kPitch + piece * 16) = wa[i];
+            *reinterpret_cast<uint4*>(smem + buf * kBufBytes + row * kPitch + piece * 16) = src[i];
             if constexpr (SUMS) {
-                const float sum = block_sum<BS>(sum_piece<BF16>(wa[i]));      // a block's pieces sit in consecutive lanes
+                const float sum = block_sum<BS>(sum_piece<BF16>(src[i]));     // a block's pieces sit in consecutive lanes
                 if (piece % kBlockLanes == 0) lds_sums[(buf * kWinBlocks + piece / kBlockLanes) * kRows + row] = sum;
             }
         }
     };
+    auto store_window = [&](int buf) { store_window_from(wa, buf); };
     // tiles [first, first + WT) of the group against window buffer `buf`
     auto compute_window = [&](const Grp& grp, int buf, int first) {
         uint32_t rr[NR * 4];
@@ -587,19 +595,52 @@ void decode_wide_kernel(PackedParams p)
 
     const int windows = p.groups * kWindowsPerGroup;
     Grp ga;
-    load_window(0);
-    store_window(0);
-    __syncthreads();
-    for (int gi = 0; gi < p.groups; ++gi) {
-        fetch_group(ga, gi);
-#pragma unroll
-        for (int h = 0; h < kWindowsPerGroup; ++h) {
-            const int win = gi * kWindowsPerGroup + h;
-            const int buf = win & 1;
-            if (win + 1 < windows) load_window(win + 1);
-            compute_window(ga, buf, h * WT);
-            if (win + 1 < windows) store_window(buf ^ 1);
+    if constexpr (DEEP) {
+        // One window per group (RB <= 2). The next window's activations sit in one register set, the one after that is
+        // in flight into the other: a pass no longer lasts at least one L2 round trip. No branch inside a pass (a branch
+        // makes the compiler wait for every load in flight): a window or group past the end loads zeros, passes run in
+        // pairs so that the register sets alternate at compile time, an odd one is peeled.
+        static_assert(!DEEP || kWindowsPerGroup == 1, "deep windows: one window per group");
+        Grp gb;
+        load_window_into(wa, 0);
+        load_window_into(wb, 1);
+        if constexpr (PF) fetch_group(ga, 0);
+        store_window_from(wa, 0);
+        __syncthreads();
+        // `ready` holds window gi + 1, `idle` receives window gi + 2
+        auto pass = [&](Grp& cur, Grp& next, int gi, const uint4* ready, uint4* idle, bool prefetch) {
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (!PF) fetch_group(cur, gi);           // needed at once: issued first, so that the wait leaves the window in flight
+            load_window_into(idle, gi + 2);
+            if constexpr (PF) {
+                if (prefetch) fetch_group(next, gi + 1);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            compute_window(cur, gi & 1, 0);
+            store_window_from(ready, (gi & 1) ^ 1);
             __syncthreads();
+        };
+        int gi = 0;
+        for (; gi + 1 < p.groups; gi += 2) {
+            pass(ga, gb, gi, wb, wa, true);
+            pass(PF ? gb : ga, ga, gi + 1, wa, wb, true);
+        }
+        if (gi < p.groups) pass(ga, gb, gi, wb, wa, false);
+    } else {
+        load_window(0);
+        store_window(0);
+        __syncthreads();
+        for (int gi = 0; gi < p.groups; ++gi) {
+            fetch_group(ga, gi);
+#pragma unroll
+            for (int h = 0; h < kWindowsPerGroup; ++h) {
+                const int win = gi * kWindowsPerGroup + h;
+                const int buf = win & 1;
+                if (win + 1 < windows) load_window(win + 1);
+                compute_window(ga, buf, h * WT);
+                if (win + 1 < windows) store_window(buf ^ 1);
+                __syncthreads();
+            }
         }
     }
 
@@ -636,13 +677,18 @@ static int launch_wide_bs(const PackedParams& p, int bs, hipStream_t stream)
         constexpr int BS = decltype(bs_tag)::value;
         // two window buffers of rows x (tiles x 256 + 16) bytes, then two tables of (blocks per window) x rows f32 sums
         constexpr int NBT = 128 / BS;
+        constexpr size_t lds16 = 2 * 16 * (4 * 256 + 16), sums16 = 2 * 4 * NBT * 16 * 4;
         if (p.m <= 16) {
-            if (grid.x >= 768) return go(decode_wide_kernel<BF16, BS, ST, 1, false>, 2 * 16 * (4 * 256 + 16));      // three or more workgroups per CU
-            return go(decode_wide_kernel<BF16, BS, ST, 1, true>, 2 * 16 * (4 * 256 + 16) + 2 * 4 * NBT * 16 * 4);
+            // Measured at 8 / 16 rows (3584 -> 152064, 3584 -> 37888, 4096 -> 16384): three or more workgroups per CU run
+            // best without the sums and with the windows two ahead (68 -> 64 us); fewer workgroups than CUs with weights
+            // and windows both ahead (17.2 -> 14.5 us); in between neither helps (20.6 us either way).
+            if (grid.x >= 768) return go(decode_wide_kernel<BF16, BS, ST, 1, false, false, true>, lds16);
+            if (grid.x < 256) return go(decode_wide_kernel<BF16, BS, ST, 1, true, true, true>, lds16 + sums16);
+            return go(decode_wide_kernel<BF16, BS, ST, 1, true, false, false>, lds16 + sums16);
         }
-        if (p.m <= 32) return go(decode_wide_kernel<BF16, BS, ST, 2, true>, 2 * 32 * (4 * 256 + 16) + 2 * 4 * NBT * 32 * 4);
+        if (p.m <= 32) return go(decode_wide_kernel<BF16, BS, ST, 2, true, false, false>, 2 * 32 * (4 * 256 + 16) + 2 * 4 * NBT * 32 * 4);
         if constexpr (BS == 32) return -1;
-        else return go(decode_wide_kernel<BF16, BS, ST, 4, true>, 2 * 64 * (2 * 256 + 16) + 2 * 2 * NBT * 64 * 4);
+        else return go(decode_wide_kernel<BF16, BS, ST, 4, true, false, false>, 2 * 64 * (2 * 256 + 16) + 2 * 2 * NBT * 64 * 4);
     };
     switch (bs) {
         case 32: return by_rows(std::integral_constant<int, 32>{});

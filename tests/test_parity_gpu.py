@@ -205,6 +205,7 @@ DECODE_CASES = [
     (E.F16, E.F16, 128, True, 13, 16385, 2048 + 8),
     (E.BF16, E.BF16, 128, True, 9, 98400, 512),         # three or more workgroups per CU: the variant with the second MFMA
     (E.F16, E.F16, 64, True, 16, 98304, 256),
+    (E.BF16, E.BF16, 128, True, 12, 98400, 1536),       # the same over three tile groups: a pair of passes and a peeled one
     (E.BF16, E.BF16, 128, True, 17, 16400, 3584),       # up to 64 rows ride on one pass over the weights
     (E.F16, E.F16, 64, True, 40, 16384, 1024 + 64),
     (E.BF16, E.F32, 128, False, 64, 16390, 2048),
