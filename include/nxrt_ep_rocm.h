@@ -72,11 +72,16 @@ NxrtRocmEp* nxrt_rocm_ep_from_vtable(const NxrtEpVtable* vtable);
 
 /* Node attributes of MatMulNBits. `present` has bit i set when attribute i was on the node:
  * 0=K 1=N 2=bits 3=block_size 4=accuracy_level 5=weight_prepacked
- * (onnx-runtime-ep-cpu/src/kernels/matmul_nbits.rs:1410-1481). */
+ * (onnx-runtime-ep-cpu/src/kernels/matmul_nbits.rs:1410-1481), and 6=folded_bias: the marker an optimizer pass sets
+ * when it folds a standalone Add into the bias input (the CUDA provider's `_cuda_matmul_nbits_folded_bias`,
+ * onnx-runtime-ep-cuda/src/optimizer.rs:35, kernels/matmul_nbits.rs:1189-1212). With folded_bias = 1 and a 16-bit
+ * output the result is round(round(acc) + bias), bit for bit what the two nodes gave; otherwise round(acc + bias).
+ * struct_size tells which fields the caller's struct has: one that ends after weight_prepacked is read as folded_bias = 0. */
 typedef struct NxrtRocmMatMulNBitsAttrs {
   uint32_t struct_size;
   uint32_t present;
   int64_t K, N, bits, block_size, accuracy_level, weight_prepacked;
+  int64_t folded_bias;
 } NxrtRocmMatMulNBitsAttrs;
 
 /* C layout of TensorView / TensorMut (crates/onnx-runtime-ep-api/src/tensor.rs:132-143, 241).

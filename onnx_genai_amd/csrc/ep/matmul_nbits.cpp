@@ -2,6 +2,7 @@
 // Attribute parsing, input validation and their messages follow the reference's CPU kernel
 // (crates/onnx-runtime-ep-cpu/src/kernels/matmul_nbits.rs:1410-1600, helpers at :10254-10378);
 // the contiguity rule follows its CUDA sibling (crates/onnx-runtime-ep-cuda/src/kernels/matmul_nbits.rs:7089-7106).
+#include <cstddef>
 #include <mutex>
 #include <string>
 #include <vector>
@@ -12,7 +13,7 @@ using namespace nxrt_rocm;
 
 namespace {
 
-enum AttrBit { kAttrK = 0, kAttrN = 1, kAttrBits = 2, kAttrBlockSize = 3, kAttrAccuracy = 4, kAttrPrepacked = 5 };
+enum AttrBit { kAttrK = 0, kAttrN = 1, kAttrBits = 2, kAttrBlockSize = 3, kAttrAccuracy = 4, kAttrPrepacked = 5, kAttrFoldedBias = 6 };
 
 std::string err(const std::string& message) { return "MatMulNBits: " + message; }   // matmul_nbits.rs:10376
 
@@ -119,6 +120,7 @@ struct NxrtRocmMatMulNBits {
     NxrtRocmEp* ep = nullptr;
     int64_t k = 0, n = 0, block_size = 0, accuracy_level = 0;
     int64_t rows_hint = -1;              // M when the create-time shape of A was static
+    bool bias_post_round = false;        // the bias is a folded Add: round(round(acc) + bias) on 16-bit outputs
     bool constant_inputs[6] = {false, false, false, false, false, false};
     std::string variant = "none";
     void* scratch = nullptr;             // kernel-owned workspace, grown on demand
@@ -227,6 +229,7 @@ bool dense_route(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& args, int& 
     if ((reinterpret_cast<uintptr_t>(args.a) & 15) != 0 || (reinterpret_cast<uintptr_t>(args.y) & 15) != 0 || (reinterpret_cast<uintptr_t>(args.b) & 3) != 0) return false;
     const uint64_t need = static_cast<uint64_t>(args.n) * static_cast<uint64_t>(args.k) * 2;
     if (need > ep.dense_gemm_max_bytes) return false;
+    if (args.bias && (args.bias_dtype & ROCM_BIAS_POST_ROUND)) return false;      // the library's epilogue adds the bias before the one rounding
     const int bias_dtype = args.bias ? args.bias_dtype : -1;
 
     std::lock_guard<std::mutex> lock(ep.dense_mu);
@@ -420,6 +423,7 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
     args.a_dtype = static_cast<int>(A.dtype);
     args.scale_dtype = static_cast<int>(S.dtype);
     args.bias_dtype = BIAS ? static_cast<int>(BIAS->dtype) : ROCM_DT_F32;
+    if (BIAS && kn.bias_post_round) args.bias_dtype |= ROCM_BIAS_POST_ROUND;
     args.y_dtype = static_cast<int>(Y.dtype);
     args.m = static_cast<int64_t>(M);
     args.n = kn.n;
@@ -597,6 +601,8 @@ NxrtStatus nxrt_rocm_matmul_nbits_create(NxrtRocmEp* ep, const NxrtRocmMatMulNBi
         kn->n = attrs->N;
         kn->block_size = attrs->block_size;
         kn->accuracy_level = (attrs->present & (1u << kAttrAccuracy)) ? attrs->accuracy_level : 0;
+        const bool has_folded_bias = attrs->struct_size >= offsetof(NxrtRocmMatMulNBitsAttrs, folded_bias) + sizeof(int64_t);
+        kn->bias_post_round = has_folded_bias && (attrs->present & (1u << kAttrFoldedBias)) && attrs->folded_bias == 1;
         // flops::leading_rows: product of A's leading dims when all are static
         if (input_shapes && n_inputs >= 1 && input_shapes[0].ndim >= 1 && input_shapes[0].dims) {
             int64_t rows = 1;

@@ -18,6 +18,10 @@ typedef void* rocm_event_t;
 
 /* element dtypes on the wire (onnx-runtime-ir DataType discriminants) */
 enum { ROCM_DT_F32 = 1, ROCM_DT_U8 = 2, ROCM_DT_I32 = 6, ROCM_DT_F16 = 10, ROCM_DT_BF16 = 16 };
+/* Or-ed into a bias dtype: the bias is a folded standalone Add. The accumulator is rounded to the output's 16-bit type
+ * first and the bias added with a second rounding, round(round(acc) + bias), which is what MatMulNBits followed by Add
+ * produces (onnx-runtime-ep-cuda/src/kernels/matmul_nbits.rs:1189-1212). Without it: round(acc + bias). */
+enum { ROCM_BIAS_POST_ROUND = 0x100 };
 
 const char* rocm_ffi_error_string(int err);
 int rocm_ffi_device_count(int* count);
@@ -51,7 +55,7 @@ typedef struct RocmMatMulNBitsArgs {
   const uint8_t* b;     /* [N, kb, bs/2] */
   const void* scales;   /* [N, kb] scale_dtype */
   const uint8_t* zp;    /* [N, ceil(kb/2)] or NULL (zero point 8) */
-  const void* bias;     /* [N] bias_dtype or NULL */
+  const void* bias;     /* [N] bias_dtype or NULL; bias_dtype may carry ROCM_BIAS_POST_ROUND */
   void* y;              /* [M, N] y_dtype */
   int a_dtype, scale_dtype, bias_dtype, y_dtype;
   int64_t m, n, k;

@@ -376,7 +376,7 @@ void decode_packed_kernel(PackedParams p)
         if (row < p.m && col < p.n) {
             float total = 0.f;
             for (int w = 0; w < waves; ++w) total += red[(w * 4 + r) * 64 + l];
-            if (p.bias) total += load_as_f32(p.bias, p.bias_dtype, col);
+            total = with_bias(total, p.bias, p.bias_dtype, col, p.y_dtype);
             store_from_f32(p.y, p.y_dtype, static_cast<int64_t>(row) * p.n + col, total);
         }
     }
@@ -647,13 +647,13 @@ void decode_wide_kernel(PackedParams p)
     if (active) {
         const int64_t col = n_base + c;
         if (col < p.n) {
-            const float bias = p.bias ? load_as_f32(p.bias, p.bias_dtype, col) : 0.f;
+            const BiasTerm bias = load_bias(p.bias, p.bias_dtype, col);
 #pragma unroll
             for (int rb = 0; rb < RB; ++rb) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const int row = rb * 16 + 4 * g + r;
-                    if (row < p.m) store_from_f32(p.y, p.y_dtype, static_cast<int64_t>(row) * p.n + col, y[rb][r] + bias);
+                    if (row < p.m) store_from_f32(p.y, p.y_dtype, static_cast<int64_t>(row) * p.n + col, add_bias(y[rb][r], bias, p.y_dtype));
                 }
             }
         }
@@ -925,7 +925,7 @@ __global__ __launch_bounds__(512) void acc4_packed_kernel(Acc4PackedParams p)
         if (col < p.n) {
             float total = 0.f;
             for (int w = 0; w < waves; ++w) total += red[w * 16 + threadIdx.x];
-            if (p.bias) total += load_as_f32(p.bias, p.bias_dtype, col);
+            total = with_bias(total, p.bias, p.bias_dtype, col, p.y_dtype);
             store_from_f32(p.y, p.y_dtype, col, total);
         }
     }

@@ -49,7 +49,7 @@ class NxrtTensorDesc(C.Structure):
 
 class Attrs(C.Structure):
     _fields_ = [("struct_size", C.c_uint32), ("present", C.c_uint32), ("K", C.c_int64), ("N", C.c_int64), ("bits", C.c_int64),
-                ("block_size", C.c_int64), ("accuracy_level", C.c_int64), ("weight_prepacked", C.c_int64)]
+                ("block_size", C.c_int64), ("accuracy_level", C.c_int64), ("weight_prepacked", C.c_int64), ("folded_bias", C.c_int64)]
 
 
 class CTensorView(C.Structure):
@@ -61,7 +61,7 @@ class WorkspaceRequirement(C.Structure):
     _fields_ = [("bytes", C.c_uint64), ("alignment", C.c_uint64)]
 
 
-_ATTR_BITS = {"K": 0, "N": 1, "bits": 2, "block_size": 3, "accuracy_level": 4, "weight_prepacked": 5}
+_ATTR_BITS = {"K": 0, "N": 1, "bits": 2, "block_size": 3, "accuracy_level": 4, "weight_prepacked": 5, "folded_bias": 6}
 _lib = None
 
 
@@ -447,7 +447,8 @@ _NP = {F32: np.float32, F16: np.float16, BF16: np.uint16, U8: np.uint8, I8: np.i
 class DeviceOperands:
     """The device-resident operands of one MatMulNBits node plus its kernel; what a session would hold."""
 
-    def __init__(self, ep, b, scales, scale_dtype, zp, n, k, bs, *, accuracy_level=0, bias=None, bias_dtype=F32, rows=None, a_dtype=None):
+    def __init__(self, ep, b, scales, scale_dtype, zp, n, k, bs, *, accuracy_level=0, bias=None, bias_dtype=F32, rows=None, a_dtype=None,
+                 folded_bias=None):
         self.ep, self.n, self.k, self.bs = ep, n, k, bs
         self.kb = -(-k // bs)
         self.scale_dtype, self.bias_dtype = scale_dtype, bias_dtype
@@ -458,7 +459,7 @@ class DeviceOperands:
         shapes = None
         if rows is not None and a_dtype is not None:
             shapes = [((rows, k), a_dtype), ((n, self.kb, bs // 2), U8), ((n, self.kb), scale_dtype)]
-        self.kernel = ep.get_kernel({"K": k, "N": n, "bits": 4, "block_size": bs, "accuracy_level": accuracy_level}, shapes)
+        self.kernel = ep.get_kernel({"K": k, "N": n, "bits": 4, "block_size": bs, "accuracy_level": accuracy_level, "folded_bias": folded_bias}, shapes)
         self.kernel.set_constant_inputs([False, True, True, True, True, True])
 
     def views(self, a_buf: DeviceBuffer, a_dtype: int, m: int):
@@ -485,12 +486,12 @@ class DeviceOperands:
                 self.ep.deallocate(buf)
 
 
-def matmul_nbits(ep, a, a_dtype, b, scales, scale_dtype, zp, n, k, bs, *, accuracy_level=0, bias=None, bias_dtype=F32, y_dtype=None):
+def matmul_nbits(ep, a, a_dtype, b, scales, scale_dtype, zp, n, k, bs, *, accuracy_level=0, bias=None, bias_dtype=F32, y_dtype=None, folded_bias=None):
     """One-shot helper: upload, execute through the C ABI, download. Returns (Y as numpy, variant name)."""
     y_dtype = a_dtype if y_dtype is None else y_dtype
     a = np.ascontiguousarray(a)
     m = a.size // k
-    ops = DeviceOperands(ep, b, scales, scale_dtype, zp, n, k, bs, accuracy_level=accuracy_level, bias=bias, bias_dtype=bias_dtype)
+    ops = DeviceOperands(ep, b, scales, scale_dtype, zp, n, k, bs, accuracy_level=accuracy_level, bias=bias, bias_dtype=bias_dtype, folded_bias=folded_bias)
     a_buf = ep.upload(a)
     y_buf = ep.allocate(max(m * n * _ITEM[y_dtype], 1))
     try:

@@ -501,6 +501,60 @@ def test_prefill_weight_tiles_are_f16_of_f32_dequant(ep, port, bs, zero_points):
 
 
 # ---------------------------------------------------------------------------------------------
+# folded bias: a standalone Add folded into the bias input keeps the two nodes' two roundings
+# ---------------------------------------------------------------------------------------------
+FOLDED_BIAS_CASES = [
+    # a_dt, bs, accuracy_level, m, n, k: one per kernel family
+    (E.BF16, 128, 0, 1, 300, 3584),        # one row over the repacked stream
+    (E.F16, 32, 0, 4, 130, 896),           # four rows over the repacked stream
+    (E.BF16, 128, 0, 8, 16400, 1024),      # shared-activation kernel
+    (E.F16, 64, 0, 16, 100, 2048),         # split-K kernel
+    (E.F16, 32, 0, 200, 136, 512),         # tiled kernel
+    (E.F16, 64, 0, 100, 130, 4096),        # tiled kernel, K in slices: the reduce kernel adds the bias
+    (E.F16, 32, 0, 1100, 136, 512),        # tall call
+    (E.BF16, 16, 0, 3, 40, 64),            # catch-all kernel
+    (E.F16, 64, 4, 1, 160, 1024),          # accuracy_level 4, one row
+    (E.F16, 64, 4, 5, 96, 512),            # accuracy_level 4, split-K
+    (E.BF16, 128, 4, 130, 200, 2560),      # accuracy_level 4, tiled, K in slices
+    (E.F16, 16, 4, 20, 64, 256),           # accuracy_level 4, catch-all
+]
+
+
+@pytest.mark.parametrize("a_dt,bs,acc,m,n,k", FOLDED_BIAS_CASES)
+def test_folded_bias_rounds_twice(ep_tiled, port, a_dt, bs, acc, m, n, k):
+    """folded_bias = 1 on a 16-bit output gives round(round(acc) + bias), i.e. exactly what the same kernel without a bias
+    followed by a 16-bit Add gives (onnx-runtime-ep-cuda/src/kernels/matmul_nbits.rs:1189-1212); without the marker the
+    bias joins the accumulator before the one rounding."""
+    ep = ep_tiled                                    # with and without a bias the same hand-written kernel must serve the call
+    b, s, zp = synth.make_weights(n, k, bs, 700 + n, zero_points=True, scale_lo=0.002, scale_hi=0.01, scale_dtype=a_dt)
+    a = synth.make_activation(m, k, 700 + m, a_dt)
+    bias = synth.to_dtype((np.random.default_rng(n).standard_normal(n) * 0.37).astype(np.float32), a_dt)
+    o_dt = oracle.F16 if a_dt == E.F16 else oracle.BF16
+    common = dict(accuracy_level=acc)
+    plain, v0 = run_op(ep, a, a_dt, b, s, a_dt, zp, n, k, bs, **common)
+    folded, v1 = run_op(ep, a, a_dt, b, s, a_dt, zp, n, k, bs, bias=bias, bias_dtype=a_dt, folded_bias=1, **common)
+    fused, _ = run_op(ep, a, a_dt, b, s, a_dt, zp, n, k, bs, bias=bias, bias_dtype=a_dt, **common)
+    fused32, _ = run_op(ep, a, a_dt, b, s, a_dt, zp, n, k, bs, bias=bias, bias_dtype=a_dt, y_dtype=E.F32, **common)
+    assert v0 == v1
+    want = port.narrow(synth.to_f32(plain, a_dt) + synth.to_f32(bias, a_dt)[None, :], o_dt)
+    assert np.array_equal(np.asarray(folded).view(np.uint16), np.asarray(want).view(np.uint16))
+    assert np.array_equal(np.asarray(fused).view(np.uint16), np.asarray(port.narrow(fused32, o_dt)).view(np.uint16))
+    assert not np.array_equal(np.asarray(folded).view(np.uint16), np.asarray(fused).view(np.uint16)) or m * n < 2000
+
+
+def test_folded_bias_keeps_tall_calls_off_the_library_gemm(ep):
+    """The library's epilogue adds a bias before the one rounding, so a folded bias stays on the hand-written kernel."""
+    a_dt, bs, m, n, k = E.F16, 32, 1100, 136, 512
+    b, s, zp = synth.make_weights(n, k, bs, 5, zero_points=False, scale_lo=0.002, scale_hi=0.01, scale_dtype=a_dt)
+    a = synth.make_activation(m, k, 5, a_dt)
+    bias = synth.to_dtype(np.linspace(-1, 1, n).astype(np.float32), a_dt)
+    _, variant = run_op(ep, a, a_dt, b, s, a_dt, zp, n, k, bs, bias=bias, bias_dtype=a_dt, folded_bias=1)
+    assert variant == "prefill_mfma_lds"
+    _, variant = run_op(ep, a, a_dt, b, s, a_dt, zp, n, k, bs, bias=bias, bias_dtype=a_dt)
+    assert variant == "dense_transient_blaslt"
+
+
+# ---------------------------------------------------------------------------------------------
 # dense route: weights expanded to 16 bits, then the library GEMM (tall calls)
 # ---------------------------------------------------------------------------------------------
 DENSE_CASES = [
