@@ -76,12 +76,19 @@ NxrtRocmEp* nxrt_rocm_ep_from_vtable(const NxrtEpVtable* vtable);
  * when it folds a standalone Add into the bias input (the CUDA provider's `_cuda_matmul_nbits_folded_bias`,
  * onnx-runtime-ep-cuda/src/optimizer.rs:35, kernels/matmul_nbits.rs:1189-1212). With folded_bias = 1 and a 16-bit
  * output the result is round(round(acc) + bias), bit for bit what the two nodes gave; otherwise round(acc + bias).
- * struct_size tells which fields the caller's struct has: one that ends after weight_prepacked is read as folded_bias = 0. */
+ * 7=gate_up_swiglu, 8=decomposed_silu: the CUDA provider's fused gate/up node (`_cuda_gate_up_swiglu`, `_cuda_decomposed_silu`,
+ * onnx-runtime-ep-cuda/src/optimizer.rs:14, 36-46; kernels/matmul_nbits.rs:9017-9130). With gate_up_swiglu = 1 the inputs are
+ * [x, W_gate, scales_gate, W_up, scales_up, (gamma: must be absent), (zp_gate, zp_up: both or neither)], x and Y Float16 or
+ * BFloat16, and Y = round16(silu(round16(x W_gate^T)) * round16(x W_up^T)) - bit for bit what the two projections followed by
+ * the 16-bit silu-and-multiply give (kernels/matmul_nbits.rs:4207-4233, 4375-4386). workspace_requirement then sizes the
+ * two 16-bit [M, N] intermediates.
+ * struct_size tells which fields the caller's struct has: fields past its end are read as 0. */
 typedef struct NxrtRocmMatMulNBitsAttrs {
   uint32_t struct_size;
   uint32_t present;
   int64_t K, N, bits, block_size, accuracy_level, weight_prepacked;
   int64_t folded_bias;
+  int64_t gate_up_swiglu, decomposed_silu;
 } NxrtRocmMatMulNBitsAttrs;
 
 /* C layout of TensorView / TensorMut (crates/onnx-runtime-ep-api/src/tensor.rs:132-143, 241).

@@ -21,6 +21,7 @@ HIP_SOURCES = [
     "kernels/decode_packed.hip",
     "kernels/prefill_mfma.hip",
     "kernels/dense_gemm.hip",
+    "kernels/swiglu.hip",
     "kernels/acc4.hip",
     "kernels/acc4_mfma.hip",
 ]

@@ -13,7 +13,7 @@ using namespace nxrt_rocm;
 
 namespace {
 
-enum AttrBit { kAttrK = 0, kAttrN = 1, kAttrBits = 2, kAttrBlockSize = 3, kAttrAccuracy = 4, kAttrPrepacked = 5, kAttrFoldedBias = 6 };
+enum AttrBit { kAttrK = 0, kAttrN = 1, kAttrBits = 2, kAttrBlockSize = 3, kAttrAccuracy = 4, kAttrPrepacked = 5, kAttrFoldedBias = 6, kAttrGateUpSwiglu = 7, kAttrDecomposedSilu = 8 };
 
 std::string err(const std::string& message) { return "MatMulNBits: " + message; }   // matmul_nbits.rs:10376
 
@@ -121,6 +121,11 @@ struct NxrtRocmMatMulNBits {
     int64_t k = 0, n = 0, block_size = 0, accuracy_level = 0;
     int64_t rows_hint = -1;              // M when the create-time shape of A was static
     bool bias_post_round = false;        // the bias is a folded Add: round(round(acc) + bias) on 16-bit outputs
+    // The fused gate/up node: two ordinary kernels (each with its own repacked copy, scratch and variant) whose 16-bit
+    // results meet in the silu(gate) * up epilogue.
+    bool gate_up_swiglu = false, decomposed_silu = false;
+    NxrtRocmMatMulNBits* gate = nullptr;
+    NxrtRocmMatMulNBits* up = nullptr;
     bool constant_inputs[6] = {false, false, false, false, false, false};
     std::string variant = "none";
     void* scratch = nullptr;             // kernel-owned workspace, grown on demand
@@ -138,6 +143,8 @@ struct NxrtRocmMatMulNBits {
 
     ~NxrtRocmMatMulNBits()
     {
+        delete gate;
+        delete up;
         if ((scratch || packed || dense || !retired.empty()) && ep && ep->bind().code == NXRT_OK) {
             rocm_ffi_stream_sync(ep->stream);
             for (void* old : retired) rocm_ffi_free(old);
@@ -512,11 +519,89 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
     return hip_status(rc, "MatMulNBits: kernel launch");
 }
 
+// The fused gate/up node of the CUDA provider (onnx-runtime-ep-cuda/src/optimizer.rs:36-46, kernels/matmul_nbits.rs:9017-9130):
+// inputs [x, W_gate, scales_gate, W_up, scales_up, (gamma), (zp_gate, zp_up)], output silu(gate) * up with both projections
+// rounded to the 16-bit type first. Here both projections run through the ordinary dispatch into scratch, then the epilogue.
+NxrtStatus execute_swiglu(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, uint32_t n_in, NxrtRocmTensorView* out, uint32_t n_out,
+                          void* workspace, uint64_t workspace_bytes)
+{
+    std::lock_guard<std::mutex> lock(kn.mu);
+    if (n_in < 5 || n_in > 8 || n_out != 1)
+        return make_status(NXRT_INVALID_ARGUMENT, err("gate/up SwiGLU fusion expects 5 to 8 inputs [x, W_gate, scales_gate, W_up, scales_up, (gamma), "
+                                                      "(zp_gate, zp_up)] and 1 output, got " + std::to_string(n_in) + " inputs and " + std::to_string(n_out) + " outputs"));
+    if (!in || !out) return make_status(NXRT_INVALID_ARGUMENT, "MatMulNBits: null tensor view array");
+    auto optional = [&](uint32_t i) -> const NxrtRocmTensorView* { return (i < n_in && in[i].data != nullptr) ? &in[i] : nullptr; };
+    if (optional(5))
+        return make_status(NXRT_INVALID_ARGUMENT, err("gate/up SwiGLU fusion with an RMS-norm prologue (gamma at input 5) is not supported on the ROCm execution "
+                                                      "provider. How to fix: leave the normalization as its own node"));
+    const NxrtRocmTensorView* zp_gate = optional(6);
+    const NxrtRocmTensorView* zp_up = optional(7);
+    if ((zp_gate != nullptr) != (zp_up != nullptr))
+        return make_status(NXRT_INVALID_ARGUMENT, err("gate/up SwiGLU fusion requires zero points for both projections or neither"));
+    const NxrtRocmTensorView& A = in[0];
+    NxrtRocmTensorView& Y = out[0];
+    if (A.dtype != NXRT_DT_FLOAT16 && A.dtype != NXRT_DT_BFLOAT16)
+        return make_status(NXRT_INVALID_ARGUMENT, err(std::string("gate/up SwiGLU fusion needs Float16 or BFloat16 activations, got ") + dtype_name(A.dtype)));
+    if (Y.dtype != A.dtype)
+        return make_status(NXRT_INVALID_ARGUMENT, err(std::string("Y must have dtype ") + dtype_name(A.dtype) + ", got " + dtype_name(Y.dtype)));
+    const uint64_t K = static_cast<uint64_t>(kn.k), N = static_cast<uint64_t>(kn.n);
+    if (A.ndim == 0 || A.shape[A.ndim - 1] != K)
+        return make_status(NXRT_INVALID_ARGUMENT, err("A must have rank >= 1 and last dimension K=" + std::to_string(K) + ", got " + shape_str(A.shape, A.ndim)));
+    std::vector<uint64_t> y_shape(A.shape, A.shape + A.ndim - 1);
+    y_shape.push_back(N);
+    if (!shape_is(Y, y_shape)) return make_status(NXRT_INVALID_ARGUMENT, err("Y must have shape " + shape_str(y_shape) + ", got " + shape_str(Y.shape, Y.ndim)));
+    if (!is_contiguous(Y)) return make_status(NXRT_INVALID_ARGUMENT, err("Y must be contiguous on the ROCm execution provider"));
+    if (Y.device_type != NXRT_DEVICE_ROCM || Y.device_index != kn.ep->device)
+        return make_status(NXRT_INVALID_ARGUMENT, err("Y must live on ROCm device " + std::to_string(kn.ep->device) + " (allocate it with this provider and copy the data in)"));
+    uint64_t M = 1;
+    for (uint32_t i = 0; i + 1 < A.ndim; ++i) M *= A.shape[i];
+    if (M == 0) return ok();
+    NxrtStatus st = kn.ep->bind();
+    if (st.code != NXRT_OK) return st;
+
+    // two 16-bit [M, N] matrices: the caller's workspace if it is large enough, else the kernel's own
+    const uint64_t each = (M * N * 2 + 255) / 256 * 256;
+    uint8_t* ws = static_cast<uint8_t*>(workspace);
+    if (!ws || workspace_bytes < 2 * each) {
+        if (kn.scratch_bytes < 2 * each) {
+            if (kn.ep->capturing)
+                return make_status(NXRT_INVALID_ARGUMENT, err("gate/up SwiGLU fusion under graph capture needs a caller workspace of " + std::to_string(2 * each) +
+                                                              " bytes (see workspace_requirement), or one eager call of this height first"));
+            const int e = grow_buffer(kn.scratch, kn.scratch_bytes, 2 * each, kn.retired);
+            if (e != 0) return hip_status(e, "MatMulNBits: workspace hipMalloc");
+        }
+        ws = static_cast<uint8_t*>(kn.scratch);
+    }
+    auto run = [&](NxrtRocmMatMulNBits& child, const NxrtRocmTensorView& w, const NxrtRocmTensorView& s, const NxrtRocmTensorView* zp, void* dst) {
+        NxrtRocmTensorView cin[4];
+        cin[0] = A;
+        cin[1] = w;
+        cin[2] = s;
+        if (zp) cin[3] = *zp;
+        NxrtRocmTensorView cy = Y;
+        cy.data = dst;
+        cy.byte_offset = 0;
+        cy.strides = nullptr;
+        return execute_impl(child, cin, zp ? 4u : 3u, &cy, 1, nullptr, 0);
+    };
+    st = run(*kn.gate, in[1], in[2], zp_gate, ws);
+    if (st.code != NXRT_OK) return st;
+    st = run(*kn.up, in[3], in[4], zp_up, ws + each);
+    if (st.code != NXRT_OK) return st;
+    void* y = static_cast<uint8_t*>(Y.data) + Y.byte_offset;
+    const int rc = rocm_launch_swiglu(ws, ws + each, static_cast<int64_t>(M * N), static_cast<int>(A.dtype), kn.decomposed_silu ? 1 : 0, y, kn.ep->stream);
+    kn.ep->launches.fetch_add(1);
+    kn.variant = "gate_up_swiglu[" + kn.gate->variant + "]";
+    return hip_status(rc, "MatMulNBits: kernel launch");
+}
+
 NxrtStatus vtable_execute(void* ctx, const void* const* inputs, uint32_t n_in, void** outputs, uint32_t n_out)
 {
     return fenced([&]() -> NxrtStatus {
         auto* kn = static_cast<NxrtRocmMatMulNBits*>(ctx);
         if (!kn || !inputs || !outputs) return make_status(NXRT_INVALID_ARGUMENT, "MatMulNBits: null pointer in kernel vtable execute");
+        if (kn->gate_up_swiglu)
+            return make_status(NXRT_INVALID_ARGUMENT, err("the fused gate/up node is not served through the raw kernel vtable; call nxrt_rocm_matmul_nbits_execute"));
         if (kn->rows_hint < 0)
             return make_status(NXRT_INVALID_ARGUMENT, err("the kernel vtable carries no shapes; create the kernel with a static shape for A"));
         const uint64_t K = kn->k, N = kn->n, BS = kn->block_size, kb = (K + BS - 1) / BS;
@@ -573,6 +658,15 @@ int nxrt_rocm_ep_supports_matmul_nbits(const NxrtRocmEp* ep, const NxrtRocmMatMu
     check_attrs(*attrs, c);
     if (c.failed) return decline(c.message);
     if (inputs) {
+        const bool swiglu = attrs->struct_size >= offsetof(NxrtRocmMatMulNBitsAttrs, gate_up_swiglu) + sizeof(int64_t) &&
+                            (attrs->present & (1u << kAttrGateUpSwiglu)) && attrs->gate_up_swiglu == 1;
+        if (swiglu) {
+            if (n_inputs < 5 || n_inputs > 8) return decline(err("gate/up SwiGLU fusion expects 5 to 8 inputs, got " + std::to_string(n_inputs)));
+            if (inputs[0].dtype != NXRT_DT_FLOAT16 && inputs[0].dtype != NXRT_DT_BFLOAT16)
+                return decline(err(std::string("gate/up SwiGLU fusion needs Float16 or BFloat16 activations, got ") + dtype_name(inputs[0].dtype)));
+            if (n_inputs > 5 && inputs[5].dtype != 0) return decline(err("gate/up SwiGLU fusion with an RMS-norm prologue (gamma at input 5) is not supported on the ROCm execution provider"));
+            return 1;
+        }
         if (n_inputs < 3 || n_inputs > 6) return decline("MatMulNBits: expected 3..=6 inputs, got " + std::to_string(n_inputs));
         if (!is_float_compute(inputs[0].dtype)) return decline(err(std::string("A must have dtype Float32, Float16, or BFloat16, got ") + dtype_name(inputs[0].dtype)));
         if (inputs[1].dtype != NXRT_DT_UINT8) return decline(err(std::string("B must have dtype Uint8, got ") + dtype_name(inputs[1].dtype)));
@@ -616,6 +710,21 @@ NxrtStatus nxrt_rocm_matmul_nbits_create(NxrtRocmEp* ep, const NxrtRocmMatMulNBi
             kn->vt_y_dtype = input_shapes[0].dtype;
             kn->vt_scale_dtype = n_inputs >= 3 ? input_shapes[2].dtype : input_shapes[0].dtype;
         }
+        const bool has_swiglu = attrs->struct_size >= offsetof(NxrtRocmMatMulNBitsAttrs, decomposed_silu) + sizeof(int64_t);
+        kn->gate_up_swiglu = has_swiglu && (attrs->present & (1u << kAttrGateUpSwiglu)) && attrs->gate_up_swiglu == 1;
+        kn->decomposed_silu = has_swiglu && (attrs->present & (1u << kAttrDecomposedSilu)) && attrs->decomposed_silu == 1;
+        if (kn->gate_up_swiglu) {
+            for (NxrtRocmMatMulNBits** child : {&kn->gate, &kn->up}) {
+                auto* c2 = new NxrtRocmMatMulNBits();
+                c2->ep = ep;
+                c2->k = kn->k;
+                c2->n = kn->n;
+                c2->block_size = kn->block_size;
+                c2->accuracy_level = kn->accuracy_level;
+                c2->rows_hint = kn->rows_hint;
+                *child = c2;
+            }
+        }
         std::memset(&kn->vtable, 0, sizeof(kn->vtable));
         kn->vtable.struct_size = sizeof(NxrtKernelVtable);
         kn->vtable.execute = vtable_execute;
@@ -629,6 +738,16 @@ NxrtStatus nxrt_rocm_matmul_nbits_create(NxrtRocmEp* ep, const NxrtRocmMatMulNBi
 void nxrt_rocm_matmul_nbits_set_constant_inputs(NxrtRocmMatMulNBits* kernel, const uint8_t* is_constant, uint32_t n)
 {
     if (!kernel) return;
+    if (kernel->gate_up_swiglu) {
+        // [x, W_gate, scales_gate, W_up, scales_up, gamma, zp_gate, zp_up] -> each projection's [x, B, scales, zero_points]
+        auto flag = [&](uint32_t i) { return is_constant && i < n && is_constant[i] != 0; };
+        const uint32_t gate_slots[4] = {0, 1, 2, 6}, up_slots[4] = {0, 3, 4, 7};
+        for (uint32_t i = 0; i < 4; ++i) {
+            kernel->gate->constant_inputs[i] = flag(gate_slots[i]);
+            kernel->up->constant_inputs[i] = flag(up_slots[i]);
+        }
+        return;
+    }
     for (uint32_t i = 0; i < 6; ++i) kernel->constant_inputs[i] = (is_constant && i < n) ? is_constant[i] != 0 : false;
 }
 
@@ -650,6 +769,11 @@ NxrtStatus nxrt_rocm_matmul_nbits_workspace_requirement(const NxrtRocmMatMulNBit
                 return make_status(NXRT_INVALID_ARGUMENT, err("workspace_requirement needs static leading dimensions of A"));
             }
             m *= static_cast<uint64_t>(inputs[0].dims[i]);
+        }
+        if (kernel->gate_up_swiglu) {
+            out->bytes = 2 * ((m * static_cast<uint64_t>(kernel->n) * 2 + 255) / 256 * 256);     // both projections, 16 bits each
+            out->alignment = 256;
+            return ok();
         }
         if (kernel->accuracy_level == 4) {
             out->bytes = acc4_workspace_bytes(*kernel, m);
@@ -678,6 +802,7 @@ NxrtStatus nxrt_rocm_matmul_nbits_execute(NxrtRocmMatMulNBits* kernel, const Nxr
 {
     return fenced([&]() -> NxrtStatus {
         if (!kernel) return make_status(NXRT_INVALID_ARGUMENT, "MatMulNBits: null kernel");
+        if (kernel->gate_up_swiglu) return execute_swiglu(*kernel, inputs, n_inputs, outputs, n_outputs, workspace_device, workspace_bytes);
         return execute_impl(*kernel, inputs, n_inputs, outputs, n_outputs, workspace_device, workspace_bytes);
     });
 }
@@ -685,7 +810,7 @@ NxrtStatus nxrt_rocm_matmul_nbits_execute(NxrtRocmMatMulNBits* kernel, const Nxr
 uint64_t nxrt_rocm_matmul_nbits_estimated_flops(const NxrtRocmMatMulNBits* kernel)
 {
     if (!kernel || kernel->rows_hint < 0) return 0;
-    return 2ull * static_cast<uint64_t>(kernel->rows_hint) * static_cast<uint64_t>(kernel->n) * static_cast<uint64_t>(kernel->k);
+    return (kernel->gate_up_swiglu ? 4ull : 2ull) * static_cast<uint64_t>(kernel->rows_hint) * static_cast<uint64_t>(kernel->n) * static_cast<uint64_t>(kernel->k);
 }
 
 const char* nxrt_rocm_matmul_nbits_last_variant(const NxrtRocmMatMulNBits* kernel) { return kernel ? kernel->variant.c_str() : ""; }

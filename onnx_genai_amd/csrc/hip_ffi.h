@@ -82,6 +82,10 @@ int rocm_dense_gemm_ready(RocmDenseGemm* g, int64_t m, int64_t n, int64_t k, int
 int rocm_dense_gemm_run(RocmDenseGemm* g, const void* w_nk, const void* a, void* y, const void* bias, int bias_dtype,
                         int64_t m, int64_t n, int64_t k, int dtype, rocm_stream_t stream);
 
+/* y = round16(silu(gate) * up) over `count` 16-bit elements (f16 or bf16): the epilogue of the fused gate/up node
+ * (onnx-runtime-ep-cuda/src/kernels/matmul_nbits.rs:4207-4233, 4375-4386). decomposed = 1: silu spelled as Sigmoid and Mul. */
+int rocm_launch_swiglu(const void* gate, const void* up, int64_t count, int dtype, int decomposed, void* y, rocm_stream_t stream);
+
 /* Any dtype mix, any K, any block size: f32 math, one wave per output column. */
 int rocm_launch_gemv_generic(const RocmMatMulNBitsArgs* args, rocm_stream_t stream);
 /* f32 activations, M <= 4, block size >= 32, K % 4 == 0, A and B 16-byte aligned: f32 FMA streaming kernel */

@@ -38,8 +38,9 @@ __global__ __launch_bounds__(256) void dequant_16_kernel(
         uint32_t pair[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const float lo = __fmul_rn(static_cast<float>((w >> (8 * i)) & 0xf) - z, s);
-            const float hi = __fmul_rn(static_cast<float>((w >> (8 * i + 4)) & 0xf) - z, s);
+            // as_f32: the f32 product is a value of its own (f32 scales: a fused product-and-convert would round once)
+            const float lo = as_f32(__fmul_rn(static_cast<float>((w >> (8 * i)) & 0xf) - z, s));
+            const float hi = as_f32(__fmul_rn(static_cast<float>((w >> (8 * i + 4)) & 0xf) - z, s));
             const uint32_t l16 = BF16 ? f32_to_bf16_bits(lo) : f32_to_f16_bits(lo);
             const uint32_t h16 = BF16 ? f32_to_bf16_bits(hi) : f32_to_f16_bits(hi);
             pair[i] = l16 | (h16 << 16);

@@ -49,7 +49,8 @@ class NxrtTensorDesc(C.Structure):
 
 class Attrs(C.Structure):
     _fields_ = [("struct_size", C.c_uint32), ("present", C.c_uint32), ("K", C.c_int64), ("N", C.c_int64), ("bits", C.c_int64),
-                ("block_size", C.c_int64), ("accuracy_level", C.c_int64), ("weight_prepacked", C.c_int64), ("folded_bias", C.c_int64)]
+                ("block_size", C.c_int64), ("accuracy_level", C.c_int64), ("weight_prepacked", C.c_int64), ("folded_bias", C.c_int64),
+                ("gate_up_swiglu", C.c_int64), ("decomposed_silu", C.c_int64)]
 
 
 class CTensorView(C.Structure):
@@ -61,7 +62,8 @@ class WorkspaceRequirement(C.Structure):
     _fields_ = [("bytes", C.c_uint64), ("alignment", C.c_uint64)]
 
 
-_ATTR_BITS = {"K": 0, "N": 1, "bits": 2, "block_size": 3, "accuracy_level": 4, "weight_prepacked": 5, "folded_bias": 6}
+_ATTR_BITS = {"K": 0, "N": 1, "bits": 2, "block_size": 3, "accuracy_level": 4, "weight_prepacked": 5, "folded_bias": 6, "gate_up_swiglu": 7,
+              "decomposed_silu": 8}
 _lib = None
 
 
@@ -505,5 +507,59 @@ def matmul_nbits(ep, a, a_dtype, b, scales, scale_dtype, zp, n, k, bs, *, accura
     return y, variant
 
 
-__all__ = ["RocmExecutionProvider", "MatMulNBitsKernel", "TensorView", "DeviceBuffer", "DeviceOperands", "EpError", "matmul_nbits",
+class GateUpOperands:
+    """Device-resident operands of the fused gate/up node (inputs [x, W_gate, scales_gate, W_up, scales_up, -, zp_gate, zp_up])."""
+
+    def __init__(self, ep, gate, up, scale_dtype, n, k, bs, *, decomposed=False, rows=None, a_dtype=None):
+        self.ep, self.n, self.k, self.bs, self.scale_dtype = ep, n, k, bs, scale_dtype
+        self.kb = -(-k // bs)
+        self.bufs = []
+        for b, s, zp in (gate, up):
+            self.bufs.append((ep.upload(np.asarray(b, np.uint8)), ep.upload(s), ep.upload(np.asarray(zp, np.uint8)) if zp is not None else None))
+        shapes = [((rows, k), a_dtype)] if rows is not None and a_dtype is not None else None
+        self.kernel = ep.get_kernel({"K": k, "N": n, "bits": 4, "block_size": bs, "gate_up_swiglu": 1, "decomposed_silu": 1 if decomposed else None}, shapes)
+        self.kernel.set_constant_inputs([False, True, True, True, True, True, True, True])
+
+    def views(self, a_buf: DeviceBuffer, a_dtype: int, m: int):
+        dev = self.ep.device_index
+        (bg, sg, zg), (bu, su, zu) = self.bufs
+        w_shape, s_shape, z_shape = (self.n, self.kb, self.bs // 2), (self.n, self.kb), (self.n, (self.kb + 1) // 2)
+        ins = [TensorView(a_buf.ptr, a_dtype, (m, self.k), device_index=dev),
+               TensorView(bg.ptr, U8, w_shape, device_index=dev), TensorView(sg.ptr, self.scale_dtype, s_shape, device_index=dev),
+               TensorView(bu.ptr, U8, w_shape, device_index=dev), TensorView(su.ptr, self.scale_dtype, s_shape, device_index=dev)]
+        if zg is not None:
+            ins += [TensorView.absent(F32), TensorView(zg.ptr, U8, z_shape, device_index=dev), TensorView(zu.ptr, U8, z_shape, device_index=dev)]
+        return ins
+
+    def run(self, a_buf: DeviceBuffer, a_dtype: int, m: int, y_buf: DeviceBuffer, workspace: DeviceBuffer | None = None) -> None:
+        out = [TensorView(y_buf.ptr, a_dtype, (m, self.n), device_index=self.ep.device_index)]
+        self.kernel.execute(self.views(a_buf, a_dtype, m), out, workspace=workspace)
+
+    def free(self) -> None:
+        self.kernel.release()
+        for group in self.bufs:
+            for buf in group:
+                if buf is not None:
+                    self.ep.deallocate(buf)
+
+
+def gate_up_swiglu(ep, a, a_dtype, gate, up, scale_dtype, n, k, bs, *, decomposed=False):
+    """One-shot helper for the fused gate/up node: gate and up are (B, scales, zero_points or None). Returns (Y, variant)."""
+    a = np.ascontiguousarray(a)
+    m = a.size // k
+    ops = GateUpOperands(ep, gate, up, scale_dtype, n, k, bs, decomposed=decomposed)
+    a_buf = ep.upload(a)
+    y_buf = ep.allocate(max(m * n * 2, 1))
+    try:
+        ops.run(a_buf, a_dtype, m, y_buf)
+        y = ep.download(y_buf, (m, n), _NP[a_dtype])
+        variant = ops.kernel.last_variant()
+    finally:
+        ep.deallocate(a_buf)
+        ep.deallocate(y_buf)
+        ops.free()
+    return y, variant
+
+
+__all__ = ["RocmExecutionProvider", "GateUpOperands", "gate_up_swiglu", "MatMulNBitsKernel", "TensorView", "DeviceBuffer", "DeviceOperands", "EpError", "matmul_nbits",
            "load_library", "make_attrs", "make_descs", "synth", "F32", "U8", "I8", "I32", "F16", "BF16"]

@@ -79,6 +79,11 @@ class Port:
         L.mnb_quantize_a.argtypes = [v, z, z, z, C.c_int, v, v]
         L.mnb_block_acc_i32.argtypes = [v, v, v, z, z, z, z, v]
         L.mnb_matmul_acc4_f32.argtypes = [v, v, v, v, v, z, z, z, z, C.c_int, v]
+        L.mnb_swiglu_silu.restype = C.c_float
+        L.mnb_swiglu_silu.argtypes = [C.c_float]
+        L.mnb_swiglu_silu_decomposed.restype = C.c_float
+        L.mnb_swiglu_silu_decomposed.argtypes = [C.c_float, C.c_int]
+        L.mnb_swiglu.argtypes = [v, v, z, C.c_int, C.c_int, v]
         L.mnb_matmul_nbits.restype = C.c_int
         L.mnb_matmul_nbits.argtypes = [v, C.c_int, v, v, C.c_int, v, v, C.c_int, v, C.c_int, z, z, z, z, C.c_int, C.c_int]
 
@@ -93,6 +98,14 @@ class Port:
         src = _c(src, np.float32)
         out = np.empty(src.shape, _NP_DT[code])
         self.lib.mnb_narrow(_ptr(src), src.size, code, _ptr(out))
+        return out
+
+    # -- the CUDA provider's fused gate/up epilogue ------------------------------------------------
+    def swiglu(self, gate16: np.ndarray, up16: np.ndarray, code: int, decomposed: bool = False) -> np.ndarray:
+        """round16(silu(gate) * up) on 16-bit inputs (f16 arrays, or bf16 bit patterns as uint16)."""
+        gate16, up16 = np.ascontiguousarray(gate16), np.ascontiguousarray(up16)
+        out = np.empty(gate16.shape, _NP_DT[code])
+        self.lib.mnb_swiglu(_ptr(gate16), _ptr(up16), gate16.size, code, int(decomposed), _ptr(out))
         return out
 
     # -- operator pieces -----------------------------------------------------------------------

@@ -275,3 +275,49 @@ int mnb_matmul_nbits(const void* a, int a_dtype, const uint8_t* b, const void* s
     free(af); free(sf); free(bf); free(yf);
     return 0;
 }
+
+
+/* ---- gate/up SwiGLU epilogue (onnx-runtime-ep-cuda/src/kernels/matmul_nbits.rs:4207-4233, 4375-4386) ---- */
+
+float mnb_swiglu_silu(float x)
+{
+    if (x >= 0.0f) {
+        const float denominator = 1.0f + (float)exp((double)-x);
+        return x / denominator;
+    }
+    const float e = (float)exp((double)x);
+    const float numerator = x * e;
+    return numerator / (1.0f + e);
+}
+
+static float round16(float v, int dtype)
+{
+    return dtype == MNB_F16 ? mnb_f16_to_f32(mnb_f32_to_f16(v)) : mnb_bf16_to_f32(mnb_f32_to_bf16(v));
+}
+
+float mnb_swiglu_silu_decomposed(float x, int dtype)
+{
+    float sigmoid;
+    if (x >= 0.0f) {
+        sigmoid = 1.0f / (1.0f + (float)exp((double)-x));
+    } else {
+        const float e = (float)exp((double)x);
+        sigmoid = e / (1.0f + e);
+    }
+    const float sigmoid_h = round16(sigmoid, dtype);
+    return round16(x * sigmoid_h, dtype);
+}
+
+void mnb_swiglu(const void* gate, const void* up, size_t count, int dtype, int decomposed, void* y)
+{
+    const uint16_t* g = (const uint16_t*)gate;
+    const uint16_t* u = (const uint16_t*)up;
+    uint16_t* out = (uint16_t*)y;
+    for (size_t i = 0; i < count; ++i) {
+        const float gate_h = dtype == MNB_F16 ? mnb_f16_to_f32(g[i]) : mnb_bf16_to_f32(g[i]);
+        const float up_h = dtype == MNB_F16 ? mnb_f16_to_f32(u[i]) : mnb_bf16_to_f32(u[i]);
+        const float silu_h = decomposed ? mnb_swiglu_silu_decomposed(gate_h, dtype) : mnb_swiglu_silu(gate_h);
+        const float prod = silu_h * up_h;
+        out[i] = dtype == MNB_F16 ? mnb_f32_to_f16(prod) : mnb_f32_to_bf16(prod);
+    }
+}

@@ -83,6 +83,18 @@ int mnb_matmul_nbits(const void* a, int a_dtype, const uint8_t* b, const void* s
                      const uint8_t* zp, const void* bias, int bias_dtype, void* y, int y_dtype,
                      size_t m, size_t n, size_t k, size_t block_size, int accuracy_level, int rounding);
 
+/* The epilogue of the CUDA provider's fused gate/up node (a "next" neighbour of the operator, not part of the CPU path):
+ * onnx-runtime-ep-cuda/src/kernels/matmul_nbits.rs:4207-4219 (silu, the form of its standalone op_silu):
+ *   x >= 0: x / (1 + (float)exp((double)-x));  x < 0: (x * e) / (1 + e) with e = (float)exp((double)x); every step one
+ *   correctly rounded f32 operation, the exponential evaluated in double and rounded to f32;
+ * :4221-4233 (decomposed silu: Sigmoid and Mul as two 16-bit ops): sigmoid = 1/(1+exp(-x)) resp. e/(1+e) in f32, rounded
+ *   to the 16-bit type, times x, rounded to the 16-bit type again;
+ * :4375-4386: gate and up arrive rounded to the 16-bit type; y = round16(silu(gate) * up), the product one f32 multiply.
+ * `dtype` is MNB_F16 or MNB_BF16 (the reference is fp16 only; bf16 follows the same steps with bf16 roundings). */
+float mnb_swiglu_silu(float x);
+float mnb_swiglu_silu_decomposed(float x, int dtype);
+void  mnb_swiglu(const void* gate, const void* up, size_t count, int dtype, int decomposed, void* y);
+
 #ifdef __cplusplus
 }
 #endif

@@ -210,3 +210,52 @@ def test_compiled_mlas_agrees_with_golden_and_oracle(port, ref, golden):
         r = ref.quantize_a(a, 512, bs)
         qa, qs = port.quantize_a(a, 512, bs, oracle.ROUND_HALF_EVEN)
         assert np.array_equal(r[0], qa) and np.array_equal(r[1].view(np.uint32), qs.view(np.uint32))
+
+
+# ---------------------------------------------------------------------------------------------
+# The fused gate/up epilogue (onnx-runtime-ep-cuda/src/kernels/matmul_nbits.rs:4207-4233, 4375-4386). No golden vector of the
+# reference covers it (its tests need a CUDA device); it is pinned by what the mathematics fixes.
+# ---------------------------------------------------------------------------------------------
+def test_swiglu_silu_against_double_precision(port):
+    """silu in f32 with a double exponential stays within three f32 ulps of the double-precision value (the negative branch
+    holds four roundings), on both branches, at the branch point, and where the exponential saturates or vanishes."""
+    xs = np.concatenate([np.linspace(-30, 30, 4001), [0.0, -0.0, 1e-8, -1e-8, 88.0, -88.0, 104.0, -104.0, 6e4, -6e4]]).astype(np.float32)
+    got = np.array([port.lib.mnb_swiglu_silu(float(x)) for x in xs], np.float32)
+    with np.errstate(over="ignore"):
+        want = xs.astype(np.float64) / (1.0 + np.exp(-xs.astype(np.float64)))
+    ulp = np.spacing(np.abs(want).astype(np.float32)).astype(np.float64)
+    assert np.all(np.abs(got.astype(np.float64) - want) <= 3.0 * ulp + 1e-37)          # 1e-37: where e = exp(x) is a denormal
+    assert port.lib.mnb_swiglu_silu(0.0) == 0.0
+    # x sigma(x) + x sigma(-x) = x: a sign slip on either branch breaks it
+    pos = np.array([port.lib.mnb_swiglu_silu(float(x)) for x in xs[:4001]], np.float64)
+    neg = np.array([port.lib.mnb_swiglu_silu(float(-x)) for x in xs[:4001]], np.float64)
+    assert np.allclose(pos - neg, xs[:4001].astype(np.float64), rtol=0, atol=4e-6)
+
+
+def test_swiglu_rounding_steps(port):
+    """Known answers that fix where the roundings sit: gate = 1, up = 3 in f16 gives f16(0.7310586 * 3) = 2.1933594 (a second
+    rounding of silu to f16 first would give 2.1914062); the decomposed form rounds sigmoid(1) to f16 0.73095703 and gives
+    f16(0.73095703 * 3) = 2.1933594 as well, but differs at gate = 3: f16(3 * f16(0.95257413)) = 2.8574219 against
+    f16(2.8577223 * 1) = 2.8574219 ... so the steps are checked one by one."""
+    f16 = lambda v: float(np.float16(v))
+    one, three = np.array([1.0], np.float16), np.array([3.0], np.float16)
+    silu1 = np.float32(1.0) / (np.float32(1.0) + np.float32(np.exp(-1.0)))
+    assert port.swiglu(one, three, oracle.F16, False)[0] == np.float16(np.float32(silu1) * np.float32(3.0))
+    # decomposed: sigmoid and x * sigmoid each rounded to f16 before the product with up
+    for x in (0.5, 1.0, 3.0, -2.0, -0.25, 7.5):
+        xf = np.float32(x)
+        sig = np.float32(1.0) / (np.float32(1.0) + np.float32(np.exp(-float(xf)))) if x >= 0 else \
+            np.float32(np.exp(float(xf))) / (np.float32(1.0) + np.float32(np.exp(float(xf))))
+        want = f16(np.float32(xf * np.float32(f16(sig))))
+        assert port.lib.mnb_swiglu_silu_decomposed(float(xf), oracle.F16) == want
+        # the two forms differ by at most the two extra roundings
+        assert abs(port.lib.mnb_swiglu_silu(float(xf)) - want) <= 2 ** -9 * max(abs(x), 1.0)
+    # bf16 follows the same steps with bf16 roundings; up = 1 makes the product exact, so y = bf16(silu(gate))
+    g = port.narrow(np.array([1.5, -0.75, 4.0], np.float32), oracle.BF16)
+    ones = port.narrow(np.ones(3, np.float32), oracle.BF16)
+    y = port.widen(port.swiglu(g, ones, oracle.BF16, False), oracle.BF16)
+    want = port.widen(port.narrow(np.array([port.lib.mnb_swiglu_silu(float(v)) for v in port.widen(g, oracle.BF16)], np.float32), oracle.BF16), oracle.BF16)
+    assert np.array_equal(y, want)
+    # silu(gate) * 0 = 0 and silu(0) * up = 0
+    z = port.swiglu(np.array([2.0, 0.0], np.float16), np.array([0.0, 5.0], np.float16), oracle.F16, False)
+    assert np.array_equal(z.view(np.uint16) & 0x7fff, np.zeros(2, np.uint16))

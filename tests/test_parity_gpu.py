@@ -555,6 +555,70 @@ def test_folded_bias_keeps_tall_calls_off_the_library_gemm(ep):
 
 
 # ---------------------------------------------------------------------------------------------
+# fused gate/up node: silu(gate) * up over both projections, rounded as the separate nodes round
+# ---------------------------------------------------------------------------------------------
+SWIGLU_CASES = [
+    # a_dt, s_dt, bs, zero points, m, n, k, decomposed
+    (E.F16, E.F16, 32, False, 1, 300, 896, False),
+    (E.F16, E.F16, 32, True, 1, 4864, 896, True),
+    (E.BF16, E.BF16, 128, True, 1, 1000, 3584, False),
+    (E.BF16, E.BF16, 128, True, 4, 520, 1024, True),
+    (E.F16, E.F32, 64, True, 3, 130, 512, False),
+    (E.F16, E.F16, 32, True, 16, 200, 1024, False),
+    (E.BF16, E.BF16, 128, False, 8, 16400, 512, False),
+    (E.F16, E.F16, 64, True, 100, 136, 1024, False),
+    (E.F16, E.F16, 32, False, 1100, 136, 512, True),
+]
+
+
+@pytest.mark.parametrize("a_dt,s_dt,bs,zero_points,m,n,k,decomposed", SWIGLU_CASES)
+def test_gate_up_swiglu(ep, port, a_dt, s_dt, bs, zero_points, m, n, k, decomposed):
+    """The fused node equals, bit for bit, the oracle's epilogue applied to this provider's own two projections (the node's
+    contract: 'identical to the separate kernels'), and is within the 16-bit bar of the epilogue applied to f64 projections."""
+    gate = synth.make_weights(n, k, bs, 810 + n, zero_points=zero_points, scale_lo=0.004, scale_hi=0.02, scale_dtype=s_dt)
+    up = synth.make_weights(n, k, bs, 811 + n, zero_points=zero_points, scale_lo=0.004, scale_hi=0.02, scale_dtype=s_dt)
+    a = synth.make_activation(m, k, 812 + m, a_dt)
+    o_dt = oracle.F16 if a_dt == E.F16 else oracle.BF16
+    y, variant = E.gate_up_swiglu(ep, a, a_dt, gate, up, s_dt, n, k, bs, decomposed=decomposed)
+    assert variant.startswith("gate_up_swiglu")
+    g16, _ = run_op(ep, a, a_dt, gate[0], gate[1], s_dt, gate[2], n, k, bs)
+    u16, _ = run_op(ep, a, a_dt, up[0], up[1], s_dt, up[2], n, k, bs)
+    want = port.swiglu(g16, u16, o_dt, decomposed)
+    assert np.array_equal(np.asarray(y).view(np.uint16), np.asarray(want).view(np.uint16))
+    g64 = oracle_f64(port, a, a_dt, gate[0], gate[1], s_dt, gate[2], n, k, bs)
+    u64 = oracle_f64(port, a, a_dt, up[0], up[1], s_dt, up[2], n, k, bs)
+    ideal = g64 / (1.0 + np.exp(-g64)) * u64
+    assert helpers.rel_l2(synth.to_f32(y, a_dt), ideal) <= 2 * TOL_HALF
+
+
+def test_gate_up_swiglu_validation(ep):
+    a_dt, bs, n, k = E.F16, 32, 64, 128
+    gate = synth.make_weights(n, k, bs, 1, zero_points=True, scale_lo=0.004, scale_hi=0.02, scale_dtype=a_dt)
+    up = synth.make_weights(n, k, bs, 2, zero_points=True, scale_lo=0.004, scale_hi=0.02, scale_dtype=a_dt)
+    ops = E.GateUpOperands(ep, gate, up, a_dt, n, k, bs)
+    a, y = ep.upload(synth.make_activation(2, k, 3, a_dt)), ep.allocate(2 * n * 2)
+    try:
+        assert ops.kernel.workspace_requirement([((2, k), a_dt)])[0] == 2 * 256
+        views = ops.views(a, a_dt, 2)
+        out = [E.TensorView(y.ptr, a_dt, (2, n), device_index=ep.device_index)]
+        with pytest.raises(E.EpError, match="both projections or neither"):
+            ops.kernel.execute(views[:7], out)
+        with pytest.raises(E.EpError, match="expects 5 to 8 inputs"):
+            ops.kernel.execute(views[:4], out)
+        gamma = list(views)
+        gamma[5] = E.TensorView(a.ptr, a_dt, (k,), device_index=ep.device_index)
+        with pytest.raises(E.EpError, match="RMS-norm prologue"):
+            ops.kernel.execute(gamma, out)
+        with pytest.raises(E.EpError, match="Y must have dtype"):
+            ops.kernel.execute(views, [E.TensorView(y.ptr, E.F32, (2, n), device_index=ep.device_index)])
+        ops.kernel.execute(views, out)                       # and the well-formed call goes through
+    finally:
+        ep.deallocate(a)
+        ep.deallocate(y)
+        ops.free()
+
+
+# ---------------------------------------------------------------------------------------------
 # dense route: weights expanded to 16 bits, then the library GEMM (tall calls)
 # ---------------------------------------------------------------------------------------------
 DENSE_CASES = [
