@@ -162,6 +162,48 @@ def small_model_step(ep):
     return out
 
 
+def swiglu_table(ep, copies=8):
+    """The fused gate/up node at the 7B shape (3584 -> 2 x 18944, bf16, block 128, zero points): one launch that reads both
+    projections and writes silu(gate) * up, over `copies` distinct weight pairs per graph; beside it the unfused pair as one
+    MatMulNBits over the concatenated 37888 columns (which a model still follows with an elementwise kernel)."""
+    k, n, bs, dt = HIDDEN, INTER, BS, A_DT
+    table = []
+    for m in (1, 4):
+        a = ep.upload(synth.make_activation(m, k, 9, dt))
+        fused, reuse = [], None
+        for i in range(copies):
+            gate = _device_random_weights(ep, n, k, bs, 300 + 2 * i, 0.002, 0.01, dt, True, reuse)
+            reuse = gate[0] if reuse is None else reuse
+            up = _device_random_weights(ep, n, k, bs, 301 + 2 * i, 0.002, 0.01, dt, True, reuse)
+            ops = E.GateUpOperands(ep, gate, up, dt, n, k, bs)
+            fused.append((ops, ep.allocate(m * n * 2)))
+        for _ in range(2):                                  # the first call makes the repacked copies, the second is the single launch
+            for ops, y in fused:
+                ops.run(a, dt, m, y)
+        ep.sync()
+        variant = fused[0][0].kernel.last_variant()
+        graph = capture(ep, lambda: [ops.run(a, dt, m, y) for ops, y in fused])
+        us = time_graph(ep, graph, 20, 2) * 1e3 / copies
+        graph.release()
+        nbytes = 2 * synth.algorithmic_bytes(m, n, k, bs, a_dtype=dt, scale_dtype=dt, zero_points=True) - m * k * 2 - m * n * 2
+        for ops, y in fused:
+            ep.deallocate(y)
+            ops.free()
+        plain = [Node(ep, "gate_up.%d" % i, k, 2 * n, bs, 400 + i, dt, m) for i in range(copies)]
+        for node in plain:
+            node.run(a)
+        ep.sync()
+        graph = capture(ep, lambda: [node.run(a) for node in plain])
+        plain_us = time_graph(ep, graph, 20, 2) * 1e3 / copies
+        graph.release()
+        for node in plain:
+            node.free(ep)
+        ep.deallocate(a)
+        table.append({"k": k, "n": n, "m": m, "us": round(us, 2), "gbs": round(nbytes / us / 1e3, 1), "hbm_frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+                      "variant": variant, "unfused_matmul_us": round(plain_us, 2)})
+    return table
+
+
 def cpu_baseline(seconds_budget=20.0, threads=None):
     """The reference's CPU path (vendored MLAS through its plain-C shim, oracle/_ref) on this host, on a bounded
     sample of the workload: the gate/up projection (3584 -> 37888), bf16 activations widened to f32 before and
@@ -328,6 +370,7 @@ def main():
         result["prefill"] = prefill_table(ep)
         result["prefill_7b_bf16"] = prefill_7b_table(ep)
         result["acc4"] = acc4_table(ep)
+        result["gate_up_swiglu"] = swiglu_table(ep)
         result["small_model_step"] = small_model_step(ep)
     ep.shutdown()
     if not args.no_cpu:

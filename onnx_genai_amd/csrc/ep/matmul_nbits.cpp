@@ -126,6 +126,7 @@ struct NxrtRocmMatMulNBits {
     bool gate_up_swiglu = false, decomposed_silu = false;
     NxrtRocmMatMulNBits* gate = nullptr;
     NxrtRocmMatMulNBits* up = nullptr;
+    bool pair_member = false;            // this kernel is one projection of a fused gate/up node
     bool constant_inputs[6] = {false, false, false, false, false, false};
     std::string variant = "none";
     void* scratch = nullptr;             // kernel-owned workspace, grown on demand
@@ -485,7 +486,8 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
             }
         }
     } else if (M <= 64 && use_packed(kn, args, rc)) {
-        if (rc == 0) rc = rocm_launch_decode_packed(&args, kn.packed, kn.ep->decode_waves, stream);
+        if (rc == 0) rc = (kn.pair_member && M <= 4) ? rocm_launch_decode_packed_pair_member(&args, kn.packed, kn.ep->decode_waves, stream)
+                                                      : rocm_launch_decode_packed(&args, kn.packed, kn.ep->decode_waves, stream);
         kn.variant = "decode_mfma_packed";
     } else if (M <= 16 && rocm_decode_mfma_eligible(&args)) {
         rc = rocm_launch_decode_mfma(&args, kn.ep->decode_waves, kn.ep->decode_col_groups, stream);
@@ -558,6 +560,40 @@ NxrtStatus execute_swiglu(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in,
     if (M == 0) return ok();
     NxrtStatus st = kn.ep->bind();
     if (st.code != NXRT_OK) return st;
+
+    // Up to four rows over constant weights: one launch over both repacked copies. The copies are made (and every weight
+    // tensor validated) by the projections' own first call below, so this path serves the calls after the first with the
+    // same weight tensors; it sums each projection exactly as that first call did.
+    if (M <= 4 && kn.gate->packed && kn.up->packed) {
+        auto current = [&](const NxrtRocmMatMulNBits& child, const NxrtRocmTensorView& w, const NxrtRocmTensorView& s, const NxrtRocmTensorView* zp) {
+            auto at = [](const NxrtRocmTensorView& v) { return static_cast<const void*>(static_cast<const uint8_t*>(v.data) + v.byte_offset); };
+            return child.packed_from[0] == at(w) && child.packed_from[1] == at(s) && child.packed_from[2] == (zp ? at(*zp) : nullptr) &&
+                   child.packed_scale_dtype == static_cast<int>(s.dtype);
+        };
+        if (current(*kn.gate, in[1], in[2], zp_gate) && current(*kn.up, in[3], in[4], zp_up) && is_contiguous(A) &&
+            A.device_type == NXRT_DEVICE_ROCM && A.device_index == kn.ep->device) {
+            RocmMatMulNBitsArgs args;
+            std::memset(&args, 0, sizeof(args));
+            args.a = static_cast<uint8_t*>(A.data) + A.byte_offset;
+            args.b = static_cast<const uint8_t*>(kn.gate->packed_from[0]);
+            args.scales = kn.gate->packed_from[1];
+            args.zp = static_cast<const uint8_t*>(kn.gate->packed_from[2]);
+            args.y = static_cast<uint8_t*>(Y.data) + Y.byte_offset;
+            args.a_dtype = args.y_dtype = static_cast<int>(A.dtype);
+            args.scale_dtype = kn.gate->packed_scale_dtype;
+            args.bias_dtype = ROCM_DT_F32;
+            args.m = static_cast<int64_t>(M);
+            args.n = kn.n;
+            args.k = kn.k;
+            args.block_size = static_cast<int>(kn.block_size);
+            if (rocm_decode_packed_eligible(&args) && rocm_decode_packed_pair_fits(&args, kn.ep->decode_waves)) {
+                const int rc = rocm_launch_decode_packed_pair(&args, kn.gate->packed, kn.up->packed, kn.decomposed_silu ? 1 : 0, kn.ep->decode_waves, kn.ep->stream);
+                kn.ep->launches.fetch_add(1);
+                kn.variant = "gate_up_swiglu_packed";
+                return hip_status(rc, "MatMulNBits: kernel launch");
+            }
+        }
+    }
 
     // two 16-bit [M, N] matrices: the caller's workspace if it is large enough, else the kernel's own
     const uint64_t each = (M * N * 2 + 255) / 256 * 256;
@@ -722,6 +758,7 @@ NxrtStatus nxrt_rocm_matmul_nbits_create(NxrtRocmEp* ep, const NxrtRocmMatMulNBi
                 c2->block_size = kn->block_size;
                 c2->accuracy_level = kn->accuracy_level;
                 c2->rows_hint = kn->rows_hint;
+                c2->pair_member = true;
                 *child = c2;
             }
         }

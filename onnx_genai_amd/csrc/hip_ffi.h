@@ -103,6 +103,15 @@ int rocm_decode_packed_eligible(const RocmMatMulNBitsArgs* args);
 uint64_t rocm_decode_packed_bytes(const RocmMatMulNBitsArgs* args);
 int rocm_launch_pack_decode(const RocmMatMulNBitsArgs* args, void* packed, rocm_stream_t stream);
 int rocm_launch_decode_packed(const RocmMatMulNBitsArgs* args, const void* packed, int waves, rocm_stream_t stream);
+/* The fused gate/up node at up to four rows: one launch over both projections' repacked copies; Y (the activations'
+ * 16-bit type) = round16(silu(round16(gate)) * round16(up)), each projection summed exactly as its own launch would.
+ * args names the shared operands (a, y, m, n, k, block_size, dtypes; b / scales / zp only for the eligibility checks).
+ * rocm_decode_packed_pair_fits: 1 when both projections' waves fit one workgroup; otherwise run them separately.
+ * rocm_launch_decode_packed_pair_member: one projection of such a pair on its own, with the pair's split of K. */
+int rocm_launch_decode_packed_pair_member(const RocmMatMulNBitsArgs* args, const void* packed, int waves, rocm_stream_t stream);
+int rocm_decode_packed_pair_fits(const RocmMatMulNBitsArgs* args, int waves);
+int rocm_launch_decode_packed_pair(const RocmMatMulNBitsArgs* args, const void* packed_gate, const void* packed_up, int decomposed, int waves,
+                                   rocm_stream_t stream);
 
 /* Prefill (M > 16), f16/bf16 activations: B tiles dequantized into LDS, 32x32x16 MFMA.
  * tile_choice: 0 = by shape, 1 = 128 x 128, 2 = 256 x 128, 3 = 256 x 256, 4 = 128 x 64 tiles of Y per workgroup. */

@@ -20,6 +20,7 @@
 #include <type_traits>
 
 #include "mfma_common.hiph"
+#include "swiglu.hiph"
 
 namespace mnb {
 
@@ -96,6 +97,8 @@ __global__ __launch_bounds__(256) void pack_decode_kernel(PackParams p)
 struct PackedParams {
     const uint16_t* a;
     const uint8_t* packed;
+    const uint8_t* packed_up;   // paired launch only: the up projection's repacked copy (`packed` is the gate's)
+    int decomposed_silu;        // paired launch only
     const void* bias;
     void* y;
     int64_t m, n, k;
@@ -178,7 +181,10 @@ __device__ __forceinline__ float block_sum(float s)
 // waves per SIMD - for launches with thousands of waves, where the other resident waves cover it better (measured on
 // 3584 -> 37888: 15.6 us against 17.0 us). With two sets the one-row, block-128, 16-bit-scale variant fits 96
 // registers without spilling (a fifth wave per SIMD); the other variants keep the compiler's own choice.
-template <bool BF16, int BS, int MR, typename ST, int SETS>
+// PAIR: the fused gate/up node. The first half of the workgroup's waves runs the gate projection's column group, the
+// second half the up projection's - each half exactly as a launch of its own would (same split of K, same order of
+// summation, so the same f32 totals) - and the epilogue writes round16(silu(round16(gate)) * round16(up)).
+template <bool BF16, int BS, int MR, typename ST, int SETS, bool PAIR>
 __global__ __launch_bounds__((BS == 128 && sizeof(ST) == 2) ? 1024 : 512)   // block 128, 16-bit scales: up to 16 waves split a long K
 __attribute__((amdgpu_waves_per_eu((BS == 128 && MR == 1 && sizeof(ST) == 2) ? (SETS == 1 ? 8 : 5) : 1)))
 void decode_packed_kernel(PackedParams p)
@@ -206,12 +212,14 @@ void decode_packed_kernel(PackedParams p)
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int waves = blockDim.x >> 6;
+    const int waves = PAIR ? static_cast<int>(blockDim.x >> 7) : static_cast<int>(blockDim.x >> 6);      // per projection
+    const bool second = PAIR && wave >= waves;                                                           // wave-uniform
+    const int split = second ? wave - waves : wave;                                                      // this wave's share of K
     const int c = lane & 15;
     const int g = lane >> 4;
     const int64_t n_base = static_cast<int64_t>(blockIdx.x) * 16;
 
-    const __amdgpu_buffer_rsrc_t srd_p = make_srd(p.packed + static_cast<int64_t>(blockIdx.x) * p.cg_stride, static_cast<uint64_t>(p.cg_stride));
+    const __amdgpu_buffer_rsrc_t srd_p = make_srd((second ? p.packed_up : p.packed) + static_cast<int64_t>(blockIdx.x) * p.cg_stride, static_cast<uint64_t>(p.cg_stride));
     const __amdgpu_buffer_rsrc_t srd_a = make_srd(p.a, static_cast<uint64_t>(p.m * p.k) * 2);
 
     const uint32_t w_off = static_cast<uint32_t>(lane * 16);
@@ -227,7 +235,7 @@ void decode_packed_kernel(PackedParams p)
     float4p_t y = {0.f, 0.f, 0.f, 0.f};
     float4p_t acc = {0.f, 0.f, 0.f, 0.f};
 
-    const int g_begin = wave * p.groups_per_wave;
+    const int g_begin = split * p.groups_per_wave;
     const int g_end = min(g_begin + p.groups_per_wave, p.groups);
 
     using Grp = PackedGroup<NR, NA>;
@@ -376,19 +384,31 @@ void decode_packed_kernel(PackedParams p)
         if (row < p.m && col < p.n) {
             float total = 0.f;
             for (int w = 0; w < waves; ++w) total += red[(w * 4 + r) * 64 + l];
-            total = with_bias(total, p.bias, p.bias_dtype, col, p.y_dtype);
-            store_from_f32(p.y, p.y_dtype, static_cast<int64_t>(row) * p.n + col, total);
+            if constexpr (PAIR) {
+                float total_up = 0.f;
+                for (int w = waves; w < 2 * waves; ++w) total_up += red[(w * 4 + r) * 64 + l];
+                const uint16_t gate16 = BF16 ? f32_to_bf16_bits(total) : f32_to_f16_bits(total);
+                const uint16_t up16 = BF16 ? f32_to_bf16_bits(total_up) : f32_to_f16_bits(total_up);
+                static_cast<uint16_t*>(p.y)[static_cast<int64_t>(row) * p.n + col] = swiglu16<BF16>(gate16, up16, p.decomposed_silu != 0);
+            } else {
+                total = with_bias(total, p.bias, p.bias_dtype, col, p.y_dtype);
+                store_from_f32(p.y, p.y_dtype, static_cast<int64_t>(row) * p.n + col, total);
+            }
         }
     }
 }
 
+// `waves` = waves per projection; a paired launch has twice as many in a workgroup.
 template <bool BF16, int BS, int MR, typename ST, int SETS>
 static int launch_packed_cfg(const PackedParams& p, int waves, hipStream_t stream)
 {
     const unsigned grid = static_cast<unsigned>((p.n + 15) / 16);
-    const size_t stage = static_cast<size_t>(waves) * 2 * (MR == 1 ? 1024 : MR * kRowPitchP);
-    const size_t red = static_cast<size_t>(waves) * 1024;
-    hipLaunchKernelGGL((decode_packed_kernel<BF16, BS, MR, ST, SETS>), dim3(grid), dim3(waves * 64), stage > red ? stage : red, stream, p);
+    const bool pair = p.packed_up != nullptr;
+    const int all = pair ? 2 * waves : waves;
+    const size_t stage = static_cast<size_t>(all) * 2 * (MR == 1 ? 1024 : MR * kRowPitchP);
+    const size_t red = static_cast<size_t>(all) * 1024;
+    if (pair) hipLaunchKernelGGL((decode_packed_kernel<BF16, BS, MR, ST, SETS, true>), dim3(grid), dim3(all * 64), stage > red ? stage : red, stream, p);
+    else hipLaunchKernelGGL((decode_packed_kernel<BF16, BS, MR, ST, SETS, false>), dim3(grid), dim3(all * 64), stage > red ? stage : red, stream, p);
     return static_cast<int>(hipGetLastError());
 }
 
@@ -1002,12 +1022,19 @@ extern "C" int rocm_launch_pack_decode(const RocmMatMulNBitsArgs* a, void* packe
     return static_cast<int>(hipGetLastError());
 }
 
-extern "C" int rocm_launch_decode_packed(const RocmMatMulNBitsArgs* a, const void* packed, int waves, rocm_stream_t stream)
+// The launch of rocm_launch_decode_packed; with `packed_up` the paired gate/up launch. `probe_only`: nothing is launched,
+// the return value says whether a paired launch with this split of K fits a workgroup (1) or not (0).
+// `pair_member`: the launch is one projection of a gate/up pair (or the paired launch itself): the split of K is chosen
+// for the pair's column groups together, so that the separate launches and the paired one add up in the same order.
+static int launch_decode_packed(const RocmMatMulNBitsArgs* a, const void* packed, const void* packed_up, int decomposed, int waves, bool probe_only,
+                                bool pair_member, rocm_stream_t stream)
 {
-    if (!rocm_decode_packed_eligible(a)) return -1;
+    if (!rocm_decode_packed_eligible(a)) return probe_only ? 0 : -1;
     mnb::PackedParams p;
     p.a = static_cast<const uint16_t*>(a->a);
     p.packed = static_cast<const uint8_t*>(packed);
+    p.packed_up = static_cast<const uint8_t*>(packed_up);
+    p.decomposed_silu = decomposed;
     p.bias = a->bias;
     p.y = a->y;
     p.m = a->m;
@@ -1025,6 +1052,7 @@ extern "C" int rocm_launch_decode_packed(const RocmMatMulNBitsArgs* a, const voi
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool f32_scales = a->scale_dtype == ROCM_DT_F32;
     if (wide_shape(a)) {
+        if (probe_only || packed_up) return probe_only ? 0 : -1;          // the shared-activation kernel has no paired form
         p.groups_per_wave = p.groups;
         if (bf16) return f32_scales ? mnb::launch_wide_bs<true, float>(p, a->block_size, s) : mnb::launch_wide_bs<true, uint16_t>(p, a->block_size, s);
         return f32_scales ? mnb::launch_wide_bs<false, float>(p, a->block_size, s) : mnb::launch_wide_bs<false, uint16_t>(p, a->block_size, s);
@@ -1033,7 +1061,7 @@ extern "C" int rocm_launch_decode_packed(const RocmMatMulNBitsArgs* a, const voi
     // Waves per workgroup. Many column groups (thousands of waves even at four per group): short waves of at most two
     // tile groups and no prefetch, so that eight of them fit a SIMD and cover each other's memory latency. Few column
     // groups: enough waves per group to reach about 8k in flight, each prefetching its next group.
-    const int64_t wgs = (a->n + 15) / 16;
+    const int64_t wgs = (a->n + 15) / 16 * (pair_member ? 2 : 1);
     int w = waves;
     bool single_set = wgs * 4 >= 6144;
     if (w <= 0) {
@@ -1053,9 +1081,34 @@ extern "C" int rocm_launch_decode_packed(const RocmMatMulNBitsArgs* a, const voi
     const int gpw = (p.groups + w - 1) / w;
     w = (p.groups + gpw - 1) / gpw;
     p.groups_per_wave = gpw;
+    // a paired launch keeps each projection's own split of K (so that it adds up in the same order) and needs twice the waves
+    if (probe_only) return a->m <= 4 && 2 * w <= w_max ? 1 : 0;
+    if (packed_up && (a->m > 4 || 2 * w > w_max)) return -1;
 
     if (bf16) return f32_scales ? mnb::launch_packed_bs<true, float>(p, a->block_size, w, single_set, s) : mnb::launch_packed_bs<true, uint16_t>(p, a->block_size, w, single_set, s);
     return f32_scales ? mnb::launch_packed_bs<false, float>(p, a->block_size, w, single_set, s) : mnb::launch_packed_bs<false, uint16_t>(p, a->block_size, w, single_set, s);
+}
+
+extern "C" int rocm_launch_decode_packed(const RocmMatMulNBitsArgs* a, const void* packed, int waves, rocm_stream_t stream)
+{
+    return launch_decode_packed(a, packed, nullptr, 0, waves, false, false, stream);
+}
+
+extern "C" int rocm_launch_decode_packed_pair_member(const RocmMatMulNBitsArgs* a, const void* packed, int waves, rocm_stream_t stream)
+{
+    return launch_decode_packed(a, packed, nullptr, 0, waves, false, true, stream);
+}
+
+extern "C" int rocm_decode_packed_pair_fits(const RocmMatMulNBitsArgs* a, int waves)
+{
+    return launch_decode_packed(a, nullptr, nullptr, 0, waves, true, true, nullptr);
+}
+
+extern "C" int rocm_launch_decode_packed_pair(const RocmMatMulNBitsArgs* a, const void* packed_gate, const void* packed_up, int decomposed, int waves,
+                                              rocm_stream_t stream)
+{
+    if (!packed_gate || !packed_up || a->y_dtype != a->a_dtype) return -1;
+    return launch_decode_packed(a, packed_gate, packed_up, decomposed, waves, false, true, stream);
 }
 
 extern "C" int rocm_acc4_packed_eligible(const RocmMatMulNBitsArgs* a)

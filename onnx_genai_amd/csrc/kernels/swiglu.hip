@@ -3,46 +3,9 @@
 // projections arrive rounded to the 16-bit type (as the separate nodes would store them), silu is evaluated in f32 with
 // the exponential taken in double and rounded to f32, and the product is rounded once. `decomposed` reproduces a graph
 // that spelled silu as Sigmoid and Mul: the sigmoid and x * sigmoid are each rounded to the 16-bit type.
-#include "common.hiph"
+#include "swiglu.hiph"
 
 namespace mnb {
-
-__device__ __forceinline__ float silu_f32(float x)
-{
-    if (x >= 0.0f) return __fdiv_rn(x, __fadd_rn(1.0f, static_cast<float>(exp(static_cast<double>(-x)))));
-    const float e = static_cast<float>(exp(static_cast<double>(x)));
-    return __fdiv_rn(__fmul_rn(x, e), __fadd_rn(1.0f, e));
-}
-
-template <bool BF16>
-__device__ __forceinline__ float round16(float v)
-{
-    return BF16 ? bf16_bits_to_f32(f32_to_bf16_bits(v)) : f16_bits_to_f32(f32_to_f16_bits(v));
-}
-
-template <bool BF16>
-__device__ __forceinline__ float silu_decomposed_f32(float x)
-{
-    float sigmoid;
-    if (x >= 0.0f) {
-        sigmoid = __fdiv_rn(1.0f, __fadd_rn(1.0f, static_cast<float>(exp(static_cast<double>(-x)))));
-    } else {
-        const float e = static_cast<float>(exp(static_cast<double>(x)));
-        sigmoid = __fdiv_rn(e, __fadd_rn(1.0f, e));
-    }
-    return round16<BF16>(as_f32(__fmul_rn(x, round16<BF16>(as_f32(sigmoid)))));
-}
-
-// 16-bit gate and up values (already rounded) -> the 16-bit result.
-template <bool BF16>
-__device__ __forceinline__ uint16_t swiglu16(uint16_t gate, uint16_t up, bool decomposed)
-{
-    const float g = BF16 ? bf16_bits_to_f32(gate) : f16_bits_to_f32(gate);
-    const float u = BF16 ? bf16_bits_to_f32(up) : f16_bits_to_f32(up);
-    const float s = decomposed ? silu_decomposed_f32<BF16>(g) : silu_f32(g);
-    const float prod = as_f32(__fmul_rn(s, u));
-    return BF16 ? f32_to_bf16_bits(prod) : f32_to_f16_bits(prod);
-}
 
 template <bool BF16>
 __global__ __launch_bounds__(256) void swiglu_kernel(const uint16_t* __restrict__ gate, const uint16_t* __restrict__ up, int64_t count, int decomposed,

@@ -572,9 +572,12 @@ SWIGLU_CASES = [
 
 
 @pytest.mark.parametrize("a_dt,s_dt,bs,zero_points,m,n,k,decomposed", SWIGLU_CASES)
-def test_gate_up_swiglu(ep, port, a_dt, s_dt, bs, zero_points, m, n, k, decomposed):
+def test_gate_up_swiglu(ep_unpacked, port, a_dt, s_dt, bs, zero_points, m, n, k, decomposed):
     """The fused node equals, bit for bit, the oracle's epilogue applied to this provider's own two projections (the node's
-    contract: 'identical to the separate kernels'), and is within the 16-bit bar of the epilogue applied to f64 projections."""
+    contract: 'identical to the separate kernels'), and is within the 16-bit bar of the epilogue applied to f64 projections.
+    Run without repacked copies: over those a pair splits K as one launch of twice the columns would, which a projection
+    launched alone does not (test_gate_up_swiglu_single_launch covers that path)."""
+    ep = ep_unpacked
     gate = synth.make_weights(n, k, bs, 810 + n, zero_points=zero_points, scale_lo=0.004, scale_hi=0.02, scale_dtype=s_dt)
     up = synth.make_weights(n, k, bs, 811 + n, zero_points=zero_points, scale_lo=0.004, scale_hi=0.02, scale_dtype=s_dt)
     a = synth.make_activation(m, k, 812 + m, a_dt)
@@ -589,6 +592,47 @@ def test_gate_up_swiglu(ep, port, a_dt, s_dt, bs, zero_points, m, n, k, decompos
     u64 = oracle_f64(port, a, a_dt, up[0], up[1], s_dt, up[2], n, k, bs)
     ideal = g64 / (1.0 + np.exp(-g64)) * u64
     assert helpers.rel_l2(synth.to_f32(y, a_dt), ideal) <= 2 * TOL_HALF
+
+
+@pytest.mark.parametrize("a_dt,s_dt,bs,zero_points,m,n,k,decomposed", [c for c in SWIGLU_CASES if c[4] <= 4] + [
+    (E.BF16, E.BF16, 128, True, 1, 18944, 3584, False),      # the 7B gate/up pair at full size: seven waves per projection
+    (E.F16, E.F16, 32, True, 2, 96, 4096, False),            # more waves per projection than half a workgroup holds: stays on two launches
+])
+def test_gate_up_swiglu_single_launch(ep, port, a_dt, s_dt, bs, zero_points, m, n, k, decomposed):
+    """From the second call on, up to four rows over constant weights run as one launch over both repacked copies, with
+    the result of the first call (two launches and the epilogue) bit for bit - also when replayed from a HIP graph."""
+    gate = synth.make_weights(n, k, bs, 810 + n, zero_points=zero_points, scale_lo=0.004, scale_hi=0.02, scale_dtype=s_dt)
+    up = synth.make_weights(n, k, bs, 811 + n, zero_points=zero_points, scale_lo=0.004, scale_hi=0.02, scale_dtype=s_dt)
+    a = synth.make_activation(m, k, 812 + m, a_dt)
+    ops = E.GateUpOperands(ep, gate, up, s_dt, n, k, bs, decomposed=decomposed)
+    ab, yb = ep.upload(a), ep.allocate(m * n * 2)
+    try:
+        ops.run(ab, a_dt, m, yb)
+        first = ep.download(yb, (m, n), np.uint16).copy()
+        assert ops.kernel.last_variant() == "gate_up_swiglu[decode_mfma_packed]"
+        ep.copy_from_host(yb, np.full(m * n * 2, 0xFF, np.uint8))
+        ops.run(ab, a_dt, m, yb)
+        single = k <= 2048 or bs == 128
+        assert ops.kernel.last_variant() == ("gate_up_swiglu_packed" if single else "gate_up_swiglu[decode_mfma_packed]")
+        assert np.array_equal(ep.download(yb, (m, n), np.uint16), first)
+        ep.sync()
+        ep.capture_begin()
+        try:
+            ops.run(ab, a_dt, m, yb)
+        finally:
+            graph = ep.capture_end()
+        ep.copy_from_host(yb, np.full(m * n * 2, 0xFF, np.uint8))
+        graph.replay()
+        assert np.array_equal(ep.download(yb, (m, n), np.uint16), first)
+        graph.release()
+        g64 = oracle_f64(port, a, a_dt, gate[0], gate[1], s_dt, gate[2], n, k, bs)
+        u64 = oracle_f64(port, a, a_dt, up[0], up[1], s_dt, up[2], n, k, bs)
+        ideal = g64 / (1.0 + np.exp(-g64)) * u64
+        assert helpers.rel_l2(synth.to_f32(first.view(NPDT[a_dt]), a_dt), ideal) <= 2 * TOL_HALF
+    finally:
+        ep.deallocate(ab)
+        ep.deallocate(yb)
+        ops.free()
 
 
 def test_gate_up_swiglu_validation(ep):
