@@ -90,7 +90,9 @@ int mnb_matmul_nbits(const void* a, int a_dtype, const uint8_t* b, const void* s
  * :4221-4233 (decomposed silu: Sigmoid and Mul as two 16-bit ops): sigmoid = 1/(1+exp(-x)) resp. e/(1+e) in f32, rounded
  *   to the 16-bit type, times x, rounded to the 16-bit type again;
  * :4375-4386: gate and up arrive rounded to the 16-bit type; y = round16(silu(gate) * up), the product one f32 multiply.
- * `dtype` is MNB_F16 or MNB_BF16 (the reference is fp16 only; bf16 follows the same steps with bf16 roundings). */
+ * `dtype` is MNB_F16 or MNB_BF16 (the reference is fp16 only; bf16 follows the same steps with bf16 roundings).
+ * Pinned by the mathematics only (the reference holds no vectors for this node): parity unpinned in the last bit of
+ * (float)exp((double)x), which is taken to round alike under every double-precision libm. */
 float mnb_swiglu_silu(float x);
 float mnb_swiglu_silu_decomposed(float x, int dtype);
 void  mnb_swiglu(const void* gate, const void* up, size_t count, int dtype, int decomposed, void* y);
