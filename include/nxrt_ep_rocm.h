@@ -82,6 +82,10 @@ NxrtRocmEp* nxrt_rocm_ep_from_vtable(const NxrtEpVtable* vtable);
  * BFloat16, and Y = round16(silu(round16(x W_gate^T)) * round16(x W_up^T)) - bit for bit what the two projections followed by
  * the 16-bit silu-and-multiply give (kernels/matmul_nbits.rs:4207-4233, 4375-4386). workspace_requirement then sizes the
  * two 16-bit [M, N] intermediates.
+ * 9=rmsnorm_prologue, 10=rmsnorm_epsilon (default 1e-5): the CUDA provider's `_cuda_matmul_nbits_rmsnorm_prologue` / `_epsilon`
+ * (optimizer.rs:48-60). The activations (Float16 or BFloat16, K % 128 == 0) are RMS-normalized before the product,
+ * x' = round16((x / sqrt(mean(x^2) + epsilon)) * gamma), with gamma [K] (Float32 or the activations' dtype) at input 6, or
+ * input 5 of the fused gate/up node - the arithmetic and summation order of kernels/matmul_nbits.rs:4125-4205.
  * struct_size tells which fields the caller's struct has: fields past its end are read as 0. */
 typedef struct NxrtRocmMatMulNBitsAttrs {
   uint32_t struct_size;
@@ -89,6 +93,8 @@ typedef struct NxrtRocmMatMulNBitsAttrs {
   int64_t K, N, bits, block_size, accuracy_level, weight_prepacked;
   int64_t folded_bias;
   int64_t gate_up_swiglu, decomposed_silu;
+  int64_t rmsnorm_prologue;
+  double rmsnorm_epsilon;
 } NxrtRocmMatMulNBitsAttrs;
 
 /* C layout of TensorView / TensorMut (crates/onnx-runtime-ep-api/src/tensor.rs:132-143, 241).

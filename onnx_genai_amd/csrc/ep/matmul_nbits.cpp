@@ -13,7 +13,7 @@ using namespace nxrt_rocm;
 
 namespace {
 
-enum AttrBit { kAttrK = 0, kAttrN = 1, kAttrBits = 2, kAttrBlockSize = 3, kAttrAccuracy = 4, kAttrPrepacked = 5, kAttrFoldedBias = 6, kAttrGateUpSwiglu = 7, kAttrDecomposedSilu = 8 };
+enum AttrBit { kAttrK = 0, kAttrN = 1, kAttrBits = 2, kAttrBlockSize = 3, kAttrAccuracy = 4, kAttrPrepacked = 5, kAttrFoldedBias = 6, kAttrGateUpSwiglu = 7, kAttrDecomposedSilu = 8, kAttrRmsnormPrologue = 9, kAttrRmsnormEpsilon = 10 };
 
 std::string err(const std::string& message) { return "MatMulNBits: " + message; }   // matmul_nbits.rs:10376
 
@@ -127,6 +127,12 @@ struct NxrtRocmMatMulNBits {
     NxrtRocmMatMulNBits* gate = nullptr;
     NxrtRocmMatMulNBits* up = nullptr;
     bool pair_member = false;            // this kernel is one projection of a fused gate/up node
+    // RMS-normalization prologue: the activations are normalized into `norm` first (gamma at input 6, or 5 of the fused node)
+    bool rmsnorm_prologue = false;
+    float rmsnorm_epsilon = 1e-5f;
+    void* norm = nullptr;
+    size_t norm_bytes = 0;
+    std::mutex norm_mu;                  // held across a normalized call: `norm` feeds the kernels enqueued under it
     bool constant_inputs[6] = {false, false, false, false, false, false};
     std::string variant = "none";
     void* scratch = nullptr;             // kernel-owned workspace, grown on demand
@@ -146,8 +152,9 @@ struct NxrtRocmMatMulNBits {
     {
         delete gate;
         delete up;
-        if ((scratch || packed || dense || !retired.empty()) && ep && ep->bind().code == NXRT_OK) {
+        if ((scratch || packed || dense || norm || !retired.empty()) && ep && ep->bind().code == NXRT_OK) {
             rocm_ffi_stream_sync(ep->stream);
+            if (norm) rocm_ffi_free(norm);
             for (void* old : retired) rocm_ffi_free(old);
             if (scratch) rocm_ffi_free(scratch);
             if (packed) rocm_ffi_free(packed);
@@ -534,8 +541,8 @@ NxrtStatus execute_swiglu(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in,
     if (!in || !out) return make_status(NXRT_INVALID_ARGUMENT, "MatMulNBits: null tensor view array");
     auto optional = [&](uint32_t i) -> const NxrtRocmTensorView* { return (i < n_in && in[i].data != nullptr) ? &in[i] : nullptr; };
     if (optional(5))
-        return make_status(NXRT_INVALID_ARGUMENT, err("gate/up SwiGLU fusion with an RMS-norm prologue (gamma at input 5) is not supported on the ROCm execution "
-                                                      "provider. How to fix: leave the normalization as its own node"));
+        return make_status(NXRT_INVALID_ARGUMENT, err("gate/up SwiGLU fusion received a normalization weight at input 5 but no RMS-norm prologue marker. "
+                                                      "How to fix: set rmsnorm_prologue = 1 on the node, or leave input 5 absent"));
     const NxrtRocmTensorView* zp_gate = optional(6);
     const NxrtRocmTensorView* zp_up = optional(7);
     if ((zp_gate != nullptr) != (zp_up != nullptr))
@@ -631,13 +638,75 @@ NxrtStatus execute_swiglu(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in,
     return hip_status(rc, "MatMulNBits: kernel launch");
 }
 
+// A node with the RMS-normalization prologue (the CUDA provider's `_cuda_matmul_nbits_rmsnorm_prologue`,
+// onnx-runtime-ep-cuda/src/optimizer.rs:48-60; kernels/matmul_nbits.rs:7739-7745, 9042-9050): gamma [K] rides at input 6
+// (input 5 of the fused gate/up node). The activations are normalized into a buffer of the kernel's own, then the node runs
+// on them as it would without the prologue.
+NxrtStatus execute_normalized(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, uint32_t n_in, NxrtRocmTensorView* out, uint32_t n_out,
+                              void* workspace, uint64_t workspace_bytes)
+{
+    std::lock_guard<std::mutex> lock(kn.norm_mu);
+    const uint32_t slot = kn.gate_up_swiglu ? 5u : 6u;
+    if (!in || n_in <= slot || in[slot].data == nullptr)
+        return make_status(NXRT_INVALID_ARGUMENT, err("rmsnorm_prologue fusion requires the normalization weight at input " + std::to_string(slot)));
+    if (n_in > (kn.gate_up_swiglu ? 8u : 7u)) return make_status(NXRT_INVALID_ARGUMENT, err("too many inputs for a node with the RMS-normalization prologue, got " + std::to_string(n_in)));
+    const NxrtRocmTensorView& A = in[0];
+    const NxrtRocmTensorView& G = in[slot];
+    const uint64_t K = static_cast<uint64_t>(kn.k);
+    if (A.dtype != NXRT_DT_FLOAT16 && A.dtype != NXRT_DT_BFLOAT16)
+        return make_status(NXRT_INVALID_ARGUMENT, err(std::string("rmsnorm_prologue fusion needs Float16 or BFloat16 activations, got ") + dtype_name(A.dtype)));
+    if (G.dtype != NXRT_DT_FLOAT32 && G.dtype != A.dtype)
+        return make_status(NXRT_INVALID_ARGUMENT, err(std::string("gamma must have dtype Float32 or the activations' dtype, got ") + dtype_name(G.dtype)));
+    if (!shape_is(G, {K})) return make_status(NXRT_INVALID_ARGUMENT, err("gamma must have shape [" + std::to_string(K) + "], got " + shape_str(G.shape, G.ndim)));
+    if (A.ndim == 0 || A.shape[A.ndim - 1] != K)
+        return make_status(NXRT_INVALID_ARGUMENT, err("A must have rank >= 1 and last dimension K=" + std::to_string(K) + ", got " + shape_str(A.shape, A.ndim)));
+    if (K % 128 != 0)
+        return make_status(NXRT_INVALID_ARGUMENT, err("rmsnorm_prologue fusion needs K to be a multiple of 128 (the reduction runs in 4-element chunks over 32 lanes), got K=" + std::to_string(K)));
+    for (const NxrtRocmTensorView* t : {&A, &G}) {
+        if (!is_contiguous(*t)) return make_status(NXRT_INVALID_ARGUMENT, err(std::string(t == &A ? "A" : "gamma") + " must be contiguous on the ROCm execution provider"));
+        if (t->device_type != NXRT_DEVICE_ROCM || t->device_index != kn.ep->device)
+            return make_status(NXRT_INVALID_ARGUMENT, err(std::string(t == &A ? "A" : "gamma") + " must live on ROCm device " + std::to_string(kn.ep->device)));
+    }
+    uint64_t M = 1;
+    for (uint32_t i = 0; i + 1 < A.ndim; ++i) M *= A.shape[i];
+    std::vector<NxrtRocmTensorView> views(in, in + n_in);
+    views[slot].data = nullptr;                                  // the node proper sees no gamma
+    uint32_t n_views = n_in;
+    if (!kn.gate_up_swiglu) n_views = n_in < 6 ? n_in : 6;
+    if (M > 0) {
+        NxrtStatus st = kn.ep->bind();
+        if (st.code != NXRT_OK) return st;
+        const uint64_t need = M * K * 2;
+        if (kn.norm_bytes < need) {
+            if (kn.ep->capturing)
+                return make_status(NXRT_INVALID_ARGUMENT, err("rmsnorm_prologue fusion under graph capture needs one eager call of this height first (the "
+                                                              "normalized activations live in a buffer the kernel may not allocate while a capture is open)"));
+            const int e = grow_buffer(kn.norm, kn.norm_bytes, need, kn.retired);
+            if (e != 0) return hip_status(e, "MatMulNBits: workspace hipMalloc");
+        }
+        const void* a = static_cast<const uint8_t*>(A.data) + A.byte_offset;
+        const void* g = static_cast<const uint8_t*>(G.data) + G.byte_offset;
+        const int rc = rocm_launch_rmsnorm16(a, g, static_cast<int>(G.dtype), static_cast<int64_t>(M), static_cast<int64_t>(K), kn.rmsnorm_epsilon,
+                                             static_cast<int>(A.dtype), kn.norm, kn.ep->stream);
+        if (rc != 0) return hip_status(rc, "MatMulNBits: kernel launch");
+        kn.ep->launches.fetch_add(1);
+        views[0].data = kn.norm;
+        views[0].byte_offset = 0;
+        views[0].strides = nullptr;
+    }
+    NxrtStatus st = kn.gate_up_swiglu ? execute_swiglu(kn, views.data(), n_views, out, n_out, workspace, workspace_bytes)
+                                      : execute_impl(kn, views.data(), n_views, out, n_out, workspace, workspace_bytes);
+    if (st.code == NXRT_OK) kn.variant = "rmsnorm+" + kn.variant;
+    return st;
+}
+
 NxrtStatus vtable_execute(void* ctx, const void* const* inputs, uint32_t n_in, void** outputs, uint32_t n_out)
 {
     return fenced([&]() -> NxrtStatus {
         auto* kn = static_cast<NxrtRocmMatMulNBits*>(ctx);
         if (!kn || !inputs || !outputs) return make_status(NXRT_INVALID_ARGUMENT, "MatMulNBits: null pointer in kernel vtable execute");
-        if (kn->gate_up_swiglu)
-            return make_status(NXRT_INVALID_ARGUMENT, err("the fused gate/up node is not served through the raw kernel vtable; call nxrt_rocm_matmul_nbits_execute"));
+        if (kn->gate_up_swiglu || kn->rmsnorm_prologue)
+            return make_status(NXRT_INVALID_ARGUMENT, err("fused nodes (gate/up, RMS-normalization prologue) are not served through the raw kernel vtable; call nxrt_rocm_matmul_nbits_execute"));
         if (kn->rows_hint < 0)
             return make_status(NXRT_INVALID_ARGUMENT, err("the kernel vtable carries no shapes; create the kernel with a static shape for A"));
         const uint64_t K = kn->k, N = kn->n, BS = kn->block_size, kb = (K + BS - 1) / BS;
@@ -696,11 +765,20 @@ int nxrt_rocm_ep_supports_matmul_nbits(const NxrtRocmEp* ep, const NxrtRocmMatMu
     if (inputs) {
         const bool swiglu = attrs->struct_size >= offsetof(NxrtRocmMatMulNBitsAttrs, gate_up_swiglu) + sizeof(int64_t) &&
                             (attrs->present & (1u << kAttrGateUpSwiglu)) && attrs->gate_up_swiglu == 1;
+        const bool rmsnorm = attrs->struct_size >= offsetof(NxrtRocmMatMulNBitsAttrs, rmsnorm_prologue) + sizeof(int64_t) &&
+                             (attrs->present & (1u << kAttrRmsnormPrologue)) && attrs->rmsnorm_prologue == 1;
+        if (rmsnorm) {
+            if (attrs->K % 128 != 0) return decline(err("rmsnorm_prologue fusion needs K to be a multiple of 128, got K=" + std::to_string(attrs->K)));
+            if (inputs[0].dtype != NXRT_DT_FLOAT16 && inputs[0].dtype != NXRT_DT_BFLOAT16)
+                return decline(err(std::string("rmsnorm_prologue fusion needs Float16 or BFloat16 activations, got ") + dtype_name(inputs[0].dtype)));
+            if (!swiglu) return n_inputs == 7 ? 1 : decline(err("rmsnorm_prologue fusion requires the normalization weight at input 6"));
+            return (n_inputs >= 6 && n_inputs <= 8 && inputs[5].dtype != 0) ? 1 : decline(err("rmsnorm_prologue fusion requires the normalization weight at input 5"));
+        }
         if (swiglu) {
             if (n_inputs < 5 || n_inputs > 8) return decline(err("gate/up SwiGLU fusion expects 5 to 8 inputs, got " + std::to_string(n_inputs)));
             if (inputs[0].dtype != NXRT_DT_FLOAT16 && inputs[0].dtype != NXRT_DT_BFLOAT16)
                 return decline(err(std::string("gate/up SwiGLU fusion needs Float16 or BFloat16 activations, got ") + dtype_name(inputs[0].dtype)));
-            if (n_inputs > 5 && inputs[5].dtype != 0) return decline(err("gate/up SwiGLU fusion with an RMS-norm prologue (gamma at input 5) is not supported on the ROCm execution provider"));
+            if (n_inputs > 5 && inputs[5].dtype != 0) return decline(err("gate/up SwiGLU fusion received a normalization weight at input 5 but no RMS-norm prologue marker"));
             return 1;
         }
         if (n_inputs < 3 || n_inputs > 6) return decline("MatMulNBits: expected 3..=6 inputs, got " + std::to_string(n_inputs));
@@ -749,6 +827,9 @@ NxrtStatus nxrt_rocm_matmul_nbits_create(NxrtRocmEp* ep, const NxrtRocmMatMulNBi
         const bool has_swiglu = attrs->struct_size >= offsetof(NxrtRocmMatMulNBitsAttrs, decomposed_silu) + sizeof(int64_t);
         kn->gate_up_swiglu = has_swiglu && (attrs->present & (1u << kAttrGateUpSwiglu)) && attrs->gate_up_swiglu == 1;
         kn->decomposed_silu = has_swiglu && (attrs->present & (1u << kAttrDecomposedSilu)) && attrs->decomposed_silu == 1;
+        const bool has_rmsnorm = attrs->struct_size >= offsetof(NxrtRocmMatMulNBitsAttrs, rmsnorm_epsilon) + sizeof(double);
+        kn->rmsnorm_prologue = has_rmsnorm && (attrs->present & (1u << kAttrRmsnormPrologue)) && attrs->rmsnorm_prologue == 1;
+        if (has_rmsnorm && (attrs->present & (1u << kAttrRmsnormEpsilon))) kn->rmsnorm_epsilon = static_cast<float>(attrs->rmsnorm_epsilon);
         if (kn->gate_up_swiglu) {
             for (NxrtRocmMatMulNBits** child : {&kn->gate, &kn->up}) {
                 auto* c2 = new NxrtRocmMatMulNBits();
@@ -839,6 +920,7 @@ NxrtStatus nxrt_rocm_matmul_nbits_execute(NxrtRocmMatMulNBits* kernel, const Nxr
 {
     return fenced([&]() -> NxrtStatus {
         if (!kernel) return make_status(NXRT_INVALID_ARGUMENT, "MatMulNBits: null kernel");
+        if (kernel->rmsnorm_prologue) return execute_normalized(*kernel, inputs, n_inputs, outputs, n_outputs, workspace_device, workspace_bytes);
         if (kernel->gate_up_swiglu) return execute_swiglu(*kernel, inputs, n_inputs, outputs, n_outputs, workspace_device, workspace_bytes);
         return execute_impl(*kernel, inputs, n_inputs, outputs, n_outputs, workspace_device, workspace_bytes);
     });

@@ -86,6 +86,11 @@ int rocm_dense_gemm_run(RocmDenseGemm* g, const void* w_nk, const void* a, void*
  * (onnx-runtime-ep-cuda/src/kernels/matmul_nbits.rs:4207-4233, 4375-4386). decomposed = 1: silu spelled as Sigmoid and Mul. */
 int rocm_launch_swiglu(const void* gate, const void* up, int64_t count, int dtype, int decomposed, void* y, rocm_stream_t stream);
 
+/* out = round16((a * inv_std) * gamma) per row of K 16-bit elements (K % 128 == 0), inv_std = 1 / sqrt(mean(a^2) + eps),
+ * summed in the reference's order (onnx-runtime-ep-cuda/src/kernels/matmul_nbits.rs:4125-4205). gamma: f32 or 16-bit. */
+int rocm_launch_rmsnorm16(const void* a, const void* gamma, int gamma_dtype, int64_t rows, int64_t k, float epsilon, int dtype, void* out,
+                          rocm_stream_t stream);
+
 /* Any dtype mix, any K, any block size: f32 math, one wave per output column. */
 int rocm_launch_gemv_generic(const RocmMatMulNBitsArgs* args, rocm_stream_t stream);
 /* f32 activations, M <= 4, block size >= 32, K % 4 == 0, A and B 16-byte aligned: f32 FMA streaming kernel */

@@ -15,7 +15,64 @@ __global__ __launch_bounds__(256) void swiglu_kernel(const uint16_t* __restrict_
         y[i] = swiglu16<BF16>(gate[i], up[i], decomposed != 0);
 }
 
+// RMS-normalization prologue (onnx-runtime-ep-cuda/src/kernels/matmul_nbits.rs:4125-4205): out = round16((a * inv_std) *
+// gamma) per row, inv_std = 1 / sqrt(mean(a^2) + eps). The sum of squares follows the reference's order exactly - 32
+// lanes, each with four running sums over its 4-element chunks, (s0 + s1) + (s2 + s3), then the shuffle tree over 32
+// lanes - so half a wavefront plays one 32-lane warp and a workgroup of one wave normalizes two rows.
+template <bool BF16>
+__global__ __launch_bounds__(64) void rmsnorm16_kernel(const uint16_t* __restrict__ a, const void* __restrict__ gamma, int gamma_dtype, int64_t rows,
+                                                       int64_t k, float epsilon, uint16_t* __restrict__ out)
+{
+    const int lane = threadIdx.x & 31;
+    const int64_t row = static_cast<int64_t>(blockIdx.x) * 2 + (threadIdx.x >> 5);
+    const bool live = row < rows;
+    const uint16_t* x = a + (live ? row : 0) * k;
+    const int chunks_per_lane = static_cast<int>(k / 128);
+    float ss0 = 0.f, ss1 = 0.f, ss2 = 0.f, ss3 = 0.f;
+    for (int item = 0; item < chunks_per_lane; ++item) {
+        const uint2 raw = reinterpret_cast<const uint2*>(x)[lane + item * 32];
+        const float v0 = BF16 ? bf16_bits_to_f32(static_cast<uint16_t>(raw.x)) : f16_bits_to_f32(static_cast<uint16_t>(raw.x));
+        const float v1 = BF16 ? bf16_bits_to_f32(static_cast<uint16_t>(raw.x >> 16)) : f16_bits_to_f32(static_cast<uint16_t>(raw.x >> 16));
+        const float v2 = BF16 ? bf16_bits_to_f32(static_cast<uint16_t>(raw.y)) : f16_bits_to_f32(static_cast<uint16_t>(raw.y));
+        const float v3 = BF16 ? bf16_bits_to_f32(static_cast<uint16_t>(raw.y >> 16)) : f16_bits_to_f32(static_cast<uint16_t>(raw.y >> 16));
+        ss0 = __fmaf_rn(v0, v0, ss0);
+        ss1 = __fmaf_rn(v1, v1, ss1);
+        ss2 = __fmaf_rn(v2, v2, ss2);
+        ss3 = __fmaf_rn(v3, v3, ss3);
+    }
+    float ss = __fadd_rn(__fadd_rn(ss0, ss1), __fadd_rn(ss2, ss3));
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) ss = __fadd_rn(ss, __shfl_down(ss, off, 32));
+    // sqrtf, not __fsqrt_rn: the latter is the hardware's approximate square root here; sqrtf and the division are
+    // correctly rounded (the compiler's default for f32 divide and sqrt)
+    float inv_std = __fdiv_rn(1.0f, sqrtf(__fadd_rn(__fdiv_rn(ss, static_cast<float>(k)), epsilon)));
+    inv_std = __shfl(inv_std, 0, 32);
+    if (!live) return;
+    for (int64_t j = lane; j < k; j += 32) {
+        const float v = BF16 ? bf16_bits_to_f32(x[j]) : f16_bits_to_f32(x[j]);
+        const float g = load_as_f32(gamma, gamma_dtype, j);
+        const float y = as_f32(__fmul_rn(__fmul_rn(v, inv_std), g));
+        out[row * k + j] = BF16 ? f32_to_bf16_bits(y) : f32_to_f16_bits(y);
+    }
+}
+
 }  // namespace mnb
+
+extern "C" int rocm_launch_rmsnorm16(const void* a, const void* gamma, int gamma_dtype, int64_t rows, int64_t k, float epsilon, int dtype, void* out,
+                                     rocm_stream_t stream)
+{
+    if (rows <= 0 || k <= 0) return 0;
+    if ((dtype != ROCM_DT_F16 && dtype != ROCM_DT_BF16) || k % 128 != 0) return static_cast<int>(hipErrorInvalidValue);
+    const unsigned blocks = static_cast<unsigned>((rows + 1) / 2);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == ROCM_DT_BF16)
+        hipLaunchKernelGGL(mnb::rmsnorm16_kernel<true>, dim3(blocks), dim3(64), 0, s, static_cast<const uint16_t*>(a), gamma, gamma_dtype, rows, k, epsilon,
+                           static_cast<uint16_t*>(out));
+    else
+        hipLaunchKernelGGL(mnb::rmsnorm16_kernel<false>, dim3(blocks), dim3(64), 0, s, static_cast<const uint16_t*>(a), gamma, gamma_dtype, rows, k, epsilon,
+                           static_cast<uint16_t*>(out));
+    return static_cast<int>(hipGetLastError());
+}
 
 extern "C" int rocm_launch_swiglu(const void* gate, const void* up, int64_t count, int dtype, int decomposed, void* y, rocm_stream_t stream)
 {

@@ -50,7 +50,7 @@ class NxrtTensorDesc(C.Structure):
 class Attrs(C.Structure):
     _fields_ = [("struct_size", C.c_uint32), ("present", C.c_uint32), ("K", C.c_int64), ("N", C.c_int64), ("bits", C.c_int64),
                 ("block_size", C.c_int64), ("accuracy_level", C.c_int64), ("weight_prepacked", C.c_int64), ("folded_bias", C.c_int64),
-                ("gate_up_swiglu", C.c_int64), ("decomposed_silu", C.c_int64)]
+                ("gate_up_swiglu", C.c_int64), ("decomposed_silu", C.c_int64), ("rmsnorm_prologue", C.c_int64), ("rmsnorm_epsilon", C.c_double)]
 
 
 class CTensorView(C.Structure):
@@ -63,7 +63,7 @@ class WorkspaceRequirement(C.Structure):
 
 
 _ATTR_BITS = {"K": 0, "N": 1, "bits": 2, "block_size": 3, "accuracy_level": 4, "weight_prepacked": 5, "folded_bias": 6, "gate_up_swiglu": 7,
-              "decomposed_silu": 8}
+              "decomposed_silu": 8, "rmsnorm_prologue": 9, "rmsnorm_epsilon": 10}
 _lib = None
 
 
@@ -157,7 +157,7 @@ def make_attrs(**kw) -> Attrs:
         if value is None:
             continue
         a.present |= 1 << _ATTR_BITS[name]
-        setattr(a, name, int(value))
+        setattr(a, name, float(value) if name == "rmsnorm_epsilon" else int(value))
     return a
 
 
@@ -450,7 +450,7 @@ class DeviceOperands:
     """The device-resident operands of one MatMulNBits node plus its kernel; what a session would hold."""
 
     def __init__(self, ep, b, scales, scale_dtype, zp, n, k, bs, *, accuracy_level=0, bias=None, bias_dtype=F32, rows=None, a_dtype=None,
-                 folded_bias=None):
+                 folded_bias=None, gamma=None, gamma_dtype=F32, rmsnorm_epsilon=None):
         self.ep, self.n, self.k, self.bs = ep, n, k, bs
         self.kb = -(-k // bs)
         self.scale_dtype, self.bias_dtype = scale_dtype, bias_dtype
@@ -458,22 +458,27 @@ class DeviceOperands:
         self.scales = ep.upload(scales)
         self.zp = ep.upload(np.asarray(zp, np.uint8)) if zp is not None else None
         self.bias = ep.upload(bias) if bias is not None else None
+        self.gamma = ep.upload(gamma) if gamma is not None else None        # RMS-normalization prologue: gamma [K] at input 6
+        self.gamma_dtype = gamma_dtype
         shapes = None
         if rows is not None and a_dtype is not None:
             shapes = [((rows, k), a_dtype), ((n, self.kb, bs // 2), U8), ((n, self.kb), scale_dtype)]
-        self.kernel = ep.get_kernel({"K": k, "N": n, "bits": 4, "block_size": bs, "accuracy_level": accuracy_level, "folded_bias": folded_bias}, shapes)
-        self.kernel.set_constant_inputs([False, True, True, True, True, True])
+        self.kernel = ep.get_kernel({"K": k, "N": n, "bits": 4, "block_size": bs, "accuracy_level": accuracy_level, "folded_bias": folded_bias,
+                                     "rmsnorm_prologue": 1 if gamma is not None else None, "rmsnorm_epsilon": rmsnorm_epsilon}, shapes)
+        self.kernel.set_constant_inputs([False, True, True, True, True, True, True])
 
     def views(self, a_buf: DeviceBuffer, a_dtype: int, m: int):
         dev = self.ep.device_index
         ins = [TensorView(a_buf.ptr, a_dtype, (m, self.k), device_index=dev),
                TensorView(self.b.ptr, U8, (self.n, self.kb, self.bs // 2), device_index=dev),
                TensorView(self.scales.ptr, self.scale_dtype, (self.n, self.kb), device_index=dev)]
-        if self.zp is not None or self.bias is not None:
+        if self.zp is not None or self.bias is not None or self.gamma is not None:
             ins.append(TensorView(self.zp.ptr, U8, (self.n, (self.kb + 1) // 2), device_index=dev) if self.zp is not None else TensorView.absent(U8))
-        if self.bias is not None:
+        if self.bias is not None or self.gamma is not None:
             ins.append(TensorView.absent(I32))
-            ins.append(TensorView(self.bias.ptr, self.bias_dtype, (self.n,), device_index=dev))
+            ins.append(TensorView(self.bias.ptr, self.bias_dtype, (self.n,), device_index=dev) if self.bias is not None else TensorView.absent(F32))
+        if self.gamma is not None:
+            ins.append(TensorView(self.gamma.ptr, self.gamma_dtype, (self.k,), device_index=dev))
         return ins
 
     def run(self, a_buf: DeviceBuffer, a_dtype: int, m: int, y_buf: DeviceBuffer, y_dtype: int | None = None) -> None:
@@ -483,17 +488,19 @@ class DeviceOperands:
 
     def free(self) -> None:
         self.kernel.release()
-        for buf in (self.b, self.scales, self.zp, self.bias):
+        for buf in (self.b, self.scales, self.zp, self.bias, self.gamma):
             if buf is not None:
                 self.ep.deallocate(buf)
 
 
-def matmul_nbits(ep, a, a_dtype, b, scales, scale_dtype, zp, n, k, bs, *, accuracy_level=0, bias=None, bias_dtype=F32, y_dtype=None, folded_bias=None):
+def matmul_nbits(ep, a, a_dtype, b, scales, scale_dtype, zp, n, k, bs, *, accuracy_level=0, bias=None, bias_dtype=F32, y_dtype=None, folded_bias=None,
+                 gamma=None, gamma_dtype=F32, rmsnorm_epsilon=None):
     """One-shot helper: upload, execute through the C ABI, download. Returns (Y as numpy, variant name)."""
     y_dtype = a_dtype if y_dtype is None else y_dtype
     a = np.ascontiguousarray(a)
     m = a.size // k
-    ops = DeviceOperands(ep, b, scales, scale_dtype, zp, n, k, bs, accuracy_level=accuracy_level, bias=bias, bias_dtype=bias_dtype, folded_bias=folded_bias)
+    ops = DeviceOperands(ep, b, scales, scale_dtype, zp, n, k, bs, accuracy_level=accuracy_level, bias=bias, bias_dtype=bias_dtype, folded_bias=folded_bias,
+                         gamma=gamma, gamma_dtype=gamma_dtype, rmsnorm_epsilon=rmsnorm_epsilon)
     a_buf = ep.upload(a)
     y_buf = ep.allocate(max(m * n * _ITEM[y_dtype], 1))
     try:
@@ -510,14 +517,17 @@ def matmul_nbits(ep, a, a_dtype, b, scales, scale_dtype, zp, n, k, bs, *, accura
 class GateUpOperands:
     """Device-resident operands of the fused gate/up node (inputs [x, W_gate, scales_gate, W_up, scales_up, -, zp_gate, zp_up])."""
 
-    def __init__(self, ep, gate, up, scale_dtype, n, k, bs, *, decomposed=False, rows=None, a_dtype=None):
+    def __init__(self, ep, gate, up, scale_dtype, n, k, bs, *, decomposed=False, rows=None, a_dtype=None, gamma=None, gamma_dtype=F32, rmsnorm_epsilon=None):
         self.ep, self.n, self.k, self.bs, self.scale_dtype = ep, n, k, bs, scale_dtype
         self.kb = -(-k // bs)
         self.bufs = []
         for b, s, zp in (gate, up):
             self.bufs.append((ep.upload(np.asarray(b, np.uint8)), ep.upload(s), ep.upload(np.asarray(zp, np.uint8)) if zp is not None else None))
         shapes = [((rows, k), a_dtype)] if rows is not None and a_dtype is not None else None
-        self.kernel = ep.get_kernel({"K": k, "N": n, "bits": 4, "block_size": bs, "gate_up_swiglu": 1, "decomposed_silu": 1 if decomposed else None}, shapes)
+        self.gamma = ep.upload(gamma) if gamma is not None else None
+        self.gamma_dtype = gamma_dtype
+        self.kernel = ep.get_kernel({"K": k, "N": n, "bits": 4, "block_size": bs, "gate_up_swiglu": 1, "decomposed_silu": 1 if decomposed else None,
+                                     "rmsnorm_prologue": 1 if gamma is not None else None, "rmsnorm_epsilon": rmsnorm_epsilon}, shapes)
         self.kernel.set_constant_inputs([False, True, True, True, True, True, True, True])
 
     def views(self, a_buf: DeviceBuffer, a_dtype: int, m: int):
@@ -527,8 +537,11 @@ class GateUpOperands:
         ins = [TensorView(a_buf.ptr, a_dtype, (m, self.k), device_index=dev),
                TensorView(bg.ptr, U8, w_shape, device_index=dev), TensorView(sg.ptr, self.scale_dtype, s_shape, device_index=dev),
                TensorView(bu.ptr, U8, w_shape, device_index=dev), TensorView(su.ptr, self.scale_dtype, s_shape, device_index=dev)]
+        gamma = TensorView(self.gamma.ptr, self.gamma_dtype, (self.k,), device_index=dev) if self.gamma is not None else None
         if zg is not None:
-            ins += [TensorView.absent(F32), TensorView(zg.ptr, U8, z_shape, device_index=dev), TensorView(zu.ptr, U8, z_shape, device_index=dev)]
+            ins += [gamma or TensorView.absent(F32), TensorView(zg.ptr, U8, z_shape, device_index=dev), TensorView(zu.ptr, U8, z_shape, device_index=dev)]
+        elif gamma is not None:
+            ins.append(gamma)
         return ins
 
     def run(self, a_buf: DeviceBuffer, a_dtype: int, m: int, y_buf: DeviceBuffer, workspace: DeviceBuffer | None = None) -> None:
@@ -537,17 +550,17 @@ class GateUpOperands:
 
     def free(self) -> None:
         self.kernel.release()
-        for group in self.bufs:
+        for group in self.bufs + [(self.gamma,)]:
             for buf in group:
                 if buf is not None:
                     self.ep.deallocate(buf)
 
 
-def gate_up_swiglu(ep, a, a_dtype, gate, up, scale_dtype, n, k, bs, *, decomposed=False):
+def gate_up_swiglu(ep, a, a_dtype, gate, up, scale_dtype, n, k, bs, *, decomposed=False, gamma=None, gamma_dtype=F32, rmsnorm_epsilon=None):
     """One-shot helper for the fused gate/up node: gate and up are (B, scales, zero_points or None). Returns (Y, variant)."""
     a = np.ascontiguousarray(a)
     m = a.size // k
-    ops = GateUpOperands(ep, gate, up, scale_dtype, n, k, bs, decomposed=decomposed)
+    ops = GateUpOperands(ep, gate, up, scale_dtype, n, k, bs, decomposed=decomposed, gamma=gamma, gamma_dtype=gamma_dtype, rmsnorm_epsilon=rmsnorm_epsilon)
     a_buf = ep.upload(a)
     y_buf = ep.allocate(max(m * n * 2, 1))
     try:

@@ -84,6 +84,7 @@ class Port:
         L.mnb_swiglu_silu_decomposed.restype = C.c_float
         L.mnb_swiglu_silu_decomposed.argtypes = [C.c_float, C.c_int]
         L.mnb_swiglu.argtypes = [v, v, z, C.c_int, C.c_int, v]
+        L.mnb_rmsnorm16.argtypes = [v, v, C.c_int, z, z, C.c_float, C.c_int, v]
         L.mnb_matmul_nbits.restype = C.c_int
         L.mnb_matmul_nbits.argtypes = [v, C.c_int, v, v, C.c_int, v, v, C.c_int, v, C.c_int, z, z, z, z, C.c_int, C.c_int]
 
@@ -106,6 +107,15 @@ class Port:
         gate16, up16 = np.ascontiguousarray(gate16), np.ascontiguousarray(up16)
         out = np.empty(gate16.shape, _NP_DT[code])
         self.lib.mnb_swiglu(_ptr(gate16), _ptr(up16), gate16.size, code, int(decomposed), _ptr(out))
+        return out
+
+    def rmsnorm16(self, a16: np.ndarray, gamma: np.ndarray, gamma_code: int, epsilon: float, code: int) -> np.ndarray:
+        """The RMS-normalization prologue on 16-bit rows [rows, K] (K % 128 == 0); gamma 16-bit of the same type or f32."""
+        a16, gamma = np.ascontiguousarray(a16), np.ascontiguousarray(gamma)
+        rows, k = a16.shape
+        assert k % 128 == 0 and gamma.size == k
+        out = np.empty(a16.shape, _NP_DT[code])
+        self.lib.mnb_rmsnorm16(_ptr(a16), _ptr(gamma), gamma_code, rows, k, float(epsilon), code, _ptr(out))
         return out
 
     # -- operator pieces -----------------------------------------------------------------------

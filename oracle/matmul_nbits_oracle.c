@@ -321,3 +321,42 @@ void mnb_swiglu(const void* gate, const void* up, size_t count, int dtype, int d
         out[i] = dtype == MNB_F16 ? mnb_f32_to_f16(prod) : mnb_f32_to_bf16(prod);
     }
 }
+
+
+/* ---- RMS-normalization prologue (onnx-runtime-ep-cuda/src/kernels/matmul_nbits.rs:4125-4205) ---- */
+
+void mnb_rmsnorm16(const void* a, const void* gamma, int gamma_dtype, size_t rows, size_t k, float epsilon, int dtype, void* out)
+{
+    const uint16_t* in = (const uint16_t*)a;
+    uint16_t* dst = (uint16_t*)out;
+    const size_t chunks_per_lane = k / (32 * 4);
+    for (size_t row = 0; row < rows; ++row) {
+        const uint16_t* x = in + row * k;
+        float lane_sum[32];
+        for (size_t lane = 0; lane < 32; ++lane) {
+            float ss[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+            for (size_t item = 0; item < chunks_per_lane; ++item) {
+                const size_t chunk = lane + item * 32;
+                for (int e = 0; e < 4; ++e) {
+                    const float v = dtype == MNB_F16 ? mnb_f16_to_f32(x[chunk * 4 + e]) : mnb_bf16_to_f32(x[chunk * 4 + e]);
+                    ss[e] = fmaf(v, v, ss[e]);
+                }
+            }
+            lane_sum[lane] = (ss[0] + ss[1]) + (ss[2] + ss[3]);
+        }
+        for (size_t off = 16; off > 0; off >>= 1) {
+            float next[32];
+            for (size_t lane = 0; lane < 32; ++lane) next[lane] = lane_sum[lane] + (lane + off < 32 ? lane_sum[lane + off] : lane_sum[lane]);
+            memcpy(lane_sum, next, sizeof(next));
+        }
+        const float inv_std = 1.0f / sqrtf(lane_sum[0] / (float)k + epsilon);
+        for (size_t j = 0; j < k; ++j) {
+            const float v = dtype == MNB_F16 ? mnb_f16_to_f32(x[j]) : mnb_bf16_to_f32(x[j]);
+            float g;
+            if (gamma_dtype == MNB_F32) g = ((const float*)gamma)[j];
+            else g = gamma_dtype == MNB_F16 ? mnb_f16_to_f32(((const uint16_t*)gamma)[j]) : mnb_bf16_to_f32(((const uint16_t*)gamma)[j]);
+            const float y = (v * inv_std) * g;
+            dst[row * k + j] = dtype == MNB_F16 ? mnb_f32_to_f16(y) : mnb_f32_to_bf16(y);
+        }
+    }
+}

@@ -97,6 +97,16 @@ float mnb_swiglu_silu(float x);
 float mnb_swiglu_silu_decomposed(float x, int dtype);
 void  mnb_swiglu(const void* gate, const void* up, size_t count, int dtype, int decomposed, void* y);
 
+/* The RMS-normalization prologue the CUDA provider folds into a following MatMulNBits
+ * (onnx-runtime-ep-cuda/src/kernels/matmul_nbits.rs:4125-4205, the same arithmetic in-kernel at :3747-3783): per row of K
+ * 16-bit elements, 32 lanes each own the 4-element chunks lane, lane + 32, ...; four running sums of squares per lane (one per
+ * element of a chunk; a * a + s as one fused multiply-add, the CUDA compiler's default contraction), combined as
+ * (s0 + s1) + (s2 + s3), then the shuffle tree off = 16, 8, 4, 2, 1 (lane += lane + off); inv_std = 1 / sqrtf(ss / K + eps),
+ * every step correctly rounded; out = round16((a * inv_std) * gamma). K % 128 == 0. gamma: 16-bit of `dtype` or f32.
+ * Pinned by the mathematics only (closed forms, a double-precision restatement): the reference holds no vectors, and
+ * whether its compiler contracts the sum of squares is an assumption - parity unpinned in that respect. */
+void mnb_rmsnorm16(const void* a, const void* gamma, int gamma_dtype, size_t rows, size_t k, float epsilon, int dtype, void* out);
+
 #ifdef __cplusplus
 }
 #endif

@@ -259,3 +259,35 @@ def test_swiglu_rounding_steps(port):
     # silu(gate) * 0 = 0 and silu(0) * up = 0
     z = port.swiglu(np.array([2.0, 0.0], np.float16), np.array([0.0, 5.0], np.float16), oracle.F16, False)
     assert np.array_equal(z.view(np.uint16) & 0x7fff, np.zeros(2, np.uint16))
+
+
+# ---------------------------------------------------------------------------------------------
+# The RMS-normalization prologue (onnx-runtime-ep-cuda/src/kernels/matmul_nbits.rs:4125-4205): pinned by the mathematics.
+# ---------------------------------------------------------------------------------------------
+def test_rmsnorm_closed_forms_and_double_precision(port):
+    k = 512
+    # a constant row c: mean square c^2 exactly (every partial sum is a small multiple of c^2), so y = f16(f32(c / sqrt(c^2 + eps)) * gamma)
+    for c, eps in ((1.0, 0.0), (0.5, 0.0), (2.0, 1e-5), (-3.0, 1e-6)):
+        a = np.full((1, k), c, np.float16)
+        gamma = np.linspace(0.5, 1.5, k).astype(np.float32)
+        inv = np.float32(1.0) / np.sqrt(np.float32(np.float32(c * c * k) / np.float32(k)) + np.float32(eps), dtype=np.float32)
+        want = (np.float32(c) * inv * gamma).astype(np.float16)
+        got = port.rmsnorm16(a, gamma, oracle.F32, eps, oracle.F16)
+        assert np.array_equal(got[0].view(np.uint16), want.view(np.uint16))
+    # random rows against a double-precision restatement: within one unit of the 16-bit grid (f32 sums of 512 squares agree
+    # with the exact sum to ~1e-6, far below the 16-bit rounding)
+    rng = np.random.default_rng(11)
+    for code, np_dt in ((oracle.F16, np.float16), (oracle.BF16, None)):
+        a32 = rng.standard_normal((5, k)).astype(np.float32)
+        a16 = port.narrow(a32, code)
+        af = port.widen(a16, code).astype(np.float64)
+        gamma = (1.0 + 0.1 * rng.standard_normal(k)).astype(np.float32)
+        want = af / np.sqrt(np.mean(af * af, axis=1, keepdims=True) + 1e-5) * gamma.astype(np.float64)
+        got = port.widen(port.rmsnorm16(a16, gamma, oracle.F32, 1e-5, code), code).astype(np.float64)
+        grid = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(want), 1e-30))) - (10 if code == oracle.F16 else 7))
+        if code == oracle.F16:
+            grid = np.maximum(grid, 2.0 ** -24)                     # f16 subnormals lie on a fixed grid
+        assert np.all(np.abs(got - want) <= 0.5 * grid + 2e-6 * np.abs(want))       # 2e-6: the f32 steps before the 16-bit rounding
+    # a zero row stays zero; gamma of the activations' own 16-bit type is read as such
+    z = port.rmsnorm16(np.zeros((1, k), np.float16), np.ones(k, np.float16), oracle.F16, 1e-5, oracle.F16)
+    assert not z.view(np.uint16).any()

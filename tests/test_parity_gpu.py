@@ -635,6 +635,66 @@ def test_gate_up_swiglu_single_launch(ep, port, a_dt, s_dt, bs, zero_points, m, 
         ops.free()
 
 
+RMSNORM_CASES = [
+    # a_dt, gamma dtype, bs, m, n, k, epsilon
+    (E.F16, E.F16, 32, 1, 300, 896, 1e-6),
+    (E.F16, E.F32, 32, 3, 136, 1024, 1e-5),
+    (E.BF16, E.BF16, 128, 1, 520, 3584, 1e-6),
+    (E.BF16, E.F32, 128, 16, 200, 1024, 1e-5),
+    (E.F16, E.F16, 64, 100, 136, 512, 1e-5),
+]
+
+
+@pytest.mark.parametrize("a_dt,g_dt,bs,m,n,k,eps", RMSNORM_CASES)
+def test_rmsnorm_prologue(ep, port, a_dt, g_dt, bs, m, n, k, eps):
+    """A node with the RMS-normalization prologue gives, bit for bit, what the same node without it gives on activations the
+    oracle normalized: the prologue's kernel equals the oracle's restatement (sums in the reference's order) on every element
+    that matters to the product."""
+    b, s, zp = synth.make_weights(n, k, bs, 820 + n, zero_points=True, scale_lo=0.002, scale_hi=0.01, scale_dtype=a_dt)
+    a = synth.make_activation(m, k, 821 + m, a_dt)
+    gamma = synth.to_dtype((1.0 + 0.25 * np.random.default_rng(k).standard_normal(k)).astype(np.float32), g_dt)
+    o_dt = oracle.F16 if a_dt == E.F16 else oracle.BF16
+    g_code = oracle.F32 if g_dt == E.F32 else o_dt
+    normalized = port.rmsnorm16(np.asarray(a).reshape(m, k), gamma, g_code, eps, o_dt)
+    y, variant = run_op(ep, a, a_dt, b, s, a_dt, zp, n, k, bs, gamma=gamma, gamma_dtype=g_dt, rmsnorm_epsilon=eps)
+    want, plain_variant = run_op(ep, normalized, a_dt, b, s, a_dt, zp, n, k, bs)
+    assert variant == "rmsnorm+" + plain_variant
+    assert np.array_equal(np.asarray(y).view(np.uint16), np.asarray(want).view(np.uint16))
+    # and the normalization is one: mean square of the normalized row over gamma^2 is 1 within the 16-bit roundings
+    nf = synth.to_f32(normalized, a_dt) / synth.to_f32(gamma, g_dt)[None, :]
+    assert np.allclose(np.mean(nf.astype(np.float64) ** 2, axis=1), 1.0, rtol=2e-2)
+
+
+def test_rmsnorm_prologue_on_the_fused_gate_up_node(ep, port):
+    a_dt, bs, m, n, k, eps = E.F16, 32, 2, 200, 1024, 1e-6
+    gate = synth.make_weights(n, k, bs, 830, zero_points=True, scale_lo=0.004, scale_hi=0.02, scale_dtype=a_dt)
+    up = synth.make_weights(n, k, bs, 831, zero_points=True, scale_lo=0.004, scale_hi=0.02, scale_dtype=a_dt)
+    a = synth.make_activation(m, k, 832, a_dt)
+    gamma = (1.0 + 0.25 * np.random.default_rng(7).standard_normal(k)).astype(np.float32)
+    normalized = port.rmsnorm16(np.asarray(a).reshape(m, k), gamma, oracle.F32, eps, oracle.F16)
+    y, variant = E.gate_up_swiglu(ep, a, a_dt, gate, up, a_dt, n, k, bs, gamma=gamma, gamma_dtype=E.F32, rmsnorm_epsilon=eps)
+    want, _ = E.gate_up_swiglu(ep, normalized, a_dt, gate, up, a_dt, n, k, bs)
+    assert variant.startswith("rmsnorm+gate_up_swiglu")
+    assert np.array_equal(np.asarray(y).view(np.uint16), np.asarray(want).view(np.uint16))
+
+
+def test_rmsnorm_prologue_validation(ep):
+    a_dt, bs, n = E.F16, 32, 64
+    for k, match in ((192, "multiple of 128"), (256, "normalization weight at input 6")):
+        b, s, zp = synth.make_weights(n, k, bs, 1, zero_points=True, scale_lo=0.004, scale_hi=0.02, scale_dtype=a_dt)
+        ops = E.DeviceOperands(ep, b, s, a_dt, zp, n, k, bs, gamma=np.ones(k, np.float32), gamma_dtype=E.F32)
+        a, y = ep.upload(synth.make_activation(2, k, 3, a_dt)), ep.allocate(2 * n * 2)
+        try:
+            views = ops.views(a, a_dt, 2)
+            out = [E.TensorView(y.ptr, a_dt, (2, n), device_index=ep.device_index)]
+            with pytest.raises(E.EpError, match=match):
+                ops.kernel.execute(views if k == 192 else views[:6], out)
+        finally:
+            ep.deallocate(a)
+            ep.deallocate(y)
+            ops.free()
+
+
 def test_gate_up_swiglu_validation(ep):
     a_dt, bs, n, k = E.F16, 32, 64, 128
     gate = synth.make_weights(n, k, bs, 1, zero_points=True, scale_lo=0.004, scale_hi=0.02, scale_dtype=a_dt)
@@ -651,7 +711,7 @@ def test_gate_up_swiglu_validation(ep):
             ops.kernel.execute(views[:4], out)
         gamma = list(views)
         gamma[5] = E.TensorView(a.ptr, a_dt, (k,), device_index=ep.device_index)
-        with pytest.raises(E.EpError, match="RMS-norm prologue"):
+        with pytest.raises(E.EpError, match="no RMS-norm prologue marker"):
             ops.kernel.execute(gamma, out)
         with pytest.raises(E.EpError, match="Y must have dtype"):
             ops.kernel.execute(views, [E.TensorView(y.ptr, E.F32, (2, n), device_index=ep.device_index)])
