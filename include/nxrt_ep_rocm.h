@@ -153,6 +153,11 @@ NxrtStatus nxrt_rocm_matmul_nbits_as_vtable(NxrtRocmMatMulNBits* kernel, NxrtKer
 NxrtStatus nxrt_rocm_matmul_nbits_dequantize(NxrtRocmEp* ep, const void* b_device, const void* scales_device, uint32_t scale_dtype,
                                              const void* zero_points_device, uint64_t n, uint64_t k, uint32_t block_size,
                                              float* out_nk_device);
+/* The same at bits = 2, 4 or 8 (NBitsLayout, matmul_nbits.rs:1276-1321): b is [N, kb, block_size * bits / 8], zero points
+ * [N, ceil(kb * bits / 8)], default zero point 1 << (bits - 1). */
+NxrtStatus nxrt_rocm_matmul_nbits_dequantize_bits(NxrtRocmEp* ep, const void* b_device, const void* scales_device, uint32_t scale_dtype,
+                                                  const void* zero_points_device, uint64_t n, uint64_t k, uint32_t block_size, uint32_t bits,
+                                                  float* out_nk_device);
 /* accuracy_level=4 activation quantizer (simd_quant.rs:131-143 / sqnbitgemm_kernel_avx512.cpp:349-426).
  * rounding: 0 = ties to even (MLAS), 1 = ties away from zero (native). qa: int8 [M, kb*bs];
  * qscale: f32 [M, kb]. */

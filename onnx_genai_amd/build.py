@@ -16,6 +16,7 @@ HIP_SOURCES = [
     "hip_ffi.hip",
     "kernels/dequant.hip",
     "kernels/gemv_generic.hip",
+    "kernels/gemv_nbits.hip",
     "kernels/gemv_f32.hip",
     "kernels/decode_mfma.hip",
     "kernels/decode_packed.hip",

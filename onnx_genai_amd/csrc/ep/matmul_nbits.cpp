@@ -96,11 +96,18 @@ void check_attrs(const NxrtRocmMatMulNBitsAttrs& a, Check& c)
     required_positive(kAttrN, "N", a.N);
     if (c.failed) return;
     const int64_t bits = (a.present & (1u << kAttrBits)) ? a.bits : 4;
-    if (bits != 4) {
+    if (bits != 2 && bits != 4 && bits != 8) {                     // the widths the CPU provider takes (matmul_nbits.rs:1424-1431)
         c.failed = true;
-        c.message = "MatMulNBits ROCm supports bits=4, got bits=" + std::to_string(bits) +
-                    ". Why: only the 4-bit packed layout has a validated gfx950 kernel. How to fix: export bits=4, "
+        c.message = "MatMulNBits ROCm supports bits in {2, 4, 8}, got bits=" + std::to_string(bits) +
+                    ". Why: only these packed layouts have gfx950 kernels. How to fix: export bits=4 (the tuned path), 2 or 8, "
                     "or select the CPU execution provider for this node";
+        return;
+    }
+    const int64_t accuracy = (a.present & (1u << kAttrAccuracy)) ? a.accuracy_level : 0;
+    if (bits != 4 && accuracy == 4) {
+        c.failed = true;
+        c.message = "MatMulNBits ROCm: accuracy_level=4 is implemented for bits=4 only, got bits=" + std::to_string(bits) +
+                    ". How to fix: use accuracy_level=0 with this bit width, or run this node on the CPU execution provider";
         return;
     }
     const int64_t prepacked = (a.present & (1u << kAttrPrepacked)) ? a.weight_prepacked : 0;
@@ -119,6 +126,7 @@ void check_attrs(const NxrtRocmMatMulNBitsAttrs& a, Check& c)
 struct NxrtRocmMatMulNBits {
     NxrtRocmEp* ep = nullptr;
     int64_t k = 0, n = 0, block_size = 0, accuracy_level = 0;
+    int64_t bits = 4;                    // 2 and 8 run on the plain kernels (and the dense route), 4 on everything
     int64_t rows_hint = -1;              // M when the create-time shape of A was static
     bool bias_post_round = false;        // the bias is a folded Add: round(round(acc) + bias) on 16-bit outputs
     // The fused gate/up node: two ordinary kernels (each with its own repacked copy, scratch and variant) whose 16-bit
@@ -239,7 +247,9 @@ bool dense_route(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& args, int& 
 {
     rc = 0;
     NxrtRocmEp& ep = *kn.ep;
-    if (ep.dense_gemm_min_rows <= 0 || args.m < ep.dense_gemm_min_rows) return false;
+    // other bit widths have no tiled kernel to fall back on, only the plain GEMV: the route pays from a few dozen rows
+    const int64_t min_rows = kn.bits == 4 ? ep.dense_gemm_min_rows : (ep.dense_gemm_min_rows < 32 ? ep.dense_gemm_min_rows : 32);
+    if (ep.dense_gemm_min_rows <= 0 || args.m < min_rows) return false;
     if ((args.a_dtype != ROCM_DT_F16 && args.a_dtype != ROCM_DT_BF16) || args.y_dtype != args.a_dtype || (args.k & 7) != 0) return false;
     if ((reinterpret_cast<uintptr_t>(args.a) & 15) != 0 || (reinterpret_cast<uintptr_t>(args.y) & 15) != 0 || (reinterpret_cast<uintptr_t>(args.b) & 3) != 0) return false;
     const uint64_t need = static_cast<uint64_t>(args.n) * static_cast<uint64_t>(args.k) * 2;
@@ -257,6 +267,11 @@ bool dense_route(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& args, int& 
     if (!rocm_dense_gemm_ready(ep.dense, args.m, args.n, args.k, args.a_dtype, bias_dtype, ep.capturing ? 0 : 1)) return false;
 
     const bool constant = kn.constant_inputs[1] && kn.constant_inputs[2] && (!args.zp || kn.constant_inputs[3]);
+    auto expand = [&](void* dst) {
+        if (kn.bits == 4) return rocm_launch_dequant_16(args.b, args.scales, args.scale_dtype, args.zp, args.n, args.k, args.block_size, args.a_dtype, dst, ep.stream);
+        return rocm_launch_dequant_nbits(args.b, args.scales, args.scale_dtype, args.zp, args.n, args.k, args.block_size, static_cast<int>(kn.bits), args.a_dtype,
+                                         dst, ep.stream);
+    };
     const void* w16 = nullptr;
     if (ep.dense_resident && constant) {
         const bool current = kn.dense && kn.dense_from[0] == args.b && kn.dense_from[1] == args.scales && kn.dense_from[2] == args.zp &&
@@ -272,7 +287,7 @@ bool dense_route(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& args, int& 
                 kn.dense = nullptr;
                 return false;                   // no memory for a dense copy: the tiled kernel reads the packed weights
             }
-            rc = rocm_launch_dequant_16(args.b, args.scales, args.scale_dtype, args.zp, args.n, args.k, args.block_size, args.a_dtype, kn.dense, ep.stream);
+            rc = expand(kn.dense);
             kn.dense_from[0] = args.b;
             kn.dense_from[1] = args.scales;
             kn.dense_from[2] = args.zp;
@@ -286,7 +301,7 @@ bool dense_route(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& args, int& 
             if (ep.capturing) return false;
             if (grow_buffer(ep.dense_scratch, ep.dense_scratch_bytes, need, ep.dense_retired) != 0) return false;
         }
-        rc = rocm_launch_dequant_16(args.b, args.scales, args.scale_dtype, args.zp, args.n, args.k, args.block_size, args.a_dtype, ep.dense_scratch, ep.stream);
+        rc = expand(ep.dense_scratch);
         w16 = ep.dense_scratch;
         kn.variant = "dense_transient_blaslt";
     }
@@ -385,12 +400,13 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
         return make_status(NXRT_INVALID_ARGUMENT, err("Y must have shape " + shape_str(y_shape) + ", got " + shape_str(Y.shape, Y.ndim)));
 
     const uint64_t kb = (K + BS - 1) / BS;
-    const uint64_t blob = BS / 2;
+    const uint64_t bits = static_cast<uint64_t>(kn.bits);
+    const uint64_t blob = BS * bits / 8;
     flat_or_matrix("scales", S, N, kb);
     const NxrtRocmTensorView* ZP = optional(3);
     if (ZP && !c.failed) {
         require_dtype("zero_points", ZP->dtype, NXRT_DT_UINT8);
-        if (!c.failed) flat_or_matrix("zero_points", *ZP, N, (kb + 1) / 2);
+        if (!c.failed) flat_or_matrix("zero_points", *ZP, N, (kb * bits + 7) / 8);
     }
     const NxrtRocmTensorView* G = optional(4);
     if (G && !c.failed) {
@@ -447,6 +463,15 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
 
     rocm_stream_t stream = kn.ep->stream;
     int rc = 0;
+    if (kn.bits != 4) {
+        // 2 and 8 bits: tall 16-bit calls expand the weights and run the library GEMM, everything else the plain f32 GEMV
+        if (!dense_route(kn, args, rc)) {
+            rc = rocm_launch_gemv_nbits(&args, static_cast<int>(kn.bits), stream);
+            kn.variant = "gemv_nbits_f32";
+        }
+        kn.ep->launches.fetch_add(1);
+        return hip_status(rc, "MatMulNBits: kernel launch");
+    }
     if (kn.accuracy_level == 4) {
         const int rounding = kn.ep->acc4_rounding == 2 ? (static_cast<int64_t>(M) < static_cast<int64_t>(kn.ep->acc4_native_below) ? 1 : 0) : kn.ep->acc4_rounding;   // matmul_nbits.rs:640-660
         int pack_rc = 0;
@@ -710,8 +735,8 @@ NxrtStatus vtable_execute(void* ctx, const void* const* inputs, uint32_t n_in, v
         if (kn->rows_hint < 0)
             return make_status(NXRT_INVALID_ARGUMENT, err("the kernel vtable carries no shapes; create the kernel with a static shape for A"));
         const uint64_t K = kn->k, N = kn->n, BS = kn->block_size, kb = (K + BS - 1) / BS;
-        const uint64_t a_shape[2] = {static_cast<uint64_t>(kn->rows_hint), K}, b_shape[3] = {N, kb, BS / 2}, s_shape[2] = {N, kb},
-                       z_shape[2] = {N, (kb + 1) / 2}, bias_shape[1] = {N}, y_shape[2] = {static_cast<uint64_t>(kn->rows_hint), N};
+        const uint64_t a_shape[2] = {static_cast<uint64_t>(kn->rows_hint), K}, b_shape[3] = {N, kb, BS * static_cast<uint64_t>(kn->bits) / 8},
+                       s_shape[2] = {N, kb}, z_shape[2] = {N, (kb * static_cast<uint64_t>(kn->bits) + 7) / 8}, bias_shape[1] = {N}, y_shape[2] = {static_cast<uint64_t>(kn->rows_hint), N};
         NxrtRocmTensorView in[6];
         std::memset(in, 0, sizeof(in));
         auto set = [&](NxrtRocmTensorView& v, const void* p, uint32_t dt, uint32_t nd, const uint64_t* sh) {
@@ -809,6 +834,7 @@ NxrtStatus nxrt_rocm_matmul_nbits_create(NxrtRocmEp* ep, const NxrtRocmMatMulNBi
         kn->n = attrs->N;
         kn->block_size = attrs->block_size;
         kn->accuracy_level = (attrs->present & (1u << kAttrAccuracy)) ? attrs->accuracy_level : 0;
+        kn->bits = (attrs->present & (1u << kAttrBits)) ? attrs->bits : 4;
         const bool has_folded_bias = attrs->struct_size >= offsetof(NxrtRocmMatMulNBitsAttrs, folded_bias) + sizeof(int64_t);
         kn->bias_post_round = has_folded_bias && (attrs->present & (1u << kAttrFoldedBias)) && attrs->folded_bias == 1;
         // flops::leading_rows: product of A's leading dims when all are static
@@ -838,6 +864,7 @@ NxrtStatus nxrt_rocm_matmul_nbits_create(NxrtRocmEp* ep, const NxrtRocmMatMulNBi
                 c2->n = kn->n;
                 c2->block_size = kn->block_size;
                 c2->accuracy_level = kn->accuracy_level;
+                c2->bits = kn->bits;
                 c2->rows_hint = kn->rows_hint;
                 c2->pair_member = true;
                 *child = c2;
@@ -955,6 +982,25 @@ NxrtStatus nxrt_rocm_matmul_nbits_dequantize(NxrtRocmEp* ep, const void* b, cons
         ep->launches.fetch_add(1);
         return hip_status(rocm_launch_dequant_f32(static_cast<const uint8_t*>(b), scales, static_cast<int>(scale_dtype), static_cast<const uint8_t*>(zp),
                                                   static_cast<int64_t>(n), static_cast<int64_t>(k), static_cast<int>(block_size), out_nk, ep->stream),
+                          "MatMulNBits dequantize launch");
+    });
+}
+
+NxrtStatus nxrt_rocm_matmul_nbits_dequantize_bits(NxrtRocmEp* ep, const void* b, const void* scales, uint32_t scale_dtype, const void* zp, uint64_t n,
+                                                  uint64_t k, uint32_t block_size, uint32_t bits, float* out_nk)
+{
+    if (bits == 4) return nxrt_rocm_matmul_nbits_dequantize(ep, b, scales, scale_dtype, zp, n, k, block_size, out_nk);
+    return fenced([&]() -> NxrtStatus {
+        if (!ep || !b || !scales || !out_nk) return make_status(NXRT_INVALID_ARGUMENT, "MatMulNBits dequantize: null pointer");
+        if (bits != 2 && bits != 8) return make_status(NXRT_INVALID_ARGUMENT, err("bits must be 2, 4 or 8, got " + std::to_string(bits)));
+        if (!is_float_compute(scale_dtype)) return make_status(NXRT_INVALID_ARGUMENT, err(std::string("scales must have dtype Float32, Float16, or BFloat16, got ") + dtype_name(scale_dtype)));
+        if (block_size < 16 || (block_size & (block_size - 1)) != 0) return make_status(NXRT_INVALID_ARGUMENT, err("block_size must be a power of two and at least 16, got " + std::to_string(block_size)));
+        NxrtStatus st = ep->bind();
+        if (st.code != NXRT_OK) return st;
+        ep->launches.fetch_add(1);
+        return hip_status(rocm_launch_dequant_nbits(static_cast<const uint8_t*>(b), scales, static_cast<int>(scale_dtype), static_cast<const uint8_t*>(zp),
+                                                    static_cast<int64_t>(n), static_cast<int64_t>(k), static_cast<int>(block_size), static_cast<int>(bits),
+                                                    ROCM_DT_F32, out_nk, ep->stream),
                           "MatMulNBits dequantize launch");
     });
 }

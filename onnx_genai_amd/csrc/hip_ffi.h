@@ -91,6 +91,13 @@ int rocm_launch_swiglu(const void* gate, const void* up, int64_t count, int dtyp
 int rocm_launch_rmsnorm16(const void* a, const void* gamma, int gamma_dtype, int64_t rows, int64_t k, float epsilon, int dtype, void* out,
                           rocm_stream_t stream);
 
+/* bits = 2 or 8 (element i of a packed row in byte i / (8 / bits) at bit (i % (8 / bits)) * bits; zero points packed alike,
+ * default 1 << (bits - 1)): w[n,k] = (q - zp) * scale as f32, f16 or bf16 [N, K] (one f32 multiply, then one rounding), and
+ * the f32 GEMV with one wave per output column (args as for 4 bits, b / zp in the wider or narrower layout). */
+int rocm_launch_dequant_nbits(const uint8_t* b, const void* scales, int scale_dtype, const uint8_t* zp, int64_t n, int64_t k, int block_size,
+                              int bits, int out_dtype, void* out_nk, rocm_stream_t stream);
+int rocm_launch_gemv_nbits(const RocmMatMulNBitsArgs* args, int bits, rocm_stream_t stream);
+
 /* Any dtype mix, any K, any block size: f32 math, one wave per output column. */
 int rocm_launch_gemv_generic(const RocmMatMulNBitsArgs* args, rocm_stream_t stream);
 /* f32 activations, M <= 4, block size >= 32, K % 4 == 0, A and B 16-byte aligned: f32 FMA streaming kernel */

@@ -121,6 +121,8 @@ def load_library() -> C.CDLL:
     L.nxrt_rocm_matmul_nbits_as_vtable.argtypes = [v, C.POINTER(v)]
     L.nxrt_rocm_matmul_nbits_dequantize.restype = S
     L.nxrt_rocm_matmul_nbits_dequantize.argtypes = [v, v, v, u32, v, u64, u64, u32, v]
+    L.nxrt_rocm_matmul_nbits_dequantize_bits.restype = S
+    L.nxrt_rocm_matmul_nbits_dequantize_bits.argtypes = [v, v, v, u32, v, u64, u64, u32, u32, v]
     L.nxrt_rocm_matmul_nbits_quantize_a.restype = S
     L.nxrt_rocm_matmul_nbits_quantize_a.argtypes = [v, v, u32, u64, u64, u32, u32, v, v]
     L.nxrt_rocm_matmul_nbits_block_acc.restype = S
@@ -309,8 +311,11 @@ class RocmExecutionProvider:
         return MatMulNBitsKernel(self, attrs, input_shapes)
 
     # -- pieces -----------------------------------------------------------------------------------
-    def dequantize(self, b: DeviceBuffer, scales: DeviceBuffer, scale_dtype: int, zp: DeviceBuffer | None, n, k, bs, out: DeviceBuffer) -> None:
-        self.lib.nxrt_rocm_matmul_nbits_dequantize(self.handle, b.ptr, scales.ptr, scale_dtype, zp.ptr if zp else None, n, k, bs, out.ptr).check()
+    def dequantize(self, b: DeviceBuffer, scales: DeviceBuffer, scale_dtype: int, zp: DeviceBuffer | None, n, k, bs, out: DeviceBuffer, bits: int = 4) -> None:
+        if bits == 4:
+            self.lib.nxrt_rocm_matmul_nbits_dequantize(self.handle, b.ptr, scales.ptr, scale_dtype, zp.ptr if zp else None, n, k, bs, out.ptr).check()
+        else:
+            self.lib.nxrt_rocm_matmul_nbits_dequantize_bits(self.handle, b.ptr, scales.ptr, scale_dtype, zp.ptr if zp else None, n, k, bs, bits, out.ptr).check()
 
     def quantize_a(self, a: DeviceBuffer, a_dtype: int, m, k, bs, rounding: int, qa: DeviceBuffer, qscale: DeviceBuffer) -> None:
         self.lib.nxrt_rocm_matmul_nbits_quantize_a(self.handle, a.ptr, a_dtype, m, k, bs, rounding, qa.ptr, qscale.ptr).check()
@@ -450,8 +455,8 @@ class DeviceOperands:
     """The device-resident operands of one MatMulNBits node plus its kernel; what a session would hold."""
 
     def __init__(self, ep, b, scales, scale_dtype, zp, n, k, bs, *, accuracy_level=0, bias=None, bias_dtype=F32, rows=None, a_dtype=None,
-                 folded_bias=None, gamma=None, gamma_dtype=F32, rmsnorm_epsilon=None):
-        self.ep, self.n, self.k, self.bs = ep, n, k, bs
+                 folded_bias=None, gamma=None, gamma_dtype=F32, rmsnorm_epsilon=None, bits=4):
+        self.ep, self.n, self.k, self.bs, self.bits = ep, n, k, bs, bits
         self.kb = -(-k // bs)
         self.scale_dtype, self.bias_dtype = scale_dtype, bias_dtype
         self.b = ep.upload(np.asarray(b, np.uint8))
@@ -462,18 +467,18 @@ class DeviceOperands:
         self.gamma_dtype = gamma_dtype
         shapes = None
         if rows is not None and a_dtype is not None:
-            shapes = [((rows, k), a_dtype), ((n, self.kb, bs // 2), U8), ((n, self.kb), scale_dtype)]
-        self.kernel = ep.get_kernel({"K": k, "N": n, "bits": 4, "block_size": bs, "accuracy_level": accuracy_level, "folded_bias": folded_bias,
+            shapes = [((rows, k), a_dtype), ((n, self.kb, bs * bits // 8), U8), ((n, self.kb), scale_dtype)]
+        self.kernel = ep.get_kernel({"K": k, "N": n, "bits": bits, "block_size": bs, "accuracy_level": accuracy_level, "folded_bias": folded_bias,
                                      "rmsnorm_prologue": 1 if gamma is not None else None, "rmsnorm_epsilon": rmsnorm_epsilon}, shapes)
         self.kernel.set_constant_inputs([False, True, True, True, True, True, True])
 
     def views(self, a_buf: DeviceBuffer, a_dtype: int, m: int):
         dev = self.ep.device_index
         ins = [TensorView(a_buf.ptr, a_dtype, (m, self.k), device_index=dev),
-               TensorView(self.b.ptr, U8, (self.n, self.kb, self.bs // 2), device_index=dev),
+               TensorView(self.b.ptr, U8, (self.n, self.kb, self.bs * self.bits // 8), device_index=dev),
                TensorView(self.scales.ptr, self.scale_dtype, (self.n, self.kb), device_index=dev)]
         if self.zp is not None or self.bias is not None or self.gamma is not None:
-            ins.append(TensorView(self.zp.ptr, U8, (self.n, (self.kb + 1) // 2), device_index=dev) if self.zp is not None else TensorView.absent(U8))
+            ins.append(TensorView(self.zp.ptr, U8, (self.n, (self.kb * self.bits + 7) // 8), device_index=dev) if self.zp is not None else TensorView.absent(U8))
         if self.bias is not None or self.gamma is not None:
             ins.append(TensorView.absent(I32))
             ins.append(TensorView(self.bias.ptr, self.bias_dtype, (self.n,), device_index=dev) if self.bias is not None else TensorView.absent(F32))
@@ -494,13 +499,13 @@ class DeviceOperands:
 
 
 def matmul_nbits(ep, a, a_dtype, b, scales, scale_dtype, zp, n, k, bs, *, accuracy_level=0, bias=None, bias_dtype=F32, y_dtype=None, folded_bias=None,
-                 gamma=None, gamma_dtype=F32, rmsnorm_epsilon=None):
+                 gamma=None, gamma_dtype=F32, rmsnorm_epsilon=None, bits=4):
     """One-shot helper: upload, execute through the C ABI, download. Returns (Y as numpy, variant name)."""
     y_dtype = a_dtype if y_dtype is None else y_dtype
     a = np.ascontiguousarray(a)
     m = a.size // k
     ops = DeviceOperands(ep, b, scales, scale_dtype, zp, n, k, bs, accuracy_level=accuracy_level, bias=bias, bias_dtype=bias_dtype, folded_bias=folded_bias,
-                         gamma=gamma, gamma_dtype=gamma_dtype, rmsnorm_epsilon=rmsnorm_epsilon)
+                         gamma=gamma, gamma_dtype=gamma_dtype, rmsnorm_epsilon=rmsnorm_epsilon, bits=bits)
     a_buf = ep.upload(a)
     y_buf = ep.allocate(max(m * n * _ITEM[y_dtype], 1))
     try:

@@ -73,6 +73,16 @@ def make_weights(n, k, bs, seed, *, zero_points: bool, scale_lo: float, scale_hi
     return b, scales, zp
 
 
+def make_weights_bits(n, k, bs, bits, seed, *, zero_points: bool, scale_lo: float, scale_hi: float, scale_dtype: int):
+    """The same for 2- or 8-bit weights: random bytes are uniform fields of any width; zero points packed alike."""
+    rng = np.random.default_rng(seed)
+    kb = -(-k // bs)
+    b = rng.integers(0, 256, size=(n, kb, bs * bits // 8), dtype=np.uint8)
+    scales = to_dtype(rng.uniform(scale_lo, scale_hi, size=(n, kb)).astype(np.float32), scale_dtype)
+    zp = rng.integers(0, 256, size=(n, -(-kb * bits // 8)), dtype=np.uint8) if zero_points else None
+    return b, scales, zp
+
+
 def make_activation(m, k, seed, dtype: int, dist: str = "normal"):
     rng = np.random.default_rng(seed + 7919)
     a = rng.standard_normal((m, k)).astype(np.float32) if dist == "normal" else rng.uniform(-1, 1, (m, k)).astype(np.float32)

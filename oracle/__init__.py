@@ -85,6 +85,8 @@ class Port:
         L.mnb_swiglu_silu_decomposed.argtypes = [C.c_float, C.c_int]
         L.mnb_swiglu.argtypes = [v, v, z, C.c_int, C.c_int, v]
         L.mnb_rmsnorm16.argtypes = [v, v, C.c_int, z, z, C.c_float, C.c_int, v]
+        L.mnb_dequantize_nk_bits.argtypes = [v, v, v, z, z, z, C.c_int, v]
+        L.mnb_matmul_f64_bits.argtypes = [v, v, v, v, v, z, z, z, z, C.c_int, v]
         L.mnb_matmul_nbits.restype = C.c_int
         L.mnb_matmul_nbits.argtypes = [v, C.c_int, v, v, C.c_int, v, v, C.c_int, v, C.c_int, z, z, z, z, C.c_int, C.c_int]
 
@@ -108,6 +110,20 @@ class Port:
         out = np.empty(gate16.shape, _NP_DT[code])
         self.lib.mnb_swiglu(_ptr(gate16), _ptr(up16), gate16.size, code, int(decomposed), _ptr(out))
         return out
+
+    # -- bits 2 / 4 / 8 ---------------------------------------------------------------------------
+    def dequantize_nk_bits(self, b, scales, zp, n, k, bs, bits) -> np.ndarray:
+        b, scales, zp = _c(b, np.uint8), _c(scales, np.float32), _c(zp, np.uint8)
+        out = np.empty((n, k), np.float32)
+        self.lib.mnb_dequantize_nk_bits(_ptr(b), _ptr(scales), _ptr(zp), n, k, bs, bits, _ptr(out))
+        return out
+
+    def matmul_f64_bits(self, a, b, scales, zp, n, k, bs, bits, bias=None) -> np.ndarray:
+        a, b, scales, zp, bias = _c(a, np.float32), _c(b, np.uint8), _c(scales, np.float32), _c(zp, np.uint8), _c(bias, np.float32)
+        m = a.size // k
+        y = np.empty((m, n), np.float64)
+        self.lib.mnb_matmul_f64_bits(_ptr(a), _ptr(b), _ptr(scales), _ptr(zp), _ptr(bias), m, n, k, bs, bits, _ptr(y))
+        return y
 
     def rmsnorm16(self, a16: np.ndarray, gamma: np.ndarray, gamma_code: int, epsilon: float, code: int) -> np.ndarray:
         """The RMS-normalization prologue on 16-bit rows [rows, K] (K % 128 == 0); gamma 16-bit of the same type or f32."""

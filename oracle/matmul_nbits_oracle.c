@@ -360,3 +360,49 @@ void mnb_rmsnorm16(const void* a, const void* gamma, int gamma_dtype, size_t row
         }
     }
 }
+
+
+/* ---- bits 2 / 4 / 8: NBitsLayout, matmul_nbits.rs:1276-1321, 1360-1363 ---------------------------- */
+
+uint8_t mnb_unpack_bits(const uint8_t* packed, size_t index, int bits)
+{
+    const size_t per_byte = 8 / (size_t)bits;
+    const uint8_t mask = bits == 8 ? 0xff : (uint8_t)((1u << bits) - 1);
+    return (uint8_t)((packed[index / per_byte] >> ((index % per_byte) * (size_t)bits)) & mask);
+}
+
+void mnb_dequantize_nk_bits(const uint8_t* b, const float* scales, const uint8_t* zp, size_t n, size_t k, size_t block_size, int bits,
+                            float* out_nk)
+{
+    const size_t kb = div_ceil(k, block_size), blob = block_size * (size_t)bits / 8, zp_row = div_ceil(kb * (size_t)bits, 8);
+    for (size_t col = 0; col < n; ++col) {
+        const uint8_t* row = b + col * kb * blob;
+        for (size_t depth = 0; depth < k; ++depth) {
+            const size_t block = depth / block_size;
+            const uint8_t q = mnb_unpack_bits(row + block * blob, depth % block_size, bits);
+            const uint8_t z = zp ? mnb_unpack_bits(zp + col * zp_row, block, bits) : (uint8_t)(1u << (bits - 1));
+            out_nk[col * k + depth] = ((float)q - (float)z) * scales[col * kb + block];
+        }
+    }
+}
+
+void mnb_matmul_f64_bits(const float* a, const uint8_t* b, const float* scales, const uint8_t* zp, const float* bias,
+                         size_t m, size_t n, size_t k, size_t block_size, int bits, double* y)
+{
+    const size_t kb = div_ceil(k, block_size), blob = block_size * (size_t)bits / 8, zp_row = div_ceil(kb * (size_t)bits, 8);
+    for (size_t row = 0; row < m; ++row)
+        for (size_t col = 0; col < n; ++col) {
+            double acc = 0.0;
+            for (size_t block = 0; block < kb; ++block) {
+                const double scale = (double)scales[col * kb + block];
+                const double z = zp ? (double)mnb_unpack_bits(zp + col * zp_row, block, bits) : (double)(1u << (bits - 1));
+                const uint8_t* blk = b + (col * kb + block) * blob;
+                for (size_t off = 0; off < block_size; ++off) {
+                    const size_t depth = block * block_size + off;
+                    if (depth >= k) break;
+                    acc += ((double)mnb_unpack_bits(blk, off, bits) - z) * scale * (double)a[row * k + depth];
+                }
+            }
+            y[row * n + col] = acc + (bias ? (double)bias[col] : 0.0);
+        }
+}

@@ -43,6 +43,16 @@ uint8_t mnb_zero_point(const uint8_t* zp_row, size_t block);
 void mnb_dequantize_nk(const uint8_t* b, const float* scales, const uint8_t* zp,
                        size_t n, size_t k, size_t block_size, float* out_nk);
 
+/* The same definition at the other bit widths the CPU provider takes (NBitsLayout, matmul_nbits.rs:1276-1321; bits 2, 4, 8):
+ * element i of a packed row sits in byte i / (8 / bits), at bit (i % (8 / bits)) * bits; zero points are packed the same
+ * way, ceil(kb * bits / 8) bytes per column, default 1 << (bits - 1); a block is block_size * bits / 8 bytes. */
+uint8_t mnb_unpack_bits(const uint8_t* packed, size_t index, int bits);
+void mnb_dequantize_nk_bits(const uint8_t* b, const float* scales, const uint8_t* zp, size_t n, size_t k, size_t block_size, int bits,
+                            float* out_nk);
+/* int4_f64_reference (matmul_nbits.rs:10890-10933) over that layout: f64 accumulation, bias added in f64. */
+void mnb_matmul_f64_bits(const float* a, const uint8_t* b, const float* scales, const uint8_t* zp, const float* bias,
+                         size_t m, size_t n, size_t k, size_t block_size, int bits, double* y);
+
 /* matmul_nbits.rs:12205-12230 (test `reference`) and mlas-sys/src/lib.rs:2997-3015 (ref_gemm_nk):
  * y[m,n] = bias[n] + sum_k a[m,k] * w[n,k], f32, k ascending. */
 void mnb_matmul_dequant_f32(const float* a, const float* w_nk, const float* bias,

@@ -190,8 +190,9 @@ def test_attribute_validation_messages(lib):
         (dict(K=64, N=8, block_size=48), "MatMulNBits: block_size must be a power of two and at least 16, got 48"),
         (dict(K=64, N=8, block_size=32, weight_prepacked=2), "weight_prepacked must be 0 (standard ONNX layout) or 1 (MLAS SQNBit packed layout), got 2"),
         (dict(K=64, N=8, block_size=32, weight_prepacked=1), "weight_prepacked=1 holds the MLAS SQNBit CPU layout"),
-        (dict(K=64, N=8, block_size=32, bits=8), "MatMulNBits ROCm supports bits=4, got bits=8"),
-        (dict(K=64, N=8, block_size=32, bits=3), "MatMulNBits ROCm supports bits=4, got bits=3"),
+        (dict(K=64, N=8, block_size=32, bits=3), "MatMulNBits ROCm supports bits in {2, 4, 8}, got bits=3"),
+        (dict(K=64, N=8, block_size=32, bits=16), "MatMulNBits ROCm supports bits in {2, 4, 8}, got bits=16"),
+        (dict(K=64, N=8, block_size=32, bits=8, accuracy_level=4), "accuracy_level=4 is implemented for bits=4 only, got bits=8"),
     ]
     for attrs, text in cases:
         st, h = create_status(lib, **attrs)
@@ -202,8 +203,10 @@ def test_attribute_validation_messages(lib):
 
 def test_supports_op_declines_with_reasons(lib):
     reason = C.create_string_buffer(512)
-    a = E.make_attrs(K=64, N=8, bits=2, block_size=32)
+    a = E.make_attrs(K=64, N=8, bits=3, block_size=32)
     assert lib.nxrt_rocm_ep_supports_matmul_nbits(None, C.byref(a), None, 0, reason, 512) == 0 and b"How to fix" in reason.value
+    a = E.make_attrs(K=64, N=8, bits=8, block_size=32)
+    assert lib.nxrt_rocm_ep_supports_matmul_nbits(None, C.byref(a), None, 0, reason, 512) == 1 and reason.value == b""
     a = E.make_attrs(K=64, N=8, bits=4, block_size=32)
     assert lib.nxrt_rocm_ep_supports_matmul_nbits(None, C.byref(a), None, 0, reason, 512) == 1 and reason.value == b""
     descs, keep = E.make_descs([((1, 64), E.F16), ((8, 2, 16), E.U8), ((8, 2), E.F16), (None, 0), ((64,), E.I32)])

@@ -291,3 +291,39 @@ def test_rmsnorm_closed_forms_and_double_precision(port):
     # a zero row stays zero; gamma of the activations' own 16-bit type is read as such
     z = port.rmsnorm16(np.zeros((1, k), np.float16), np.ones(k, np.float16), oracle.F16, 1e-5, oracle.F16)
     assert not z.view(np.uint16).any()
+
+
+# ---------------------------------------------------------------------------------------------
+# bits 2 and 8 (NBitsLayout, onnx-runtime-ep-cpu/src/kernels/matmul_nbits.rs:1276-1321)
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("bits", [2, 4, 8])
+@pytest.mark.parametrize("zero_points", [False, True])
+def test_nbits_layout_against_numpy_unpacking(port, bits, zero_points):
+    """The bit-width-generic restatement against an independent unpacking with numpy (unpackbits on little-endian bit
+    order), at 4 bits also against the 4-bit functions the compiled MLAS pins; default zero point 1 << (bits - 1)."""
+    rng = np.random.default_rng(bits)
+    n, k, bs = 7, 200, 32
+    kb = -(-k // bs)
+    b = rng.integers(0, 256, size=(n, kb, bs * bits // 8), dtype=np.uint8)
+    scales = rng.uniform(0.01, 0.1, size=(n, kb)).astype(np.float32)
+    zp = rng.integers(0, 256, size=(n, -(-kb * bits // 8)), dtype=np.uint8) if zero_points else None
+    fields = np.unpackbits(b.reshape(n, -1), axis=1, bitorder="little").reshape(n, -1, bits)
+    q = (fields * (1 << np.arange(bits))).sum(axis=2)[:, :kb * bs].reshape(n, kb, bs)
+    if zero_points:
+        zf = np.unpackbits(zp, axis=1, bitorder="little").reshape(n, -1, bits)
+        z = (zf * (1 << np.arange(bits))).sum(axis=2)[:, :kb]
+    else:
+        z = np.full((n, kb), 1 << (bits - 1))
+    want = ((q.astype(np.float32) - z[:, :, None].astype(np.float32)) * scales[:, :, None]).reshape(n, kb * bs)[:, :k]
+    got = port.dequantize_nk_bits(b, scales, zp, n, k, bs, bits)
+    assert np.array_equal(got, want)
+    a = rng.standard_normal((3, k)).astype(np.float32)
+    y = port.matmul_f64_bits(a, b, scales, zp, n, k, bs, bits)
+    exact = ((q.astype(np.float64) - z[:, :, None]) * scales.astype(np.float64)[:, :, None]).reshape(n, kb * bs)[:, :k]       # no f32 rounding
+    assert np.allclose(y, a.astype(np.float64) @ exact.T, rtol=1e-12, atol=1e-12)
+    if bits == 4:
+        assert np.array_equal(got, port.dequantize_nk(b, scales, zp, n, k, bs))
+    # known answer: byte 0xe4 holds 2-bit fields 0,1,2,3 from the low end; as one 8-bit field it is 228
+    one = np.array([[[0xe4] * (16 * bits // 8)]], np.uint8)
+    w = port.dequantize_nk_bits(one, np.ones((1, 1), np.float32), None, 1, 16, 16, bits)[0]
+    assert list(w[:4]) == {2: [-2.0, -1.0, 0.0, 1.0], 4: [-4.0, 6.0, -4.0, 6.0], 8: [100.0] * 4}[bits]

@@ -555,6 +555,75 @@ def test_folded_bias_keeps_tall_calls_off_the_library_gemm(ep):
 
 
 # ---------------------------------------------------------------------------------------------
+# bits = 2 and 8: the CPU provider's other widths, on the plain kernels and the dense route
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("bits", [2, 8])
+@pytest.mark.parametrize("bs,zero_points,s_dt", [(16, True, E.F32), (32, False, E.F16), (128, True, E.BF16)])
+def test_dequantize_bits_bit_exact(ep, port, bits, bs, zero_points, s_dt):
+    n, k = 37, 5 * bs - 8
+    b, s, zp = synth.make_weights_bits(n, k, bs, bits, 40 + bits, zero_points=zero_points, scale_lo=0.001, scale_hi=0.05, scale_dtype=s_dt)
+    bb, sb, zb, ob = ep.upload(b), ep.upload(s), ep.upload(zp) if zp is not None else None, ep.allocate(n * k * 4)
+    try:
+        ep.dequantize(bb, sb, s_dt, zb, n, k, bs, ob, bits=bits)
+        got = ep.download(ob, (n, k), np.float32)
+        assert np.array_equal(got, port.dequantize_nk_bits(b, synth.to_f32(s, s_dt), zp, n, k, bs, bits))
+    finally:
+        for buf in (bb, sb, zb, ob):
+            if buf is not None:
+                ep.deallocate(buf)
+
+
+NBITS_CASES = [
+    # a_dt, s_dt, bs, zp, m, n, k
+    (E.F32, E.F32, 32, True, 1, 300, 896),
+    (E.F16, E.F16, 32, False, 1, 130, 1024),
+    (E.BF16, E.BF16, 128, True, 5, 200, 3584),
+    (E.F16, E.F32, 16, True, 13, 64, 200),        # K ends inside a block
+    (E.F16, E.F16, 64, True, 40, 136, 512),       # tall enough for the dense route at these widths
+    (E.BF16, E.BF16, 128, True, 300, 256, 1024),
+    (E.F32, E.F16, 64, True, 20, 72, 256),        # f32 activations stay on the plain kernel at any height
+    (E.BF16, E.BF16, 128, True, 1, 1030, 3584),   # 8 bits: the 16-byte-load GEMV (one row), ragged column count
+    (E.F16, E.F16, 16, False, 4, 70, 1040),       # 8 bits: four rows, a K that leaves the last step half empty
+    (E.F16, E.F16, 32, True, 3, 40, 72),          # K % 16 != 0: the plain kernel
+]
+
+
+@pytest.mark.parametrize("bits", [2, 8])
+@pytest.mark.parametrize("a_dt,s_dt,bs,zero_points,m,n,k", NBITS_CASES)
+def test_other_bit_widths_match_oracle(ep, port, bits, a_dt, s_dt, bs, zero_points, m, n, k):
+    b, s, zp = synth.make_weights_bits(n, k, bs, bits, 50 + bits + n, zero_points=zero_points, scale_lo=0.002 if bits == 8 else 0.02,
+                                       scale_hi=0.004 if bits == 8 else 0.04, scale_dtype=s_dt)
+    a = synth.make_activation(m, k, 51 + m, a_dt)
+    bias = synth.to_dtype(np.linspace(-1, 1, n).astype(np.float32), a_dt)
+    y, variant = run_op(ep, a, a_dt, b, s, s_dt, zp, n, k, bs, bias=bias, bias_dtype=a_dt, bits=bits)
+    tall = a_dt != E.F32 and m >= 32 and k % 8 == 0
+    assert variant == ("dense_transient_blaslt" if tall else "gemv_nbits_f32")
+    want = port.matmul_f64_bits(synth.to_f32(a, a_dt), b, synth.to_f32(s, s_dt), zp, n, k, bs, bits, bias=synth.to_f32(bias, a_dt))
+    assert helpers.rel_l2(synth.to_f32(y, a_dt), want) <= (TOL_F32 if a_dt == E.F32 else TOL_HALF)
+
+
+def test_other_bit_widths_validation(ep):
+    with pytest.raises(E.EpError, match="bits in {2, 4, 8}"):
+        ep.get_kernel({"K": 64, "N": 8, "bits": 3, "block_size": 32})
+    with pytest.raises(E.EpError, match="accuracy_level=4 is implemented for bits=4 only"):
+        ep.get_kernel({"K": 64, "N": 8, "bits": 8, "block_size": 32, "accuracy_level": 4})
+    n, k, bs = 8, 64, 32
+    b4, s, _ = synth.make_weights(n, k, bs, 1, zero_points=False, scale_lo=0.01, scale_hi=0.02, scale_dtype=E.F16)
+    a = synth.make_activation(1, k, 1, E.F16)
+    ops = E.DeviceOperands(ep, b4, s, E.F16, None, n, k, bs, bits=8)       # 4-bit sized B on an 8-bit node
+    ab, yb = ep.upload(a), ep.allocate(n * 2)
+    try:
+        views = ops.views(ab, E.F16, 1)
+        views[1] = E.TensorView(ops.b.ptr, E.U8, (n, k // bs, bs // 2), device_index=ep.device_index)
+        with pytest.raises(E.EpError, match=r"B must have shape \[8, 2, 32\]"):
+            ops.kernel.execute(views, [E.TensorView(yb.ptr, E.F16, (1, n), device_index=ep.device_index)])
+    finally:
+        ep.deallocate(ab)
+        ep.deallocate(yb)
+        ops.free()
+
+
+# ---------------------------------------------------------------------------------------------
 # fused gate/up node: silu(gate) * up over both projections, rounded as the separate nodes round
 # ---------------------------------------------------------------------------------------------
 SWIGLU_CASES = [
