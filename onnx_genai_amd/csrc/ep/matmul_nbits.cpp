@@ -135,6 +135,7 @@ struct NxrtRocmMatMulNBits {
     NxrtRocmMatMulNBits* gate = nullptr;
     NxrtRocmMatMulNBits* up = nullptr;
     bool pair_member = false;            // this kernel is one projection of a fused gate/up node
+    const void* g_idx_checked = nullptr; // the g_idx tensor whose groups were found in range
     // RMS-normalization prologue: the activations are normalized into `norm` first (gamma at input 6, or 5 of the fused node)
     bool rmsnorm_prologue = false;
     float rmsnorm_epsilon = 1e-5f;
@@ -248,7 +249,8 @@ bool dense_route(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& args, int& 
     rc = 0;
     NxrtRocmEp& ep = *kn.ep;
     // other bit widths have no tiled kernel to fall back on, only the plain GEMV: the route pays from a few dozen rows
-    const int64_t min_rows = kn.bits == 4 ? ep.dense_gemm_min_rows : (ep.dense_gemm_min_rows < 32 ? ep.dense_gemm_min_rows : 32);
+    const bool plain_only = kn.bits != 4 || args.g_idx != nullptr;
+    const int64_t min_rows = !plain_only ? ep.dense_gemm_min_rows : (ep.dense_gemm_min_rows < 32 ? ep.dense_gemm_min_rows : 32);
     if (ep.dense_gemm_min_rows <= 0 || args.m < min_rows) return false;
     if ((args.a_dtype != ROCM_DT_F16 && args.a_dtype != ROCM_DT_BF16) || args.y_dtype != args.a_dtype || (args.k & 7) != 0) return false;
     if ((reinterpret_cast<uintptr_t>(args.a) & 15) != 0 || (reinterpret_cast<uintptr_t>(args.y) & 15) != 0 || (reinterpret_cast<uintptr_t>(args.b) & 3) != 0) return false;
@@ -266,8 +268,11 @@ bool dense_route(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& args, int& 
     }
     if (!rocm_dense_gemm_ready(ep.dense, args.m, args.n, args.k, args.a_dtype, bias_dtype, ep.capturing ? 0 : 1)) return false;
 
-    const bool constant = kn.constant_inputs[1] && kn.constant_inputs[2] && (!args.zp || kn.constant_inputs[3]);
+    const bool constant = kn.constant_inputs[1] && kn.constant_inputs[2] && (!args.zp || kn.constant_inputs[3]) && !args.g_idx;
     auto expand = [&](void* dst) {
+        if (args.g_idx)
+            return rocm_launch_dequant_gidx(args.b, args.scales, args.scale_dtype, args.zp, args.g_idx, args.n, args.k, args.block_size, static_cast<int>(kn.bits),
+                                            args.a_dtype, dst, ep.stream);
         if (kn.bits == 4) return rocm_launch_dequant_16(args.b, args.scales, args.scale_dtype, args.zp, args.n, args.k, args.block_size, args.a_dtype, dst, ep.stream);
         return rocm_launch_dequant_nbits(args.b, args.scales, args.scale_dtype, args.zp, args.n, args.k, args.block_size, static_cast<int>(kn.bits), args.a_dtype,
                                          dst, ep.stream);
@@ -413,9 +418,9 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
         require_dtype("g_idx", G->dtype, NXRT_DT_INT32);
         if (!c.failed && !shape_is(*G, {K}) && !shape_is(*G, {kb * BS}))
             c.fail("g_idx must have shape [" + std::to_string(K) + "] or [" + std::to_string(kb * BS) + "], got " + shape_str(G->shape, G->ndim));
-        if (!c.failed)
-            c.fail("g_idx is not supported on the ROCm execution provider. Why: its kernels stream contiguous K blocks. "
-                   "How to fix: export the weight without act-order, or run this node on the CPU execution provider");
+        if (!c.failed && kn.accuracy_level == 4)
+            c.fail("accuracy_level=4 does not take g_idx on the ROCm execution provider. Why: its int8 kernels scale whole contiguous K blocks. "
+                   "How to fix: export the weight without act-order, use accuracy_level=0, or run this node on the CPU execution provider");
     }
     if (!c.failed && !shape_is(B, {N, kb, blob}))
         c.fail("B must have shape " + shape_str({N, kb, blob}) + ", got " + shape_str(B.shape, B.ndim));
@@ -427,7 +432,7 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
     if (c.failed) return make_status(NXRT_INVALID_ARGUMENT, c.message);
 
     struct Named { const char* name; const NxrtRocmTensorView* v; };
-    const Named all[] = {{"A", &A}, {"B", &B}, {"scales", &S}, {"zero_points", ZP}, {"bias", BIAS}, {"Y", &Y}};
+    const Named all[] = {{"A", &A}, {"B", &B}, {"scales", &S}, {"zero_points", ZP}, {"g_idx", G}, {"bias", BIAS}, {"Y", &Y}};
     for (const Named& t : all) {
         if (!t.v) continue;
         if (!is_contiguous(*t.v)) return make_status(NXRT_INVALID_ARGUMENT, err(std::string(t.name) + " must be contiguous on the ROCm execution provider"));
@@ -460,11 +465,23 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
     args.n = kn.n;
     args.k = kn.k;
     args.block_size = static_cast<int>(kn.block_size);
+    args.g_idx = G ? static_cast<const int32_t*>(at(*G)) : nullptr;
 
     rocm_stream_t stream = kn.ep->stream;
     int rc = 0;
-    if (kn.bits != 4) {
-        // 2 and 8 bits: tall 16-bit calls expand the weights and run the library GEMM, everything else the plain f32 GEMV
+    if (G && kn.g_idx_checked != args.g_idx) {
+        // matmul_nbits.rs:3515-3521: every group must lie in 0..kb. Checked once per tensor (a device pass and a read-back).
+        if (kn.ep->capturing)
+            return make_status(NXRT_INVALID_ARGUMENT, err("g_idx has not been range-checked yet and a graph capture is open; run this node once eagerly first"));
+        int64_t bad = -1;
+        const int e = rocm_g_idx_first_bad(args.g_idx, static_cast<int64_t>(K), static_cast<int64_t>(kb), &bad, stream);
+        if (e != 0) return hip_status(e, "MatMulNBits: g_idx check");
+        if (bad >= 0) return make_status(NXRT_INVALID_ARGUMENT, err("g_idx[" + std::to_string(bad) + "] is outside 0.." + std::to_string(kb)));
+        kn.g_idx_checked = args.g_idx;
+    }
+    if (kn.bits != 4 || G) {
+        // 2 and 8 bits, and act-order weights of any width: tall 16-bit calls expand the weights and run the library GEMM,
+        // everything else the plain f32 GEMV
         if (!dense_route(kn, args, rc)) {
             rc = rocm_launch_gemv_nbits(&args, static_cast<int>(kn.bits), stream);
             kn.variant = "gemv_nbits_f32";
@@ -810,9 +827,10 @@ int nxrt_rocm_ep_supports_matmul_nbits(const NxrtRocmEp* ep, const NxrtRocmMatMu
         if (!is_float_compute(inputs[0].dtype)) return decline(err(std::string("A must have dtype Float32, Float16, or BFloat16, got ") + dtype_name(inputs[0].dtype)));
         if (inputs[1].dtype != NXRT_DT_UINT8) return decline(err(std::string("B must have dtype Uint8, got ") + dtype_name(inputs[1].dtype)));
         if (!is_float_compute(inputs[2].dtype)) return decline(err(std::string("scales must have dtype Float32, Float16, or BFloat16, got ") + dtype_name(inputs[2].dtype)));
-        if (n_inputs > 4 && inputs[4].dtype != 0)
-            return decline(err("g_idx is not supported on the ROCm execution provider. Why: its kernels stream contiguous K blocks. "
-                               "How to fix: export the weight without act-order, or run this node on the CPU execution provider"));
+        const int64_t accuracy = (attrs->present & (1u << kAttrAccuracy)) ? attrs->accuracy_level : 0;
+        if (n_inputs > 4 && inputs[4].dtype != 0 && accuracy == 4)
+            return decline(err("accuracy_level=4 does not take g_idx on the ROCm execution provider. Why: its int8 kernels scale whole contiguous K blocks. "
+                               "How to fix: export the weight without act-order, use accuracy_level=0, or run this node on the CPU execution provider"));
     }
     return 1;
 }

@@ -60,6 +60,7 @@ typedef struct RocmMatMulNBitsArgs {
   int a_dtype, scale_dtype, bias_dtype, y_dtype;
   int64_t m, n, k;
   int block_size;
+  const int32_t* g_idx;  /* [K] group of every element (act-order), or NULL: group = k / block_size. Only the plain kernels read it. */
 } RocmMatMulNBitsArgs;
 
 /* w[n,k] = (q - zp) * scale as f32 [N, K]. */
@@ -97,6 +98,11 @@ int rocm_launch_rmsnorm16(const void* a, const void* gamma, int gamma_dtype, int
 int rocm_launch_dequant_nbits(const uint8_t* b, const void* scales, int scale_dtype, const uint8_t* zp, int64_t n, int64_t k, int block_size,
                               int bits, int out_dtype, void* out_nk, rocm_stream_t stream);
 int rocm_launch_gemv_nbits(const RocmMatMulNBitsArgs* args, int bits, rocm_stream_t stream);
+/* The same with g_idx (bits 2, 4 or 8): scale and zero point of element k come from group g_idx[k]. */
+int rocm_launch_dequant_gidx(const uint8_t* b, const void* scales, int scale_dtype, const uint8_t* zp, const int32_t* g_idx, int64_t n, int64_t k,
+                             int block_size, int bits, int out_dtype, void* out_nk, rocm_stream_t stream);
+/* First index whose group lies outside 0..kb, or -1: synchronizes the stream and allocates (never inside a graph capture). */
+int rocm_g_idx_first_bad(const int32_t* g_idx, int64_t count, int64_t kb, int64_t* first_bad, rocm_stream_t stream);
 
 /* Any dtype mix, any K, any block size: f32 math, one wave per output column. */
 int rocm_launch_gemv_generic(const RocmMatMulNBitsArgs* args, rocm_stream_t stream);

@@ -24,9 +24,11 @@ __device__ __forceinline__ float zero_point_bits(const uint8_t* zrow, int64_t bl
 
 // One thread per packed dword (32 / BITS consecutive k of one column; a dword never straddles a block: block >= 16).
 // OUT: 0 = f32, 1 = f16, 2 = bf16.
+// `g`: per-element group indices (act-order), or null.
 template <int BITS, int OUT>
 __global__ __launch_bounds__(256) void dequant_nbits_kernel(const uint8_t* __restrict__ b, const void* __restrict__ scales, int scale_dtype,
-                                                            const uint8_t* __restrict__ zp, int64_t n, int64_t k, int bs_log2, int64_t kb, void* __restrict__ out)
+                                                            const uint8_t* __restrict__ zp, const int32_t* __restrict__ g, int64_t n, int64_t k, int bs_log2,
+                                                            int64_t kb, void* __restrict__ out)
 {
     constexpr int W = 32 / BITS;                                         // weights per dword
     const int64_t row_dwords = ((kb << bs_log2) * BITS) >> 5;
@@ -38,11 +40,17 @@ __global__ __launch_bounds__(256) void dequant_nbits_kernel(const uint8_t* __res
         if (k0 >= k) continue;
         const int64_t blk = k0 >> bs_log2;
         const uint32_t w = reinterpret_cast<const uint32_t*>(b)[idx];
-        const float s = load_as_f32(scales, scale_dtype, col * kb + blk);
-        const float z = zero_point_bits<BITS>(zp ? zp + col * zp_row : nullptr, blk);
+        const uint8_t* zrow = zp ? zp + col * zp_row : nullptr;
+        float s = load_as_f32(scales, scale_dtype, col * kb + blk);
+        float z = zero_point_bits<BITS>(zrow, blk);
 #pragma unroll
         for (int i = 0; i < W; ++i) {
             if (k0 + i >= k) break;
+            if (g) {
+                const int64_t group = g[k0 + i];
+                s = load_as_f32(scales, scale_dtype, col * kb + group);
+                z = zero_point_bits<BITS>(zrow, group);
+            }
             const float v = as_f32(__fmul_rn(static_cast<float>(field<BITS>(w, i)) - z, s));
             const int64_t at = col * k + k0 + i;
             if constexpr (OUT == 0) static_cast<float*>(out)[at] = v;
@@ -74,11 +82,16 @@ __global__ __launch_bounds__(256) void gemv_nbits_kernel(RocmMatMulNBitsArgs p, 
         if (k0 >= p.k) break;
         const int64_t blk = k0 >> bs_log2;
         const uint32_t w = brow[d];
-        const float s = load_as_f32(p.scales, p.scale_dtype, col * kb + blk);
-        const float z = zero_point_bits<BITS>(zrow, blk);
+        float s = load_as_f32(p.scales, p.scale_dtype, col * kb + blk);
+        float z = zero_point_bits<BITS>(zrow, blk);
 #pragma unroll
         for (int i = 0; i < W; ++i) {
             if (k0 + i < p.k) {
+                if (p.g_idx) {
+                    const int64_t group = p.g_idx[k0 + i];
+                    s = load_as_f32(p.scales, p.scale_dtype, col * kb + group);
+                    z = zero_point_bits<BITS>(zrow, group);
+                }
                 const float wv = __fmul_rn(static_cast<float>(field<BITS>(w, i)) - z, s);
 #pragma unroll
                 for (int r = 0; r < ROWS; ++r)
@@ -158,8 +171,8 @@ __global__ __launch_bounds__(256) void gemv_q8_kernel(RocmMatMulNBitsArgs p, int
 }
 
 template <int BITS>
-static int launch_dequant(const uint8_t* b, const void* scales, int scale_dtype, const uint8_t* zp, int64_t n, int64_t k, int block_size, int out_dtype,
-                          void* out, hipStream_t s)
+static int launch_dequant(const uint8_t* b, const void* scales, int scale_dtype, const uint8_t* zp, const int32_t* g, int64_t n, int64_t k, int block_size,
+                          int out_dtype, void* out, hipStream_t s)
 {
     const int bs_log2 = __builtin_ctz(static_cast<unsigned>(block_size));
     const int64_t kb = (k + block_size - 1) / block_size;
@@ -167,9 +180,9 @@ static int launch_dequant(const uint8_t* b, const void* scales, int scale_dtype,
     int64_t blocks = (total + 255) / 256;
     if (blocks > 262144) blocks = 262144;
     const dim3 grid(static_cast<unsigned>(blocks));
-    if (out_dtype == ROCM_DT_F32) hipLaunchKernelGGL((dequant_nbits_kernel<BITS, 0>), grid, dim3(256), 0, s, b, scales, scale_dtype, zp, n, k, bs_log2, kb, out);
-    else if (out_dtype == ROCM_DT_F16) hipLaunchKernelGGL((dequant_nbits_kernel<BITS, 1>), grid, dim3(256), 0, s, b, scales, scale_dtype, zp, n, k, bs_log2, kb, out);
-    else hipLaunchKernelGGL((dequant_nbits_kernel<BITS, 2>), grid, dim3(256), 0, s, b, scales, scale_dtype, zp, n, k, bs_log2, kb, out);
+    if (out_dtype == ROCM_DT_F32) hipLaunchKernelGGL((dequant_nbits_kernel<BITS, 0>), grid, dim3(256), 0, s, b, scales, scale_dtype, zp, g, n, k, bs_log2, kb, out);
+    else if (out_dtype == ROCM_DT_F16) hipLaunchKernelGGL((dequant_nbits_kernel<BITS, 1>), grid, dim3(256), 0, s, b, scales, scale_dtype, zp, g, n, k, bs_log2, kb, out);
+    else hipLaunchKernelGGL((dequant_nbits_kernel<BITS, 2>), grid, dim3(256), 0, s, b, scales, scale_dtype, zp, g, n, k, bs_log2, kb, out);
     return static_cast<int>(hipGetLastError());
 }
 
@@ -186,7 +199,49 @@ static int launch_gemv(const RocmMatMulNBitsArgs* args, hipStream_t s)
     return static_cast<int>(hipGetLastError());
 }
 
+// The smallest index whose group lies outside 0..kb, through an atomic minimum (count when every group is in range).
+__global__ __launch_bounds__(256) void g_idx_check_kernel(const int32_t* __restrict__ g, int64_t count, int64_t kb, unsigned long long* first_bad)
+{
+    for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < count; i += static_cast<int64_t>(gridDim.x) * blockDim.x)
+        if (g[i] < 0 || g[i] >= kb) atomicMin(first_bad, static_cast<unsigned long long>(i));
+}
+
 }  // namespace mnb
+
+extern "C" int rocm_g_idx_first_bad(const int32_t* g_idx, int64_t count, int64_t kb, int64_t* first_bad, rocm_stream_t stream)
+{
+    *first_bad = -1;
+    if (count <= 0) return 0;
+    unsigned long long* dev = nullptr;
+    hipError_t e = hipMalloc(&dev, sizeof(unsigned long long));
+    if (e != hipSuccess) return static_cast<int>(e);
+    unsigned long long host = static_cast<unsigned long long>(count);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    e = hipMemcpyAsync(dev, &host, sizeof(host), hipMemcpyHostToDevice, s);
+    if (e == hipSuccess) {
+        int64_t blocks = (count + 255) / 256;
+        if (blocks > 4096) blocks = 4096;
+        hipLaunchKernelGGL(mnb::g_idx_check_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, g_idx, count, kb, dev);
+        e = hipGetLastError();
+    }
+    if (e == hipSuccess) e = hipMemcpyAsync(&host, dev, sizeof(host), hipMemcpyDeviceToHost, s);
+    if (e == hipSuccess) e = hipStreamSynchronize(s);
+    (void)hipFree(dev);
+    if (e == hipSuccess && host < static_cast<unsigned long long>(count)) *first_bad = static_cast<int64_t>(host);
+    return static_cast<int>(e);
+}
+
+extern "C" int rocm_launch_dequant_gidx(const uint8_t* b, const void* scales, int scale_dtype, const uint8_t* zp, const int32_t* g_idx, int64_t n, int64_t k,
+                                        int block_size, int bits, int out_dtype, void* out_nk, rocm_stream_t stream)
+{
+    if (n <= 0 || k <= 0) return 0;
+    if (out_dtype != ROCM_DT_F32 && out_dtype != ROCM_DT_F16 && out_dtype != ROCM_DT_BF16) return static_cast<int>(hipErrorInvalidValue);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (bits == 2) return mnb::launch_dequant<2>(b, scales, scale_dtype, zp, g_idx, n, k, block_size, out_dtype, out_nk, s);
+    if (bits == 4) return mnb::launch_dequant<4>(b, scales, scale_dtype, zp, g_idx, n, k, block_size, out_dtype, out_nk, s);
+    if (bits == 8) return mnb::launch_dequant<8>(b, scales, scale_dtype, zp, g_idx, n, k, block_size, out_dtype, out_nk, s);
+    return static_cast<int>(hipErrorInvalidValue);
+}
 
 extern "C" int rocm_launch_dequant_nbits(const uint8_t* b, const void* scales, int scale_dtype, const uint8_t* zp, int64_t n, int64_t k, int block_size,
                                          int bits, int out_dtype, void* out_nk, rocm_stream_t stream)
@@ -194,8 +249,8 @@ extern "C" int rocm_launch_dequant_nbits(const uint8_t* b, const void* scales, i
     if (n <= 0 || k <= 0) return 0;
     if (out_dtype != ROCM_DT_F32 && out_dtype != ROCM_DT_F16 && out_dtype != ROCM_DT_BF16) return static_cast<int>(hipErrorInvalidValue);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (bits == 2) return mnb::launch_dequant<2>(b, scales, scale_dtype, zp, n, k, block_size, out_dtype, out_nk, s);
-    if (bits == 8) return mnb::launch_dequant<8>(b, scales, scale_dtype, zp, n, k, block_size, out_dtype, out_nk, s);
+    if (bits == 2) return mnb::launch_dequant<2>(b, scales, scale_dtype, zp, nullptr, n, k, block_size, out_dtype, out_nk, s);
+    if (bits == 8) return mnb::launch_dequant<8>(b, scales, scale_dtype, zp, nullptr, n, k, block_size, out_dtype, out_nk, s);
     return static_cast<int>(hipErrorInvalidValue);
 }
 
@@ -204,7 +259,7 @@ extern "C" int rocm_launch_gemv_nbits(const RocmMatMulNBitsArgs* args, int bits,
     if (args->m <= 0 || args->n <= 0) return 0;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool half_in = args->a_dtype == ROCM_DT_F16 || args->a_dtype == ROCM_DT_BF16;
-    if (bits == 8 && half_in && args->m <= 4 && args->k % 16 == 0 && (reinterpret_cast<uintptr_t>(args->a) & 15) == 0 &&
+    if (bits == 8 && !args->g_idx && half_in && args->m <= 4 && args->k % 16 == 0 && (reinterpret_cast<uintptr_t>(args->a) & 15) == 0 &&
         (reinterpret_cast<uintptr_t>(args->b) & 15) == 0) {
         const int bs_log2 = __builtin_ctz(static_cast<unsigned>(args->block_size));
         const int64_t kb = (args->k + args->block_size - 1) / args->block_size;
@@ -220,6 +275,7 @@ extern "C" int rocm_launch_gemv_nbits(const RocmMatMulNBitsArgs* args, int bits,
         return static_cast<int>(hipGetLastError());
     }
     if (bits == 2) return mnb::launch_gemv<2>(args, s);
+    if (bits == 4) return mnb::launch_gemv<4>(args, s);            // 4 bits come here with g_idx only
     if (bits == 8) return mnb::launch_gemv<8>(args, s);
     return static_cast<int>(hipErrorInvalidValue);
 }

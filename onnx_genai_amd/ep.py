@@ -455,8 +455,9 @@ class DeviceOperands:
     """The device-resident operands of one MatMulNBits node plus its kernel; what a session would hold."""
 
     def __init__(self, ep, b, scales, scale_dtype, zp, n, k, bs, *, accuracy_level=0, bias=None, bias_dtype=F32, rows=None, a_dtype=None,
-                 folded_bias=None, gamma=None, gamma_dtype=F32, rmsnorm_epsilon=None, bits=4):
+                 folded_bias=None, gamma=None, gamma_dtype=F32, rmsnorm_epsilon=None, bits=4, g_idx=None):
         self.ep, self.n, self.k, self.bs, self.bits = ep, n, k, bs, bits
+        self.g_idx = ep.upload(np.ascontiguousarray(g_idx, np.int32)) if g_idx is not None else None      # act-order groups, input 4
         self.kb = -(-k // bs)
         self.scale_dtype, self.bias_dtype = scale_dtype, bias_dtype
         self.b = ep.upload(np.asarray(b, np.uint8))
@@ -477,10 +478,12 @@ class DeviceOperands:
         ins = [TensorView(a_buf.ptr, a_dtype, (m, self.k), device_index=dev),
                TensorView(self.b.ptr, U8, (self.n, self.kb, self.bs * self.bits // 8), device_index=dev),
                TensorView(self.scales.ptr, self.scale_dtype, (self.n, self.kb), device_index=dev)]
-        if self.zp is not None or self.bias is not None or self.gamma is not None:
+        if self.zp is not None or self.bias is not None or self.gamma is not None or self.g_idx is not None:
             ins.append(TensorView(self.zp.ptr, U8, (self.n, (self.kb * self.bits + 7) // 8), device_index=dev) if self.zp is not None else TensorView.absent(U8))
+        if self.g_idx is not None and self.bias is None and self.gamma is None:
+            ins.append(TensorView(self.g_idx.ptr, I32, (self.k,), device_index=dev))
         if self.bias is not None or self.gamma is not None:
-            ins.append(TensorView.absent(I32))
+            ins.append(TensorView(self.g_idx.ptr, I32, (self.k,), device_index=dev) if self.g_idx is not None else TensorView.absent(I32))
             ins.append(TensorView(self.bias.ptr, self.bias_dtype, (self.n,), device_index=dev) if self.bias is not None else TensorView.absent(F32))
         if self.gamma is not None:
             ins.append(TensorView(self.gamma.ptr, self.gamma_dtype, (self.k,), device_index=dev))
@@ -493,19 +496,19 @@ class DeviceOperands:
 
     def free(self) -> None:
         self.kernel.release()
-        for buf in (self.b, self.scales, self.zp, self.bias, self.gamma):
+        for buf in (self.b, self.scales, self.zp, self.bias, self.gamma, self.g_idx):
             if buf is not None:
                 self.ep.deallocate(buf)
 
 
 def matmul_nbits(ep, a, a_dtype, b, scales, scale_dtype, zp, n, k, bs, *, accuracy_level=0, bias=None, bias_dtype=F32, y_dtype=None, folded_bias=None,
-                 gamma=None, gamma_dtype=F32, rmsnorm_epsilon=None, bits=4):
+                 gamma=None, gamma_dtype=F32, rmsnorm_epsilon=None, bits=4, g_idx=None):
     """One-shot helper: upload, execute through the C ABI, download. Returns (Y as numpy, variant name)."""
     y_dtype = a_dtype if y_dtype is None else y_dtype
     a = np.ascontiguousarray(a)
     m = a.size // k
     ops = DeviceOperands(ep, b, scales, scale_dtype, zp, n, k, bs, accuracy_level=accuracy_level, bias=bias, bias_dtype=bias_dtype, folded_bias=folded_bias,
-                         gamma=gamma, gamma_dtype=gamma_dtype, rmsnorm_epsilon=rmsnorm_epsilon, bits=bits)
+                         gamma=gamma, gamma_dtype=gamma_dtype, rmsnorm_epsilon=rmsnorm_epsilon, bits=bits, g_idx=g_idx)
     a_buf = ep.upload(a)
     y_buf = ep.allocate(max(m * n * _ITEM[y_dtype], 1))
     try:

@@ -87,6 +87,8 @@ class Port:
         L.mnb_rmsnorm16.argtypes = [v, v, C.c_int, z, z, C.c_float, C.c_int, v]
         L.mnb_dequantize_nk_bits.argtypes = [v, v, v, z, z, z, C.c_int, v]
         L.mnb_matmul_f64_bits.argtypes = [v, v, v, v, v, z, z, z, z, C.c_int, v]
+        L.mnb_dequantize_nk_gidx.restype = C.c_long
+        L.mnb_dequantize_nk_gidx.argtypes = [v, v, v, v, z, z, z, C.c_int, v]
         L.mnb_matmul_nbits.restype = C.c_int
         L.mnb_matmul_nbits.argtypes = [v, C.c_int, v, v, C.c_int, v, v, C.c_int, v, C.c_int, z, z, z, z, C.c_int, C.c_int]
 
@@ -124,6 +126,15 @@ class Port:
         y = np.empty((m, n), np.float64)
         self.lib.mnb_matmul_f64_bits(_ptr(a), _ptr(b), _ptr(scales), _ptr(zp), _ptr(bias), m, n, k, bs, bits, _ptr(y))
         return y
+
+    def dequantize_nk_gidx(self, b, scales, zp, g_idx, n, k, bs, bits=4) -> np.ndarray:
+        """Dequantized [N, K] with scale / zero point of element k taken from group g_idx[k]; raises on an index outside 0..kb."""
+        b, scales, zp, g_idx = _c(b, np.uint8), _c(scales, np.float32), _c(zp, np.uint8), _c(g_idx, np.int32)
+        out = np.empty((n, k), np.float32)
+        rc = self.lib.mnb_dequantize_nk_gidx(_ptr(b), _ptr(scales), _ptr(zp), _ptr(g_idx), n, k, bs, bits, _ptr(out))
+        if rc != 0:
+            raise ValueError("g_idx[%d] is outside 0..kb" % (-1 - rc))
+        return out
 
     def rmsnorm16(self, a16: np.ndarray, gamma: np.ndarray, gamma_code: int, epsilon: float, code: int) -> np.ndarray:
         """The RMS-normalization prologue on 16-bit rows [rows, K] (K % 128 == 0); gamma 16-bit of the same type or f32."""

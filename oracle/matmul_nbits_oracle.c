@@ -406,3 +406,26 @@ void mnb_matmul_f64_bits(const float* a, const uint8_t* b, const float* scales, 
             y[row * n + col] = acc + (bias ? (double)bias[col] : 0.0);
         }
 }
+
+
+/* ---- g_idx: matmul_nbits.rs:3515-3521, 3636-3658 --------------------------------------------------- */
+
+long mnb_dequantize_nk_gidx(const uint8_t* b, const float* scales, const uint8_t* zp, const int32_t* g_idx, size_t n, size_t k, size_t block_size,
+                            int bits, float* out_nk)
+{
+    const size_t kb = div_ceil(k, block_size), blob = block_size * (size_t)bits / 8, zp_row = div_ceil(kb * (size_t)bits, 8);
+    if (g_idx)
+        for (size_t depth = 0; depth < k; ++depth)
+            if (g_idx[depth] < 0 || (size_t)g_idx[depth] >= kb) return -1 - (long)depth;
+    for (size_t col = 0; col < n; ++col) {
+        const uint8_t* row = b + col * kb * blob;
+        for (size_t depth = 0; depth < k; ++depth) {
+            const size_t block = depth / block_size;
+            const size_t group = g_idx ? (size_t)g_idx[depth] : block;
+            const uint8_t q = mnb_unpack_bits(row + block * blob, depth % block_size, bits);
+            const uint8_t z = zp ? mnb_unpack_bits(zp + col * zp_row, group, bits) : (uint8_t)(1u << (bits - 1));
+            out_nk[col * k + depth] = ((float)q - (float)z) * scales[col * kb + group];
+        }
+    }
+    return 0;
+}

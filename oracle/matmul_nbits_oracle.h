@@ -49,6 +49,11 @@ void mnb_dequantize_nk(const uint8_t* b, const float* scales, const uint8_t* zp,
 uint8_t mnb_unpack_bits(const uint8_t* packed, size_t index, int bits);
 void mnb_dequantize_nk_bits(const uint8_t* b, const float* scales, const uint8_t* zp, size_t n, size_t k, size_t block_size, int bits,
                             float* out_nk);
+/* With g_idx (matmul_nbits.rs:3636-3658): scale and zero point of element k come from group g_idx[k] instead of block
+ * k / block_size; the packed weights stay where they are. g_idx NULL: the functions above. Returns -1 - index of the first
+ * entry outside 0..kb (matmul_nbits.rs:3515-3521 raises there), 0 otherwise. */
+long mnb_dequantize_nk_gidx(const uint8_t* b, const float* scales, const uint8_t* zp, const int32_t* g_idx, size_t n, size_t k, size_t block_size,
+                            int bits, float* out_nk);
 /* int4_f64_reference (matmul_nbits.rs:10890-10933) over that layout: f64 accumulation, bias added in f64. */
 void mnb_matmul_f64_bits(const float* a, const uint8_t* b, const float* scales, const uint8_t* zp, const float* bias,
                          size_t m, size_t n, size_t k, size_t block_size, int bits, double* y);

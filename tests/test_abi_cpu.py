@@ -210,7 +210,9 @@ def test_supports_op_declines_with_reasons(lib):
     a = E.make_attrs(K=64, N=8, bits=4, block_size=32)
     assert lib.nxrt_rocm_ep_supports_matmul_nbits(None, C.byref(a), None, 0, reason, 512) == 1 and reason.value == b""
     descs, keep = E.make_descs([((1, 64), E.F16), ((8, 2, 16), E.U8), ((8, 2), E.F16), (None, 0), ((64,), E.I32)])
-    assert lib.nxrt_rocm_ep_supports_matmul_nbits(None, C.byref(a), descs, 5, reason, 512) == 0 and b"g_idx is not supported" in reason.value
+    assert lib.nxrt_rocm_ep_supports_matmul_nbits(None, C.byref(a), descs, 5, reason, 512) == 1                      # act-order weights are taken
+    a4 = E.make_attrs(K=64, N=8, bits=4, block_size=32, accuracy_level=4)
+    assert lib.nxrt_rocm_ep_supports_matmul_nbits(None, C.byref(a4), descs, 5, reason, 512) == 0 and b"does not take g_idx" in reason.value
     descs, keep = E.make_descs([((1, 64), E.I32), ((8, 2, 16), E.U8), ((8, 2), E.F16)])
     assert lib.nxrt_rocm_ep_supports_matmul_nbits(None, C.byref(a), descs, 3, reason, 512) == 0
     assert reason.value == b"MatMulNBits: A must have dtype Float32, Float16, or BFloat16, got Int32"

@@ -327,3 +327,28 @@ def test_nbits_layout_against_numpy_unpacking(port, bits, zero_points):
     one = np.array([[[0xe4] * (16 * bits // 8)]], np.uint8)
     w = port.dequantize_nk_bits(one, np.ones((1, 1), np.float32), None, 1, 16, 16, bits)[0]
     assert list(w[:4]) == {2: [-2.0, -1.0, 0.0, 1.0], 4: [-4.0, 6.0, -4.0, 6.0], 8: [100.0] * 4}[bits]
+
+
+def test_g_idx_against_numpy_gather(port):
+    """g_idx: scale and zero point gathered per element (matmul_nbits.rs:3636-3658), against numpy fancy indexing; the identity
+    g_idx[k] = k / block_size gives the plain dequantization; an index outside 0..kb is an error (:3515-3521)."""
+    rng = np.random.default_rng(5)
+    n, k, bs = 6, 160, 32
+    kb = k // bs
+    for bits in (4, 8):
+        b = rng.integers(0, 256, size=(n, kb, bs * bits // 8), dtype=np.uint8)
+        scales = rng.uniform(0.01, 0.1, size=(n, kb)).astype(np.float32)
+        zp = rng.integers(0, 256, size=(n, -(-kb * bits // 8)), dtype=np.uint8)
+        plain = port.dequantize_nk_bits(b, scales, zp, n, k, bs, bits)
+        ident = (np.arange(k) // bs).astype(np.int32)
+        assert np.array_equal(port.dequantize_nk_gidx(b, scales, zp, ident, n, k, bs, bits), plain)
+        g = rng.integers(0, kb, size=k).astype(np.int32)
+        zf = np.unpackbits(zp, axis=1, bitorder="little").reshape(n, -1, bits)
+        z = (zf * (1 << np.arange(bits))).sum(axis=2)[:, :kb].astype(np.float32)
+        q = plain / scales[:, ident] + z[:, ident]                       # recover the integers (exact: small integers times a scale)
+        want = (np.rint(q).astype(np.float32) - z[:, g]) * scales[:, g]
+        assert np.array_equal(port.dequantize_nk_gidx(b, scales, zp, g, n, k, bs, bits), want)
+        bad = g.copy()
+        bad[17] = kb
+        with pytest.raises(ValueError, match="g_idx\\[17\\]"):
+            port.dequantize_nk_gidx(b, scales, zp, bad, n, k, bs, bits)

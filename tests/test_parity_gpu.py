@@ -602,6 +602,46 @@ def test_other_bit_widths_match_oracle(ep, port, bits, a_dt, s_dt, bs, zero_poin
     assert helpers.rel_l2(synth.to_f32(y, a_dt), want) <= (TOL_F32 if a_dt == E.F32 else TOL_HALF)
 
 
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("a_dt,bs,zero_points,m,n,k,with_bias", [
+    (E.F32, 32, True, 1, 100, 256, False),
+    (E.F16, 32, False, 3, 130, 1024, True),
+    (E.BF16, 128, True, 16, 72, 1024, False),
+    (E.F16, 64, True, 48, 136, 512, True),          # tall: dense route over weights expanded with their groups
+])
+def test_g_idx_matches_oracle(ep, port, bits, a_dt, bs, zero_points, m, n, k, with_bias):
+    """Act-order weights (g_idx at input 4): scale and zero point of element k come from group g_idx[k] (matmul_nbits.rs:3636-3658)."""
+    kb = k // bs
+    if bits == 4:
+        b, s, zp = synth.make_weights(n, k, bs, 60 + n, zero_points=zero_points, scale_lo=0.005, scale_hi=0.02, scale_dtype=a_dt)
+    else:
+        b, s, zp = synth.make_weights_bits(n, k, bs, bits, 60 + n, zero_points=zero_points, scale_lo=0.001, scale_hi=0.003, scale_dtype=a_dt)
+    g = np.random.default_rng(k + bits).integers(0, kb, size=k).astype(np.int32)
+    a = synth.make_activation(m, k, 61 + m, a_dt)
+    bias = synth.to_dtype(np.linspace(-1, 1, n).astype(np.float32), a_dt) if with_bias else None
+    y, variant = run_op(ep, a, a_dt, b, s, a_dt, zp, n, k, bs, bias=bias, bias_dtype=a_dt, bits=bits, g_idx=g)
+    assert variant == ("dense_transient_blaslt" if (m >= 32 and a_dt != E.F32) else "gemv_nbits_f32")
+    w = port.dequantize_nk_gidx(b, synth.to_f32(s, a_dt), zp, g, n, k, bs, bits).astype(np.float64)
+    want = synth.to_f32(a, a_dt).astype(np.float64) @ w.T + (synth.to_f32(bias, a_dt).astype(np.float64) if with_bias else 0.0)
+    assert helpers.rel_l2(synth.to_f32(y, a_dt), want) <= (TOL_F32 if a_dt == E.F32 else TOL_HALF)
+    if m == 1:                                         # the identity grouping is the plain operator
+        ident = (np.arange(k) // bs).astype(np.int32)
+        y0, _ = run_op(ep, a, a_dt, b, s, a_dt, zp, n, k, bs, bits=bits, g_idx=ident)
+        plain = port.matmul_f64_bits(synth.to_f32(a, a_dt), b, synth.to_f32(s, a_dt), zp, n, k, bs, bits)
+        assert helpers.rel_l2(synth.to_f32(y0, a_dt), plain) <= TOL_F32
+
+
+def test_g_idx_out_of_range_is_an_error(ep):
+    a_dt, bs, n, k = E.F16, 32, 16, 128
+    b, s, zp = synth.make_weights(n, k, bs, 3, zero_points=True, scale_lo=0.005, scale_hi=0.02, scale_dtype=a_dt)
+    g = (np.arange(k) // bs).astype(np.int32)
+    g[77] = k // bs
+    with pytest.raises(E.EpError, match=r"g_idx\[77\] is outside 0\.\.4"):
+        run_op(ep, synth.make_activation(1, k, 1, a_dt), a_dt, b, s, a_dt, zp, n, k, bs, g_idx=g)
+    with pytest.raises(E.EpError, match="accuracy_level=4 does not take g_idx"):
+        run_op(ep, synth.make_activation(1, k, 1, a_dt), a_dt, b, s, a_dt, zp, n, k, bs, g_idx=(np.arange(k) // bs).astype(np.int32), accuracy_level=4)
+
+
 def test_other_bit_widths_validation(ep):
     with pytest.raises(E.EpError, match="bits in {2, 4, 8}"):
         ep.get_kernel({"K": 64, "N": 8, "bits": 3, "block_size": 32})
@@ -1150,8 +1190,8 @@ def test_execute_validation_messages(ep):
     bad = list(good_in)
     bad[0] = E.TensorView(ab.ptr, E.F32, (2, k), strides=(2 * k, 1))
     fails(bad, good_out, "MatMulNBits: A must be contiguous on the ROCm execution provider")
-    bad = list(good_in) + [E.TensorView(ab.ptr, E.I32, (k,))]
-    fails(bad, good_out, "g_idx is not supported on the ROCm execution provider")
+    bad = list(good_in) + [E.TensorView(ops.b.ptr, E.I32, (k,))]
+    fails(bad, good_out, "] is outside 0..2")                    # 256 random weight bytes read as 64 group indices: far out of range
     bad = list(good_in)
     bad[0] = E.TensorView(ab.ptr, E.F32, (2, k), device_type=0)
     fails(bad, good_out, "must live on ROCm device 0")
