@@ -72,7 +72,8 @@ NxrtRocmEp* nxrt_rocm_ep_from_vtable(const NxrtEpVtable* vtable);
 
 /* Node attributes of MatMulNBits. `present` has bit i set when attribute i was on the node:
  * 0=K 1=N 2=bits 3=block_size 4=accuracy_level 5=weight_prepacked
- * (onnx-runtime-ep-cpu/src/kernels/matmul_nbits.rs:1410-1481), and 6=folded_bias: the marker an optimizer pass sets
+ * (onnx-runtime-ep-cpu/src/kernels/matmul_nbits.rs:1410-1481; bits 2, 4 (default) or 8 as there - 4 is the tuned path, and the
+ * only one with accuracy_level = 4; weight_prepacked must be 0), and 6=folded_bias: the marker an optimizer pass sets
  * when it folds a standalone Add into the bias input (the CUDA provider's `_cuda_matmul_nbits_folded_bias`,
  * onnx-runtime-ep-cuda/src/optimizer.rs:35, kernels/matmul_nbits.rs:1189-1212). With folded_bias = 1 and a 16-bit
  * output the result is round(round(acc) + bias), bit for bit what the two nodes gave; otherwise round(acc + bias).
@@ -133,7 +134,9 @@ NxrtStatus nxrt_rocm_matmul_nbits_workspace_requirement(const NxrtRocmMatMulNBit
                                                         uint32_t n_inputs, NxrtRocmWorkspaceRequirement* out);
 /* Kernel::execute / execute_with_workspace (matmul_nbits.rs:1490-1600, 2320-2330).
  * inputs: A, B, scales, [zero_points], [g_idx], [bias]; outputs: Y. workspace may be NULL: the
- * kernel then keeps its own scratch, grown on demand (an allocation inside the call). */
+ * kernel then keeps its own scratch, grown on demand (an allocation inside the call). B is [N, kb, block_size * bits / 8],
+ * zero_points [N, ceil(kb * bits / 8)]; g_idx (Int32 [K] or [kb * block_size], accuracy_level 0 only) is range-checked on first
+ * use (matmul_nbits.rs:3515-3521). Fused nodes (gate_up_swiglu, rmsnorm_prologue) take their own input lists, see the attributes. */
 NxrtStatus nxrt_rocm_matmul_nbits_execute(NxrtRocmMatMulNBits* kernel, const NxrtRocmTensorView* inputs, uint32_t n_inputs,
                                           NxrtRocmTensorView* outputs, uint32_t n_outputs,
                                           void* workspace_device, uint64_t workspace_bytes);
