@@ -1276,6 +1276,52 @@ def test_random_shapes_against_oracle(ep, port, a_dt, s_dt, bs, zero_points, m, 
         assert helpers.rel_l2(y32, want) <= tol, variant
 
 
+def test_concurrent_dense_calls_share_one_buffer(port):
+    """Two host threads drive two kernels whose tall calls expand their weights into the provider's one dense buffer: the
+    expansion and the GEMM of a call are enqueued as a pair, so neither call multiplies by the other's weights."""
+    import threading
+    provider = E.RocmExecutionProvider(0, {"dense_gemm_min_rows": "64"})
+    a_dt, bs, m, n, k = E.F16, 32, 96, 136, 512
+    sets = []
+    try:
+        for i in range(2):
+            b, s, zp = synth.make_weights(n, k, bs, 90 + i, zero_points=True, scale_lo=0.002, scale_hi=0.01, scale_dtype=a_dt)
+            a = synth.make_activation(m, k, 92 + i, a_dt)
+            ops = E.DeviceOperands(provider, b, s, a_dt, zp, n, k, bs)
+            ops.kernel.set_constant_inputs([False] * 6)          # weights not constant: every call refills the shared buffer
+            sets.append((ops, a, b, s, zp, provider.upload(a), provider.allocate(m * n * 2)))
+        for ops, a, _, _, _, ab, yb in sets:                     # first calls, one after the other: set-up happens here
+            ops.run(ab, a_dt, m, yb)
+        provider.sync()
+        errors = []
+
+        def work(item):
+            try:
+                ops, _, _, _, _, ab, yb = item
+                for _ in range(50):
+                    ops.run(ab, a_dt, m, yb)
+            except Exception as exc:                               # noqa: BLE001 - reported below
+                errors.append(exc)
+
+        threads = [threading.Thread(target=work, args=(item,)) for item in sets]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join()
+        provider.sync()
+        assert not errors, errors
+        for ops, a, b, s, zp, ab, yb in sets:
+            assert ops.kernel.last_variant() == "dense_transient_blaslt"
+            got = synth.to_f32(provider.download(yb, (m, n), np.float16), a_dt)
+            assert helpers.rel_l2(got, oracle_f64(port, a, a_dt, b, s, a_dt, zp, n, k, bs)) <= TOL_HALF
+    finally:
+        for ops, _, _, _, _, ab, yb in sets:
+            provider.deallocate(ab)
+            provider.deallocate(yb)
+            ops.free()
+        provider.shutdown()
+
+
 def test_concurrent_execute_on_one_kernel(ep, port):
     """Two host threads drive the same kernel object (the plugin contract asks for thread-safe vtables): every call
     must see consistent per-object state (repacked copy, scratch) and produce its own result."""
