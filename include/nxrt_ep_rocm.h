@@ -136,7 +136,8 @@ NxrtStatus nxrt_rocm_matmul_nbits_workspace_requirement(const NxrtRocmMatMulNBit
  * inputs: A, B, scales, [zero_points], [g_idx], [bias]; outputs: Y. workspace may be NULL: the
  * kernel then keeps its own scratch, grown on demand (an allocation inside the call). B is [N, kb, block_size * bits / 8],
  * zero_points [N, ceil(kb * bits / 8)]; g_idx (Int32 [K] or [kb * block_size], accuracy_level 0 only) is range-checked on first
- * use (matmul_nbits.rs:3515-3521). Fused nodes (gate_up_swiglu, rmsnorm_prologue) take their own input lists, see the attributes. */
+ * use (matmul_nbits.rs:3515-3521). bias is [N], or Y's shape: a per-token residual folded into the bias slot
+ * (onnx-runtime-ep-cuda/src/kernels/matmul_nbits.rs:7891-7897). Fused nodes (gate_up_swiglu, rmsnorm_prologue) take their own input lists, see the attributes. */
 NxrtStatus nxrt_rocm_matmul_nbits_execute(NxrtRocmMatMulNBits* kernel, const NxrtRocmTensorView* inputs, uint32_t n_inputs,
                                           NxrtRocmTensorView* outputs, uint32_t n_outputs,
                                           void* workspace_device, uint64_t workspace_bytes);

@@ -256,7 +256,7 @@ bool dense_route(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& args, int& 
     if ((reinterpret_cast<uintptr_t>(args.a) & 15) != 0 || (reinterpret_cast<uintptr_t>(args.y) & 15) != 0 || (reinterpret_cast<uintptr_t>(args.b) & 3) != 0) return false;
     const uint64_t need = static_cast<uint64_t>(args.n) * static_cast<uint64_t>(args.k) * 2;
     if (need > ep.dense_gemm_max_bytes) return false;
-    if (args.bias && (args.bias_dtype & ROCM_BIAS_POST_ROUND)) return false;      // the library's epilogue adds the bias before the one rounding
+    if (args.bias && (args.bias_dtype & (ROCM_BIAS_POST_ROUND | ROCM_BIAS_PER_ROW))) return false;      // the library's epilogue adds a [N] bias before the one rounding
     const int bias_dtype = args.bias ? args.bias_dtype : -1;
 
     std::lock_guard<std::mutex> lock(ep.dense_mu);
@@ -314,6 +314,14 @@ bool dense_route(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& args, int& 
     return true;
 }
 
+// The bias of a pass that starts at row `row0`: a per-token residual moves with the rows, a broadcast bias stays.
+const void* rows_of_bias(const RocmMatMulNBitsArgs& args, int64_t row0)
+{
+    if (!args.bias || !(args.bias_dtype & ROCM_BIAS_PER_ROW)) return args.bias;
+    const size_t elem = (args.bias_dtype & 0xff) == ROCM_DT_F32 ? 4 : 2;
+    return static_cast<const uint8_t*>(args.bias) + static_cast<size_t>(row0) * static_cast<size_t>(args.n) * elem;
+}
+
 // 17..32 rows as two blocks of at most 16 through the decode kernels. The tiled kernel needs a few hundred rows to
 // pay for itself; below that a call costs what streaming the weights costs, and two streams are still cheaper than
 // one under-filled tiled launch (measured at the 7B shapes: 19.8 against 22.6 us, 38 against 55 us; three are not). Returns false (nothing launched) when the decode kernels do not take the shape.
@@ -331,6 +339,7 @@ bool decode_in_row_blocks(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& ar
         part.m = args.m - row0 < 16 ? args.m - row0 : 16;
         part.a = static_cast<const uint8_t*>(args.a) + static_cast<size_t>(row0) * static_cast<size_t>(args.k) * a_elem;
         part.y = static_cast<uint8_t*>(args.y) + static_cast<size_t>(row0) * static_cast<size_t>(args.n) * y_elem;
+        part.bias = rows_of_bias(args, row0);
         int pack_rc = 0;
         if (use_packed(kn, part, pack_rc)) {
             rc = pack_rc != 0 ? pack_rc : rocm_launch_decode_packed(&part, kn.packed, kn.ep->decode_waves, kn.ep->stream);
@@ -357,6 +366,7 @@ bool f32_in_row_blocks(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& args,
         part.m = args.m - row0 < 4 ? args.m - row0 : 4;
         part.a = static_cast<const uint8_t*>(args.a) + static_cast<size_t>(row0) * static_cast<size_t>(args.k) * 4;
         part.y = static_cast<uint8_t*>(args.y) + static_cast<size_t>(row0) * static_cast<size_t>(args.n) * y_elem;
+        part.bias = rows_of_bias(args, row0);
         rc = rocm_launch_gemv_f32(&part, kn.ep->stream);
     }
     kn.variant = "gemv_f32_valu";
@@ -425,9 +435,18 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
     if (!c.failed && !shape_is(B, {N, kb, blob}))
         c.fail("B must have shape " + shape_str({N, kb, blob}) + ", got " + shape_str(B.shape, B.ndim));
     const NxrtRocmTensorView* BIAS = optional(5);
+    // A folded residual epilogue passes a per-token residual in the bias slot: Y's shape (or M * N elements flat), indexed
+    // with row stride N (onnx-runtime-ep-cuda/src/kernels/matmul_nbits.rs:7891-7897). A genuine bias is [N].
+    bool bias_per_row = false;
     if (BIAS && !c.failed) {
         require_float("bias", BIAS->dtype);
-        if (!c.failed && !shape_is(*BIAS, {N})) c.fail("bias must have shape " + shape_str({N}) + ", got " + shape_str(BIAS->shape, BIAS->ndim));
+        if (!c.failed && !shape_is(*BIAS, {N})) {
+            uint64_t rows = 1;
+            for (uint32_t i = 0; i + 1 < A.ndim; ++i) rows *= A.shape[i];
+            bias_per_row = rows * N != N && (shape_is(*BIAS, y_shape) || shape_is(*BIAS, {rows * N}) || shape_is(*BIAS, {rows, N}));
+            if (!bias_per_row)
+                c.fail("bias must have shape " + shape_str({N}) + " (or Y's shape " + shape_str(y_shape) + " for a folded residual), got " + shape_str(BIAS->shape, BIAS->ndim));
+        }
     }
     if (c.failed) return make_status(NXRT_INVALID_ARGUMENT, c.message);
 
@@ -460,6 +479,7 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
     args.scale_dtype = static_cast<int>(S.dtype);
     args.bias_dtype = BIAS ? static_cast<int>(BIAS->dtype) : ROCM_DT_F32;
     if (BIAS && kn.bias_post_round) args.bias_dtype |= ROCM_BIAS_POST_ROUND;
+    if (BIAS && bias_per_row) args.bias_dtype |= ROCM_BIAS_PER_ROW;
     args.y_dtype = static_cast<int>(Y.dtype);
     args.m = static_cast<int64_t>(M);
     args.n = kn.n;

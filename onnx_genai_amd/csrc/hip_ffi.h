@@ -22,6 +22,9 @@ enum { ROCM_DT_F32 = 1, ROCM_DT_U8 = 2, ROCM_DT_I32 = 6, ROCM_DT_F16 = 10, ROCM_
  * first and the bias added with a second rounding, round(round(acc) + bias), which is what MatMulNBits followed by Add
  * produces (onnx-runtime-ep-cuda/src/kernels/matmul_nbits.rs:1189-1212). Without it: round(acc + bias). */
 enum { ROCM_BIAS_POST_ROUND = 0x100 };
+/* Or-ed into a bias dtype: the bias slot carries a per-token residual [M, N] (row stride N) instead of a broadcast [N] - what
+ * the CUDA provider's folded residual epilogue passes (kernels/matmul_nbits.rs:7891-7897). */
+enum { ROCM_BIAS_PER_ROW = 0x200 };
 
 const char* rocm_ffi_error_string(int err);
 int rocm_ffi_device_count(int* count);

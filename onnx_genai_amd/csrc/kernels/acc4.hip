@@ -147,7 +147,7 @@ __global__ __launch_bounds__(256) void acc4_gemv_kernel(RocmMatMulNBitsArgs p, c
     for (int r = 0; r < ROWS; ++r) {
         const float total = wave_sum(acc[r]);
         if (lane == 0 && r < rows) {
-            store_from_f32(p.y, p.y_dtype, (row0 + r) * p.n + col, with_bias(total, p.bias, p.bias_dtype, col, p.y_dtype));
+            store_from_f32(p.y, p.y_dtype, (row0 + r) * p.n + col, with_bias(total, p.bias, p.bias_dtype, row0 + r, p.n, col, p.y_dtype));
         }
     }
 }

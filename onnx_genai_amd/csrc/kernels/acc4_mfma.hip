@@ -256,7 +256,7 @@ __global__ __launch_bounds__(512) void acc4_decode_kernel(Acc4DecodeParams p)
         if (row < p.m && col < p.n) {
             float total = 0.f;
             for (int w = 0; w < waves; ++w) total += red[(w * 4 + r) * 64 + l];
-            total = with_bias(total, p.bias, p.bias_dtype, col, p.y_dtype);
+            total = with_bias(total, p.bias, p.bias_dtype, row, p.n, col, p.y_dtype);
             store_from_f32(p.y, p.y_dtype, static_cast<int64_t>(row) * p.n + col, total);
         }
     }
@@ -549,7 +549,9 @@ __global__ __launch_bounds__(512) void acc4_prefill_kernel(Acc4PrefillParams p)
     for (int j = 0; j < TN; ++j) {
         const int64_t col = n_base + wn * 64 + j * 32 + col_in_tile;
         if (col >= p.n) continue;
-        const BiasTerm bias = load_bias(p.partial ? nullptr : p.bias, p.bias_dtype, col);     // slices: the reduce kernel adds it
+        const void* bias_ptr = p.partial ? nullptr : p.bias;                                   // slices: the reduce kernel adds it
+        const bool per_row = (p.bias_dtype & ROCM_BIAS_PER_ROW) != 0;
+        const BiasTerm bias = load_bias(bias_ptr, p.bias_dtype, 0, p.n, col);
         float* part = p.partial ? p.partial + static_cast<int64_t>(blockIdx.z) * p.m * p.n : nullptr;
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
@@ -558,7 +560,7 @@ __global__ __launch_bounds__(512) void acc4_prefill_kernel(Acc4PrefillParams p)
                 const int64_t row = m_base + wm * 32 + q * 8 + row_group + r;
                 if (row >= p.m) continue;
                 if (part) part[row * p.n + col] = y[j][q * 4 + r];
-                else store_from_f32(p.y, p.y_dtype, row * p.n + col, add_bias(y[j][q * 4 + r], bias, p.y_dtype));
+                else store_from_f32(p.y, p.y_dtype, row * p.n + col, add_bias(y[j][q * 4 + r], per_row ? load_bias(bias_ptr, p.bias_dtype, row, p.n, col) : bias, p.y_dtype));
             }
         }
     }

@@ -303,7 +303,7 @@ __global__ __launch_bounds__(512) void decode_mfma_kernel(DecodeParams p)
         if (row < p.m && col < p.n) {
             float total = 0.f;
             for (int w = 0; w < waves; ++w) total += red[((w * CG + cg) * 4 + r) * 64 + l];
-            total = with_bias(total, p.bias, p.bias_dtype, col, p.y_dtype);
+            total = with_bias(total, p.bias, p.bias_dtype, row, p.n, col, p.y_dtype);
             store_from_f32(p.y, p.y_dtype, static_cast<int64_t>(row) * p.n + col, total);
         }
     }

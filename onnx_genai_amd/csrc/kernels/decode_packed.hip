@@ -391,7 +391,7 @@ void decode_packed_kernel(PackedParams p)
                 const uint16_t up16 = BF16 ? f32_to_bf16_bits(total_up) : f32_to_f16_bits(total_up);
                 static_cast<uint16_t*>(p.y)[static_cast<int64_t>(row) * p.n + col] = swiglu16<BF16>(gate16, up16, p.decomposed_silu != 0);
             } else {
-                total = with_bias(total, p.bias, p.bias_dtype, col, p.y_dtype);
+                total = with_bias(total, p.bias, p.bias_dtype, row, p.n, col, p.y_dtype);
                 store_from_f32(p.y, p.y_dtype, static_cast<int64_t>(row) * p.n + col, total);
             }
         }
@@ -667,13 +667,14 @@ void decode_wide_kernel(PackedParams p)
     if (active) {
         const int64_t col = n_base + c;
         if (col < p.n) {
-            const BiasTerm bias = load_bias(p.bias, p.bias_dtype, col);
+            const bool per_row = (p.bias_dtype & ROCM_BIAS_PER_ROW) != 0;
+            const BiasTerm bias = load_bias(p.bias, p.bias_dtype, 0, p.n, col);
 #pragma unroll
             for (int rb = 0; rb < RB; ++rb) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const int row = rb * 16 + 4 * g + r;
-                    if (row < p.m) store_from_f32(p.y, p.y_dtype, static_cast<int64_t>(row) * p.n + col, add_bias(y[rb][r], bias, p.y_dtype));
+                    if (row < p.m) store_from_f32(p.y, p.y_dtype, static_cast<int64_t>(row) * p.n + col, add_bias(y[rb][r], per_row ? load_bias(p.bias, p.bias_dtype, row, p.n, col) : bias, p.y_dtype));
                 }
             }
         }
@@ -945,7 +946,7 @@ __global__ __launch_bounds__(512) void acc4_packed_kernel(Acc4PackedParams p)
         if (col < p.n) {
             float total = 0.f;
             for (int w = 0; w < waves; ++w) total += red[w * 16 + threadIdx.x];
-            total = with_bias(total, p.bias, p.bias_dtype, col, p.y_dtype);
+            total = with_bias(total, p.bias, p.bias_dtype, 0, p.n, col, p.y_dtype);       // one row
             store_from_f32(p.y, p.y_dtype, col, total);
         }
     }

@@ -163,7 +163,7 @@ __global__ __launch_bounds__(kF32Waves * 64) void gemv_f32_kernel(GemvF32Params 
         v += __shfl_xor(v, 4, 64);
         v += __shfl_xor(v, 8, 64);
         if (sub == 0 && live && r < p.m) {
-            v = with_bias(v, p.bias, p.bias_dtype, col, p.y_dtype);
+            v = with_bias(v, p.bias, p.bias_dtype, r, p.n, col, p.y_dtype);
             store_from_f32(p.y, p.y_dtype, r * p.n + col, v);
         }
     }

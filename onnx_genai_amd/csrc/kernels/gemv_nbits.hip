@@ -102,7 +102,7 @@ __global__ __launch_bounds__(256) void gemv_nbits_kernel(RocmMatMulNBitsArgs p, 
 #pragma unroll
     for (int r = 0; r < ROWS; ++r) {
         const float total = wave_sum(acc[r]);
-        if (lane == 0 && r < rows) store_from_f32(p.y, p.y_dtype, (row0 + r) * p.n + col, with_bias(total, p.bias, p.bias_dtype, col, p.y_dtype));
+        if (lane == 0 && r < rows) store_from_f32(p.y, p.y_dtype, (row0 + r) * p.n + col, with_bias(total, p.bias, p.bias_dtype, row0 + r, p.n, col, p.y_dtype));
     }
 }
 
@@ -166,7 +166,7 @@ __global__ __launch_bounds__(256) void gemv_q8_kernel(RocmMatMulNBitsArgs p, int
 #pragma unroll
     for (int r = 0; r < ROWS; ++r) {
         const float total = wave_sum(acc[r]);
-        if (lane == 0 && r < p.m) store_from_f32(p.y, p.y_dtype, r * p.n + col, with_bias(total, p.bias, p.bias_dtype, col, p.y_dtype));
+        if (lane == 0 && r < p.m) store_from_f32(p.y, p.y_dtype, r * p.n + col, with_bias(total, p.bias, p.bias_dtype, r, p.n, col, p.y_dtype));
     }
 }
 

@@ -286,7 +286,9 @@ __global__ __launch_bounds__(512) void prefill_mfma_kernel(PrefillParams p)
     for (int j = 0; j < TN; ++j) {
         const int64_t col = n_base + wn * WN + j * 32 + col_in_tile;
         if (col >= p.n) continue;
-        const BiasTerm bias = load_bias(p.partial ? nullptr : p.bias, p.bias_dtype, col);     // slices: the reduce kernel adds it
+        const void* bias_ptr = p.partial ? nullptr : p.bias;                                   // slices: the reduce kernel adds it
+        const bool per_row = (p.bias_dtype & ROCM_BIAS_PER_ROW) != 0;
+        const BiasTerm bias = load_bias(bias_ptr, p.bias_dtype, 0, p.n, col);
         float* part = p.partial ? p.partial + static_cast<int64_t>(blockIdx.z) * p.m * p.n : nullptr;
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
@@ -297,7 +299,7 @@ __global__ __launch_bounds__(512) void prefill_mfma_kernel(PrefillParams p)
                     const int64_t row = m_base + wm * WM + i * 32 + q * 8 + row_group + r;
                     if (row >= p.m) continue;
                     if (part) part[row * p.n + col] = acc[i][j][q * 4 + r];
-                    else store_from_f32(p.y, p.y_dtype, row * p.n + col, add_bias(acc[i][j][q * 4 + r], bias, p.y_dtype));
+                    else store_from_f32(p.y, p.y_dtype, row * p.n + col, add_bias(acc[i][j][q * 4 + r], per_row ? load_bias(bias_ptr, p.bias_dtype, row, p.n, col) : bias, p.y_dtype));
                 }
             }
         }
@@ -312,7 +314,7 @@ __global__ __launch_bounds__(256) void prefill_reduce_kernel(const float* __rest
     for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < total; i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
         float sum = 0.f;
         for (int z = 0; z < splits; ++z) sum += partial[z * total + i];
-        store_from_f32(y, y_dtype, i, with_bias(sum, bias, bias_dtype, i % n, y_dtype));
+        store_from_f32(y, y_dtype, i, with_bias(sum, bias, bias_dtype, i / n, n, i % n, y_dtype));
     }
 }
 

@@ -464,6 +464,7 @@ class DeviceOperands:
         self.scales = ep.upload(scales)
         self.zp = ep.upload(np.asarray(zp, np.uint8)) if zp is not None else None
         self.bias = ep.upload(bias) if bias is not None else None
+        self.bias_per_row = bias is not None and np.asarray(bias).size != n      # a folded residual [M, N] in the bias slot
         self.gamma = ep.upload(gamma) if gamma is not None else None        # RMS-normalization prologue: gamma [K] at input 6
         self.gamma_dtype = gamma_dtype
         shapes = None
@@ -484,7 +485,8 @@ class DeviceOperands:
             ins.append(TensorView(self.g_idx.ptr, I32, (self.k,), device_index=dev))
         if self.bias is not None or self.gamma is not None:
             ins.append(TensorView(self.g_idx.ptr, I32, (self.k,), device_index=dev) if self.g_idx is not None else TensorView.absent(I32))
-            ins.append(TensorView(self.bias.ptr, self.bias_dtype, (self.n,), device_index=dev) if self.bias is not None else TensorView.absent(F32))
+            bias_shape = (m, self.n) if self.bias_per_row else (self.n,)
+            ins.append(TensorView(self.bias.ptr, self.bias_dtype, bias_shape, device_index=dev) if self.bias is not None else TensorView.absent(F32))
         if self.gamma is not None:
             ins.append(TensorView(self.gamma.ptr, self.gamma_dtype, (self.k,), device_index=dev))
         return ins

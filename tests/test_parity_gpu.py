@@ -542,6 +542,30 @@ def test_folded_bias_rounds_twice(ep_tiled, port, a_dt, bs, acc, m, n, k):
     assert not np.array_equal(np.asarray(folded).view(np.uint16), np.asarray(fused).view(np.uint16)) or m * n < 2000
 
 
+@pytest.mark.parametrize("folded", [1, None])
+@pytest.mark.parametrize("a_dt,bs,acc,m,n,k", [c for c in FOLDED_BIAS_CASES if c[3] > 1] + [(E.F16, 32, 0, 25, 130, 896), (E.F32, 32, 0, 7, 100, 256)])
+def test_residual_in_the_bias_slot(ep_tiled, port, folded, a_dt, bs, acc, m, n, k):
+    """A bias of Y's shape is a per-token residual (row stride N) - what the CUDA provider's folded residual epilogue passes
+    (kernels/matmul_nbits.rs:7891-7897). With folded_bias it is added after the accumulator was rounded, else before."""
+    ep = ep_tiled
+    b, s, zp = synth.make_weights(n, k, bs, 710 + n, zero_points=True, scale_lo=0.002, scale_hi=0.01, scale_dtype=a_dt)
+    a = synth.make_activation(m, k, 710 + m, a_dt)
+    residual = synth.to_dtype((np.random.default_rng(n + m).standard_normal((m, n)) * 0.5).astype(np.float32), a_dt)
+    o_dt = {E.F16: oracle.F16, E.BF16: oracle.BF16, E.F32: oracle.F32}[a_dt]
+    got, v1 = run_op(ep, a, a_dt, b, s, a_dt, zp, n, k, bs, accuracy_level=acc, bias=residual, bias_dtype=a_dt, folded_bias=folded)
+    if folded and a_dt != E.F32:
+        plain, v0 = run_op(ep, a, a_dt, b, s, a_dt, zp, n, k, bs, accuracy_level=acc)
+        want = port.narrow(synth.to_f32(plain, a_dt) + synth.to_f32(residual, a_dt), o_dt)
+    else:
+        plain32, v0 = run_op(ep, a, a_dt, b, s, a_dt, zp, n, k, bs, accuracy_level=acc, y_dtype=E.F32)
+        want = port.narrow(plain32 + synth.to_f32(residual, a_dt), o_dt) if a_dt != E.F32 else plain32 + residual
+    assert v0 == v1
+    if a_dt == E.F32:
+        assert np.array_equal(np.asarray(got), np.asarray(want))
+    else:
+        assert np.array_equal(np.asarray(got).view(np.uint16), np.asarray(want).view(np.uint16))
+
+
 def test_folded_bias_keeps_tall_calls_off_the_library_gemm(ep):
     """The library's epilogue adds a bias before the one rounding, so a folded bias stays on the hand-written kernel."""
     a_dt, bs, m, n, k = E.F16, 32, 1100, 136, 512
