@@ -280,26 +280,72 @@ __global__ __launch_bounds__(512) void prefill_mfma_kernel(PrefillParams p)
     }
 
     // Epilogue. A 32x32 accumulator holds, in lane l, column l % 32 and rows 8 q + 4 (l / 32) + r (q, r = 0..3).
+    // The three forms (slice partials, one bias per column, one bias per element) are separate loops behind
+    // wave-uniform branches; the first two are fully unrolled over the accumulators and must stay small, or the
+    // compiler keeps the accumulators of the 256x256 tile in scratch memory for the whole kernel.
     const int col_in_tile = lane & 31;
     const int row_group = (lane >> 5) * 4;
+    const bool per_row = (p.bias_dtype & ROCM_BIAS_PER_ROW) != 0;
+    auto for_each = [&](auto&& store) {
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-        const int64_t col = n_base + wn * WN + j * 32 + col_in_tile;
-        if (col >= p.n) continue;
-        const void* bias_ptr = p.partial ? nullptr : p.bias;                                   // slices: the reduce kernel adds it
-        const bool per_row = (p.bias_dtype & ROCM_BIAS_PER_ROW) != 0;
-        const BiasTerm bias = load_bias(bias_ptr, p.bias_dtype, 0, p.n, col);
-        float* part = p.partial ? p.partial + static_cast<int64_t>(blockIdx.z) * p.m * p.n : nullptr;
+        for (int j = 0; j < TN; ++j) {
+            const int64_t col = n_base + wn * WN + j * 32 + col_in_tile;
+            if (col >= p.n) continue;
 #pragma unroll
-        for (int i = 0; i < TM; ++i) {
+            for (int i = 0; i < TM; ++i) {
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
+                for (int q = 0; q < 4; ++q) {
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int64_t row = m_base + wm * WM + i * 32 + q * 8 + row_group + r;
-                    if (row >= p.m) continue;
-                    if (part) part[row * p.n + col] = acc[i][j][q * 4 + r];
-                    else store_from_f32(p.y, p.y_dtype, row * p.n + col, add_bias(acc[i][j][q * 4 + r], per_row ? load_bias(bias_ptr, p.bias_dtype, row, p.n, col) : bias, p.y_dtype));
+                    for (int r = 0; r < 4; ++r) {
+                        const int64_t row = m_base + wm * WM + i * 32 + q * 8 + row_group + r;
+                        if (row >= p.m) continue;
+                        store(row, col, acc[i][j][q * 4 + r]);
+                    }
+                }
+            }
+        }
+    };
+    if (p.partial) {                                                                           // slices: the reduce kernel adds the bias
+        float* part = p.partial + static_cast<int64_t>(blockIdx.z) * p.m * p.n;
+        for_each([&](int64_t row, int64_t col, float v) { part[row * p.n + col] = v; });
+    } else if (per_row) {
+        // The bias differs per element, so its load (a choice among three types) sits in a loop that is not
+        // unrolled: sixteen accumulators at a time go through the wave's own 4 KiB of LDS, which gives that loop a
+        // run-time index. The tiles in LDS are dead once every wave is past its last step.
+        __syncthreads();
+        float* stage = reinterpret_cast<float*>(smem) + wave * (16 * 64) + lane;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int64_t col = n_base + wn * WN + j * 32 + col_in_tile;
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) stage[e * 64] = acc[i][j][e];
+                if (col >= p.n) continue;
+#pragma unroll 1
+                for (int e = 0; e < 16; ++e) {
+                    const int64_t row = m_base + wm * WM + i * 32 + (e >> 2) * 8 + row_group + (e & 3);
+                    if (row >= p.m) break;
+                    store_from_f32(p.y, p.y_dtype, row * p.n + col, with_bias(stage[e * 64], p.bias, p.bias_dtype, row, p.n, col, p.y_dtype));
+                }
+            }
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int64_t col = n_base + wn * WN + j * 32 + col_in_tile;
+            if (col >= p.n) continue;
+            const BiasTerm bias = load_bias(p.bias, p.bias_dtype, 0, p.n, col);
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const int64_t row = m_base + wm * WM + i * 32 + q * 8 + row_group + r;
+                        if (row >= p.m) continue;
+                        store_from_f32(p.y, p.y_dtype, row * p.n + col, add_bias(acc[i][j][q * 4 + r], bias, p.y_dtype));
+                    }
                 }
             }
         }
