@@ -704,12 +704,22 @@ static int launch_wide_bs(const PackedParams& p, int bs, hipStream_t stream)
             // best without the sums and with the windows two ahead (68 -> 64 us); fewer workgroups than CUs with weights
             // and windows both ahead (17.2 -> 14.5 us); in between neither helps (20.6 us either way).
             if (grid.x >= 768) return go(decode_wide_kernel<BF16, BS, ST, 1, false, false, true>, lds16);
-            if (grid.x < 256) return go(decode_wide_kernel<BF16, BS, ST, 1, true, true, true>, lds16 + sums16);
+            // (block size 32 carries four times the scales per window: with both ahead it spills)
+            if constexpr (BS != 32) {
+                if (grid.x < 256) return go(decode_wide_kernel<BF16, BS, ST, 1, true, true, true>, lds16 + sums16);
+            }
             return go(decode_wide_kernel<BF16, BS, ST, 1, true, false, false>, lds16 + sums16);
         }
-        if (p.m <= 32) return go(decode_wide_kernel<BF16, BS, ST, 2, true, false, false>, 2 * 32 * (4 * 256 + 16) + 2 * 4 * NBT * 32 * 4);
+        // More row blocks per wave only where they fit the register file: two from block size 64, four at 128. The
+        // spilling forms ran several times slower than the routes that take those calls instead (3584 -> 37888: 153 us
+        // at block 32 and 32 rows against 2 x 37 us in blocks of 16 rows; 258 us at block 64 and 64 rows against 83 us
+        // in the tiled kernel).
         if constexpr (BS == 32) return -1;
-        else return go(decode_wide_kernel<BF16, BS, ST, 4, true, false, false>, 2 * 64 * (2 * 256 + 16) + 2 * 2 * NBT * 64 * 4);
+        else {
+            if (p.m <= 32) return go(decode_wide_kernel<BF16, BS, ST, 2, true, false, false>, 2 * 32 * (4 * 256 + 16) + 2 * 4 * NBT * 32 * 4);
+            if constexpr (BS == 64) return -1;
+            else return go(decode_wide_kernel<BF16, BS, ST, 4, true, false, false>, 2 * 64 * (2 * 256 + 16) + 2 * 2 * NBT * 64 * 4);
+        }
     };
     switch (bs) {
         case 32: return by_rows(std::integral_constant<int, 32>{});
@@ -983,8 +993,12 @@ static int packed_chunk_bytes(const RocmMatMulNBitsArgs* a)
 }  // namespace mnb
 
 // Rows 5..64 only run from the repacked copy in the shared-activation kernel, which wants many column groups.
-// (block size 32 stops at 32 rows: four row blocks of it do not fit the register file)
-static bool wide_shape(const RocmMatMulNBitsArgs* a) { return a->m >= 5 && a->m <= (a->block_size == 32 ? 32 : 64) && a->n >= 16384; }
+// (16 rows at block size 32, 32 at 64, 64 at 128: more row blocks than that do not fit the register file)
+static bool wide_shape(const RocmMatMulNBitsArgs* a)
+{
+    const int64_t max_rows = a->block_size == 32 ? 16 : a->block_size == 64 ? 32 : 64;
+    return a->m >= 5 && a->m <= max_rows && a->n >= 16384;
+}
 
 extern "C" int rocm_decode_packed_eligible(const RocmMatMulNBitsArgs* a)
 {

@@ -232,3 +232,40 @@ def test_bench_refuses_more_than_one_gpu():
     import sys
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert r.returncode != 0 and "one GPU only" in (r.stderr + r.stdout)
+
+
+def test_build_reads_kernel_resource_remarks():
+    """The build refuses kernels that use scratch memory; this pins how it reads the compiler's resource remarks."""
+    from onnx_genai_amd import build
+    tag = "[" + build.REMARKS + "]"
+    err = "\n".join([
+        "k.hip:25:1: remark: Function Name: kernel_a " + tag,
+        "   25 | {",
+        "      | ^",
+        "k.hip:25:1: remark:     VGPRs: 17 " + tag,
+        "k.hip:25:1: remark:     ScratchSize [bytes/lane]: 0 " + tag,
+        "k.hip:25:1: remark:     VGPRs Spill: 0 " + tag,
+        "k.hip:90:1: remark: Function Name: kernel_b " + tag,
+        "k.hip:90:1: remark:     VGPRs: 256 " + tag,
+        "k.hip:90:1: remark:     ScratchSize [bytes/lane]: 524 " + tag,
+        "k.hip:90:1: remark:     VGPRs Spill: 158 " + tag,
+        "k.hip:3:1: warning: unused variable 'x'",
+        "    3 | int x;",
+        "      | ^",
+    ])
+    usage = build._resource_usage(err)
+    assert usage["kernel_a"] == {"VGPRs": 17, "ScratchSize [bytes/lane]": 0, "VGPRs Spill": 0}
+    assert usage["kernel_b"]["ScratchSize [bytes/lane]"] == 524 and usage["kernel_b"]["VGPRs Spill"] == 158
+    assert build._diagnostics(err) == "k.hip:3:1: warning: unused variable 'x'\n    3 | int x;\n      | ^"
+
+
+def test_built_kernels_use_no_scratch():
+    """The report the last build wrote lists every kernel with zero scratch bytes and zero spilled registers."""
+    from onnx_genai_amd import build
+    report = os.path.join(build.OBJ, "kernel_resources.txt")
+    if not os.path.exists(report):
+        pytest.skip("no build report in this tree")
+    lines = [l for l in open(report).read().splitlines() if l.strip()]
+    assert len(lines) > 100
+    for line in lines:
+        assert "ScratchSize [bytes/lane]=0" in line and "VGPRs Spill=0" in line, line

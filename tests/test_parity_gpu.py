@@ -207,7 +207,8 @@ DECODE_CASES = [
     (E.F16, E.F16, 64, True, 16, 98304, 256),
     (E.BF16, E.BF16, 128, True, 12, 98400, 1536),       # the same over three tile groups: a pair of passes and a peeled one
     (E.BF16, E.BF16, 128, True, 17, 16400, 3584),       # up to 64 rows ride on one pass over the weights
-    (E.F16, E.F16, 64, True, 40, 16384, 1024 + 64),
+    (E.F16, E.F16, 64, True, 40, 16384, 1024 + 64),     # block size 64 stops at 32 rows per pass: the tiled kernel takes this one
+    (E.F16, E.F16, 64, True, 25, 16384, 1024 + 64),
     (E.BF16, E.F32, 128, False, 64, 16390, 2048),
     (E.F16, E.F16, 32, True, 30, 16384, 1000),
 ]
@@ -228,7 +229,9 @@ def test_decode_matches_oracle(ep, ep_unpacked, port, prepack, a_dt, s_dt, bs, z
         assert variant == ("decode_mfma_packed" if prepack and (m <= 4 or n >= 16384) else "decode_mfma_splitk")   # m 2..4 at large n: the 4-row kernel
     else:
         unpacked = "decode_mfma_splitk" if m <= 32 else "prefill_mfma_lds" if k % 64 == 0 else "gemv_generic_f32"   # m <= 32: two row blocks
-        assert variant == ("decode_mfma_packed" if prepack else unpacked)
+        # rows per pass over the repacked weights: 16 at block size 32 (17..32 rows go as two such passes), 32 at 64, 64 at 128
+        packed_rows = 32 if bs <= 64 else 64
+        assert variant == ("decode_mfma_packed" if prepack and m <= packed_rows else unpacked)
     # The kernel carries each weight as (2^10 + q) in f16 or (2^7 + q) in bf16 and cancels the offset inside the
     # f32 accumulator, which costs 10 (7) of its 24 bits: a few 1e-5 on outputs that themselves cancel.
     # (The tiled kernel, which serves these row counts when nothing is repacked, rounds weights to 16 bits in LDS.)
