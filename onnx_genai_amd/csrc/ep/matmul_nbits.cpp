@@ -323,14 +323,26 @@ const void* rows_of_bias(const RocmMatMulNBitsArgs& args, int64_t row0)
 }
 
 // 17..32 rows as two blocks of at most 16 through the decode kernels. The tiled kernel needs a few hundred rows to
-// pay for itself; below that a call costs what streaming the weights costs, and two streams are still cheaper than
-// one under-filled tiled launch (measured at the 7B shapes: 19.8 against 22.6 us, 38 against 55 us; three are not). Returns false (nothing launched) when the decode kernels do not take the shape.
+// pay for itself; below that a call costs what streaming the weights costs, and two streams can be cheaper than one
+// under-filled tiled launch. Measured against the tiled kernel (which slices K for small grids), bf16:
+//   block 128, 3584 -> 3584 / 4096 -> 4096 / 18944 -> 3584 / 14336 -> 4096: blocks win at 17, 24 and 32 rows
+//     (11.9-13.1 against 14.5-15.8 us; 12.3-13.8 against 16.2-16.7; 28-36 against 38-39; 25-31 against 34-35);
+//   block 128, 4096 -> 14336: 26.7 against 30.0 us at 17 rows, 31.5 against 30.3 at 24, 35.9 against 31.1 at 32;
+//   block 64, 4096 -> 14336: the tiled kernel wins throughout (33-47 against 30-31.5 us);
+//   block 32, 896 -> 4864 / 4864 -> 896 / 2048 -> 8192: the tiled kernel wins or ties (10.5-18.8 against 11.0-15.9 us).
+// So: blocks over the repacked copy whenever it applies (one pass per block at full stream rate); otherwise blocks only
+// at block size 128, and there up to 8192 columns or up to 24 rows. Returns false (nothing launched) when the decode
+// kernels do not take the shape or the tiled kernel is the better route.
 bool decode_in_row_blocks(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& args, int& rc)
 {
     rc = 0;
     RocmMatMulNBitsArgs probe = args;
     probe.m = 16;
     if (!rocm_decode_mfma_eligible(&probe)) return false;
+    int probe_rc = 0;
+    if (!use_packed(kn, probe, probe_rc) && rocm_prefill_mfma_eligible(&args) &&
+        !(args.block_size >= 128 && (args.n <= 8192 || args.m <= 24)))
+        return false;
     const size_t a_elem = 2;                                            // eligibility means f16 / bf16 activations
     const size_t y_elem = args.y_dtype == ROCM_DT_F32 ? 4 : 2;
     bool all_packed = true;

@@ -228,7 +228,9 @@ def test_decode_matches_oracle(ep, ep_unpacked, port, prepack, a_dt, s_dt, bs, z
     if m <= 16:
         assert variant == ("decode_mfma_packed" if prepack and (m <= 4 or n >= 16384) else "decode_mfma_splitk")   # m 2..4 at large n: the 4-row kernel
     else:
-        unpacked = "decode_mfma_splitk" if m <= 32 else "prefill_mfma_lds" if k % 64 == 0 else "gemv_generic_f32"   # m <= 32: two row blocks
+        # m <= 32: two row blocks through the decode kernel where that beats the tiled kernel (block 128, few columns or rows)
+        row_blocks = m <= 32 and (k % 64 != 0 or (bs >= 128 and (n <= 8192 or m <= 24)))
+        unpacked = "decode_mfma_splitk" if row_blocks else "prefill_mfma_lds" if k % 64 == 0 else "gemv_generic_f32"
         # rows per pass over the repacked weights: 16 at block size 32 (17..32 rows go as two such passes), 32 at 64, 64 at 128
         packed_rows = 32 if bs <= 64 else 64
         assert variant == ("decode_mfma_packed" if prepack and m <= packed_rows else unpacked)
@@ -464,7 +466,7 @@ def test_prefill_matches_oracle(ep_tiled, port, a_dt, s_dt, bs, zero_points, m, 
     bias = synth.to_dtype(np.random.default_rng(n).standard_normal(n).astype(np.float32), a_dt)
     want64 = oracle_f64(port, a, a_dt, b, s, s_dt, zp, n, k, bs, bias, a_dt)
     y32, variant = run_op(ep, a, a_dt, b, s, s_dt, zp, n, k, bs, bias=bias, bias_dtype=a_dt, y_dtype=E.F32)
-    assert variant == "prefill_mfma_lds" if m > 32 else variant.startswith("decode_mfma")    # up to 32 rows: row blocks through the decode kernels
+    assert variant == "prefill_mfma_lds" if m > 32 else variant in ("prefill_mfma_lds", "decode_mfma_splitk", "decode_mfma_packed")   # up to 32 rows: row blocks through the decode kernels where they pay
     assert helpers.rel_l2(y32, want64) <= TOL_HALF
     y, _ = run_op(ep, a, a_dt, b, s, s_dt, zp, n, k, bs, bias=bias, bias_dtype=a_dt)
     assert helpers.rel_l2(synth.to_f32(y, a_dt), want64) <= TOL_HALF
