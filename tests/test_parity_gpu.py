@@ -485,6 +485,20 @@ def test_prefill_tile_shapes_agree(port, tile, a_dt, s_dt, bs, zero_points):
         y32, variant = run_op(provider, a, a_dt, b, s, s_dt, zp, n, k, bs, y_dtype=E.F32)
         assert variant == "prefill_mfma_lds"
         assert helpers.rel_l2(y32, oracle_f64(port, a, a_dt, b, s, s_dt, zp, n, k, bs)) <= TOL_HALF
+        # The epilogue forms of each tile against that f32 output, bit for bit: a bias per column, a residual per element
+        # (added before the one rounding) and a folded residual (added after the accumulator was rounded).
+        o_dt = {E.F16: oracle.F16, E.BF16: oracle.BF16}[a_dt]
+        bits = lambda t: np.asarray(t).view(np.uint16)
+        rng = np.random.default_rng(tile)
+        bias = synth.to_dtype(rng.standard_normal(n).astype(np.float32), a_dt)
+        residual = synth.to_dtype((rng.standard_normal((m, n)) * 0.5).astype(np.float32), a_dt)
+        y, _ = run_op(provider, a, a_dt, b, s, s_dt, zp, n, k, bs, bias=bias, bias_dtype=a_dt)
+        assert np.array_equal(bits(y), bits(port.narrow(y32 + synth.to_f32(bias, a_dt)[None, :], o_dt)))
+        y, _ = run_op(provider, a, a_dt, b, s, s_dt, zp, n, k, bs, bias=residual, bias_dtype=a_dt)
+        assert np.array_equal(bits(y), bits(port.narrow(y32 + synth.to_f32(residual, a_dt), o_dt)))
+        y, _ = run_op(provider, a, a_dt, b, s, s_dt, zp, n, k, bs, bias=residual, bias_dtype=a_dt, folded_bias=1)
+        rounded = synth.to_f32(port.narrow(y32, o_dt), a_dt)
+        assert np.array_equal(bits(y), bits(port.narrow(rounded + synth.to_f32(residual, a_dt), o_dt)))
     finally:
         provider.shutdown()
 
