@@ -567,13 +567,17 @@ __global__ __launch_bounds__(512) void acc4_prefill_kernel(Acc4PrefillParams p)
 }
 
 // Slices of K for a grid that leaves CUs idle. Two workgroups of the two-set variant share a CU, so up to 512 run at
-// once: slices bring the grid to at most that, with at least 8 steps each, a whole number of blocks per slice, at most 8.
+// once (block size 32 keeps four register sets: one workgroup per CU, 256 at once): slices bring the grid to at most
+// that, with at least 8 steps each, a whole number of blocks per slice, at most 8.
 static int acc4_prefill_slices(int64_t m, int64_t n, int64_t padded_k, int block_size)
 {
     const int64_t tiles = ((n + kTile - 1) / kTile) * ((m + kTile - 1) / kTile);
     const int64_t steps = (padded_k + kStep - 1) / kStep;
-    if (block_size < 64 || tiles > 170) return 1;          // block size 32 keeps four register sets: one workgroup per CU
-    int64_t want = 512 / tiles;
+    const int64_t resident = block_size < 64 ? 256 : 512;
+    // Two slices pay at block size 32 (4096 -> 14336, 17..128 rows: 70-78 -> 44-56 us) and not from 64 up, where they
+    // fill the second workgroup slot of each CU (8192 -> 28672 at block 64, 64 / 128 rows: 112 -> 120 us, 123 -> 137 us).
+    if (tiles > (block_size < 64 ? resident / 2 : resident / 3)) return 1;
+    int64_t want = resident / tiles;
     if (want > 8) want = 8;
     if (want > steps / 8) want = steps / 8;
     return want < 2 ? 1 : static_cast<int>(want);

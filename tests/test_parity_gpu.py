@@ -1061,6 +1061,8 @@ ACC4_CASES = [
     (E.BF16, 128, True, 130, 200, 128 * 20),  # five slices of whole blocks (two steps per block)
     (E.F16, 256, False, 64, 130, 256 * 9),    # slices rounded up to whole blocks of four steps
     (E.F16, 64, True, 40, 96, 64 * 17),       # two unequal slices
+    (E.F16, 32, True, 130, 200, 32 * 80),     # block size 32 (two blocks per step): five slices
+    (E.BF16, 32, False, 40, 96, 32 * 35),     # block size 32, two slices, K ends in the middle of a step
     (E.F16, 32, False, 17, 130, 200),         # K ends inside a block
     (E.F16, 16, True, 20, 64, 256),           # block size 16: not a matrix-core shape
 ]
