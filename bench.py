@@ -295,6 +295,8 @@ def main():
                     help="run only the roofline leg (decode kernel on the gate_up shape) and one 256 MiB device copy: the command profiles are taken from")
     ap.add_argument("--only-tables", action="store_true",
                     help="run only the prefill and accuracy_level=4 tables, one JSON line per row (the command their profiles are taken from)")
+    ap.add_argument("--row-sweep", action="store_true",
+                    help="run only a sweep of the row count M across the dispatch boundaries (1 .. 2048), one JSON line per call shape")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (no collectives exist on the MatMulNBits path); use --gpus 1")
@@ -303,6 +305,10 @@ def main():
     info = ep.device_info()
     if args.only_roofline:
         return roofline_only(ep, args)
+    if args.row_sweep:
+        for row in row_sweep(ep):
+            print(json.dumps(row), flush=True)
+        return
     if args.only_tables:
         for row in prefill_table(ep) + prefill_7b_table(ep) + acc4_table(ep):
             print(json.dumps(row), flush=True)
@@ -444,6 +450,37 @@ def sweep(ep, nodes, a_bufs, args):
     for clone in extra:
         clone.free(ep)
     return table
+
+
+ROW_SWEEP_ROWS = (1, 2, 4, 5, 8, 16, 17, 24, 32, 33, 48, 64, 65, 128, 256, 512, 1023, 1024, 2048)
+ROW_SWEEP_SHAPES = (   # block size, K, N, accuracy_level
+    (128, 4096, 14336, 0), (32, 4096, 14336, 0), (64, 4096, 14336, 0), (128, 3584, 37888, 0), (32, 3584, 37888, 0), (64, 3584, 37888, 0),
+    (128, 4096, 14336, 4), (32, 4096, 14336, 4),
+)
+
+
+def row_sweep(ep):
+    """Time per call against the row count M, bf16 with zero points, on the default dispatch: each step in the table should
+    cost no more than the rows it adds (a step that does marks a kernel boundary placed at the wrong M). Two copies of the
+    weights per graph, replayed after a warm-up that also brings the GPU clock up."""
+    out = []
+    for bs, k, n, acc in ROW_SWEEP_SHAPES:
+        for m in ROW_SWEEP_ROWS:
+            nodes = [Node(ep, f"w{i}", k, n, bs, i, E.BF16, m, accuracy_level=acc) for i in range(2)]
+            a = ep.upload(synth.make_activation(m, k, 5, E.BF16))
+            for nd in nodes:
+                nd.run(a)
+            ep.sync()
+            graph = capture(ep, lambda: [nd.run(a) for nd in nodes])
+            # the first of a shape follows the previous shape's tall GEMMs and host-side weight generation: ~50 ms of replays first
+            ms = time_graph(ep, graph, 20, 2000 if m == 1 else 20) / len(nodes)
+            out.append({"block_size": bs, "k": k, "n": n, "accuracy_level": acc, "m": m, "us": round(ms * 1e3, 1),
+                        "tflops": round(nodes[0].flops / ms / 1e9, 1), "gbs": round(nodes[0].bytes / ms / 1e6, 1),
+                        "variant": nodes[0].ops.kernel.last_variant()})
+            for nd in nodes:
+                nd.free(ep)
+            ep.deallocate(a)
+    return out
 
 
 def prefill_routes(ep):
