@@ -331,7 +331,8 @@ const void* rows_of_bias(const RocmMatMulNBitsArgs& args, int64_t row0)
 //   block 64, 4096 -> 14336: the tiled kernel wins throughout (33-47 against 30-31.5 us);
 //   block 32, 896 -> 4864 / 4864 -> 896 / 2048 -> 8192: the tiled kernel wins or ties (10.5-18.8 against 11.0-15.9 us).
 // So: blocks over the repacked copy whenever it applies (one pass per block at full stream rate); otherwise blocks only
-// at block size 128, and there up to 8192 columns or up to 24 rows. Returns false (nothing launched) when the decode
+// at block size 128, and there up to 8192 columns or up to 20 rows (a second block of at most four rows is the cheap one;
+// at 24 rows the two routes tie or the tiled kernel leads). Returns false (nothing launched) when the decode
 // kernels do not take the shape or the tiled kernel is the better route.
 bool decode_in_row_blocks(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& args, int& rc)
 {
@@ -341,7 +342,7 @@ bool decode_in_row_blocks(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& ar
     if (!rocm_decode_mfma_eligible(&probe)) return false;
     int probe_rc = 0;
     if (!use_packed(kn, probe, probe_rc) && rocm_prefill_mfma_eligible(&args) &&
-        !(args.block_size >= 128 && (args.n <= 8192 || args.m <= 24)))
+        !(args.block_size >= 128 && (args.n <= 8192 || args.m <= 20)))
         return false;
     const size_t a_elem = 2;                                            // eligibility means f16 / bf16 activations
     const size_t y_elem = args.y_dtype == ROCM_DT_F32 ? 4 : 2;

@@ -229,7 +229,7 @@ def test_decode_matches_oracle(ep, ep_unpacked, port, prepack, a_dt, s_dt, bs, z
         assert variant == ("decode_mfma_packed" if prepack and (m <= 4 or n >= 16384) else "decode_mfma_splitk")   # m 2..4 at large n: the 4-row kernel
     else:
         # m <= 32: two row blocks through the decode kernel where that beats the tiled kernel (block 128, few columns or rows)
-        row_blocks = m <= 32 and (k % 64 != 0 or (bs >= 128 and (n <= 8192 or m <= 24)))
+        row_blocks = m <= 32 and (k % 64 != 0 or (bs >= 128 and (n <= 8192 or m <= 20)))
         unpacked = "decode_mfma_splitk" if row_blocks else "prefill_mfma_lds" if k % 64 == 0 else "gemv_generic_f32"
         # rows per pass over the repacked weights: 16 at block size 32 (17..32 rows go as two such passes), 32 at 64, 64 at 128
         packed_rows = 32 if bs <= 64 else 64
