@@ -206,6 +206,8 @@ DECODE_CASES = [
     (E.BF16, E.BF16, 128, True, 9, 98400, 512),         # three or more workgroups per CU: the variant with the second MFMA
     (E.F16, E.F16, 64, True, 16, 98304, 256),
     (E.BF16, E.BF16, 128, True, 12, 98400, 1536),       # the same over three tile groups: a pair of passes and a peeled one
+    (E.BF16, E.BF16, 128, True, 16, 14336, 1024),       # the narrowest shape the shared-activation kernel takes (fewer workgroups than CUs)
+    (E.F16, E.F16, 64, True, 11, 14400, 512),
     (E.BF16, E.BF16, 128, True, 17, 16400, 3584),       # up to 64 rows ride on one pass over the weights
     (E.F16, E.F16, 64, True, 40, 16384, 1024 + 64),     # block size 64 stops at 32 rows per pass: the tiled kernel takes this one
     (E.F16, E.F16, 64, True, 25, 16384, 1024 + 64),
@@ -226,7 +228,8 @@ def test_decode_matches_oracle(ep, ep_unpacked, port, prepack, a_dt, s_dt, bs, z
     # f32 output: the arithmetic itself, before any narrowing
     y32, variant = run_op(ep, a, a_dt, b, s, s_dt, zp, n, k, bs, bias=bias, bias_dtype=a_dt, y_dtype=E.F32)
     if m <= 16:
-        assert variant == ("decode_mfma_packed" if prepack and (m <= 4 or n >= 16384) else "decode_mfma_splitk")   # m 2..4 at large n: the 4-row kernel
+        wide = n >= 16384 or (n >= 14336 and bs >= 64)      # columns from which the shared-activation kernel takes 5..16 rows
+        assert variant == ("decode_mfma_packed" if prepack and (m <= 4 or wide) else "decode_mfma_splitk")   # m 2..4 at large n: the 4-row kernel
     else:
         # m <= 32: two row blocks through the decode kernel where that beats the tiled kernel (block 128, few columns or rows)
         row_blocks = m <= 32 and (k % 64 != 0 or (bs >= 128 and (n <= 8192 or m <= 20)))
