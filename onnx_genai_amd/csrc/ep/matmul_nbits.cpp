@@ -341,7 +341,9 @@ bool decode_in_row_blocks(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& ar
     probe.m = 16;
     if (!rocm_decode_mfma_eligible(&probe)) return false;
     int probe_rc = 0;
-    if (!use_packed(kn, probe, probe_rc) && rocm_prefill_mfma_eligible(&args) &&
+    // (block size 32 below 16384 columns: two repacked passes of 16 rows take 41 us where the tiled kernel takes 32)
+    const bool packed_blocks = use_packed(kn, probe, probe_rc) && !(args.block_size == 32 && args.n < 16384);
+    if (!packed_blocks && rocm_prefill_mfma_eligible(&args) &&
         !(args.block_size >= 128 && (args.n <= 8192 || args.m <= 20)))
         return false;
     const size_t a_elem = 2;                                            // eligibility means f16 / bf16 activations

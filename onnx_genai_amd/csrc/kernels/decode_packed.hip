@@ -1000,8 +1000,8 @@ static bool wide_shape(const RocmMatMulNBitsArgs* a)
     // Columns from which it beats the split-K and tiled kernels (bf16, 4096 -> 14336: 19.9 -> 14.6 us at 16 rows and
     // 30.6 -> 24.4 at 32 with block 128, 20-24 -> 16 and 31.5 -> 25.7 with block 64; at 12288 columns it ties at 16 rows
     // and loses 2 us at 5-8; at 9216 and below it loses throughout, and so do 33-64 rows below 16384 columns:
-    // 32.9 -> 38.7 us). Block size 32 stays at 16384: its 17-32 rows would go as two passes (41 us against 32 tiled).
-    const int64_t min_cols = (a->block_size == 32 || a->m > 32) ? 16384 : 14336;
+    // 32.9 -> 38.7 us). Block size 32: 20.7 -> 20.3 us at 5-8 rows, 26.1 -> 20.4 at 16 (one pass of 16 rows is all it takes).
+    const int64_t min_cols = a->m > 32 ? 16384 : 14336;
     return a->m >= 5 && a->m <= max_rows && a->n >= min_cols;
 }
 

@@ -208,6 +208,7 @@ DECODE_CASES = [
     (E.BF16, E.BF16, 128, True, 12, 98400, 1536),       # the same over three tile groups: a pair of passes and a peeled one
     (E.BF16, E.BF16, 128, True, 16, 14336, 1024),       # the narrowest shape the shared-activation kernel takes (fewer workgroups than CUs)
     (E.F16, E.F16, 64, True, 11, 14400, 512),
+    (E.F16, E.F16, 32, True, 9, 14336, 512),
     (E.BF16, E.BF16, 128, True, 17, 16400, 3584),       # up to 64 rows ride on one pass over the weights
     (E.F16, E.F16, 64, True, 40, 16384, 1024 + 64),     # block size 64 stops at 32 rows per pass: the tiled kernel takes this one
     (E.F16, E.F16, 64, True, 25, 16384, 1024 + 64),
@@ -228,7 +229,7 @@ def test_decode_matches_oracle(ep, ep_unpacked, port, prepack, a_dt, s_dt, bs, z
     # f32 output: the arithmetic itself, before any narrowing
     y32, variant = run_op(ep, a, a_dt, b, s, s_dt, zp, n, k, bs, bias=bias, bias_dtype=a_dt, y_dtype=E.F32)
     if m <= 16:
-        wide = n >= 16384 or (n >= 14336 and bs >= 64)      # columns from which the shared-activation kernel takes 5..16 rows
+        wide = n >= 14336                                   # columns from which the shared-activation kernel takes 5..16 rows
         assert variant == ("decode_mfma_packed" if prepack and (m <= 4 or wide) else "decode_mfma_splitk")   # m 2..4 at large n: the 4-row kernel
     else:
         # m <= 32: two row blocks through the decode kernel where that beats the tiled kernel (block 128, few columns or rows)
@@ -297,6 +298,18 @@ def test_row_blocks_through_the_decode_kernels(ep, ep_unpacked, port, prepack, m
     assert helpers.rel_l2(y32, oracle_f64(port, a, a_dt, b, s, a_dt, zp, n, k, bs, bias, a_dt)) <= 1e-4
     y, _ = run_op(ep, a, a_dt, b, s, a_dt, zp, n, k, bs, bias=bias, bias_dtype=a_dt)
     assert np.array_equal(np.asarray(y).view(np.uint16), np.asarray(port.narrow(y32, a_dt)).view(np.uint16))
+
+
+def test_block_32_between_14336_and_16384_columns(ep, port):
+    """Block size 32 at 14336 columns: up to 16 rows ride the shared-activation kernel; 17..32 rows go to the tiled kernel,
+    not to two repacked passes."""
+    a_dt, bs, n, k = E.F16, 32, 14336, 256
+    b, s, zp = synth.make_weights(n, k, bs, 77, zero_points=True, scale_lo=0.002, scale_hi=0.01, scale_dtype=a_dt)
+    for m, expected in ((16, "decode_mfma_packed"), (24, "prefill_mfma_lds")):
+        a = synth.make_activation(m, k, 77 + m, a_dt)
+        y32, variant = run_op(ep, a, a_dt, b, s, a_dt, zp, n, k, bs, y_dtype=E.F32)
+        assert variant == expected
+        assert helpers.rel_l2(y32, oracle_f64(port, a, a_dt, b, s, a_dt, zp, n, k, bs)) <= TOL_HALF
 
 
 GRAPH_CASES = [
