@@ -47,7 +47,9 @@ typedef struct NxrtRocmMatMulNBits NxrtRocmMatMulNBits;   /* one kernel = one Ma
  * NXRT_ROCM_DECODE_COL_GROUPS, NXRT_ROCM_PREFILL_TILE when the map does not give them. */
 NxrtStatus nxrt_rocm_ep_create(uint32_t device_ordinal, const char* const* config_keys,
                                const char* const* config_values, uint32_t n_config, NxrtRocmEp** out_ep);
-/* shutdown + drop. Frees the stream and every buffer the provider still owns. */
+/* shutdown + drop. Frees the stream and every buffer the provider still owns. Kernels and allocator vtables made from the
+ * provider each hold a reference to it: the host may release them and the provider in any order, and the provider's
+ * resources go with the last of them. */
 void nxrt_rocm_ep_release(NxrtRocmEp* ep);
 /* name() / device_type() / device_id() / memory_vendor_id() — provider.rs:708-731. */
 const char* nxrt_rocm_ep_name(const NxrtRocmEp* ep);                   /* "RocmExecutionProvider" */
@@ -136,8 +138,10 @@ NxrtStatus nxrt_rocm_matmul_nbits_workspace_requirement(const NxrtRocmMatMulNBit
  * inputs: A, B, scales, [zero_points], [g_idx], [bias]; outputs: Y. workspace may be NULL: the
  * kernel then keeps its own scratch, grown on demand (an allocation inside the call). B is [N, kb, block_size * bits / 8],
  * zero_points [N, ceil(kb * bits / 8)]; g_idx (Int32 [K] or [kb * block_size], accuracy_level 0 only) is range-checked on first
- * use (matmul_nbits.rs:3515-3521). bias is [N], or Y's shape: a per-token residual folded into the bias slot
- * (onnx-runtime-ep-cuda/src/kernels/matmul_nbits.rs:7891-7897). Fused nodes (gate_up_swiglu, rmsnorm_prologue) take their own input lists, see the attributes. */
+ * use (matmul_nbits.rs:3515-3521). bias has N elements in any shape ([N], [1, N], [1, 1, N]: broadcast over the rows), or
+ * rows * N elements: a per-token residual folded into the bias slot, row stride N
+ * (onnx-runtime-ep-cuda/src/kernels/matmul_nbits.rs:7728-7735, 7891-7897). A required tensor with a NULL data pointer is
+ * refused with a status, never launched. Fused nodes (gate_up_swiglu, rmsnorm_prologue) take their own input lists, see the attributes. */
 NxrtStatus nxrt_rocm_matmul_nbits_execute(NxrtRocmMatMulNBits* kernel, const NxrtRocmTensorView* inputs, uint32_t n_inputs,
                                           NxrtRocmTensorView* outputs, uint32_t n_outputs,
                                           void* workspace_device, uint64_t workspace_bytes);
@@ -172,6 +176,15 @@ NxrtStatus nxrt_rocm_matmul_nbits_quantize_a(NxrtRocmEp* ep, const void* a_devic
 NxrtStatus nxrt_rocm_matmul_nbits_block_acc(NxrtRocmEp* ep, const int8_t* qa_device, const void* b_device,
                                             const void* zero_points_device, uint64_t m, uint64_t n, uint64_t k,
                                             uint32_t block_size, int32_t* acc_device);
+
+/* The same integers as the production kernels hold them: with a probe buffer set (int32 [M, N, kb] device memory, NULL
+ * clears it), every later accuracy_level=4 execute of this kernel that runs on the int8 matrix cores also stores each
+ * block accumulator at the moment it is scaled into the f32 result (matmul_nbits.rs:9159-9177: `acc` of `int8_row`).
+ * The launch is the same kernel with the store compiled in; a call the dot-product catch-all would serve is refused. */
+NxrtStatus nxrt_rocm_matmul_nbits_set_block_acc_probe(NxrtRocmMatMulNBits* kernel, int32_t* acc_device, uint64_t capacity_elements);
+/* Device buffers the kernel object has replaced (outgrown scratch, a repacked or dense copy of weights that changed) and
+ * keeps until it is released, because a HIP graph recorded earlier may still replay through them. */
+uint64_t nxrt_rocm_matmul_nbits_retired_buffers(const NxrtRocmMatMulNBits* kernel);
 
 /* ---- timing on the provider's stream (HIP events) ---------------------------------------------- */
 

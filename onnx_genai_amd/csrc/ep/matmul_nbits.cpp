@@ -136,6 +136,8 @@ struct NxrtRocmMatMulNBits {
     NxrtRocmMatMulNBits* up = nullptr;
     bool pair_member = false;            // this kernel is one projection of a fused gate/up node
     const void* g_idx_checked = nullptr; // the g_idx tensor whose groups were found in range
+    int32_t* acc_probe = nullptr;        // accuracy_level 4: where the int8 matrix-core kernels also store their block accumulators (tests)
+    uint64_t acc_probe_elems = 0;
     // RMS-normalization prologue: the activations are normalized into `norm` first (gamma at input 6, or 5 of the fused node)
     bool rmsnorm_prologue = false;
     float rmsnorm_epsilon = 1e-5f;
@@ -157,11 +159,15 @@ struct NxrtRocmMatMulNBits {
     NxrtKernelVtable vtable;
     uint32_t vt_a_dtype = 0, vt_scale_dtype = 0, vt_y_dtype = 0;
 
+    explicit NxrtRocmMatMulNBits(NxrtRocmEp* provider) : ep(provider) { ep->retain(); }     // the kernel keeps its provider alive
+    NxrtRocmMatMulNBits(const NxrtRocmMatMulNBits&) = delete;
+    NxrtRocmMatMulNBits& operator=(const NxrtRocmMatMulNBits&) = delete;
+
     ~NxrtRocmMatMulNBits()
     {
         delete gate;
         delete up;
-        if ((scratch || packed || dense || norm || !retired.empty()) && ep && ep->bind().code == NXRT_OK) {
+        if ((scratch || packed || dense || norm || !retired.empty()) && ep->bind().code == NXRT_OK) {
             rocm_ffi_stream_sync(ep->stream);
             if (norm) rocm_ffi_free(norm);
             for (void* old : retired) rocm_ffi_free(old);
@@ -169,6 +175,7 @@ struct NxrtRocmMatMulNBits {
             if (packed) rocm_ffi_free(packed);
             if (dense) rocm_ffi_free(dense);
         }
+        nxrt_rocm_ep_release(ep);
     }
 };
 
@@ -223,8 +230,7 @@ bool use_packed(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& args, int& r
     if (current) return true;
     if (kn.ep->capturing) return false;
     if (kn.packed) {
-        rocm_ffi_stream_sync(kn.ep->stream);
-        rocm_ffi_free(kn.packed);
+        kn.retired.push_back(kn.packed);    // not freed: a HIP graph recorded over the old weights may still replay through it
         kn.packed = nullptr;
     }
     if (rocm_ffi_malloc(&kn.packed, rocm_decode_packed_bytes(&args)) != 0) {
@@ -232,6 +238,11 @@ bool use_packed(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& args, int& r
         return false;                       // no memory for a second copy: stream the caller's tensors instead
     }
     rc = rocm_launch_pack_decode(&args, kn.packed, kn.ep->stream);
+    if (rc != 0) {                          // a copy that was not made must not pass for current on the next call
+        rocm_ffi_free(kn.packed);
+        kn.packed = nullptr;
+        return false;
+    }
     kn.packed_from[0] = args.b;
     kn.packed_from[1] = args.scales;
     kn.packed_from[2] = args.zp;
@@ -284,8 +295,7 @@ bool dense_route(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& args, int& 
         if (!current) {
             if (ep.capturing) return false;
             if (kn.dense) {
-                rocm_ffi_stream_sync(ep.stream);
-                rocm_ffi_free(kn.dense);
+                kn.retired.push_back(kn.dense);     // kept for graphs recorded over the old weights
                 kn.dense = nullptr;
             }
             if (rocm_ffi_malloc(&kn.dense, need) != 0) {
@@ -340,9 +350,10 @@ bool decode_in_row_blocks(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& ar
     RocmMatMulNBitsArgs probe = args;
     probe.m = 16;
     if (!rocm_decode_mfma_eligible(&probe)) return false;
-    int probe_rc = 0;
-    // (block size 32 below 16384 columns: two repacked passes of 16 rows take 41 us where the tiled kernel takes 32)
-    const bool packed_blocks = use_packed(kn, probe, probe_rc) && !(args.block_size == 32 && args.n < 16384);
+    int probe_rc = 0;       // stays 0: a repack that fails leaves no copy behind and use_packed then answers false
+    // (block size 32 below 16384 columns: two repacked passes of 16 rows take 41 us where the tiled kernel takes 32 -
+    // asked first, so that no repacked copy is made for a call the tiled kernel then takes)
+    const bool packed_blocks = !(args.block_size == 32 && args.n < 16384) && use_packed(kn, probe, probe_rc);
     if (!packed_blocks && rocm_prefill_mfma_eligible(&args) &&
         !(args.block_size >= 128 && (args.n <= 8192 || args.m <= 20)))
         return false;
@@ -456,11 +467,15 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
     if (BIAS && !c.failed) {
         require_float("bias", BIAS->dtype);
         if (!c.failed && !shape_is(*BIAS, {N})) {
-            uint64_t rows = 1;
+            // By element count, as the CUDA sibling does (matmul_nbits.rs:7728-7735): N elements in any shape ([1, N],
+            // [1, 1, N] - the residual of a one-row decode step) broadcast with stride 0, rows * N elements are per-token.
+            uint64_t rows = 1, numel = 1;
             for (uint32_t i = 0; i + 1 < A.ndim; ++i) rows *= A.shape[i];
-            bias_per_row = rows * N != N && (shape_is(*BIAS, y_shape) || shape_is(*BIAS, {rows * N}) || shape_is(*BIAS, {rows, N}));
-            if (!bias_per_row)
-                c.fail("bias must have shape " + shape_str({N}) + " (or Y's shape " + shape_str(y_shape) + " for a folded residual), got " + shape_str(BIAS->shape, BIAS->ndim));
+            for (uint32_t i = 0; i < BIAS->ndim; ++i) numel *= BIAS->shape[i];
+            bias_per_row = numel == rows * N && rows * N != N;
+            if (!bias_per_row && numel != N)
+                c.fail("bias must have " + std::to_string(N) + " elements (broadcast [N]) or " + std::to_string(rows * N) + " elements (a per-token residual of Y's shape " +
+                       shape_str(y_shape) + "), got " + shape_str(BIAS->shape, BIAS->ndim));
         }
     }
     if (c.failed) return make_status(NXRT_INVALID_ARGUMENT, c.message);
@@ -478,6 +493,9 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
     uint64_t M = 1;
     for (uint32_t i = 0; i + 1 < A.ndim; ++i) M *= A.shape[i];
     if (M == 0) return ok();
+    // A required tensor without memory behind it would reach a kernel as address 0: a GPU memory fault instead of a status.
+    for (const Named& t : {Named{"A", &A}, Named{"B", &B}, Named{"scales", &S}, Named{"Y", &Y}})
+        if (t.v->data == nullptr) return make_status(NXRT_INVALID_ARGUMENT, err(std::string(t.name) + " has a null data pointer"));
 
     NxrtStatus st = kn.ep->bind();
     if (st.code != NXRT_OK) return st;
@@ -501,6 +519,14 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
     args.k = kn.k;
     args.block_size = static_cast<int>(kn.block_size);
     args.g_idx = G ? static_cast<const int32_t*>(at(*G)) : nullptr;
+    args.acc_probe = nullptr;
+    if (kn.acc_probe) {
+        if (kn.accuracy_level != 4) return make_status(NXRT_INVALID_ARGUMENT, err("the block-accumulator probe needs accuracy_level=4"));
+        if (M * N * kb > kn.acc_probe_elems)
+            return make_status(NXRT_INVALID_ARGUMENT, err("the block-accumulator probe buffer holds " + std::to_string(kn.acc_probe_elems) + " int32 values, this call needs " +
+                                                          std::to_string(M * N * kb)));
+        args.acc_probe = kn.acc_probe;
+    }
 
     rocm_stream_t stream = kn.ep->stream;
     int rc = 0;
@@ -565,6 +591,7 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
                 rc = rocm_launch_acc4_mfma(&args, &w4, kn.ep->decode_waves, stream);
                 kn.variant = "acc4_mfma_i8";
             } else {
+                if (args.acc_probe) return make_status(NXRT_INVALID_ARGUMENT, err("the block-accumulator probe covers the int8 matrix-core kernels only; this shape runs on the dot-product kernel"));
                 rc = rocm_launch_acc4_gemv(&args, &w4, stream);
                 kn.variant = "acc4_gemv_dot4";
             }
@@ -642,13 +669,20 @@ NxrtStatus execute_swiglu(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in,
     uint64_t M = 1;
     for (uint32_t i = 0; i + 1 < A.ndim; ++i) M *= A.shape[i];
     if (M == 0) return ok();
+    {
+        const char* names[5] = {"x", "W_gate", "scales_gate", "W_up", "scales_up"};
+        for (uint32_t i = 0; i < 5; ++i)
+            if (in[i].data == nullptr) return make_status(NXRT_INVALID_ARGUMENT, err(std::string(names[i]) + " has a null data pointer"));
+        if (Y.data == nullptr) return make_status(NXRT_INVALID_ARGUMENT, err("Y has a null data pointer"));
+    }
     NxrtStatus st = kn.ep->bind();
     if (st.code != NXRT_OK) return st;
 
     // Up to four rows over constant weights: one launch over both repacked copies. The copies are made (and every weight
     // tensor validated) by the projections' own first call below, so this path serves the calls after the first with the
     // same weight tensors; it sums each projection exactly as that first call did.
-    if (M <= 4 && kn.gate->packed && kn.up->packed) {
+    // (accuracy_level 4 stays on its own int8 kernels for every call: the paired launch is the float path)
+    if (M <= 4 && kn.accuracy_level != 4 && kn.gate->packed && kn.up->packed) {
         auto current = [&](const NxrtRocmMatMulNBits& child, const NxrtRocmTensorView& w, const NxrtRocmTensorView& s, const NxrtRocmTensorView* zp) {
             auto at = [](const NxrtRocmTensorView& v) { return static_cast<const void*>(static_cast<const uint8_t*>(v.data) + v.byte_offset); };
             return child.packed_from[0] == at(w) && child.packed_from[1] == at(s) && child.packed_from[2] == (zp ? at(*zp) : nullptr) &&
@@ -881,8 +915,7 @@ NxrtStatus nxrt_rocm_matmul_nbits_create(NxrtRocmEp* ep, const NxrtRocmMatMulNBi
         check_attrs(*attrs, c);
         if (c.failed) return make_status(NXRT_INVALID_ARGUMENT, c.message);
         if (!ep) return make_status(NXRT_INVALID_ARGUMENT, "MatMulNBits: null provider");
-        auto* kn = new NxrtRocmMatMulNBits();
-        kn->ep = ep;
+        auto* kn = new NxrtRocmMatMulNBits(ep);
         kn->k = attrs->K;
         kn->n = attrs->N;
         kn->block_size = attrs->block_size;
@@ -911,8 +944,7 @@ NxrtStatus nxrt_rocm_matmul_nbits_create(NxrtRocmEp* ep, const NxrtRocmMatMulNBi
         if (has_rmsnorm && (attrs->present & (1u << kAttrRmsnormEpsilon))) kn->rmsnorm_epsilon = static_cast<float>(attrs->rmsnorm_epsilon);
         if (kn->gate_up_swiglu) {
             for (NxrtRocmMatMulNBits** child : {&kn->gate, &kn->up}) {
-                auto* c2 = new NxrtRocmMatMulNBits();
-                c2->ep = ep;
+                auto* c2 = new NxrtRocmMatMulNBits(ep);
                 c2->k = kn->k;
                 c2->n = kn->n;
                 c2->block_size = kn->block_size;
@@ -1015,6 +1047,18 @@ uint64_t nxrt_rocm_matmul_nbits_estimated_flops(const NxrtRocmMatMulNBits* kerne
 const char* nxrt_rocm_matmul_nbits_last_variant(const NxrtRocmMatMulNBits* kernel) { return kernel ? kernel->variant.c_str() : ""; }
 
 void nxrt_rocm_matmul_nbits_release(NxrtRocmMatMulNBits* kernel) { vtable_release(kernel); }
+
+NxrtStatus nxrt_rocm_matmul_nbits_set_block_acc_probe(NxrtRocmMatMulNBits* kernel, int32_t* acc_device, uint64_t capacity_elements)
+{
+    if (!kernel) return make_status(NXRT_INVALID_ARGUMENT, "MatMulNBits: null kernel");
+    if (kernel->gate_up_swiglu) return make_status(NXRT_INVALID_ARGUMENT, err("the block-accumulator probe is not offered on the fused gate/up node"));
+    std::lock_guard<std::mutex> lock(kernel->mu);
+    kernel->acc_probe = acc_device;
+    kernel->acc_probe_elems = acc_device ? capacity_elements : 0;
+    return ok();
+}
+
+uint64_t nxrt_rocm_matmul_nbits_retired_buffers(const NxrtRocmMatMulNBits* kernel) { return kernel ? kernel->retired.size() : 0; }
 
 NxrtStatus nxrt_rocm_matmul_nbits_as_vtable(NxrtRocmMatMulNBits* kernel, NxrtKernelVtable** out_vtable)
 {

@@ -51,7 +51,13 @@ NxrtStatus sync_cb(void* ctx)
     if (!h) return make_status(NXRT_INVALID_ARGUMENT, "allocator: null ctx");
     return nxrt_rocm_ep_sync(h->ep);
 }
-void allocator_release_cb(void* ctx) { delete static_cast<AllocatorHandle*>(ctx); }
+void allocator_release_cb(void* ctx)
+{
+    auto* h = static_cast<AllocatorHandle*>(ctx);
+    if (!h) return;
+    nxrt_rocm_ep_release(h->ep);                // the handle's reference: the provider outlives every allocator it handed out
+    delete h;
+}
 
 // ---- EP vtable (vtable.rs:126-168) ----
 NxrtStatus get_capability_cb(void* ctx, const uint8_t* const* op_types, const NxrtTensorDesc* const* input_descs, const uint32_t* num_inputs_per_node,
@@ -64,14 +70,16 @@ NxrtStatus get_capability_cb(void* ctx, const uint8_t* const* op_types, const Nx
         uint32_t claimed = 0;
         for (uint32_t i = 0; i < num_nodes; ++i) {
             if (!op_types[i] || std::strcmp(reinterpret_cast<const char*>(op_types[i]), "MatMulNBits") != 0) continue;
-            // Claim on dtypes alone; attributes are checked when the kernel is created.
+            // Claimed on arity and dtypes alone: this slot carries no attributes, so bits, block_size, weight_prepacked and
+            // accuracy_level (which decides whether a g_idx input is taken) are checked when the kernel is created, and a
+            // node can still be declined there with the reason.
             if (input_descs && num_inputs_per_node && input_descs[i]) {
                 const uint32_t n = num_inputs_per_node[i];
                 const NxrtTensorDesc* d = input_descs[i];
                 if (n < 3 || n > 6) continue;
                 const auto is_float = [](uint32_t dt) { return dt == NXRT_DT_FLOAT32 || dt == NXRT_DT_FLOAT16 || dt == NXRT_DT_BFLOAT16; };
                 if (!is_float(d[0].dtype) || d[1].dtype != NXRT_DT_UINT8 || !is_float(d[2].dtype)) continue;
-                if (n > 4 && d[4].dtype != 0) continue;   // g_idx present: left to another provider
+                if (n > 4 && d[4].dtype != 0 && d[4].dtype != NXRT_DT_INT32) continue;   // g_idx, when present, is int32
             }
             if (claimed < max_claims && out_claims) {
                 out_claims[claimed].node_index = i;
@@ -101,6 +109,7 @@ NxrtStatus get_allocator_cb(void* ctx, NxrtAllocatorVtable** out_allocator)
         auto* h = new AllocatorHandle();
         std::memset(&h->vtable, 0, sizeof(h->vtable));
         h->ep = static_cast<NxrtRocmEp*>(ctx);
+        h->ep->retain();
         h->vtable.struct_size = sizeof(NxrtAllocatorVtable);
         h->vtable.alloc = alloc_cb;
         h->vtable.free = free_cb;

@@ -110,6 +110,7 @@ NxrtStatus nxrt_rocm_ep_create(uint32_t device_ordinal, const char* const* keys,
 
 void nxrt_rocm_ep_release(NxrtRocmEp* ep)
 {
+    if (!ep || ep->refs.fetch_sub(1) != 1) return;      // kernels and allocator handles still hold it
     try {
         delete ep;
     } catch (...) {

@@ -34,6 +34,11 @@ struct NxrtRocmEp {
     std::unordered_map<void*, size_t> live;       // allocations handed out and not yet returned
     std::atomic<uint64_t> launches{0};
     bool capturing = false;                       // a stream capture is open: nothing may allocate or synchronise
+    // The host may release the provider, its kernels and its allocators in any order (each vtable is released exactly
+    // once, independently): every kernel object and allocator handle holds one reference, the creator holds the first,
+    // and the provider dies with the last.
+    std::atomic<uint32_t> refs{1};
+    void retain() { refs.fetch_add(1); }
     NxrtEpVtable vtable;                          // ctx points back at this object
 
     NxrtRocmEp();

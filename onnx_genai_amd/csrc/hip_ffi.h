@@ -64,6 +64,9 @@ typedef struct RocmMatMulNBitsArgs {
   int64_t m, n, k;
   int block_size;
   const int32_t* g_idx;  /* [K] group of every element (act-order), or NULL: group = k / block_size. Only the plain kernels read it. */
+  int32_t* acc_probe;    /* accuracy_level 4, int8 matrix-core kernels only: int32 [M, N, kb], or NULL. When set, the kernel also
+                            stores every block accumulator sum_k code * (q - zp) it flushes - the integer its f32 result is built
+                            from - so that a test can compare the production kernels' integers bit for bit. */
 } RocmMatMulNBitsArgs;
 
 /* w[n,k] = (q - zp) * scale as f32 [N, K]. */

@@ -46,6 +46,7 @@ struct Acc4DecodeParams {
     int tiles_per_wave;     // multiple of the group size
     int bias_dtype, y_dtype;
     int scales_bf16;        // 16-bit scales are bf16 (else f16)
+    int32_t* acc_probe;     // PROBE builds: int32 [M, N, kb] block accumulators, as flushed
 };
 
 constexpr int kCodePitch = 144;   // bytes between activation rows of one tile in LDS: 128 + 16
@@ -68,7 +69,9 @@ struct Acc4Group {
 // the activation-side pairs; scale and zero point reach the other lane groups by shuffle when a block ends.
 // SETS: 2 = the next group's loads are in flight while this one is multiplied (few waves per launch); 1 = no prefetch,
 // fewer registers, more waves per SIMD (launches with thousands of waves, where occupancy hides latency better).
-template <int BS, int MR, typename ST, int SETS>
+// PROBE: every flushed block accumulator (the integer acc - zp * code_sum that is about to be scaled) is also stored to
+// p.acc_probe; the same code otherwise, for tests that compare the integers themselves.
+template <int BS, int MR, typename ST, int SETS, bool PROBE>
 __global__ __launch_bounds__(512) void acc4_decode_kernel(Acc4DecodeParams p)
 {
     constexpr bool kTranspose = BS < 128;
@@ -170,6 +173,9 @@ __global__ __launch_bounds__(512) void acc4_decode_kernel(Acc4DecodeParams p)
             const float qs = __int_as_float(__builtin_amdgcn_readlane(static_cast<int>(grp.x.y), bi));
             const float f = fmaf(-zf, qs, static_cast<float>(acc[0]));
             y[0] = fmaf(f, __fmul_rn(sa, sb), y[0]);
+            if constexpr (PROBE) {                                          // row 0 sits in lanes 0..15
+                if (g == 0 && n_base + c < p.n) p.acc_probe[(n_base + c) * p.kb + static_cast<int64_t>(t0) * NBT + bi] = static_cast<int>(f);
+            }
         } else {
             const float4* rows = reinterpret_cast<const float4*>(aux_stage + parity * kAuxStage + bi * 128 + g * 32);
             const float4 r01 = rows[0], r23 = rows[1];
@@ -179,6 +185,10 @@ __global__ __launch_bounds__(512) void acc4_decode_kernel(Acc4DecodeParams p)
             for (int r = 0; r < 4; ++r) {
                 const float f = fmaf(-zf, qs[r], static_cast<float>(acc[r]));
                 y[r] = fmaf(f, __fmul_rn(sa[r], sb), y[r]);
+                if constexpr (PROBE) {
+                    const int64_t row = 4 * g + r;
+                    if (row < p.m && n_base + c < p.n) p.acc_probe[(row * p.n + n_base + c) * p.kb + static_cast<int64_t>(t0) * NBT + bi] = static_cast<int>(f);
+                }
             }
         }
     };
@@ -268,7 +278,8 @@ static int launch_acc4_decode(const Acc4DecodeParams& p, int waves, hipStream_t 
     const unsigned grid = static_cast<unsigned>((p.n + 15) / 16);
     const size_t stage = static_cast<size_t>(waves) * (MR == 1 ? 2048 : 2 * 16 * kCodePitch + 2048);
     const size_t red = static_cast<size_t>(waves) * 1024;
-    hipLaunchKernelGGL((acc4_decode_kernel<BS, MR, ST, SETS>), dim3(grid), dim3(waves * 64), stage > red ? stage : red, stream, p);
+    if (p.acc_probe) hipLaunchKernelGGL((acc4_decode_kernel<BS, MR, ST, SETS, true>), dim3(grid), dim3(waves * 64), stage > red ? stage : red, stream, p);
+    else hipLaunchKernelGGL((acc4_decode_kernel<BS, MR, ST, SETS, false>), dim3(grid), dim3(waves * 64), stage > red ? stage : red, stream, p);
     return static_cast<int>(hipGetLastError());
 }
 
@@ -316,6 +327,7 @@ struct Acc4PrefillParams {
     int bias_dtype, y_dtype;
     int steps_per_slice;    // K steps per grid.z slice (a whole number of blocks); all steps when there is one slice
     float* partial;         // [slices, M, N] f32 partial sums when K is cut into slices, else NULL
+    int32_t* acc_probe;     // PROBE builds: int32 [M, N, kb] block accumulators, as flushed
 };
 
 constexpr int kTile = 128;           // rows and columns of Y per workgroup
@@ -327,7 +339,8 @@ constexpr int kPitch8 = 80;          // bytes per LDS row: 64 codes + 16 of padd
 // Eight waves, 4 (rows) x 2 (columns); each owns a 32 x 64 sub-tile: two MFMA tiles, 32 f32 results per lane. The
 // small per-wave state leaves room for four waves per SIMD, which is what overlaps one wave's flush arithmetic
 // with another's MFMAs.
-template <int NBS, bool SF32, int D>
+// PROBE: every int32 tile that is flushed is also stored to p.acc_probe ([M, N, kb]); the same code otherwise.
+template <int NBS, bool SF32, int D, bool PROBE>
 __global__ __launch_bounds__(512) void acc4_prefill_kernel(Acc4PrefillParams p)
 {
     constexpr int kSlots = NBS == 2 ? 2 : 1;                   // scale slots per step
@@ -367,6 +380,12 @@ __global__ __launch_bounds__(512) void acc4_prefill_kernel(Acc4PrefillParams p)
     const uint32_t sa_goff = (sa_slot < kSlots && m_base + sa_row < p.m) ? static_cast<uint32_t>(m_base + sa_row) * 4u : kOutOfRange;
     constexpr int kSaOff = 2 * kTile * kPitch8;                 // [kSlots][128] f32 activation scales of the step
     constexpr int kSbOff = kSaOff + kSlots * kTile * 4;         // [kSlots][128] f32 weight scales of the step
+
+    // PROBE: this lane's first accumulator element, (row m_base + wm * 32 + 4 (lane / 32), column n_base + wn * 64 + lane % 32),
+    // as a byte offset into the [M, N, kb] probe (the launcher refuses probes of 2^31 bytes or more)
+    const int64_t probe_row = m_base + wm * 32 + (lane >> 5) * 4;
+    const uint32_t probe_voff = PROBE ? static_cast<uint32_t>((probe_row * p.n + n_base + wn * 64 + (lane & 31)) * p.kb) * 4u : 0u;
+    const __amdgpu_buffer_rsrc_t srd_probe = make_srd(PROBE ? p.acc_probe : nullptr, PROBE ? static_cast<uint64_t>(p.m * p.n * p.kb) * 4 : 0);
 
     // MFMA operand reads: lane (r = lane % 32, h = lane / 32) reads 16 consecutive codes of row r.
     const uint32_t frag_off = static_cast<uint32_t>((lane & 31) * kPitch8 + (lane >> 5) * 16);
@@ -453,6 +472,23 @@ __global__ __launch_bounds__(512) void acc4_prefill_kernel(Acc4PrefillParams p)
 #pragma unroll
         for (int i = 0; i < 16; ++i) y[j][i] = fmaf(static_cast<float>(tile[i]), sc[j * 16 + i], y[j][i]);
     };
+    // PROBE: the finished int32 tile j of block `blk`, stored before its scale products are formed (fewer registers live
+    // than at the flush itself; the integers are final once the block's last MFMA has written them).
+    auto probe_tile = [&](const int16_t_v& tile, int j, int64_t blk) {
+        if constexpr (PROBE) {
+            // lane l holds column l % 32 and rows 8 q + 4 (l / 32) + r of the 32 x 32 tile in component 4 q + r. One vector
+            // offset per lane (its first row, tile 0's column), everything else in the scalar offset; a row or column past
+            // the matrix gets an offset beyond the buffer's range, which stores nothing.
+            const bool col_ok = n_base + wn * 64 + j * 32 + (lane & 31) < p.n && blk < p.kb;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int rowoff = (i >> 2) * 8 + (i & 3);
+                const bool ok = col_ok && probe_row + rowoff < p.m;
+                const uint32_t soff = static_cast<uint32_t>((static_cast<int64_t>(rowoff) * p.n + j * 32) * p.kb + blk) * 4u;
+                __builtin_amdgcn_raw_buffer_store_b32(tile[i], srd_probe, static_cast<int>(ok ? probe_voff : kOutOfRange), static_cast<int>(soff), 0);
+            }
+        }
+    };
     auto mfma = [](const u32x4_t& a, const u32x4_t& b, const int16_t_v& c) {
         return __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(int4_t, a), __builtin_bit_cast(int4_t, b), c, 0, 0, 0);
     };
@@ -474,6 +510,8 @@ __global__ __launch_bounds__(512) void acc4_prefill_kernel(Acc4PrefillParams p)
             int16_t_v t1 = mfma(fa[0], fb[0][1], zero);
             t0 = mfma(fa[1], fb[1][0], t0);
             t1 = mfma(fa[1], fb[1][1], t1);
+            probe_tile(t0, 0, kt);
+            probe_tile(t1, 1, kt);
             const float32_v sc = scale_tiles(buf, 0);
             if (store_next) store_part(next, buf ^ 1, 0);
             flush_tile(t0, sc, 0);
@@ -485,6 +523,10 @@ __global__ __launch_bounds__(512) void acc4_prefill_kernel(Acc4PrefillParams p)
             const int16_t_v t1 = mfma(fa[0], fb[0][1], zero);
             const int16_t_v u0 = mfma(fa[1], fb[1][0], zero);
             const int16_t_v u1 = mfma(fa[1], fb[1][1], zero);
+            probe_tile(t0, 0, 2 * static_cast<int64_t>(kt));
+            probe_tile(t1, 1, 2 * static_cast<int64_t>(kt));
+            probe_tile(u0, 0, 2 * static_cast<int64_t>(kt) + 1);           // (a second block past K is not stored: blk < kb)
+            probe_tile(u1, 1, 2 * static_cast<int64_t>(kt) + 1);
             const float32_v sc0 = scale_tiles(buf, 0);
             const float32_v sc1 = scale_tiles(buf, 1);
             if (store_next) store_part(next, buf ^ 1, 0);
@@ -507,6 +549,8 @@ __global__ __launch_bounds__(512) void acc4_prefill_kernel(Acc4PrefillParams p)
                 if (store_next) store_part(next, buf ^ 1, j);
             }
             if (closes) {
+#pragma unroll
+                for (int j = 0; j < TN; ++j) probe_tile(acc[j], j, (static_cast<int64_t>(kt) * kStep) >> p.bs_log2);
                 const float32_v sc = scale_tiles(buf, 0);
 #pragma unroll
                 for (int j = 0; j < TN; ++j) flush_tile(acc[j], sc, j);
@@ -598,8 +642,17 @@ static int launch_acc4_prefill(const Acc4PrefillParams& p, int slices, hipStream
     const dim3 grid(static_cast<unsigned>((p.n + kTile - 1) / kTile), static_cast<unsigned>((p.m + kTile - 1) / kTile), static_cast<unsigned>(slices));
     const size_t lds = 2 * (2 * kTile * kPitch8 + 2 * (NBS == 2 ? 2 : 1) * kTile * 4);
     const bool deep = NBS == 2 || static_cast<uint64_t>(grid.x) * grid.y * grid.z <= 256;    // at most one workgroup per CU anyway
-    if (deep) hipLaunchKernelGGL((acc4_prefill_kernel<NBS, SF32, 4>), grid, dim3(512), lds, stream, p);
-    else hipLaunchKernelGGL((acc4_prefill_kernel<NBS, SF32, NBS == 2 ? 4 : 2>), grid, dim3(512), lds, stream, p);
+    if (p.acc_probe) {
+        // (block size 32 with four register sets in flight has no room left for the probe's stores: its probe build keeps two -
+        // the depth of the load pipeline changes when a step's operands arrive, not what is computed from them)
+        if constexpr (NBS == 2) {
+            hipLaunchKernelGGL((acc4_prefill_kernel<NBS, SF32, 2, true>), grid, dim3(512), lds, stream, p);
+        } else {
+            if (deep) hipLaunchKernelGGL((acc4_prefill_kernel<NBS, SF32, 4, true>), grid, dim3(512), lds, stream, p);
+            else hipLaunchKernelGGL((acc4_prefill_kernel<NBS, SF32, 2, true>), grid, dim3(512), lds, stream, p);
+        }
+    } else if (deep) hipLaunchKernelGGL((acc4_prefill_kernel<NBS, SF32, 4, false>), grid, dim3(512), lds, stream, p);
+    else hipLaunchKernelGGL((acc4_prefill_kernel<NBS, SF32, NBS == 2 ? 4 : 2, false>), grid, dim3(512), lds, stream, p);
     return static_cast<int>(hipGetLastError());
 }
 
@@ -650,6 +703,8 @@ extern "C" int rocm_launch_acc4_mfma(const RocmMatMulNBitsArgs* a, const RocmAcc
         q.scales_bf16 = a->scale_dtype == ROCM_DT_BF16;
         q.bias_dtype = a->bias_dtype;
         q.y_dtype = a->y_dtype;
+        q.acc_probe = a->acc_probe;
+        if (q.acc_probe && q.m * q.n * q.kb * 4 >= 0x7fffffff) return -1;            // the probe is addressed with 32-bit offsets
         const bool sf32 = a->scale_dtype == ROCM_DT_F32;
         // slices of K when the grid is small and the workspace has room for their partial sums
         int slices = mnb::acc4_prefill_slices(a->m, a->n, q.padded_k, a->block_size);
@@ -686,6 +741,7 @@ extern "C" int rocm_launch_acc4_mfma(const RocmMatMulNBitsArgs* a, const RocmAcc
     p.bias_dtype = a->bias_dtype;
     p.y_dtype = a->y_dtype;
     p.scales_bf16 = a->scale_dtype == ROCM_DT_BF16;
+    p.acc_probe = a->acc_probe;
 
     const int group_tiles = a->m <= 1 ? 4 : 2;
     const int64_t wgs = (a->n + 15) / 16;

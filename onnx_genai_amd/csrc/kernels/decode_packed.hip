@@ -754,6 +754,7 @@ struct Acc4PackedParams {
     int groups, groups_per_wave, chunk_bytes;
     int bias_dtype, y_dtype;
     int scales_bf16;
+    int32_t* acc_probe;     // PROBE builds: int32 [N, kb] block accumulators of the one row, as flushed
 };
 
 template <int NR>
@@ -769,7 +770,9 @@ struct Acc4PackedGroup {
 // (one correctly rounded divide each for scale and inverse, one multiply and one rounding per element) - a lane holds
 // 8 consecutive activations, a block is BS / 8 consecutive lanes. That is redundant across workgroups but saves the
 // separate launch, which at one row costs about as much as a fifth of this kernel.
-template <int BS, typename ST, int SETS, int FUSE>
+// PROBE: every flushed block accumulator (the integer acc - zp * code_sum that is about to be scaled) is also stored to
+// p.acc_probe; the same code otherwise, for tests that compare the integers themselves.
+template <int BS, typename ST, int SETS, int FUSE, bool PROBE>
 __global__ __launch_bounds__(512) void acc4_packed_kernel(Acc4PackedParams p)
 {
     constexpr int U = kGroupTiles;
@@ -917,6 +920,10 @@ __global__ __launch_bounds__(512) void acc4_packed_kernel(Acc4PackedParams p)
                     const float qs = __int_as_float(__builtin_amdgcn_readlane(FUSE ? __float_as_int(qs_lane) : static_cast<int>(grp.x.y), src));
                     const float f = fmaf(-zf, qs, static_cast<float>(acc[0]));   // both terms are integers below 2^24: exact
                     y = fmaf(f, __fmul_rn(sa, sb), y);
+                    if constexpr (PROBE) {                                       // row 0 sits in lanes 0..15
+                        const int64_t blk = static_cast<int64_t>(gi) * NB + bi;
+                        if (lane < 16 && n_base + lane < p.n && blk < p.kb) p.acc_probe[(n_base + lane) * p.kb + blk] = static_cast<int>(f);
+                    }
                 }
             }
         }
@@ -969,8 +976,11 @@ static int launch_acc4_packed(const Acc4PackedParams& p, int waves, bool single_
     const size_t lds = static_cast<size_t>(waves) * 1024;
     auto go = [&](auto fuse) {
         constexpr int F = decltype(fuse)::value;
-        if (single_set) hipLaunchKernelGGL((acc4_packed_kernel<BS, ST, 1, F>), dim3(grid), dim3(waves * 64), lds, stream, p);
-        else hipLaunchKernelGGL((acc4_packed_kernel<BS, ST, 2, F>), dim3(grid), dim3(waves * 64), lds, stream, p);
+        if (p.acc_probe) {
+            if (single_set) hipLaunchKernelGGL((acc4_packed_kernel<BS, ST, 1, F, true>), dim3(grid), dim3(waves * 64), lds, stream, p);
+            else hipLaunchKernelGGL((acc4_packed_kernel<BS, ST, 2, F, true>), dim3(grid), dim3(waves * 64), lds, stream, p);
+        } else if (single_set) hipLaunchKernelGGL((acc4_packed_kernel<BS, ST, 1, F, false>), dim3(grid), dim3(waves * 64), lds, stream, p);
+        else hipLaunchKernelGGL((acc4_packed_kernel<BS, ST, 2, F, false>), dim3(grid), dim3(waves * 64), lds, stream, p);
     };
     if (fuse == 1) go(std::integral_constant<int, 1>{});
     else if (fuse == 2) go(std::integral_constant<int, 2>{});
@@ -1168,6 +1178,7 @@ extern "C" int rocm_launch_acc4_packed(const RocmMatMulNBitsArgs* a, const void*
     p.bias_dtype = a->bias_dtype;
     p.y_dtype = a->y_dtype;
     p.scales_bf16 = a->scale_dtype == ROCM_DT_BF16;
+    p.acc_probe = a->acc_probe;
 
     const int64_t wgs = (a->n + 15) / 16;
     int w = waves;

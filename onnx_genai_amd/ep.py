@@ -117,6 +117,10 @@ def load_library() -> C.CDLL:
     L.nxrt_rocm_matmul_nbits_last_variant.argtypes = [v]
     L.nxrt_rocm_matmul_nbits_release.restype = None
     L.nxrt_rocm_matmul_nbits_release.argtypes = [v]
+    L.nxrt_rocm_matmul_nbits_set_block_acc_probe.restype = S
+    L.nxrt_rocm_matmul_nbits_set_block_acc_probe.argtypes = [v, v, u64]
+    L.nxrt_rocm_matmul_nbits_retired_buffers.restype = u64
+    L.nxrt_rocm_matmul_nbits_retired_buffers.argtypes = [v]
     L.nxrt_rocm_matmul_nbits_as_vtable.restype = S
     L.nxrt_rocm_matmul_nbits_as_vtable.argtypes = [v, C.POINTER(v)]
     L.nxrt_rocm_matmul_nbits_dequantize.restype = S
@@ -435,6 +439,13 @@ class MatMulNBitsKernel:
     def last_variant(self) -> str:
         return self.lib.nxrt_rocm_matmul_nbits_last_variant(self.handle).decode()
 
+    def set_block_acc_probe(self, buf: DeviceBuffer | None) -> None:
+        """accuracy_level 4: later executes also store their int32 block accumulators [M, N, kb] into `buf` (None clears)."""
+        self.lib.nxrt_rocm_matmul_nbits_set_block_acc_probe(self.handle, buf.ptr if buf else None, buf.nbytes // 4 if buf else 0).check()
+
+    def retired_buffers(self) -> int:
+        return self.lib.nxrt_rocm_matmul_nbits_retired_buffers(self.handle)
+
     def release(self) -> None:
         if self.handle:
             self.lib.nxrt_rocm_matmul_nbits_release(self.handle)
@@ -442,8 +453,7 @@ class MatMulNBitsKernel:
 
     def __del__(self):
         try:
-            if self.ep.handle:
-                self.release()
+            self.release()              # safe after the provider's own release: the kernel holds a reference to it
         except Exception:
             pass
 
@@ -455,8 +465,9 @@ class DeviceOperands:
     """The device-resident operands of one MatMulNBits node plus its kernel; what a session would hold."""
 
     def __init__(self, ep, b, scales, scale_dtype, zp, n, k, bs, *, accuracy_level=0, bias=None, bias_dtype=F32, rows=None, a_dtype=None,
-                 folded_bias=None, gamma=None, gamma_dtype=F32, rmsnorm_epsilon=None, bits=4, g_idx=None):
+                 folded_bias=None, gamma=None, gamma_dtype=F32, rmsnorm_epsilon=None, bits=4, g_idx=None, bias_shape=None):
         self.ep, self.n, self.k, self.bs, self.bits = ep, n, k, bs, bits
+        self.bias_shape = bias_shape                                          # the shape the bias view declares (default: [N], or [M, N] for a residual)
         self.g_idx = ep.upload(np.ascontiguousarray(g_idx, np.int32)) if g_idx is not None else None      # act-order groups, input 4
         self.kb = -(-k // bs)
         self.scale_dtype, self.bias_dtype = scale_dtype, bias_dtype
@@ -485,7 +496,7 @@ class DeviceOperands:
             ins.append(TensorView(self.g_idx.ptr, I32, (self.k,), device_index=dev))
         if self.bias is not None or self.gamma is not None:
             ins.append(TensorView(self.g_idx.ptr, I32, (self.k,), device_index=dev) if self.g_idx is not None else TensorView.absent(I32))
-            bias_shape = (m, self.n) if self.bias_per_row else (self.n,)
+            bias_shape = self.bias_shape or ((m, self.n) if self.bias_per_row else (self.n,))
             ins.append(TensorView(self.bias.ptr, self.bias_dtype, bias_shape, device_index=dev) if self.bias is not None else TensorView.absent(F32))
         if self.gamma is not None:
             ins.append(TensorView(self.gamma.ptr, self.gamma_dtype, (self.k,), device_index=dev))
@@ -504,13 +515,13 @@ class DeviceOperands:
 
 
 def matmul_nbits(ep, a, a_dtype, b, scales, scale_dtype, zp, n, k, bs, *, accuracy_level=0, bias=None, bias_dtype=F32, y_dtype=None, folded_bias=None,
-                 gamma=None, gamma_dtype=F32, rmsnorm_epsilon=None, bits=4, g_idx=None):
+                 gamma=None, gamma_dtype=F32, rmsnorm_epsilon=None, bits=4, g_idx=None, bias_shape=None):
     """One-shot helper: upload, execute through the C ABI, download. Returns (Y as numpy, variant name)."""
     y_dtype = a_dtype if y_dtype is None else y_dtype
     a = np.ascontiguousarray(a)
     m = a.size // k
     ops = DeviceOperands(ep, b, scales, scale_dtype, zp, n, k, bs, accuracy_level=accuracy_level, bias=bias, bias_dtype=bias_dtype, folded_bias=folded_bias,
-                         gamma=gamma, gamma_dtype=gamma_dtype, rmsnorm_epsilon=rmsnorm_epsilon, bits=bits, g_idx=g_idx)
+                         gamma=gamma, gamma_dtype=gamma_dtype, rmsnorm_epsilon=rmsnorm_epsilon, bits=bits, g_idx=g_idx, bias_shape=bias_shape)
     a_buf = ep.upload(a)
     y_buf = ep.allocate(max(m * n * _ITEM[y_dtype], 1))
     try:
@@ -527,7 +538,8 @@ def matmul_nbits(ep, a, a_dtype, b, scales, scale_dtype, zp, n, k, bs, *, accura
 class GateUpOperands:
     """Device-resident operands of the fused gate/up node (inputs [x, W_gate, scales_gate, W_up, scales_up, -, zp_gate, zp_up])."""
 
-    def __init__(self, ep, gate, up, scale_dtype, n, k, bs, *, decomposed=False, rows=None, a_dtype=None, gamma=None, gamma_dtype=F32, rmsnorm_epsilon=None):
+    def __init__(self, ep, gate, up, scale_dtype, n, k, bs, *, decomposed=False, rows=None, a_dtype=None, gamma=None, gamma_dtype=F32, rmsnorm_epsilon=None,
+                 accuracy_level=None):
         self.ep, self.n, self.k, self.bs, self.scale_dtype = ep, n, k, bs, scale_dtype
         self.kb = -(-k // bs)
         self.bufs = []
@@ -537,7 +549,7 @@ class GateUpOperands:
         self.gamma = ep.upload(gamma) if gamma is not None else None
         self.gamma_dtype = gamma_dtype
         self.kernel = ep.get_kernel({"K": k, "N": n, "bits": 4, "block_size": bs, "gate_up_swiglu": 1, "decomposed_silu": 1 if decomposed else None,
-                                     "rmsnorm_prologue": 1 if gamma is not None else None, "rmsnorm_epsilon": rmsnorm_epsilon}, shapes)
+                                     "accuracy_level": accuracy_level, "rmsnorm_prologue": 1 if gamma is not None else None, "rmsnorm_epsilon": rmsnorm_epsilon}, shapes)
         self.kernel.set_constant_inputs([False, True, True, True, True, True, True, True])
 
     def views(self, a_buf: DeviceBuffer, a_dtype: int, m: int):

@@ -3,7 +3,13 @@
  * crates/onnx-runtime-ep-cuda/tests/matmul_nbits_gpu.rs:223-352): dlopen, negotiate, create the
  * factory and the provider, take its allocator, then build one MatMulNBits kernel through the kernel
  * mirror, run it at accuracy_level 0 and 4 on inputs made from integer formulas, and check the
- * result against a scalar loop in this file. Prints one line per step; exit status 0 = all good.
+ * result against a scalar loop in this file. A second part does the same with every tensor of the call
+ * allocated through the nxmem allocator plugin the library also exports
+ * (crates/onnx-runtime-memory-abi/include/nxmem_memory_abi.h:581-610, 698-718): negotiate, create the
+ * factories, open the allocator of device 0, allocate, run, deallocate, and ask for the unload report;
+ * it also checks the refusals (wrong mechanism, wrong device, unknown allocation, a capability that is
+ * not offered) and that the provider, its kernels and its allocators may be released in any order.
+ * Prints one line per step; exit status 0 = all good.
  *
  *   nxrt_roundtrip <path to libnxrt_ep_rocm.so>
  */
@@ -13,6 +19,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include "nxmem_abi.h"
 #include "nxrt_abi.h"
 #include "nxrt_ep_rocm.h"
 
@@ -39,6 +46,9 @@ typedef NxrtStatus (*nxrt_rocm_matmul_nbits_execute_fn)(NxrtRocmMatMulNBits*, co
 typedef const char* (*nxrt_rocm_matmul_nbits_last_variant_fn)(const NxrtRocmMatMulNBits*);
 typedef void (*nxrt_rocm_matmul_nbits_release_fn)(NxrtRocmMatMulNBits*);
 typedef uint64_t (*nxrt_rocm_live_provider_count_fn)(void);
+typedef NxmemStatus (*NxmemNegotiate_fn)(const NxmemNegotiateRequest*, NxmemNegotiateResponse*);
+typedef NxmemStatus (*NxmemCreateAllocatorFactories_fn)(const NxmemAllocatorFactoryVtable**, uint64_t, uint64_t*);
+typedef NxmemStatus (*NxmemQueryUnloadReadiness_fn)(NxmemUnloadReport*);
 
 enum { M = 3, N = 70, K = 320, BS = 32, KB = K / BS };
 
@@ -69,6 +79,9 @@ int main(int argc, char** argv)
   LOAD(nxrt_rocm_matmul_nbits_last_variant);
   LOAD(nxrt_rocm_matmul_nbits_release);
   LOAD(nxrt_rocm_live_provider_count);
+  LOAD(NxmemNegotiate);
+  LOAD(NxmemCreateAllocatorFactories);
+  LOAD(NxmemQueryUnloadReadiness);
 
   /* negotiate: host speaks 1.0 .. 1.x */
   NxrtNegotiateRequest req = {sizeof(req), {1, 1, 0}};
@@ -171,8 +184,148 @@ int main(int argc, char** argv)
 
   void* frees[6] = {da, db, ds, dz, dbias, dy};
   for (int i = 0; i < 6; ++i) alloc->free(alloc->ctx, frees[i]);
+
+  /* ---- the same call with every tensor allocated through the nxmem allocator plugin ---- */
+  NxmemNegotiateRequest mreq;
+  memset(&mreq, 0, sizeof(mreq));
+  mreq.struct_size = sizeof(mreq);
+  mreq.host_range.major_min = 1;
+  mreq.host_range.major_max = 1;
+  mreq.host_range.minor_min = 0;
+  mreq.host_range.minor_max = NXMEM_ABI_VERSION_MINOR;
+  mreq.host_capability_flags = NXMEM_CAP_ALLOCATOR | NXMEM_CAP_DEFERRED_RELEASE;
+  NxmemNegotiateResponse mresp;
+  memset(&mresp, 0, sizeof(mresp));
+#define MOK(st, what) do { NxmemStatus s_ = (st); CHECK(s_.code == NXMEM_STATUS_OK, "%s: code %u %s", what, s_.code, (const char*)s_.message); } while (0)
+#define MREFUSED(st, want, what) do { NxmemStatus s_ = (st); CHECK(s_.code == (want), "%s: expected status %d, got %u %s", what, (int)(want), s_.code, (const char*)s_.message); } while (0)
+  MOK(NxmemNegotiate_p(&mreq, &mresp), "NxmemNegotiate");
+  CHECK(mresp.agreed_major == 1 && mresp.capability_flags == NXMEM_CAP_ALLOCATOR, "nxmem negotiated %u.%u caps %llx", mresp.agreed_major, mresp.agreed_minor,
+        (unsigned long long)mresp.capability_flags);
+  const NxmemAllocatorFactoryVtable* mfactories[16];
+  uint64_t n_mfactories = 0;
+  MOK(NxmemCreateAllocatorFactories_p(mfactories, 16, &n_mfactories), "NxmemCreateAllocatorFactories");
+  CHECK(n_mfactories >= 1 && mfactories[0]->device.tier == NXMEM_TIER_DEVICE && mfactories[0]->device.index == 0, "no nxmem factory for device 0");
+  const NxmemAllocatorFactoryVtable* mf = mfactories[0];
+  NxmemOpenRequest open_req;
+  memset(&open_req, 0, sizeof(open_req));
+  open_req.struct_size = sizeof(open_req);
+  open_req.abi_minor = mresp.agreed_minor;
+  open_req.device.tier = NXMEM_TIER_DEVICE;
+  open_req.device.index = 0;
+  open_req.required_capability_flags = NXMEM_CAP_ALLOCATOR;
+  const NxmemAllocatorVtable* mal = NULL;
+  NxmemOpenRequest bad_open = open_req;
+  bad_open.required_capability_flags = NXMEM_CAP_ALLOCATOR | NXMEM_CAP_VIRTUAL_BACKING;
+  MREFUSED(mf->open_allocator(mf->ctx, &bad_open, &mal), NXMEM_STATUS_UNSUPPORTED_CAPABILITY, "open_allocator with virtual backing required");
+  bad_open = open_req;
+  bad_open.device.index = 7;
+  MREFUSED(mf->open_allocator(mf->ctx, &bad_open, &mal), NXMEM_STATUS_WRONG_DEVICE, "open_allocator for another device");
+  MOK(mf->open_allocator(mf->ctx, &open_req, &mal), "open_allocator");
+  CHECK(mal && mal->allocate && mal->deallocate && mal->retain && mal->release, "a required allocator slot is NULL");
+  CHECK(!mal->virtual_backing && !mal->shared_mapping && !mal->enqueue_release && !mal->drain_releases && !mal->pending_release_count && !mal->release_allocation,
+        "an optional slot that is not offered must be NULL");
+  printf("nxmem allocator %s, mechanism %llx\n", (const char*)mal->name, (unsigned long long)mal->mechanism_id);
+
+  const size_t sizes[6] = {sizeof(a), sizeof(b), sizeof(scales), sizeof(zp), sizeof(bias), sizeof(y)};
+  const void* hosts[6] = {a, b, scales, zp, bias, NULL};
+  NxmemAllocation held[6];
+  for (int i = 0; i < 6; ++i) {
+    NxmemAllocRequest ar;
+    memset(&ar, 0, sizeof(ar));
+    ar.struct_size = sizeof(ar);
+    ar.mechanism_id = mal->mechanism_id;
+    ar.allocation_id = 1000 + (uint64_t)i;
+    ar.device = mal->device;
+    ar.bytes = sizes[i];
+    ar.align = 256;
+    NxmemAllocResult res;
+    memset(&res, 0, sizeof(res));
+    if (i == 0) {
+      NxmemAllocRequest wrong = ar;
+      wrong.mechanism_id ^= 1;
+      MREFUSED(mal->allocate(mal->ctx, &wrong, &res), NXMEM_STATUS_WRONG_MECHANISM, "allocate for another mechanism");
+      wrong = ar;
+      wrong.device.index = 5;
+      MREFUSED(mal->allocate(mal->ctx, &wrong, &res), NXMEM_STATUS_WRONG_DEVICE, "allocate for another device");
+      wrong = ar;
+      wrong.struct_size = 8;
+      MREFUSED(mal->allocate(mal->ctx, &wrong, &res), NXMEM_STATUS_SHORT_STRUCT, "allocate with a short request");
+    }
+    MOK(mal->allocate(mal->ctx, &ar, &res), "nxmem allocate");
+    CHECK(res.ptr != NULL && res.owned_bytes >= sizes[i] && res.mapped_bytes >= sizes[i] && ((uintptr_t)res.ptr & 255) == 0, "nxmem allocate result");
+    memset(&held[i], 0, sizeof(held[i]));
+    held[i].struct_size = sizeof(held[i]);
+    held[i].mechanism_id = ar.mechanism_id;
+    held[i].allocation_id = ar.allocation_id;
+    held[i].device = ar.device;
+    held[i].ptr = res.ptr;
+    held[i].bytes = sizes[i];
+    held[i].align = 256;
+    if (hosts[i]) OK(alloc->copy_from_host(alloc->ctx, res.ptr, (const uint8_t*)hosts[i], sizes[i]), "copy_from_host into nxmem memory");
+  }
+  NxmemUnloadReport report;
+  MOK(NxmemQueryUnloadReadiness_p(&report), "NxmemQueryUnloadReadiness");
+  CHECK(report.struct_size == sizeof(report) && report.live_allocators == 1 && report.live_allocations == 6, "unload report with the call's tensors live: %llu allocators, %llu allocations",
+        (unsigned long long)report.live_allocators, (unsigned long long)report.live_allocations);
+  {
+    NxrtRocmMatMulNBitsAttrs attrs;
+    memset(&attrs, 0, sizeof(attrs));
+    attrs.struct_size = sizeof(attrs);
+    attrs.present = 0x1f;
+    attrs.K = K;
+    attrs.N = N;
+    attrs.bits = 4;
+    attrs.block_size = BS;
+    attrs.accuracy_level = 0;
+    NxrtRocmMatMulNBits* kernel = NULL;
+    OK(nxrt_rocm_matmul_nbits_create_p(ep, &attrs, NULL, 0, &kernel), "matmul_nbits_create (nxmem)");
+    nxrt_rocm_matmul_nbits_set_constant_inputs_p(kernel, constant, 6);
+    NxrtRocmTensorView in[6];
+    in[0] = view(held[0].ptr, NXRT_DT_FLOAT32, 2, sh_a);
+    in[1] = view(held[1].ptr, NXRT_DT_UINT8, 3, sh_b);
+    in[2] = view(held[2].ptr, NXRT_DT_FLOAT32, 2, sh_s);
+    in[3] = view(held[3].ptr, NXRT_DT_UINT8, 2, sh_z);
+    in[4] = view(NULL, NXRT_DT_INT32, 0, NULL);
+    in[5] = view(held[4].ptr, NXRT_DT_FLOAT32, 1, sh_bias);
+    NxrtRocmTensorView out = view(held[5].ptr, NXRT_DT_FLOAT32, 2, sh_y);
+    OK(nxrt_rocm_matmul_nbits_execute_p(kernel, in, 6, &out, 1, NULL, 0), "matmul_nbits_execute (nxmem)");
+    static float ym[M * N];
+    OK(alloc->copy_to_host(alloc->ctx, (uint8_t*)ym, held[5].ptr, sizeof(ym)), "copy_to_host from nxmem memory");
+    OK(alloc->sync(alloc->ctx), "sync");
+    CHECK(memcmp(ym, y, sizeof(ym)) == 0, "the call over nxmem-allocated tensors differs from the call over the provider's allocator");
+    printf("nxmem-allocated tensors: variant %s, same bits as before\n", nxrt_rocm_matmul_nbits_last_variant_p(kernel));
+    /* any order: the provider's vtable goes first, the kernel and the allocator handle keep the provider alive */
+    ep_vt->release(ep_vt->ctx);
+    CHECK(nxrt_rocm_live_provider_count_p() == 1, "the provider died while a kernel and an allocator still referred to it");
+    nxrt_rocm_matmul_nbits_release_p(kernel);
+    CHECK(nxrt_rocm_live_provider_count_p() == 1, "the provider died while an allocator still referred to it");
+  }
+  uint64_t unmapped = 0;
+  {
+    NxmemAllocation wrong = held[0];
+    wrong.allocation_id = 4242;
+    MREFUSED(mal->deallocate(mal->ctx, &wrong, &unmapped), NXMEM_STATUS_UNKNOWN_ALLOCATION, "deallocate of an unknown id");
+    wrong = held[0];
+    wrong.mechanism_id ^= 1;
+    MREFUSED(mal->deallocate(mal->ctx, &wrong, &unmapped), NXMEM_STATUS_WRONG_MECHANISM, "deallocate for another mechanism");
+    wrong = held[0];
+    wrong.device.index = 3;
+    MREFUSED(mal->deallocate(mal->ctx, &wrong, &unmapped), NXMEM_STATUS_WRONG_DEVICE, "deallocate for another device");
+  }
+  for (int i = 0; i < 6; ++i) {
+    unmapped = 0;
+    MOK(mal->deallocate(mal->ctx, &held[i], &unmapped), "nxmem deallocate");
+    CHECK(unmapped == sizes[i], "deallocate reported %llu unmapped bytes of %llu", (unsigned long long)unmapped, (unsigned long long)sizes[i]);
+  }
+  MREFUSED(mal->deallocate(mal->ctx, &held[0], &unmapped), NXMEM_STATUS_UNKNOWN_ALLOCATION, "second deallocate of one allocation");
+  mal->release(mal->ctx);
+  mf->release(mf->ctx);
+  MOK(NxmemQueryUnloadReadiness_p(&report), "NxmemQueryUnloadReadiness");
+  CHECK(report.live_allocators == 0 && report.live_allocations == 0 && report.live_views == 0 && report.queued_releases == 0,
+        "unload report after release: %llu allocators, %llu allocations", (unsigned long long)report.live_allocators, (unsigned long long)report.live_allocations);
+  printf("nxmem unload report: nothing live\n");
+
   alloc->release(alloc->ctx);
-  ep_vt->release(ep_vt->ctx);
   factory->release(factory->ctx);
   CHECK(nxrt_rocm_live_provider_count_p() == 0, "a provider outlived its release");
   printf("released; roundtrip ok\n");

@@ -423,8 +423,11 @@ def test_packed_copy_follows_the_weights(ep, port):
     y1 = ep.download(yb, (m, n), np.float32)
     views2 = [E.TensorView(ab.ptr, a_dt, (m, k)), E.TensorView(other[0].ptr, E.U8, (n, kb, bs // 2)),
               E.TensorView(other[1].ptr, a_dt, (n, kb)), E.TensorView(other[2].ptr, E.U8, (n, (kb + 1) // 2))]
+    assert first.kernel.retired_buffers() == 0
     first.kernel.execute(views2, [E.TensorView(yb.ptr, E.F32, (m, n))])
     assert first.kernel.last_variant() == "decode_mfma_packed"
+    # the copy made from the first weights is kept, not freed: a graph recorded over it may still be replayed
+    assert first.kernel.retired_buffers() == 1
     y2 = ep.download(yb, (m, n), np.float32)
     assert helpers.rel_l2(y1, oracle_f64(port, a, a_dt, b1, s1, a_dt, zp1, n, k, bs)) <= 1e-4
     assert helpers.rel_l2(y2, oracle_f64(port, a, a_dt, b2, s2, a_dt, zp2, n, k, bs)) <= 1e-4
@@ -599,6 +602,27 @@ def test_residual_in_the_bias_slot(ep_tiled, port, folded, a_dt, bs, acc, m, n, 
         assert np.array_equal(np.asarray(got), np.asarray(want))
     else:
         assert np.array_equal(np.asarray(got).view(np.uint16), np.asarray(want).view(np.uint16))
+
+
+@pytest.mark.parametrize("folded", [1, None])
+@pytest.mark.parametrize("bias_shape", ["[1, N]", "[1, 1, N]"])
+@pytest.mark.parametrize("a_dt,bs,acc,n,k", [(E.BF16, 128, 0, 300, 3584), (E.F16, 64, 4, 160, 1024), (E.F32, 32, 0, 100, 256)])
+def test_one_row_residual_in_the_bias_slot(ep, port, folded, bias_shape, a_dt, bs, acc, n, k):
+    """A one-row decode step passes its residual as [1, N] or [1, 1, N]: N elements, so it broadcasts like a bias [N]
+    (the CUDA provider accepts the bias slot by element count, kernels/matmul_nbits.rs:7728-7735, 7891-7897)."""
+    b, s, zp = synth.make_weights(n, k, bs, 720 + n, zero_points=True, scale_lo=0.002, scale_hi=0.01, scale_dtype=a_dt)
+    a = synth.make_activation(1, k, 721, a_dt)
+    residual = synth.to_dtype((np.random.default_rng(n).standard_normal(n) * 0.5).astype(np.float32), a_dt)
+    shape = (1, n) if bias_shape == "[1, N]" else (1, 1, n)
+    common = dict(accuracy_level=acc, bias=residual, bias_dtype=a_dt, folded_bias=folded)
+    got, v1 = run_op(ep, a, a_dt, b, s, a_dt, zp, n, k, bs, bias_shape=shape, **common)
+    flat, v0 = run_op(ep, a, a_dt, b, s, a_dt, zp, n, k, bs, **common)            # the same values declared as [N]
+    assert v0 == v1
+    view = np.float32 if a_dt == E.F32 else np.uint16
+    assert np.array_equal(np.asarray(got).view(view), np.asarray(flat).view(view))
+    with pytest.raises(E.EpError) as e:
+        run_op(ep, a, a_dt, b, s, a_dt, zp, n, k, bs, bias_shape=(n - 1,), **common)
+    assert f"bias must have {n} elements" in str(e.value)
 
 
 def test_folded_bias_keeps_tall_calls_off_the_library_gemm(ep):
@@ -811,6 +835,29 @@ RMSNORM_CASES = [
     (E.BF16, E.F32, 128, 16, 200, 1024, 1e-5),
     (E.F16, E.F16, 64, 100, 136, 512, 1e-5),
 ]
+
+
+def test_gate_up_swiglu_at_accuracy_level_4_stays_on_the_int8_kernels(ep):
+    """A fused gate/up node with accuracy_level 4 runs both projections through the int8 path on every call: the float
+    single-launch form (which the repacked copies of the first call would make available) must not take later calls."""
+    a_dt, bs, m, n, k = E.F16, 64, 1, 160, 1024
+    gate = synth.make_weights(n, k, bs, 801, zero_points=True, scale_lo=0.002, scale_hi=0.01, scale_dtype=a_dt)
+    up = synth.make_weights(n, k, bs, 802, zero_points=True, scale_lo=0.002, scale_hi=0.01, scale_dtype=a_dt)
+    a = synth.make_activation(m, k, 803, a_dt)
+    ops = E.GateUpOperands(ep, gate, up, a_dt, n, k, bs, accuracy_level=4)
+    ab, yb = ep.upload(a), ep.allocate(m * n * 2)
+    try:
+        outs, variants = [], []
+        for _ in range(3):
+            ops.run(ab, a_dt, m, yb)
+            outs.append(ep.download(yb, (m, n), np.uint16).copy())
+            variants.append(ops.kernel.last_variant())
+        assert variants[0] == variants[1] == variants[2] == "gate_up_swiglu[acc4_mfma_i8_packed]", variants
+        assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
+    finally:
+        ep.deallocate(ab)
+        ep.deallocate(yb)
+        ops.free()
 
 
 @pytest.mark.parametrize("a_dt,g_dt,bs,m,n,k,eps", RMSNORM_CASES)
@@ -1051,6 +1098,89 @@ def test_block_accumulators_bit_exact(ep, port, bs, zero_points):
     assert np.array_equal(want.astype(np.int64), brute)
 
 
+def _production_block_acc(provider, port, a, a_dt, bs, zero_points, n, k, rounding, seed):
+    """Runs one accuracy_level=4 call with the accumulator probe set; returns (probe contents, oracle accumulators, y32, oracle y, variant)."""
+    m = a.shape[0]
+    kb = -(-k // bs)
+    b, s, zp = synth.make_weights(n, k, bs, seed, zero_points=zero_points, scale_lo=0.002, scale_hi=0.01, scale_dtype=a_dt)
+    ops = E.DeviceOperands(provider, b, s, a_dt, zp, n, k, bs, accuracy_level=4)
+    probe = provider.upload(np.full(m * n * kb, 0x7FFFFFFF, np.int32))                     # a sentinel no accumulator can reach
+    ab, yb = provider.upload(a), provider.allocate(m * n * 4)
+    try:
+        ops.kernel.set_block_acc_probe(probe)
+        ops.run(ab, a_dt, m, yb, E.F32)
+        got = provider.download(probe, (m, n, kb), np.int32)
+        y32 = provider.download(yb, (m, n), np.float32)
+        variant = ops.kernel.last_variant()
+        ops.kernel.set_block_acc_probe(None)
+        provider.copy_from_host(probe, np.full(m * n * kb, 0x7FFFFFFF, np.int32))
+        ops.run(ab, a_dt, m, yb, E.F32)                                                      # without the probe: same result, nothing stored
+        assert np.array_equal(provider.download(yb, (m, n), np.float32), y32)
+        assert (provider.download(probe, (m, n, kb), np.int32) == 0x7FFFFFFF).all()
+    finally:
+        for buf in (probe, ab, yb):
+            provider.deallocate(buf)
+        ops.free()
+    af, sf = synth.to_f32(a, a_dt), synth.to_f32(s, a_dt)
+    qa, _ = port.quantize_a(af, k, bs, rounding)
+    want = port.block_acc_i32(qa, b, zp, n, k, bs)
+    return got, want, y32, port.matmul_acc4_f32(af, b, sf, zp, n, k, bs, rounding), variant
+
+
+PRODUCTION_ACC_CASES = [
+    # bs, zero points, m, n, k, prepack - one row over the repacked stream and over the caller's layout, the split-K kernel at 5
+    # rows, the tiled kernel at 40; each with K short (one wave / one slice) and long (several waves / K in slices)
+    (32, True, 1, 100, 32 * 11, True), (64, True, 1, 333, 64 * 37, True), (128, False, 1, 160, 128 * 40, True),
+    (32, False, 1, 48, 32 * 9, False), (64, True, 1, 100, 64 * 50, False), (128, True, 1, 64, 128 * 24, False),
+    (32, True, 5, 48, 32 * 9, True), (64, True, 5, 100, 64 * 50, True), (128, False, 5, 77, 128 * 33, True), (64, True, 16, 40, 200, True),
+    (32, True, 40, 96, 32 * 35, True), (64, True, 40, 96, 64 * 17, True), (128, True, 130, 200, 128 * 20, True), (64, False, 40, 200, 64 * 3, True),
+    (256, True, 40, 96, 256 * 3, True), (32, False, 33, 64, 200, True),
+]
+
+
+@pytest.mark.parametrize("a_dt", [E.F16, E.BF16, E.F32])
+@pytest.mark.parametrize("bs,zero_points,m,n,k,prepack", PRODUCTION_ACC_CASES)
+def test_production_kernels_block_accumulators_bit_exact(port, a_dt, bs, zero_points, m, n, k, prepack):
+    """The int32 block accumulators as the production int8 matrix-core kernels hold them when they scale them into the result
+    (matmul_nbits.rs:9159-9177; canonical form acc[m,n,b] = sum_k code[m,k] * (q[n,k] - zp[n,b])): read out of the one-row
+    kernel over the repacked stream (with its fused quantizer for 16-bit rows), the split-K kernel and the tiled kernel, and
+    compared bit for bit with the oracle's integers."""
+    provider = E.RocmExecutionProvider(0, {"prepack": "1" if prepack else "0"})
+    try:
+        a = _tie_heavy_activation(m, k, bs, 300 + m, a_dt) if k % bs == 0 else synth.make_activation(m, k, 300 + m, a_dt)
+        got, want, y32, y_want, variant = _production_block_acc(provider, port, a, a_dt, bs, zero_points, n, k, oracle.ROUND_HALF_EVEN, 310 + n)
+        assert variant == ("acc4_mfma_i8_packed" if prepack and m == 1 else "acc4_mfma_i8")
+        assert not (got == 0x7FFFFFFF).any(), "an accumulator was never stored"
+        assert np.array_equal(got, want)
+        assert helpers.rel_l2(y32, y_want) <= TOL_F32
+    finally:
+        provider.shutdown()
+
+
+@pytest.mark.parametrize("a_dt", [E.F16, E.BF16])
+@pytest.mark.parametrize("bs", [32, 64, 128])
+@pytest.mark.parametrize("rounding", ["mlas", "native"])
+def test_fused_quantizer_on_ties_zero_blocks_and_extremes(port, a_dt, bs, rounding):
+    """The quantizer inside the one-row kernel over the repacked stream (every f16 / bf16 decode call at accuracy_level 4 over
+    constant weights) on the fixture that separates the two rounding rules: exact .5 ties, an all-zero block (scale 0, codes
+    0, no division by zero), +-max codes. Codes are checked through the integers they produce, bit for bit."""
+    n, k = 96, bs * 6
+    provider = E.RocmExecutionProvider(0, {"acc4_rounding": rounding})
+    try:
+        rule = oracle.ROUND_HALF_EVEN if rounding == "mlas" else oracle.ROUND_HALF_AWAY
+        a = _tie_heavy_activation(1, k, bs, 400 + bs, a_dt)
+        got, want, y32, y_want, variant = _production_block_acc(provider, port, a, a_dt, bs, True, n, k, rule, 410 + bs)
+        assert variant == "acc4_mfma_i8_packed"
+        assert np.array_equal(got, want)
+        assert (got[0, :, 0] == 0).all()                                   # the all-zero block
+        assert np.isfinite(y32).all() and helpers.rel_l2(y32, y_want) <= TOL_F32
+        af = synth.to_f32(a, a_dt)
+        other = port.quantize_a(af, k, bs, 1 - rule)[0]
+        assert (other != port.quantize_a(af, k, bs, rule)[0]).any()        # the fixture does separate the two rules
+    finally:
+        provider.shutdown()
+
+
 ACC4_CASES = [
     (E.F16, 64, True, 1, 160, 1024),
     (E.F16, 64, True, 5, 96, 512),
@@ -1257,6 +1387,15 @@ def test_execute_validation_messages(ep):
     bad[0] = E.TensorView(ab.ptr, E.F32, (2, k), device_type=0)
     fails(bad, good_out, "must live on ROCm device 0")
 
+    # a required tensor without memory behind it is refused before anything is launched
+    launches = ep.kernel_launch_count()
+    for slot, name in ((0, "A"), (1, "B"), (2, "scales")):
+        bad = list(good_in)
+        bad[slot] = E.TensorView(None, good_in[slot].dtype, good_in[slot].shape)
+        fails(bad, good_out, f"MatMulNBits: {name} has a null data pointer")
+    fails(good_in, [E.TensorView(None, E.F32, (2, n))], "MatMulNBits: Y has a null data pointer")
+    assert ep.kernel_launch_count() == launches
+
     # flat scales / zero points are accepted, as in the reference
     flat = list(good_in)
     flat[2] = E.TensorView(ops.scales.ptr, E.F32, (n * 2,))
@@ -1429,7 +1568,7 @@ def test_plain_c_host_roundtrip():
     assert os.path.exists(exe), "tests/harness/nxrt_roundtrip is built by __graft_entry__.build()"
     run = subprocess.run([exe, E.LIB_PATH], capture_output=True, text=True, timeout=100)
     assert run.returncode == 0, run.stdout + run.stderr
-    assert "roundtrip ok" in run.stdout and "accuracy_level 4" in run.stdout
+    assert "roundtrip ok" in run.stdout and "accuracy_level 4" in run.stdout and "nxmem unload report: nothing live" in run.stdout
 
 
 def test_launch_counter_proves_native_path(ep):
