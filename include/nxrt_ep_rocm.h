@@ -145,6 +145,23 @@ NxrtStatus nxrt_rocm_matmul_nbits_workspace_requirement(const NxrtRocmMatMulNBit
 NxrtStatus nxrt_rocm_matmul_nbits_execute(NxrtRocmMatMulNBits* kernel, const NxrtRocmTensorView* inputs, uint32_t n_inputs,
                                           NxrtRocmTensorView* outputs, uint32_t n_outputs,
                                           void* workspace_device, uint64_t workspace_bytes);
+/* execute for callers that cannot allocate: code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc. It has no counterpart in the reference. Same inputs, outputs, validation and results as
+ * nxrt_rocm_matmul_nbits_execute on a plain MatMulNBits node (fused gate/up and RMS-normalization nodes are refused), but the
+ * call allocates and frees nothing and calls no library routine that might: whatever scratch its kernels need (activation
+ * codes and scales of accuracy_level 4; partial sums of a tall call that cuts K into slices) lives in a static device array
+ * of NXRT_ROCM_STATIC_SCRATCH_BYTES that is part of the library's code object - one copy per GPU, held until the process
+ * ends, its address resolved once when the provider is created. Consequences:
+ *   - a call whose scratch does not fit is refused with INVALID_ARGUMENT and the sizes (accuracy_level 4 needs about
+ *     rows * K * (1 + 12 / block_size) bytes: at K = 8192, block 64, up to ~860 rows); optional scratch (K slices) shrinks to fit;
+ *   - nothing is set up on the fly: constant weights that have no repacked copy yet are streamed in the caller's layout, the
+ *     library GEMM route is not taken, a g_idx tensor must have been range-checked by an earlier execute;
+ *   - every call on one GPU shares that GPU's array, which keeps the last call's contents (the kernels overwrite all they
+ *     read). Calls through one provider are ordered by its stream; calls through different providers on the same GPU, or a
+ *     static call concurrent with another one's kernels still running on another stream, race on the array. */
+#define NXRT_ROCM_STATIC_SCRATCH_BYTES (8u << 20)
+NxrtStatus nxrt_rocm_matmul_nbits_execute_static(NxrtRocmMatMulNBits* kernel, const NxrtRocmTensorView* inputs, uint32_t n_inputs,
+                                                 NxrtRocmTensorView* outputs, uint32_t n_outputs);
 /* Kernel::estimated_flops (matmul_nbits.rs:2338): 2*M*N*K, 0 when M is not known from the shapes. */
 uint64_t nxrt_rocm_matmul_nbits_estimated_flops(const NxrtRocmMatMulNBits* kernel);
 /* record_kernel_variant (kernel.rs:361): which kernel served the last execute. */
@@ -209,6 +226,8 @@ void nxrt_rocm_ep_graph_release(NxrtRocmEp* ep, NxrtRocmGraph* graph);
  * (the role of nxrt_ep_compiled_node_count in ep-cuda-plugin/src/lib.rs:345-372). */
 uint64_t nxrt_rocm_ep_kernel_launch_count(const NxrtRocmEp* ep);
 uint64_t nxrt_rocm_live_provider_count(void);
+/* Device allocations (hipMalloc calls) the library has made in this process so far. */
+uint64_t nxrt_rocm_device_allocation_count(void);
 
 #ifdef __cplusplus
 }

@@ -156,6 +156,7 @@ struct NxrtRocmMatMulNBits {
     const void* dense_from[3] = {nullptr, nullptr, nullptr};
     int dense_dtype = 0, dense_scale_dtype = 0;
     std::mutex mu;                       // one execute at a time per kernel object: scratch, repacked copy and variant are per-object state
+    bool no_alloc = false;               // the call in progress (under `mu`) may not allocate or free device memory
     NxrtKernelVtable vtable;
     uint32_t vt_a_dtype = 0, vt_scale_dtype = 0, vt_y_dtype = 0;
 
@@ -180,6 +181,10 @@ struct NxrtRocmMatMulNBits {
 };
 
 namespace {
+
+// True while nothing may allocate, free or synchronise: a graph capture is open, or the call came in through the entry point
+// that allocates nothing.
+bool frozen(const NxrtRocmMatMulNBits& kn) { return kn.ep->capturing || kn.no_alloc; }
 
 // Scratch of accuracy_level=4 for M rows: int8 codes, (scale, code sum) pairs, and a block-major copy of the
 // pairs (M <= 16) or of the scales (M > 16) for the matrix-core kernels.
@@ -228,7 +233,7 @@ bool use_packed(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& args, int& r
     const bool current = kn.packed && kn.packed_from[0] == args.b && kn.packed_from[1] == args.scales && kn.packed_from[2] == args.zp &&
                          kn.packed_scale_dtype == args.scale_dtype;
     if (current) return true;
-    if (kn.ep->capturing) return false;
+    if (frozen(kn)) return false;
     if (kn.packed) {
         kn.retired.push_back(kn.packed);    // not freed: a HIP graph recorded over the old weights may still replay through it
         kn.packed = nullptr;
@@ -259,6 +264,7 @@ bool dense_route(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& args, int& 
 {
     rc = 0;
     NxrtRocmEp& ep = *kn.ep;
+    if (kn.no_alloc) return false;              // the library GEMM and its buffers are out of bounds for a call that may not allocate
     // other bit widths have no tiled kernel to fall back on, only the plain GEMV: the route pays from a few dozen rows
     const bool plain_only = kn.bits != 4 || args.g_idx != nullptr;
     const int64_t min_rows = !plain_only ? ep.dense_gemm_min_rows : (ep.dense_gemm_min_rows < 32 ? ep.dense_gemm_min_rows : 32);
@@ -400,9 +406,14 @@ bool f32_in_row_blocks(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& args,
 }
 
 NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, uint32_t n_in, NxrtRocmTensorView* out, uint32_t n_out,
-                        void* workspace, uint64_t workspace_bytes)
+                        void* workspace, uint64_t workspace_bytes, bool no_alloc = false)
 {
     std::lock_guard<std::mutex> lock(kn.mu);
+    struct Mode {
+        NxrtRocmMatMulNBits& k;
+        Mode(NxrtRocmMatMulNBits& kernel, bool on) : k(kernel) { k.no_alloc = on; }
+        ~Mode() { k.no_alloc = false; }
+    } mode(kn, no_alloc);
     // kernels/mod.rs:1898-1919 (check_arity)
     if (n_in < 3 || n_in > 6) return make_status(NXRT_INVALID_ARGUMENT, "MatMulNBits: expected 3..=6 inputs, got " + std::to_string(n_in));
     if (n_out < 1) return make_status(NXRT_INVALID_ARGUMENT, "MatMulNBits: expected at least 1 output(s), got " + std::to_string(n_out));
@@ -532,8 +543,9 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
     int rc = 0;
     if (G && kn.g_idx_checked != args.g_idx) {
         // matmul_nbits.rs:3515-3521: every group must lie in 0..kb. Checked once per tensor (a device pass and a read-back).
-        if (kn.ep->capturing)
-            return make_status(NXRT_INVALID_ARGUMENT, err("g_idx has not been range-checked yet and a graph capture is open; run this node once eagerly first"));
+        if (frozen(kn))
+            return make_status(NXRT_INVALID_ARGUMENT, err("g_idx has not been range-checked yet and this call may not allocate or synchronise (a graph capture is open, or it came "
+                                                          "through execute_static); run this node once through execute first"));
         int64_t bad = -1;
         const int e = rocm_g_idx_first_bad(args.g_idx, static_cast<int64_t>(K), static_cast<int64_t>(kb), &bad, stream);
         if (e != 0) return hip_status(e, "MatMulNBits: g_idx check");
@@ -561,9 +573,18 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
             kn.ep->launches.fetch_add(1);
             return hip_status(rc, "MatMulNBits: kernel launch");
         }
-        const uint64_t need = acc4_workspace_bytes(kn, M);
+        const Acc4Layout lay = acc4_layout(kn, M);
+        const uint64_t need = lay.total, mandatory = lay.codes + lay.pairs + lay.aux;
         uint8_t* ws = static_cast<uint8_t*>(workspace);
-        if (!ws || workspace_bytes < need) {
+        uint64_t partial_bytes = lay.partial;
+        if (kn.no_alloc) {
+            // the static scratch: codes, pairs and their block-major copy must fit; partial sums of K slices get what is left
+            // (with less room the tiled kernel cuts K into fewer slices, or none)
+            if (!ws || workspace_bytes < mandatory)
+                return make_status(NXRT_INVALID_ARGUMENT, err("accuracy_level=4 at " + std::to_string(M) + " rows needs " + std::to_string(mandatory) + " bytes of scratch and the static scratch of "
+                                                              "execute_static holds " + std::to_string(workspace_bytes) + "; call execute with a workspace of workspace_requirement() bytes instead"));
+            if (partial_bytes > workspace_bytes - mandatory) partial_bytes = (workspace_bytes - mandatory) / 256 * 256;
+        } else if (!ws || workspace_bytes < need) {
             if (kn.scratch_bytes < need) {
                 if (kn.ep->capturing)
                     return make_status(NXRT_INVALID_ARGUMENT, err("accuracy_level=4 under graph capture needs a caller workspace of " + std::to_string(need) +
@@ -573,14 +594,13 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
             }
             ws = static_cast<uint8_t*>(kn.scratch);
         }
-        const Acc4Layout lay = acc4_layout(kn, M);
         RocmAcc4Workspace w4;
         w4.qa = reinterpret_cast<int8_t*>(ws);
         w4.aq = reinterpret_cast<float*>(ws + lay.codes);
         w4.aux = reinterpret_cast<float*>(ws + lay.codes + lay.pairs);
         w4.code_order = packed ? 2 : 1;
-        w4.partial = lay.partial ? reinterpret_cast<float*>(ws + lay.codes + lay.pairs + lay.aux) : nullptr;
-        w4.partial_bytes = lay.partial;
+        w4.partial = partial_bytes ? reinterpret_cast<float*>(ws + lay.codes + lay.pairs + lay.aux) : nullptr;
+        w4.partial_bytes = partial_bytes;
         rc = rocm_launch_quantize_a_workspace(args.a, args.a_dtype, args.m, args.k, args.block_size, rounding, &w4, stream);
         if (rc == 0 && pack_rc != 0) rc = pack_rc;
         if (rc == 0) {
@@ -614,7 +634,7 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
         void* scratch = workspace;
         uint64_t scratch_bytes = workspace ? workspace_bytes : 0;
         if (need > scratch_bytes) {
-            if (kn.scratch_bytes < need && !kn.ep->capturing) (void)grow_buffer(kn.scratch, kn.scratch_bytes, need, kn.retired);   // on failure: slice less
+            if (kn.scratch_bytes < need && !frozen(kn)) (void)grow_buffer(kn.scratch, kn.scratch_bytes, need, kn.retired);   // on failure: slice less
             if (kn.scratch_bytes > scratch_bytes) {
                 scratch = kn.scratch;
                 scratch_bytes = kn.scratch_bytes;
@@ -1035,6 +1055,20 @@ NxrtStatus nxrt_rocm_matmul_nbits_execute(NxrtRocmMatMulNBits* kernel, const Nxr
         if (kernel->rmsnorm_prologue) return execute_normalized(*kernel, inputs, n_inputs, outputs, n_outputs, workspace_device, workspace_bytes);
         if (kernel->gate_up_swiglu) return execute_swiglu(*kernel, inputs, n_inputs, outputs, n_outputs, workspace_device, workspace_bytes);
         return execute_impl(*kernel, inputs, n_inputs, outputs, n_outputs, workspace_device, workspace_bytes);
+    });
+}
+
+NxrtStatus nxrt_rocm_matmul_nbits_execute_static(NxrtRocmMatMulNBits* kernel, const NxrtRocmTensorView* inputs, uint32_t n_inputs, NxrtRocmTensorView* outputs,
+                                                 uint32_t n_outputs)
+{
+    return fenced([&]() -> NxrtStatus {
+        if (!kernel) return make_status(NXRT_INVALID_ARGUMENT, "MatMulNBits: null kernel");
+        if (kernel->rmsnorm_prologue || kernel->gate_up_swiglu)
+            return make_status(NXRT_INVALID_ARGUMENT, err("execute_static serves plain MatMulNBits nodes; fused nodes (gate/up, RMS-normalization prologue) keep intermediates of their own - "
+                                                          "call execute with a workspace"));
+        NxrtRocmEp* ep = kernel->ep;
+        if (!ep->static_scratch) return make_status(NXRT_INTERNAL_ERROR, err("the static scratch of this GPU was not resolved when the provider was created"));
+        return execute_impl(*kernel, inputs, n_inputs, outputs, n_outputs, ep->static_scratch, ep->static_scratch_bytes, true);
     });
 }
 

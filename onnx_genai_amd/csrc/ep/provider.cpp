@@ -98,6 +98,7 @@ NxrtStatus nxrt_rocm_ep_create(uint32_t device_ordinal, const char* const* keys,
         if ((it = ep->config.find("dense_gemm_min_rows")) != ep->config.end()) ep->dense_gemm_min_rows = parse_int(it->second, ep->dense_gemm_min_rows);
         NxrtStatus st = ep->bind();
         if (st.code == NXRT_OK) st = hip_status(rocm_ffi_stream_create(&ep->stream), "hipStreamCreate");
+        if (st.code == NXRT_OK) st = hip_status(rocm_ffi_static_scratch(static_cast<int>(ep->device), &ep->static_scratch, &ep->static_scratch_bytes), "hipGetSymbolAddress(static scratch)");
         if (st.code != NXRT_OK) {
             delete ep;
             return st;
@@ -307,5 +308,6 @@ void nxrt_rocm_ep_graph_release(NxrtRocmEp* ep, NxrtRocmGraph* graph)
 
 uint64_t nxrt_rocm_ep_kernel_launch_count(const NxrtRocmEp* ep) { return ep ? ep->launches.load() : 0; }
 uint64_t nxrt_rocm_live_provider_count(void) { return g_live_providers.load(); }
+uint64_t nxrt_rocm_device_allocation_count(void) { return rocm_ffi_malloc_calls(); }
 
 }  // extern "C"

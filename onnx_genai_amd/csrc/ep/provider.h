@@ -33,6 +33,8 @@ struct NxrtRocmEp {
     std::mutex mu;
     std::unordered_map<void*, size_t> live;       // allocations handed out and not yet returned
     std::atomic<uint64_t> launches{0};
+    void* static_scratch = nullptr;               // this GPU's static scratch array (device address), resolved when the provider is created
+    size_t static_scratch_bytes = 0;
     bool capturing = false;                       // a stream capture is open: nothing may allocate or synchronise
     // The host may release the provider, its kernels and its allocators in any order (each vtable is released exactly
     // once, independently): every kernel object and allocator handle holds one reference, the creator holds the first,

@@ -32,6 +32,12 @@ int rocm_ffi_set_device(int device);
 int rocm_ffi_device_info(int device, char* arch, size_t arch_len, int* compute_units, size_t* total_mem);
 int rocm_ffi_malloc(void** ptr, size_t bytes);
 int rocm_ffi_free(void* ptr);
+/* How many times rocm_ffi_malloc has been called in this process (every device allocation of the library goes through it). */
+uint64_t rocm_ffi_malloc_calls(void);
+/* Device address and size of the library's static scratch array on `device` (a __device__ array of the code object, 256-byte
+ * aligned, one per GPU, never freed). The first call for a device makes that device current and resolves the address; later
+ * calls only read it back. Shared by every caller on that GPU and never cleared: contents are whatever the last user left. */
+int rocm_ffi_static_scratch(int device, void** ptr, size_t* bytes);
 int rocm_ffi_memcpy_h2d(void* dst, const void* src, size_t bytes, rocm_stream_t stream);
 int rocm_ffi_memcpy_d2h(void* dst, const void* src, size_t bytes, rocm_stream_t stream);
 int rocm_ffi_memcpy_d2d(void* dst, const void* src, size_t bytes, rocm_stream_t stream);

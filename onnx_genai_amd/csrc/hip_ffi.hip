@@ -1,11 +1,23 @@
 // HIP runtime half of hip_ffi.h: device memory, the stream, events. No kernels live here.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstring>
+#include <mutex>
 
 #include "hip_ffi.h"
 
 namespace {
+// Scratch for the entry point that may not allocate (rocm_ffi_static_scratch): one array per GPU, part of the code object,
+// alive from the moment the library is loaded on a device until the process ends. Host code never uses this name as an
+// address - it is a host-side stand-in; the device address is asked for once per device (hipGetSymbolAddress) and kept.
+constexpr size_t kStaticScratchBytes = 8u << 20;
+__device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+constexpr int kMaxScratchDevices = 64;
+void* g_scratch_ptr[kMaxScratchDevices] = {};
+std::mutex g_scratch_mu;
+std::atomic<uint64_t> g_device_allocations{0};
+
 __global__ void fill_u32_kernel(uint32_t* dst, uint32_t value, size_t count)
 {
     for (size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; i < count; i += static_cast<size_t>(gridDim.x) * blockDim.x) dst[i] = value;
@@ -38,7 +50,30 @@ int rocm_ffi_device_info(int device, char* arch, size_t arch_len, int* compute_u
     return 0;
 }
 
-int rocm_ffi_malloc(void** ptr, size_t bytes) { return static_cast<int>(hipMalloc(ptr, bytes)); }
+int rocm_ffi_malloc(void** ptr, size_t bytes)
+{
+    g_device_allocations.fetch_add(1);
+    return static_cast<int>(hipMalloc(ptr, bytes));
+}
+uint64_t rocm_ffi_malloc_calls(void) { return g_device_allocations.load(); }
+
+int rocm_ffi_static_scratch(int device, void** ptr, size_t* bytes)
+{
+    if (!ptr || !bytes || device < 0 || device >= kMaxScratchDevices) return static_cast<int>(hipErrorInvalidValue);
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (!g_scratch_ptr[device]) {
+        // every GPU holds its own copy of the array at its own address: ask with that GPU current
+        hipError_t e = hipSetDevice(device);
+        void* p = nullptr;
+        if (e == hipSuccess) e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return static_cast<int>(e);
+        if (!p) return static_cast<int>(hipErrorInvalidSymbol);
+        g_scratch_ptr[device] = p;
+    }
+    *ptr = g_scratch_ptr[device];
+    *bytes = kStaticScratchBytes;
+    return 0;
+}
 int rocm_ffi_free(void* ptr) { return static_cast<int>(hipFree(ptr)); }
 
 int rocm_ffi_memcpy_h2d(void* dst, const void* src, size_t bytes, rocm_stream_t stream)

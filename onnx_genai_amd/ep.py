@@ -111,6 +111,10 @@ def load_library() -> C.CDLL:
     L.nxrt_rocm_matmul_nbits_workspace_requirement.argtypes = [v, C.POINTER(NxrtTensorDesc), u32, C.POINTER(WorkspaceRequirement)]
     L.nxrt_rocm_matmul_nbits_execute.restype = S
     L.nxrt_rocm_matmul_nbits_execute.argtypes = [v, C.POINTER(CTensorView), u32, C.POINTER(CTensorView), u32, v, u64]
+    L.nxrt_rocm_matmul_nbits_execute_static.restype = S
+    L.nxrt_rocm_matmul_nbits_execute_static.argtypes = [v, C.POINTER(CTensorView), u32, C.POINTER(CTensorView), u32]
+    L.nxrt_rocm_device_allocation_count.restype = u64
+    L.nxrt_rocm_device_allocation_count.argtypes = []
     L.nxrt_rocm_matmul_nbits_estimated_flops.restype = u64
     L.nxrt_rocm_matmul_nbits_estimated_flops.argtypes = [v]
     L.nxrt_rocm_matmul_nbits_last_variant.restype = C.c_char_p
@@ -432,6 +436,12 @@ class MatMulNBitsKernel:
         cout, k2 = _c_views(outputs)
         self.lib.nxrt_rocm_matmul_nbits_execute(self.handle, cin, len(inputs), cout, len(outputs),
                                                 workspace.ptr if workspace else None, workspace.nbytes if workspace else 0).check()
+
+    def execute_static(self, inputs, outputs) -> None:
+        """execute without any device allocation: scratch comes from the library's static per-GPU array."""
+        cin, k1 = _c_views(inputs)
+        cout, k2 = _c_views(outputs)
+        self.lib.nxrt_rocm_matmul_nbits_execute_static(self.handle, cin, len(inputs), cout, len(outputs)).check()
 
     def estimated_flops(self) -> int:
         return self.lib.nxrt_rocm_matmul_nbits_estimated_flops(self.handle)

@@ -1,0 +1,96 @@
+"""The entry point that allocates nothing (nxrt_rocm_matmul_nbits_execute_static) against nxrt_rocm_matmul_nbits_execute.
+
+Collected last on purpose (the file name sorts after every other test file): the round-end run stops at the first
+failure, and a failure here should not hide the parity tests.
+"""
+import numpy as np
+import pytest
+
+from onnx_genai_amd import ep as E
+from onnx_genai_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+
+def _both_ways(provider, a_dt, bs, acc, m, n, k, y_dt, seed):
+    """One node, the same inputs through execute and through execute_static; returns both outputs, the variant of each, and
+    the number of device allocations the static call made."""
+    lib = provider.lib
+    b, s, zp = synth.make_weights(n, k, bs, seed, zero_points=True, scale_lo=0.002, scale_hi=0.01, scale_dtype=a_dt)
+    a = synth.make_activation(m, k, seed + 1, a_dt)
+    bias = synth.to_dtype(np.linspace(-1, 1, n).astype(np.float32), a_dt)
+    ops = E.DeviceOperands(provider, b, s, a_dt, zp, n, k, bs, accuracy_level=acc, bias=bias, bias_dtype=a_dt)
+    item = 4 if y_dt == E.F32 else 2
+    np_dt = np.float32 if y_dt == E.F32 else np.uint16
+    ab, y1, y2 = provider.upload(a), provider.allocate(m * n * item), provider.allocate(m * n * item)
+    try:
+        views = ops.views(ab, a_dt, m)
+        ops.kernel.execute(views, [E.TensorView(y1.ptr, y_dt, (m, n))])
+        v1 = ops.kernel.last_variant()
+        want = provider.download(y1, (m, n), np_dt)
+        provider.copy_from_host(y2, np.full(m * n * item, 0xEE, np.uint8))
+        before = lib.nxrt_rocm_device_allocation_count()
+        ops.kernel.execute_static(views, [E.TensorView(y2.ptr, y_dt, (m, n))])
+        allocations = lib.nxrt_rocm_device_allocation_count() - before
+        v2 = ops.kernel.last_variant()
+        got = provider.download(y2, (m, n), np_dt)
+    finally:
+        for buf in (ab, y1, y2):
+            provider.deallocate(buf)
+        ops.free()
+    return want, got, v1, v2, allocations
+
+
+def test_execute_static_matches_execute_and_allocates_nothing():
+    # weights streamed as given (no repacked copy, no dense copy): both entry points then run the same kernels
+    provider = E.RocmExecutionProvider(0, {"prepack": "0", "dense_gemm_min_rows": "0"})
+    try:
+        calls = [
+            # a_dt, block, accuracy_level, m, n, k, y dtype - each pair: a larger call, then a smaller one over the same scratch
+            (E.F16, 64, 4, 40, 96, 64 * 17, E.F32),       # int8 tiled kernel, K in two slices: codes, scales and partial sums in scratch
+            (E.F16, 64, 4, 3, 50, 256, E.F32),            # int8 split-K kernel, a few KB of codes
+            (E.F16, 64, 0, 100, 130, 4096, E.F16),        # float tiled kernel, K in slices: f32 partial sums in scratch
+            (E.BF16, 128, 0, 40, 72, 2048, E.BF16),       # the same kernel, smaller, fewer slices
+            (E.F16, 32, 4, 1, 48, 4100, E.F32),           # one row, K % 8 != 0: the separate quantizer fills the scratch
+            (E.BF16, 128, 0, 4, 300, 3584, E.BF16),       # a decode call: no scratch at all
+        ]
+        for i, (a_dt, bs, acc, m, n, k, y_dt) in enumerate(calls):
+            want, got, v1, v2, allocations = _both_ways(provider, a_dt, bs, acc, m, n, k, y_dt, 900 + i)
+            assert v1 == v2, (calls[i], v1, v2)
+            assert allocations == 0, (calls[i], allocations)
+            assert np.array_equal(want, got), (calls[i], v1)            # same kernels, same order of summation: the same bits
+    finally:
+        provider.shutdown()
+
+
+def test_execute_static_refuses_what_does_not_fit():
+    provider = E.RocmExecutionProvider(0, {"prepack": "0", "dense_gemm_min_rows": "0"})
+    try:
+        a_dt, bs, m, n, k = E.F16, 64, 2048, 64, 8192                    # 16 MiB of activation codes: beyond the 8 MiB array
+        b, s, zp = synth.make_weights(n, k, bs, 950, zero_points=True, scale_lo=0.002, scale_hi=0.01, scale_dtype=a_dt)
+        ops = E.DeviceOperands(provider, b, s, a_dt, zp, n, k, bs, accuracy_level=4)
+        ab, yb = provider.upload(synth.make_activation(m, k, 951, a_dt)), provider.allocate(m * n * 2)
+        try:
+            launches = provider.kernel_launch_count()
+            with pytest.raises(E.EpError) as e:
+                ops.kernel.execute_static(ops.views(ab, a_dt, m), [E.TensorView(yb.ptr, a_dt, (m, n))])
+            assert "bytes of scratch and the static scratch of execute_static holds 8388608" in str(e.value)
+            assert provider.kernel_launch_count() == launches
+            ops.kernel.execute(ops.views(ab, a_dt, m), [E.TensorView(yb.ptr, a_dt, (m, n))])          # the allocating entry point takes it
+        finally:
+            provider.deallocate(ab)
+            provider.deallocate(yb)
+            ops.free()
+        fused = E.GateUpOperands(provider, synth.make_weights(32, 128, 32, 1, zero_points=False, scale_lo=0.01, scale_hi=0.02, scale_dtype=E.F16),
+                                 synth.make_weights(32, 128, 32, 2, zero_points=False, scale_lo=0.01, scale_hi=0.02, scale_dtype=E.F16), E.F16, 32, 128, 32)
+        ab, yb = provider.upload(synth.make_activation(1, 128, 3, E.F16)), provider.allocate(64)
+        try:
+            with pytest.raises(E.EpError) as e:
+                fused.kernel.execute_static(fused.views(ab, E.F16, 1), [E.TensorView(yb.ptr, E.F16, (1, 32))])
+            assert "execute_static serves plain MatMulNBits nodes" in str(e.value)
+        finally:
+            provider.deallocate(ab)
+            provider.deallocate(yb)
+            fused.free()
+    finally:
+        provider.shutdown()
