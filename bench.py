@@ -41,9 +41,55 @@ BS = 128
 A_DT = E.BF16
 
 
-# HBM bytes one gate/up launch (M=1, repacked weights) moves, from two rocprofv3 counter runs of `bench.py --only-roofline`:
-# FETCH_SIZE 35,282.4 KiB-units x 1.9997 (what the same counter reads for a 256 MiB copy) plus WRITE_SIZE 74.0 KiB.
-GATE_UP_HBM_BYTES_PER_LAUNCH = 72_324_100
+# HBM bytes one gate/up launch (M=1, repacked weights) moves come from two rocprofv3 counter runs of `bench.py --only-roofline`
+# (FETCH_SIZE, then WRITE_SIZE, each scaled by what the same counter reads for the 256 MiB copy that run ends with).
+# `bench.py --traffic-from <fetch csv> <write csv>` turns the two counter files into this tracked JSON; the benchmark line
+# reports its figure only while the kernel variant it was taken on is still the one that runs.
+TRAFFIC_JSON = os.path.join(ROOT, "profiles", "decode_gate_up_m1_traffic.json")
+
+
+def traffic_from_counters(fetch_csv, write_csv):
+    """Reads two rocprofv3 `--pmc` counter files of `bench.py --only-roofline` and writes TRAFFIC_JSON."""
+    import csv
+    copy_bytes = 256 << 20
+
+    def per_kernel(path, counter):
+        by = {}
+        for r in csv.DictReader(open(path)):
+            if r["Counter_Name"] == counter:
+                by.setdefault(r["Kernel_Name"], []).append(float(r["Counter_Value"]))
+        return {k: sum(v) / len(v) for k, v in by.items()}, {k: len(v) for k, v in by.items()}
+
+    fetch, n_fetch = per_kernel(fetch_csv, "FETCH_SIZE")
+    write, _ = per_kernel(write_csv, "WRITE_SIZE")
+    copy = next(k for k in fetch if "copy_kernel" in k)
+    decode = max((k for k in fetch if "decode" in k and "pack_decode" not in k), key=lambda k: n_fetch[k])
+    fetch_factor = (copy_bytes / 1024.0) / fetch[copy]
+    write_factor = (copy_bytes / 1024.0) / write[copy]
+    hbm = (fetch[decode] * fetch_factor + write[decode] * write_factor) * 1024.0
+    out = {"kernel": decode, "workload": "gate_up 3584->37888, M=1, bf16, block 128, zero points, repacked weights",
+           "fetch_size_kib_per_dispatch": round(fetch[decode], 1), "write_size_kib_per_dispatch": round(write[decode], 1),
+           "copy_kernel_fetch_size_kib": round(fetch[copy], 1), "copy_kernel_write_size_kib": round(write[copy], 1),
+           "fetch_scale": round(fetch_factor, 4), "write_scale": round(write_factor, 4), "dispatches": n_fetch[decode],
+           "hbm_bytes_per_launch": int(round(hbm)),
+           "commands": ["rocprofv3 --pmc FETCH_SIZE --output-format csv -d <dir> -o run -- python3 bench.py --only-roofline --steps 2 --warmup 1",
+                        "rocprofv3 --pmc WRITE_SIZE --output-format csv -d <dir> -o run -- python3 bench.py --only-roofline --steps 2 --warmup 1",
+                        "python3 bench.py --traffic-from <fetch run_counter_collection.csv> <write run_counter_collection.csv>"]}
+    with open(TRAFFIC_JSON, "w") as f:
+        json.dump(out, f, indent=1)
+        f.write("\n")
+    return out
+
+
+def measured_traffic(kernel_template_hint):
+    """HBM bytes per launch of the gate/up decode kernel from the tracked counter summary, or None when there is none
+    or it was taken on another kernel."""
+    try:
+        with open(TRAFFIC_JSON) as f:
+            t = json.load(f)
+    except (OSError, ValueError):
+        return None
+    return t["hbm_bytes_per_launch"] if kernel_template_hint in t.get("kernel", "") else None
 
 
 def _device_random_weights(ep, n, k, bs, seed, scale_lo, scale_hi, dtype, zero_points=True, reuse=None):
@@ -213,6 +259,7 @@ def cpu_baseline(seconds_budget=20.0, threads=None):
     if not oracle.Ref.available():
         return None
     ref, port = oracle.Ref(), oracle.Port()
+    # the GPU box gives one job the CPU share of one GPU (16 hardware threads), whatever os.cpu_count() shows of the host
     threads = threads or min(16, os.cpu_count() or 1)
     k, n, m = HIDDEN, 2 * INTER, 1
     copies = 3                                         # 3 x 68 MB of packed weights: larger than the last-level cache
@@ -264,21 +311,29 @@ def cpu_baseline(seconds_budget=20.0, threads=None):
         dt = (time.perf_counter() - t0) / calls
         result[label] = {"gbs": nbytes / dt / 1e9, "us": dt * 1e6, "calls": calls}
     pool.shutdown()
-    cpu_model = ""
+    cpu_model, cpu_ids = "", {}
     try:
         with open("/proc/cpuinfo") as f:
             for line in f:
-                if line.startswith("model name"):
-                    cpu_model = line.split(":", 1)[1].strip()
-                    break
+                key, _, value = line.partition(":")
+                key = key.strip()
+                if key == "model name" and not cpu_model:
+                    cpu_model = value.strip()
+                if key in ("cpu family", "model", "stepping", "cpu MHz") and key not in cpu_ids:
+                    cpu_ids[key] = value.strip()
     except OSError:
         pass
+    try:
+        usable = len(os.sched_getaffinity(0))
+    except (AttributeError, OSError):
+        usable = os.cpu_count() or 1
     best = result[str(threads)]
     return {"value": round(best["gbs"], 2), "unit": "GB/s", "cores": threads, "kind": "reference",
             "sample": f"MLAS SQNBit CompFp32 (oracle/_ref), gate_up 3584->37888, M=1, bf16 in/out widened+narrowed in the timed region, "
                       f"block 128 with zero points, {best['calls']} calls rotating over {copies} weight copies, N-sharded over {threads} threads",
             "us_per_call": round(best["us"], 1), "single_thread_gbs": round(result["1"]["gbs"], 2),
-            "dispatch": ref.dispatch_id(), "cpu": cpu_model}
+            "dispatch": ref.dispatch_id(), "cpu": cpu_model, "cpu_ids": cpu_ids, "host_logical_cpus": os.cpu_count(), "usable_cpus": usable,
+            "note": "cores = worker threads used: the CPU share a one-GPU job is given on this host (16), not every core of the machine"}
 
 
 def main():
@@ -295,11 +350,16 @@ def main():
                     help="run only the roofline leg (decode kernel on the gate_up shape) and one 256 MiB device copy: the command profiles are taken from")
     ap.add_argument("--only-tables", action="store_true",
                     help="run only the prefill and accuracy_level=4 tables, one JSON line per row (the command their profiles are taken from)")
+    ap.add_argument("--traffic-from", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
+                    help="no GPU work: turn two rocprofv3 counter files of --only-roofline runs (FETCH_SIZE, WRITE_SIZE) into profiles/decode_gate_up_m1_traffic.json")
     ap.add_argument("--row-sweep", action="store_true",
                     help="run only a sweep of the row count M across the dispatch boundaries (1 .. 2048), one JSON line per call shape")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (no collectives exist on the MatMulNBits path); use --gpus 1")
+    if args.traffic_from:
+        print(json.dumps(traffic_from_counters(*args.traffic_from)), flush=True)
+        return
 
     ep = E.RocmExecutionProvider(0)
     info = ep.device_info()
@@ -350,7 +410,8 @@ def main():
     roofline = {"bound": "hbm", "kernel": "%s<bf16, block 128> on gate_up 3584->37888, M=%d" % (gate_up[0].ops.kernel.last_variant(), args.m),
                 "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                 "bytes_per_launch": gate_up[0].bytes, "us_per_launch": round(launch_us, 2),
-                "traffic": GATE_UP_HBM_BYTES_PER_LAUNCH if args.m == 1 and gate_up[0].ops.kernel.last_variant() == "decode_mfma_packed" else None}
+                "traffic": measured_traffic("decode_packed_kernel") if args.m == 1 and gate_up[0].ops.kernel.last_variant() == "decode_mfma_packed" else None,
+                "traffic_source": os.path.relpath(TRAFFIC_JSON, ROOT)}
     g2.release()
 
     result = {
@@ -485,11 +546,12 @@ def row_sweep(ep):
 
 
 def prefill_routes(ep):
-    """The three ways a tall 16-bit call can run, each as its own provider: the hand-written tiled kernel only; the
-    default dispatch (from 1024 rows: weights expanded into one shared 16-bit buffer per call, then the library GEMM);
-    constant weights keeping a resident 16-bit copy (the call is the library GEMM alone)."""
-    return [("tiled", E.RocmExecutionProvider(0, {"dense_gemm_min_rows": "0"}), True), ("default", ep, False),
-            ("resident", E.RocmExecutionProvider(0, {"dense_weights": "resident"}), True)]
+    """The ways a tall 16-bit call can run, each as its own provider: the default dispatch (this provider's own tiled
+    kernel at every height); and, for comparison, the two opt-in forms of the dense route - weights expanded into one
+    shared 16-bit buffer per call and then the library GEMM (from 1024 rows), or constant weights keeping a resident
+    16-bit copy (the call is the library GEMM alone)."""
+    return [("default", ep, False), ("library_transient", E.RocmExecutionProvider(0, {"dense_gemm_min_rows": "1024"}), True),
+            ("library_resident", E.RocmExecutionProvider(0, {"dense_weights": "resident"}), True)]
 
 
 def prefill_table(ep, shapes=((4096, 14336), (14336, 4096)), rows=(512, 2048, 8192), dtype=E.F16, bs=32, zero_points=False):

@@ -35,8 +35,9 @@ typedef struct NxrtRocmMatMulNBits NxrtRocmMatMulNBits;   /* one kernel = one Ma
  *             "acc4_native_below" rows, else mlas: the CPU provider's route, matmul_nbits.rs:640-660);
  *             "prepack" = "1" (default: constant weights are copied once into the decode kernels' streaming order) | "0";
  *             "dense_gemm_min_rows" = rows from which a 16-bit call expands the weights to a dense [N, K] matrix and runs
- *             the library GEMM ("0" = never; default 1024, or 256 with resident copies; the CUDA provider's
- *             dequantize + cuBLASLt route, onnx-runtime-ep-cuda/src/kernels/matmul_nbits.rs:6176-6222);
+ *             the library GEMM (hipBLASLt) instead of this provider's own tiled kernel: opt-in, default "0" = never (256 once
+ *             "dense_weights" = "resident" is chosen; the CUDA provider's dequantize + cuBLASLt route,
+ *             onnx-runtime-ep-cuda/src/kernels/matmul_nbits.rs:6176-6222);
  *             "dense_gemm_max_mb" = largest dense copy of one weight (default 1024, as matmul_nbits.rs:6212);
  *             "dense_weights" = "transient" (default: one buffer per provider, refilled by every such call) |
  *             "resident" (a constant weight keeps its dense copy: 2 bytes per weight of HBM for a call that is the

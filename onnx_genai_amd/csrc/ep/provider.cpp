@@ -27,10 +27,11 @@ NxrtRocmEp::~NxrtRocmEp()
 
 NxrtStatus NxrtRocmEp::bind() const { return hip_status(rocm_ffi_set_device(static_cast<int>(device)), "hipSetDevice"); }
 
-// Rows from which the dense route (expand the weights, then the library GEMM) is the default. Measured at 8B / 7B MLP
-// shapes against the tiled kernel: refilling the dense buffer on every call pays from about a thousand rows; a
-// resident copy (no expansion per call) from a few hundred.
-constexpr int kDenseGemmMinRows = 1024;
+// The dense route (expand the weights to 16 bits, then the library GEMM) is opt-in: by default every call runs on this
+// provider's own kernels. `dense_gemm_min_rows` > 0 turns it on from that many rows; `dense_weights = resident` turns it
+// on from kDenseGemmMinRowsResident rows unless `dense_gemm_min_rows` says otherwise. Measured at 8B / 7B MLP shapes
+// against the tiled kernel: refilling the dense buffer on every call pays from about a thousand rows; a resident copy
+// (no expansion per call) from a few hundred.
 constexpr int kDenseGemmMinRowsResident = 256;
 
 static int parse_int(const std::string& v, int fallback)
@@ -94,7 +95,7 @@ NxrtStatus nxrt_rocm_ep_create(uint32_t device_ordinal, const char* const* keys,
                 return make_status(NXRT_INVALID_ARGUMENT, "RocmExecutionProvider: dense_weights must be 'transient' or 'resident'");
             }
         }
-        ep->dense_gemm_min_rows = ep->dense_resident ? kDenseGemmMinRowsResident : kDenseGemmMinRows;
+        ep->dense_gemm_min_rows = ep->dense_resident ? kDenseGemmMinRowsResident : 0;
         if ((it = ep->config.find("dense_gemm_min_rows")) != ep->config.end()) ep->dense_gemm_min_rows = parse_int(it->second, ep->dense_gemm_min_rows);
         NxrtStatus st = ep->bind();
         if (st.code == NXRT_OK) st = hip_status(rocm_ffi_stream_create(&ep->stream), "hipStreamCreate");

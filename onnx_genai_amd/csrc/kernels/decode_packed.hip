@@ -1094,6 +1094,17 @@ static int launch_decode_packed(const RocmMatMulNBitsArgs* a, const void* packed
     const int64_t wgs = (a->n + 15) / 16 * (pair_member ? 2 : 1);
     int w = waves;
     bool single_set = wgs * 4 >= 6144;
+    // One row (not a member of a gate/up pair, whose split of K is fixed by the paired launch): one tile group per wave where
+    // the workgroup can hold that many waves, no prefetch, offset and zero point through the activation sums. Every byte
+    // of the call is then requested as soon as its wave starts, and what a wave computes between its loads and the
+    // reduction is the least any variant here does. Measured against the few-wave prefetching build it replaced on the
+    // small shapes (bf16, block 128): 3584 -> 4608 5.06 -> 4.78 us, 3584 -> 3584 4.17 -> 3.97, 18944 -> 3584 9.94 -> 9.41,
+    // 3584 -> 37888 15.81 -> 15.48.
+    const bool one_row = a->m <= 1 && !pair_member;
+    if (one_row && w <= 0) {
+        single_set = true;
+        w = p.groups;
+    } else
     if (w <= 0) {
         if (single_set) {
             w = (p.groups + 1) / 2;
@@ -1105,6 +1116,7 @@ static int launch_decode_packed(const RocmMatMulNBitsArgs* a, const void* packed
     } else {
         single_set = wgs * w >= 6144;
     }
+    if (one_row) single_set = true;
     const int w_max = (a->block_size == 128 && !f32_scales) ? 16 : 8;      // see the kernel's launch bounds
     if (w > w_max) w = w_max;
     if (w > p.groups) w = p.groups;

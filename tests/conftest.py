@@ -52,8 +52,19 @@ def ep_unpacked():
 
 @pytest.fixture(scope="session")
 def ep_tiled():
-    """A provider whose tall 16-bit calls stay on the hand-written tiled kernel (no dense copy, no library GEMM)."""
+    """A provider whose tall 16-bit calls stay on the hand-written tiled kernel (no dense copy, no library GEMM) - the
+    default, spelled out."""
     from onnx_genai_amd.ep import RocmExecutionProvider
     provider = RocmExecutionProvider(0, {"dense_gemm_min_rows": "0"})
+    yield provider
+    provider.shutdown()
+
+
+@pytest.fixture(scope="session")
+def ep_dense():
+    """A provider with the opt-in dense route on: from 1024 rows (32 for bit widths and act-order weights that have no tiled
+    kernel) a 16-bit call expands the weights and runs the library GEMM."""
+    from onnx_genai_amd.ep import RocmExecutionProvider
+    provider = RocmExecutionProvider(0, {"dense_gemm_min_rows": "1024"})
     yield provider
     provider.shutdown()

@@ -625,8 +625,10 @@ def test_one_row_residual_in_the_bias_slot(ep, port, folded, bias_shape, a_dt, b
     assert f"bias must have {n} elements" in str(e.value)
 
 
-def test_folded_bias_keeps_tall_calls_off_the_library_gemm(ep):
-    """The library's epilogue adds a bias before the one rounding, so a folded bias stays on the hand-written kernel."""
+def test_folded_bias_keeps_tall_calls_off_the_library_gemm(ep_dense):
+    """The library's epilogue adds a bias before the one rounding, so a folded bias stays on the hand-written kernel even
+    where the opt-in dense route is on."""
+    ep = ep_dense
     a_dt, bs, m, n, k = E.F16, 32, 1100, 136, 512
     b, s, zp = synth.make_weights(n, k, bs, 5, zero_points=False, scale_lo=0.002, scale_hi=0.01, scale_dtype=a_dt)
     a = synth.make_activation(m, k, 5, a_dt)
@@ -673,13 +675,15 @@ NBITS_CASES = [
 
 @pytest.mark.parametrize("bits", [2, 8])
 @pytest.mark.parametrize("a_dt,s_dt,bs,zero_points,m,n,k", NBITS_CASES)
-def test_other_bit_widths_match_oracle(ep, port, bits, a_dt, s_dt, bs, zero_points, m, n, k):
+def test_other_bit_widths_match_oracle(ep, ep_dense, port, bits, a_dt, s_dt, bs, zero_points, m, n, k):
+    tall = a_dt != E.F32 and m >= 32 and k % 8 == 0
+    if tall:
+        ep = ep_dense                                  # with the opt-in dense route tall calls leave the plain kernel
     b, s, zp = synth.make_weights_bits(n, k, bs, bits, 50 + bits + n, zero_points=zero_points, scale_lo=0.002 if bits == 8 else 0.02,
                                        scale_hi=0.004 if bits == 8 else 0.04, scale_dtype=s_dt)
     a = synth.make_activation(m, k, 51 + m, a_dt)
     bias = synth.to_dtype(np.linspace(-1, 1, n).astype(np.float32), a_dt)
     y, variant = run_op(ep, a, a_dt, b, s, s_dt, zp, n, k, bs, bias=bias, bias_dtype=a_dt, bits=bits)
-    tall = a_dt != E.F32 and m >= 32 and k % 8 == 0
     assert variant == ("dense_transient_blaslt" if tall else "gemv_nbits_f32")
     want = port.matmul_f64_bits(synth.to_f32(a, a_dt), b, synth.to_f32(s, s_dt), zp, n, k, bs, bits, bias=synth.to_f32(bias, a_dt))
     assert helpers.rel_l2(synth.to_f32(y, a_dt), want) <= (TOL_F32 if a_dt == E.F32 else TOL_HALF)
@@ -692,8 +696,10 @@ def test_other_bit_widths_match_oracle(ep, port, bits, a_dt, s_dt, bs, zero_poin
     (E.BF16, 128, True, 16, 72, 1024, False),
     (E.F16, 64, True, 48, 136, 512, True),          # tall: dense route over weights expanded with their groups
 ])
-def test_g_idx_matches_oracle(ep, port, bits, a_dt, bs, zero_points, m, n, k, with_bias):
+def test_g_idx_matches_oracle(ep, ep_dense, port, bits, a_dt, bs, zero_points, m, n, k, with_bias):
     """Act-order weights (g_idx at input 4): scale and zero point of element k come from group g_idx[k] (matmul_nbits.rs:3636-3658)."""
+    if m >= 32 and a_dt != E.F32:
+        ep = ep_dense                                  # the opt-in dense route; the default provider runs the plain kernel at any height
     kb = k // bs
     if bits == 4:
         b, s, zp = synth.make_weights(n, k, bs, 60 + n, zero_points=zero_points, scale_lo=0.005, scale_hi=0.02, scale_dtype=a_dt)
