@@ -175,7 +175,7 @@ __device__ __forceinline__ float block_sum(float s)
     return s;
 }
 
-// BF16: activation element type. BS: block size. MR: rows staged (1 or 4; M <= MR). ST: storage type of the scales.
+// BF16: activation element type. BS: block size. MR: rows staged (1, 4 or 16; M <= MR). ST: storage type of the scales.
 // SETS: register sets of one group each. 2: the next group's loads are in flight while this one is multiplied - for
 // launches with few waves, where each wave must cover memory latency by itself. 1: no prefetch, 62 registers, eight
 // waves per SIMD - for launches with thousands of waves, where the other resident waves cover it better (measured on
@@ -185,7 +185,7 @@ __device__ __forceinline__ float block_sum(float s)
 // second half the up projection's - each half exactly as a launch of its own would (same split of K, same order of
 // summation, so the same f32 totals) - and the epilogue writes round16(silu(round16(gate)) * round16(up)).
 template <bool BF16, int BS, int MR, typename ST, int SETS, bool PAIR>
-__global__ __launch_bounds__((BS == 128 && sizeof(ST) == 2) ? 1024 : 512)   // block 128, 16-bit scales: up to 16 waves split a long K
+__global__ __launch_bounds__((BS == 128 && sizeof(ST) == 2 && (MR != 16 || BF16)) ? 1024 : 512)   // block 128, 16-bit scales, up to 4 rows: up to 16 waves split a long K
 __attribute__((amdgpu_waves_per_eu((BS == 128 && MR == 1 && sizeof(ST) == 2) ? (SETS == 1 ? 8 : 5) : 1)))
 void decode_packed_kernel(PackedParams p)
 {
@@ -194,7 +194,8 @@ void decode_packed_kernel(PackedParams p)
     constexpr int NB = U * NBT;
     constexpr int R = packed_record_bytes(BS, static_cast<int>(sizeof(ST)));
     constexpr int NR = R / 16;
-    constexpr int NA = MR == 1 ? 1 : U;
+    constexpr int RQ = MR == 1 ? 1 : MR / 4;       // loads per tile: each covers four rows (row g + 4 i, piece c)
+    constexpr int NA = MR == 1 ? 1 : U * RQ;
     constexpr int kStageBytes = MR == 1 ? 1024 : MR * kRowPitchP;
     constexpr float kMagicF = BF16 ? 128.0f : 1024.0f;
     constexpr uint32_t kMagicNeg = BF16 ? 0xC300C300u : 0xE400E400u;
@@ -224,7 +225,7 @@ void decode_packed_kernel(PackedParams p)
 
     const uint32_t w_off = static_cast<uint32_t>(lane * 16);
     const uint32_t r_off = static_cast<uint32_t>(kChunkWeights + c * R);
-    // compact activation load. MR = 1: piece c of tile g of the group. MR = 4: row g, piece c of one tile.
+    // compact activation load. MR = 1: piece c of tile g of the group. MR = 4 / 16: row g (+ 4 i), piece c of one tile.
     const uint32_t a_off = MR == 1 ? static_cast<uint32_t>(g * 256 + c * 16) : static_cast<uint32_t>(g) * static_cast<uint32_t>(p.k) * 2u + static_cast<uint32_t>(c * 16);
     unsigned char* stage = smem + wave * (2 * kStageBytes);
     const uint32_t st_write = MR == 1 ? static_cast<uint32_t>(lane * 16) : static_cast<uint32_t>(g * kRowPitchP + c * 16);
@@ -250,10 +251,12 @@ void decode_packed_kernel(PackedParams p)
         // that an outstanding load still owns, and then waits for it
         uint32_t a_voff[NA];
 #pragma unroll
-        for (int u = 0; u < NA; ++u) {
+        for (int x = 0; x < NA; ++x) {
+            const int u = x / RQ, i = x % RQ;
             const int tile = MR == 1 ? t0 + g : t0 + u;
             const bool beyond = static_cast<int64_t>(tile) * 128 + c * 8 + 8 > p.k;        // K is a multiple of 8: a piece is all in or all out
-            a_voff[u] = (beyond ? kOutOfRange : a_off) | oor;
+            // rows past M lie past the end of the activations' range and read as zeros
+            a_voff[x] = (beyond ? kOutOfRange : a_off + static_cast<uint32_t>(4 * i) * static_cast<uint32_t>(p.k) * 2u) | oor;
         }
         const uint32_t w_voff = w_off | oor, r_voff = r_off | oor;
         __builtin_amdgcn_sched_barrier(0);
@@ -262,14 +265,15 @@ void decode_packed_kernel(PackedParams p)
 #pragma unroll
         for (int i = 0; i < NR; ++i) grp.r[i] = load16(srd_p, r_voff + static_cast<uint32_t>(i * 16), soff);
 #pragma unroll
-        for (int u = 0; u < NA; ++u) grp.a[u] = load16(srd_a, a_voff[u], static_cast<uint32_t>(MR == 1 ? t0 : t0 + u) * 256u);
+        for (int x = 0; x < NA; ++x) grp.a[x] = load16(srd_a, a_voff[x], static_cast<uint32_t>(MR == 1 ? t0 : t0 + x / RQ) * 256u);
         __builtin_amdgcn_sched_barrier(0);
     };
     // `asum` (with SUMS): this lane's block sum of the group's tile lane / 16 (one load covers the group's four tiles).
     auto compute_tile = [&](const Grp& grp, int u, int parity, float asum) {
         unsigned char* st = stage + (MR == 1 ? parity : (u & 1)) * kStageBytes;
         if constexpr (MR != 1) {
-            *reinterpret_cast<uint4*>(st + st_write) = grp.a[u];
+#pragma unroll
+            for (int i = 0; i < RQ; ++i) *reinterpret_cast<uint4*>(st + st_write + i * 4 * kRowPitchP) = grp.a[u * RQ + i];
             lds_order();
         }
         uint4 av[4];
@@ -407,8 +411,19 @@ static int launch_packed_cfg(const PackedParams& p, int waves, hipStream_t strea
     const int all = pair ? 2 * waves : waves;
     const size_t stage = static_cast<size_t>(all) * 2 * (MR == 1 ? 1024 : MR * kRowPitchP);
     const size_t red = static_cast<size_t>(all) * 1024;
-    if (pair) hipLaunchKernelGGL((decode_packed_kernel<BF16, BS, MR, ST, SETS, true>), dim3(grid), dim3(all * 64), stage > red ? stage : red, stream, p);
-    else hipLaunchKernelGGL((decode_packed_kernel<BF16, BS, MR, ST, SETS, false>), dim3(grid), dim3(all * 64), stage > red ? stage : red, stream, p);
+    const size_t lds = stage > red ? stage : red;
+    if constexpr (MR == 16) {
+        // sixteen staged rows of sixteen waves outgrow the 64 KiB a kernel gets without asking
+        if (lds > 65536) {
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(decode_packed_kernel<BF16, BS, MR, ST, SETS, false>),
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+            if (e != hipSuccess) return static_cast<int>(e);
+        }
+        hipLaunchKernelGGL((decode_packed_kernel<BF16, BS, MR, ST, SETS, false>), dim3(grid), dim3(all * 64), lds, stream, p);
+    } else {
+        if (pair) hipLaunchKernelGGL((decode_packed_kernel<BF16, BS, MR, ST, SETS, true>), dim3(grid), dim3(all * 64), lds, stream, p);
+        else hipLaunchKernelGGL((decode_packed_kernel<BF16, BS, MR, ST, SETS, false>), dim3(grid), dim3(all * 64), lds, stream, p);
+    }
     return static_cast<int>(hipGetLastError());
 }
 
@@ -416,7 +431,9 @@ template <bool BF16, int BS, typename ST>
 static int launch_packed_mr(const PackedParams& p, int waves, bool single_set, hipStream_t stream)
 {
     if (p.m <= 1) return single_set ? launch_packed_cfg<BF16, BS, 1, ST, 1>(p, waves, stream) : launch_packed_cfg<BF16, BS, 1, ST, 2>(p, waves, stream);
-    return single_set ? launch_packed_cfg<BF16, BS, 4, ST, 1>(p, waves, stream) : launch_packed_cfg<BF16, BS, 4, ST, 2>(p, waves, stream);
+    if (p.m <= 4) return single_set ? launch_packed_cfg<BF16, BS, 4, ST, 1>(p, waves, stream) : launch_packed_cfg<BF16, BS, 4, ST, 2>(p, waves, stream);
+    // 5 .. 16 rows: one register set (64 registers of activations per group; a second set in flight measured slower)
+    return launch_packed_cfg<BF16, BS, 16, ST, 1>(p, waves, stream);
 }
 
 template <bool BF16, typename ST>
@@ -1021,7 +1038,7 @@ extern "C" int rocm_decode_packed_eligible(const RocmMatMulNBitsArgs* a)
     if (base.m > 16) base.m = 16;                         // the shared-activation kernel takes up to 64 rows
     if (!rocm_decode_mfma_eligible(&base)) return 0;
     if (a->m * a->k * 2 >= 0x7ffffff0) return 0;
-    if (a->m > 4 && !wide_shape(a)) return 0;
+    if (a->m > 16 && !wide_shape(a)) return 0;           // up to 16 rows the split-K kernel stages the rows per wave
     return static_cast<int64_t>(mnb::packed_groups(a)) * mnb::packed_chunk_bytes(a) < 0x7fffffff;
 }
 
@@ -1117,7 +1134,7 @@ static int launch_decode_packed(const RocmMatMulNBitsArgs* a, const void* packed
         single_set = wgs * w >= 6144;
     }
     if (one_row) single_set = true;
-    const int w_max = (a->block_size == 128 && !f32_scales) ? 16 : 8;      // see the kernel's launch bounds
+    const int w_max = (a->block_size == 128 && !f32_scales && (a->m <= 4 || a->a_dtype == ROCM_DT_BF16)) ? 16 : 8;      // see the kernel's launch bounds
     if (w > w_max) w = w_max;
     if (w > p.groups) w = p.groups;
     const int gpw = (p.groups + w - 1) / w;

@@ -49,7 +49,8 @@ def sampled_f64(port, a_f32, b, s_f32, zp, cols, k, bs, rows=None):
 DECODE_SHAPES = [
     # name, dtype, block, zero points, K, N, rows, scale range
     ("7b lm_head", E.BF16, 128, True, 3584, 152064, (1, 16), (0.002, 0.01)),
-    ("7b down", E.BF16, 128, True, 18944, 3584, (1, 16), (0.002, 0.01)),
+    ("7b down", E.BF16, 128, True, 18944, 3584, (1, 5, 16), (0.002, 0.01)),
+    ("7b qkv", E.BF16, 128, True, 3584, 4608, (1, 9, 16), (0.002, 0.01)),
     ("7b gate_up", E.BF16, 128, True, 3584, 37888, (4, 8), (0.002, 0.01)),
     ("0.5b lm_head", E.F16, 32, True, 896, 151936, (1,), (0.002, 0.01)),
 ]

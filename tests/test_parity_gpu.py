@@ -229,8 +229,8 @@ def test_decode_matches_oracle(ep, ep_unpacked, port, prepack, a_dt, s_dt, bs, z
     # f32 output: the arithmetic itself, before any narrowing
     y32, variant = run_op(ep, a, a_dt, b, s, s_dt, zp, n, k, bs, bias=bias, bias_dtype=a_dt, y_dtype=E.F32)
     if m <= 16:
-        wide = n >= 14336                                   # columns from which the shared-activation kernel takes 5..16 rows
-        assert variant == ("decode_mfma_packed" if prepack and (m <= 4 or wide) else "decode_mfma_splitk")   # m 2..4 at large n: the 4-row kernel
+        # up to 16 rows read the repacked stream at every width (the shared-activation kernel from 14336 columns and 5 rows)
+        assert variant == ("decode_mfma_packed" if prepack else "decode_mfma_splitk")
     else:
         # m <= 32: two row blocks through the decode kernel where that beats the tiled kernel (block 128, few columns or rows)
         row_blocks = m <= 32 and (k % 64 != 0 or (bs >= 128 and (n <= 8192 or m <= 20)))
@@ -256,7 +256,7 @@ def test_decode_matches_oracle(ep, ep_unpacked, port, prepack, a_dt, s_dt, bs, z
 @pytest.mark.parametrize("waves,cg", [(1, 1), (3, 2), (16, 4), (7, 1)])
 def test_decode_launch_shapes_agree(port, waves, cg):
     """Every split of the work over waves and column groups gives the same answer (to f32 rounding)."""
-    provider = E.RocmExecutionProvider(0, {"decode_waves": waves, "decode_col_groups": cg})
+    provider = E.RocmExecutionProvider(0, {"decode_waves": waves, "decode_col_groups": cg, "prepack": "0"})
     try:
         a_dt, bs, m, n, k = E.BF16, 128, 6, 200, 3584
         b, s, zp = synth.make_weights(n, k, bs, 77, zero_points=True, scale_lo=0.002, scale_hi=0.01, scale_dtype=a_dt)
@@ -274,7 +274,7 @@ def test_packed_decode_wave_counts_agree(port, waves):
     try:
         a_dt, bs, n, k = E.BF16, 128, 200, 3584
         b, s, zp = synth.make_weights(n, k, bs, 78, zero_points=True, scale_lo=0.002, scale_hi=0.01, scale_dtype=a_dt)
-        for m in (1, 3):
+        for m in (1, 3, 7, 16):
             a = synth.make_activation(m, k, 78 + m, a_dt)
             y32, variant = run_op(provider, a, a_dt, b, s, a_dt, zp, n, k, bs, y_dtype=E.F32)
             assert variant == "decode_mfma_packed"
@@ -293,8 +293,8 @@ def test_row_blocks_through_the_decode_kernels(ep, ep_unpacked, port, prepack, m
     a = synth.make_activation(m, k, 55 + m, a_dt)
     bias = synth.to_dtype(np.linspace(-2, 2, n).astype(np.float32), a_dt)
     y32, variant = run_op(ep, a, a_dt, b, s, a_dt, zp, n, k, bs, bias=bias, bias_dtype=a_dt, y_dtype=E.F32)
-    # with the repacked copy, blocks of more than 4 rows still stream the caller's layout at this width
-    assert variant == "decode_mfma_splitk"
+    # with the repacked copy, both row blocks read it
+    assert variant == ("decode_mfma_packed" if prepack else "decode_mfma_splitk")
     assert helpers.rel_l2(y32, oracle_f64(port, a, a_dt, b, s, a_dt, zp, n, k, bs, bias, a_dt)) <= 1e-4
     y, _ = run_op(ep, a, a_dt, b, s, a_dt, zp, n, k, bs, bias=bias, bias_dtype=a_dt)
     assert np.array_equal(np.asarray(y).view(np.uint16), np.asarray(port.narrow(y32, a_dt)).view(np.uint16))
