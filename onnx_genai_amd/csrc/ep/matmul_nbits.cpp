@@ -565,7 +565,7 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
     if (kn.accuracy_level == 4) {
         const int rounding = kn.ep->acc4_rounding == 2 ? (static_cast<int64_t>(M) < static_cast<int64_t>(kn.ep->acc4_native_below) ? 1 : 0) : kn.ep->acc4_rounding;   // matmul_nbits.rs:640-660
         int pack_rc = 0;
-        const bool packed = M == 1 && use_packed(kn, args, pack_rc);
+        const bool packed = M <= 16 && use_packed(kn, args, pack_rc);       // up to 16 rows read the repacked stream
         if (packed && rocm_acc4_packed_fuses_quantizer(&args)) {
             // one f16 / bf16 row over the repacked stream: the kernel quantizes the row itself, no workspace and no second launch
             rc = pack_rc != 0 ? pack_rc : rocm_launch_acc4_packed(&args, kn.packed, nullptr, rounding, kn.ep->decode_waves, stream);

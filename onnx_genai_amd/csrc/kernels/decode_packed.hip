@@ -746,7 +746,7 @@ static int launch_wide_bs(const PackedParams& p, int bs, hipStream_t stream)
 }
 
 // ---------------------------------------------------------------------------------------------
-// accuracy_level = 4, one row, over the same repacked stream: v_mfma_i32_16x16x32_i8.
+// accuracy_level = 4, up to 16 rows, over the same repacked stream: v_mfma_i32_16x16x32_i8.
 // ---------------------------------------------------------------------------------------------
 //
 // `w & 0x0f0f0f0f` and `(w >> 4) & 0x0f0f0f0f` turn a repacked dword into the eight weights as unsigned bytes in the
@@ -757,8 +757,10 @@ static int launch_wide_bs(const PackedParams& p, int bs, hipStream_t stream)
 typedef __attribute__((ext_vector_type(4))) int int4p_t;
 
 struct Acc4PackedParams {
-    const int8_t* qa;       // [padded_k] codes of the one row, packed order
-    const float* aq;        // [kb, 2]: scale_a, f32(sum of codes)
+    const int8_t* qa;       // [m, padded_k] codes, packed order
+    const float* aq;        // one row: [kb, 2] = scale_a, f32(sum of codes)
+    const float* aux16;     // 2 .. 16 rows: [kb, 16, 2], the same pairs block-major
+    int64_t m;
     const void* a;          // FUSE: the one row itself, f16 or bf16 [k]; every wave quantizes the groups it multiplies
     int64_t k;
     int rounding;           // FUSE: 0 = ties to even, 1 = ties away from zero
@@ -771,15 +773,17 @@ struct Acc4PackedParams {
     int groups, groups_per_wave, chunk_bytes;
     int bias_dtype, y_dtype;
     int scales_bf16;
-    int32_t* acc_probe;     // PROBE builds: int32 [N, kb] block accumulators of the one row, as flushed
+    int32_t* acc_probe;     // PROBE builds: int32 [M, N, kb] block accumulators, as flushed
 };
 
-template <int NR>
+constexpr int kCodePitchP = 144;   // bytes between the rows of one tile of codes in LDS: 128 + 16
+
+template <int NR, int NA, int NX>
 struct Acc4PackedGroup {
     uint4 w[kGroupTiles];
     uint4 r[NR];
-    uint4 a;      // 16 codes of the group (lanes 0..31)
-    uint2 x;      // (scale_a, code sum) of block `lane` of the group
+    uint4 a[NA];  // one row: 16 codes of the group (lanes 0..31). 16 rows: per tile, row lane / 8 (+ 8), piece lane % 8
+    uint4 x[NX];  // one row: .x/.y = (scale_a, code sum) of block `lane` of the group. 16 rows: 16 bytes of the group's aux16 rows
 };
 
 // FUSE: 0 = codes and (scale, sum) pairs come from the workspace a quantizer kernel filled; 1 / 2 = the row arrives as
@@ -789,14 +793,26 @@ struct Acc4PackedGroup {
 // separate launch, which at one row costs about as much as a fifth of this kernel.
 // PROBE: every flushed block accumulator (the integer acc - zp * code_sum that is about to be scaled) is also stored to
 // p.acc_probe; the same code otherwise, for tests that compare the integers themselves.
-template <int BS, typename ST, int SETS, int FUSE, bool PROBE>
+// MR: rows staged, 1, 4, 8 or 16 (M <= MR). Beyond one row the codes come from the workspace (FUSE = 0): per tile a wave
+// loads the rows' 128 codes, stages them in LDS at a padded pitch and reads MFMA operand j of row lane % 16 from there;
+// the activation-side (scale, sum) pairs of the group's blocks are staged once per group and read when a block ends.
+// With 4 (8), call row r sits in matrix row 4 r (2 r) and the rows between stay zero, so that a lane finds its rows in
+// component 0 (0 and 2) of its accumulator and a block's end scales one (two) values per lane instead of four.
+template <int BS, typename ST, int SETS, int FUSE, bool PROBE, int MR = 1>
 __global__ __launch_bounds__(512) void acc4_packed_kernel(Acc4PackedParams p)
 {
+    static_assert(MR == 1 || ((MR == 4 || MR == 8 || MR == 16) && FUSE == 0 && SETS == 1), "several rows: codes from the workspace, one register set");
     constexpr int U = kGroupTiles;
     constexpr int NBT = 128 / BS;
     constexpr int NB = U * NBT;
     constexpr int R = packed_record_bytes(BS, static_cast<int>(sizeof(ST)));
     constexpr int NR = R / 16;
+    constexpr int NA = MR == 16 ? 2 * U : MR == 1 ? 1 : U;
+    constexpr int SP = MR == 1 ? 1 : 16 / MR;                                     // matrix rows per call row
+    constexpr int NX = MR == 1 ? 1 : (NB * 8 + 63) / 64;
+    constexpr int kCodeStage = 16 * kCodePitchP;                                  // 16 rows: one tile of codes
+    constexpr int kWaveBytes = MR == 1 ? SETS * 512 : 2 * kCodeStage + NB * 128;  // 16 rows: two tiles in turn + the group's pairs
+    constexpr int kRowsKept = MR == 1 ? 1 : MR / 4;                               // call rows per lane: g * kRowsKept + r
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
     const int lane = threadIdx.x & 63;
@@ -808,24 +824,34 @@ __global__ __launch_bounds__(512) void acc4_packed_kernel(Acc4PackedParams p)
     const bool bf16_scales = p.scales_bf16 != 0;
 
     const __amdgpu_buffer_rsrc_t srd_p = make_srd(p.packed + static_cast<int64_t>(blockIdx.x) * p.cg_stride, static_cast<uint64_t>(p.cg_stride));
-    const __amdgpu_buffer_rsrc_t srd_a = FUSE ? make_srd(p.a, static_cast<uint64_t>(p.k) * 2) : make_srd(p.qa, static_cast<uint64_t>(p.padded_k));
-    const __amdgpu_buffer_rsrc_t srd_x = make_srd(p.aq, FUSE ? 0 : static_cast<uint64_t>(p.kb) * 8);
+    const __amdgpu_buffer_rsrc_t srd_a = FUSE ? make_srd(p.a, static_cast<uint64_t>(p.k) * 2) : make_srd(p.qa, static_cast<uint64_t>(p.m * p.padded_k));
+    const __amdgpu_buffer_rsrc_t srd_x = MR == 1 ? make_srd(p.aq, FUSE ? 0 : static_cast<uint64_t>(p.kb) * 8) : make_srd(p.aux16, static_cast<uint64_t>(p.kb) * 128);
     constexpr int kBlockLanes = BS / 8;
 
     const uint32_t w_off = static_cast<uint32_t>(lane * 16);
     const uint32_t r_off = static_cast<uint32_t>(kChunkWeights + c * R);
-    unsigned char* stage = smem + wave * (SETS * 512);
-    // operand of MFMA j of tile u: the 8 codes of elements u*128 + j*32 + g*8 .. +8 (only row 0 matters: every lane
-    // of a lane group reads the same 8 bytes)
-    const uint32_t st_read = static_cast<uint32_t>(g * 8);
+    unsigned char* stage = smem + wave * kWaveBytes;
+    unsigned char* aux_stage = stage + 2 * kCodeStage;            // 16 rows only
+    // operand of MFMA j of tile u: the 8 codes of elements u*128 + j*32 + g*8 .. +8. One row: only row 0 matters, every
+    // lane of a lane group reads the same 8 bytes of the group's 512. 16 rows: row lane % 16 of the staged tile.
+    const uint32_t st_read = MR == 1 ? static_cast<uint32_t>(g * 8) : static_cast<uint32_t>(c * kCodePitchP + g * 8);
+    // several rows: a tile's codes arrive as row lane / 8 (+ 8), piece lane % 8, and go to matrix row SP * row
+    const uint32_t a_off16 = static_cast<uint32_t>(lane >> 3) * static_cast<uint32_t>(p.padded_k) + static_cast<uint32_t>((lane & 7) * 16);
+    const uint32_t st_write16 = static_cast<uint32_t>((lane >> 3) * SP * kCodePitchP + (lane & 7) * 16);
+    if constexpr (MR == 4 || MR == 8) {
+        for (int i = lane; i < 2 * kCodeStage / 16; i += 64) *reinterpret_cast<uint4*>(stage + i * 16) = make_uint4(0, 0, 0, 0);
+        lds_order();
+    }
 
-    float y = 0.f;
+    float y[kRowsKept];
+#pragma unroll
+    for (int r = 0; r < kRowsKept; ++r) y[r] = 0.f;
     int4p_t acc = {0, 0, 0, 0};
 
     const int g_begin = wave * p.groups_per_wave;
     const int g_end = min(g_begin + p.groups_per_wave, p.groups);
 
-    using Grp = Acc4PackedGroup<NR>;
+    using Grp = Acc4PackedGroup<NR, NA, NX>;
     // No branch in here (a branch would make the compiler wait for every load in flight, the prefetch included): a group
     // past the wave's last one gets every offset out of range, fetches nothing and reads as zeros - it adds nothing.
     auto fetch_group = [&](Grp& grp, int gi) {
@@ -835,19 +861,36 @@ __global__ __launch_bounds__(512) void acc4_packed_kernel(Acc4PackedParams p)
         for (int u = 0; u < U; ++u) grp.w[u] = load16(srd_p, (w_off + static_cast<uint32_t>(u * 1024)) | oor, soff);
 #pragma unroll
         for (int i = 0; i < NR; ++i) grp.r[i] = load16(srd_p, (r_off + static_cast<uint32_t>(i * 16)) | oor, soff);
-        if constexpr (FUSE) {
-            grp.a = load16(srd_a, static_cast<uint32_t>(lane * 16) | oor, static_cast<uint32_t>(gi) * 1024u);   // 8 activations; K % 8 == 0 and the range ends the row
+        if constexpr (MR != 1) {
+#pragma unroll
+            for (int x = 0; x < NA; ++x) {
+                const int u = MR == 16 ? x / 2 : x, i = MR == 16 ? x % 2 : 0;
+                // a piece past the end of its row would read the next row's codes (rows past M lie past the range and read as zeros)
+                const bool beyond = static_cast<int64_t>(gi * U + u) * 128 + (lane & 7) * 16 >= p.padded_k || (MR == 4 && lane >= 32);
+                const uint32_t off = beyond ? kOutOfRange : a_off16 + static_cast<uint32_t>(i * 8) * static_cast<uint32_t>(p.padded_k);
+                grp.a[x] = load16(srd_a, off | oor, static_cast<uint32_t>(gi * U + u) * 128u);
+            }
+#pragma unroll
+            for (int x = 0; x < NX; ++x)
+                grp.x[x] = load16(srd_x, (lane + 64 * x < NB * 8 ? static_cast<uint32_t>((lane + 64 * x) * 16) : kOutOfRange) | oor, static_cast<uint32_t>(gi * NB) * 128u);
+        } else if constexpr (FUSE) {
+            grp.a[0] = load16(srd_a, static_cast<uint32_t>(lane * 16) | oor, static_cast<uint32_t>(gi) * 1024u);   // 8 activations; K % 8 == 0 and the range ends the row
         } else {
-            grp.a = load16(srd_a, (lane < 32 ? static_cast<uint32_t>(lane * 16) : kOutOfRange) | oor, static_cast<uint32_t>(gi) * 512u);   // the range ends the row at padded_k
+            grp.a[0] = load16(srd_a, (lane < 32 ? static_cast<uint32_t>(lane * 16) : kOutOfRange) | oor, static_cast<uint32_t>(gi) * 512u);   // the range ends the row at padded_k
             const auto v = __builtin_amdgcn_raw_buffer_load_b64(srd_x, static_cast<int>((lane < NB ? static_cast<uint32_t>(lane * 8) : kOutOfRange) | oor), static_cast<int>(gi * NB * 8), 0);
-            grp.x = make_uint2(v[0], v[1]);
+            grp.x[0].x = v[0];
+            grp.x[0].y = v[1];
         }
     };
     auto compute_group = [&](const Grp& grp, int gi, int slot) {
         unsigned char* st = stage + slot * 512;
         float sa_lane = 0.f, qs_lane = 0.f;          // FUSE: scale and f32(code sum) of the block this lane's activations lie in
-        if constexpr (FUSE) {
-            const uint32_t d[4] = {grp.a.x, grp.a.y, grp.a.z, grp.a.w};
+        if constexpr (MR != 1) {
+#pragma unroll
+            for (int x = 0; x < NX; ++x)
+                if (lane + 64 * x < NB * 8) *reinterpret_cast<uint4*>(aux_stage + (lane + 64 * x) * 16) = grp.x[x];
+        } else if constexpr (FUSE) {
+            const uint32_t d[4] = {grp.a[0].x, grp.a[0].y, grp.a[0].z, grp.a[0].w};
             float v[8];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
@@ -892,7 +935,7 @@ __global__ __launch_bounds__(512) void acc4_packed_kernel(Acc4PackedParams p)
             const uint32_t hi = (q[2] & 0xff) | ((q[6] & 0xff) << 8) | ((q[3] & 0xff) << 16) | (static_cast<uint32_t>(q[7]) << 24);
             *reinterpret_cast<uint2*>(st + lane * 8) = make_uint2(lo, hi);
         } else {
-            if (lane < 32) *reinterpret_cast<uint4*>(st + lane * 16) = grp.a;
+            if (lane < 32) *reinterpret_cast<uint4*>(st + lane * 16) = grp.a[0];
         }
         lds_order();
         uint32_t rr[NR * 4];
@@ -910,8 +953,21 @@ __global__ __launch_bounds__(512) void acc4_packed_kernel(Acc4PackedParams p)
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             long av[4];
+            if constexpr (MR != 1) {
+                unsigned char* tile = stage + (u & 1) * kCodeStage;
+                if constexpr (MR != 16) {
+                    if (MR == 8 || lane < 32) *reinterpret_cast<uint4*>(tile + st_write16) = grp.a[u];
+                } else {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) av[j] = *reinterpret_cast<const long*>(st + st_read + u * 128 + j * 32);
+                    for (int i = 0; i < 2; ++i) *reinterpret_cast<uint4*>(tile + st_write16 + i * 8 * kCodePitchP) = grp.a[u * 2 + i];
+                }
+                lds_order();
+#pragma unroll
+                for (int j = 0; j < 4; ++j) av[j] = *reinterpret_cast<const long*>(tile + st_read + j * 32);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) av[j] = *reinterpret_cast<const long*>(st + st_read + u * 128 + j * 32);
+            }
             const uint32_t wd[4] = {grp.w[u].x, grp.w[u].y, grp.w[u].z, grp.w[u].w};
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
@@ -932,14 +988,30 @@ __global__ __launch_bounds__(512) void acc4_packed_kernel(Acc4PackedParams p)
                         const uint32_t raw = (rr[bi / 2] >> ((bi % 2) * 16)) & 0xffffu;
                         sb = bf16_scales ? __uint_as_float(raw << 16) : f16_bits_to_f32(static_cast<uint16_t>(raw));
                     }
-                    const int src = FUSE ? bi * kBlockLanes : bi;         // a lane of the block, or the lane that loaded its pair
-                    const float sa = __int_as_float(__builtin_amdgcn_readlane(FUSE ? __float_as_int(sa_lane) : static_cast<int>(grp.x.x), src));
-                    const float qs = __int_as_float(__builtin_amdgcn_readlane(FUSE ? __float_as_int(qs_lane) : static_cast<int>(grp.x.y), src));
-                    const float f = fmaf(-zf, qs, static_cast<float>(acc[0]));   // both terms are integers below 2^24: exact
-                    y = fmaf(f, __fmul_rn(sa, sb), y);
-                    if constexpr (PROBE) {                                       // row 0 sits in lanes 0..15
-                        const int64_t blk = static_cast<int64_t>(gi) * NB + bi;
-                        if (lane < 16 && n_base + lane < p.n && blk < p.kb) p.acc_probe[(n_base + lane) * p.kb + blk] = static_cast<int>(f);
+                    if constexpr (MR != 1) {
+                        // this lane's call rows g * kRowsKept + r sit in components SP * r of its accumulator
+                        const float2* pairs = reinterpret_cast<const float2*>(aux_stage + bi * 128 + g * kRowsKept * 8);
+#pragma unroll
+                        for (int r = 0; r < kRowsKept; ++r) {
+                            const float2 pr = pairs[r];                                           // (scale, sum of codes)
+                            const float f = fmaf(-zf, pr.y, static_cast<float>(acc[SP * r]));      // both terms are integers below 2^24: exact
+                            y[r] = fmaf(f, __fmul_rn(pr.x, sb), y[r]);
+                            if constexpr (PROBE) {
+                                const int64_t blk = static_cast<int64_t>(gi) * NB + bi;
+                                const int64_t row = g * kRowsKept + r;
+                                if (row < p.m && n_base + c < p.n && blk < p.kb) p.acc_probe[(row * p.n + n_base + c) * p.kb + blk] = static_cast<int>(f);
+                            }
+                        }
+                    } else {
+                        const int src = FUSE ? bi * kBlockLanes : bi;         // a lane of the block, or the lane that loaded its pair
+                        const float sa = __int_as_float(__builtin_amdgcn_readlane(FUSE ? __float_as_int(sa_lane) : static_cast<int>(grp.x[0].x), src));
+                        const float qs = __int_as_float(__builtin_amdgcn_readlane(FUSE ? __float_as_int(qs_lane) : static_cast<int>(grp.x[0].y), src));
+                        const float f = fmaf(-zf, qs, static_cast<float>(acc[0]));   // both terms are integers below 2^24: exact
+                        y[0] = fmaf(f, __fmul_rn(sa, sb), y[0]);
+                        if constexpr (PROBE) {                                       // row 0 sits in lanes 0..15
+                            const int64_t blk = static_cast<int64_t>(gi) * NB + bi;
+                            if (lane < 16 && n_base + lane < p.n && blk < p.kb) p.acc_probe[(n_base + lane) * p.kb + blk] = static_cast<int>(f);
+                        }
                     }
                 }
             }
@@ -970,18 +1042,36 @@ __global__ __launch_bounds__(512) void acc4_packed_kernel(Acc4PackedParams p)
         }
     }
 
-    // ---- split-K reduction across the waves of this workgroup, in wave order; row 0 lives in lanes 0..15 ----
+    // ---- split-K reduction across the waves of this workgroup, in wave order ----
     __syncthreads();
-    float* red = reinterpret_cast<float*>(smem);       // [waves][16]
-    if (lane < 16) red[wave * 16 + lane] = y;
-    __syncthreads();
-    if (threadIdx.x < 16) {
-        const int64_t col = n_base + threadIdx.x;
-        if (col < p.n) {
-            float total = 0.f;
-            for (int w = 0; w < waves; ++w) total += red[w * 16 + threadIdx.x];
-            total = with_bias(total, p.bias, p.bias_dtype, 0, p.n, col, p.y_dtype);       // one row
-            store_from_f32(p.y, p.y_dtype, col, total);
+    float* red = reinterpret_cast<float*>(smem);
+    if constexpr (MR != 1) {                           // [waves][kRowsKept][64]: lane (c, g) holds rows g * kRowsKept + r of column c
+#pragma unroll
+        for (int r = 0; r < kRowsKept; ++r) red[(wave * kRowsKept + r) * 64 + lane] = y[r];
+        __syncthreads();
+        for (int idx = threadIdx.x; idx < kRowsKept * 64; idx += blockDim.x) {
+            const int r = idx >> 6;
+            const int l = idx & 63;
+            const int row = (l >> 4) * kRowsKept + r;
+            const int64_t col = n_base + (l & 15);
+            if (row < p.m && col < p.n) {
+                float total = 0.f;
+                for (int w = 0; w < waves; ++w) total += red[(w * kRowsKept + r) * 64 + l];
+                total = with_bias(total, p.bias, p.bias_dtype, row, p.n, col, p.y_dtype);
+                store_from_f32(p.y, p.y_dtype, static_cast<int64_t>(row) * p.n + col, total);
+            }
+        }
+    } else {                                           // [waves][16]: row 0 lives in lanes 0..15
+        if (lane < 16) red[wave * 16 + lane] = y[0];
+        __syncthreads();
+        if (threadIdx.x < 16) {
+            const int64_t col = n_base + threadIdx.x;
+            if (col < p.n) {
+                float total = 0.f;
+                for (int w = 0; w < waves; ++w) total += red[w * 16 + threadIdx.x];
+                total = with_bias(total, p.bias, p.bias_dtype, 0, p.n, col, p.y_dtype);       // one row
+                store_from_f32(p.y, p.y_dtype, col, total);
+            }
         }
     }
 }
@@ -990,6 +1080,19 @@ template <int BS, typename ST>
 static int launch_acc4_packed(const Acc4PackedParams& p, int waves, bool single_set, int fuse, hipStream_t stream)
 {
     const unsigned grid = static_cast<unsigned>((p.n + 15) / 16);
+    if (p.m > 1) {
+        // two tiles of codes in turn + the group's pairs per wave; the reduction reuses the space (1 KiB per wave)
+        const size_t lds16 = static_cast<size_t>(waves) * (2 * 16 * kCodePitchP + kGroupTiles * (128 / BS) * 128);
+        if (p.m <= 4) {
+            if (p.acc_probe) hipLaunchKernelGGL((acc4_packed_kernel<BS, ST, 1, 0, true, 4>), dim3(grid), dim3(waves * 64), lds16, stream, p);
+            else hipLaunchKernelGGL((acc4_packed_kernel<BS, ST, 1, 0, false, 4>), dim3(grid), dim3(waves * 64), lds16, stream, p);
+        } else if (p.m <= 8) {
+            if (p.acc_probe) hipLaunchKernelGGL((acc4_packed_kernel<BS, ST, 1, 0, true, 8>), dim3(grid), dim3(waves * 64), lds16, stream, p);
+            else hipLaunchKernelGGL((acc4_packed_kernel<BS, ST, 1, 0, false, 8>), dim3(grid), dim3(waves * 64), lds16, stream, p);
+        } else if (p.acc_probe) hipLaunchKernelGGL((acc4_packed_kernel<BS, ST, 1, 0, true, 16>), dim3(grid), dim3(waves * 64), lds16, stream, p);
+        else hipLaunchKernelGGL((acc4_packed_kernel<BS, ST, 1, 0, false, 16>), dim3(grid), dim3(waves * 64), lds16, stream, p);
+        return static_cast<int>(hipGetLastError());
+    }
     const size_t lds = static_cast<size_t>(waves) * 1024;
     auto go = [&](auto fuse) {
         constexpr int F = decltype(fuse)::value;
@@ -1173,14 +1276,16 @@ extern "C" int rocm_launch_decode_packed_pair(const RocmMatMulNBitsArgs* a, cons
 extern "C" int rocm_acc4_packed_eligible(const RocmMatMulNBitsArgs* a)
 {
     const bool bs_ok = a->block_size == 32 || a->block_size == 64 || a->block_size == 128;
-    if (!(bs_ok && a->m == 1 && a->n >= 1)) return 0;
+    if (!(bs_ok && a->m >= 1 && a->m <= 16 && a->n >= 1)) return 0;
     if ((reinterpret_cast<uintptr_t>(a->b) & 15) != 0 || (reinterpret_cast<uintptr_t>(a->scales) & 3) != 0) return 0;
+    const int64_t padded_k = (a->k + a->block_size - 1) / a->block_size * a->block_size;
+    if (a->m * padded_k >= 0x7fffffff) return 0;                          // the codes are addressed with 32-bit offsets
     return static_cast<int64_t>(mnb::packed_groups(a)) * mnb::packed_chunk_bytes(a) < 0x7fffffff;
 }
 
 extern "C" int rocm_acc4_packed_fuses_quantizer(const RocmMatMulNBitsArgs* a)
 {
-    return rocm_acc4_packed_eligible(a) && (a->a_dtype == ROCM_DT_F16 || a->a_dtype == ROCM_DT_BF16) && a->k % 8 == 0 &&
+    return rocm_acc4_packed_eligible(a) && a->m == 1 && (a->a_dtype == ROCM_DT_F16 || a->a_dtype == ROCM_DT_BF16) && a->k % 8 == 0 &&
            (reinterpret_cast<uintptr_t>(a->a) & 15) == 0;
 }
 
@@ -1192,6 +1297,8 @@ extern "C" int rocm_launch_acc4_packed(const RocmMatMulNBitsArgs* a, const void*
     mnb::Acc4PackedParams p;
     p.qa = ws ? ws->qa : nullptr;
     p.aq = ws ? ws->aq : nullptr;
+    p.aux16 = ws ? ws->aux : nullptr;
+    p.m = a->m;
     p.a = a->a;
     p.k = a->k;
     p.rounding = rounding;

@@ -113,7 +113,7 @@ def test_prefill_configs_at_full_size(ep, ep_tiled, port, route, k, n, m):
     assert helpers.rel_l2(y[np.ix_(rows, cols)].astype(np.float64), want) <= TOL_HALF, variant
 
 
-ACC4_SHAPES = [(8192, 28672, 1), (8192, 28672, 256), (28672, 8192, 1), (28672, 8192, 256), (8192, 10240, 4096)]
+ACC4_SHAPES = [(8192, 28672, 1), (8192, 28672, 8), (28672, 8192, 16), (8192, 28672, 256), (28672, 8192, 1), (28672, 8192, 256), (8192, 10240, 4096)]
 
 
 @pytest.mark.parametrize("k,n,m", ACC4_SHAPES)

@@ -1134,11 +1134,13 @@ def _production_block_acc(provider, port, a, a_dt, bs, zero_points, n, k, roundi
 
 
 PRODUCTION_ACC_CASES = [
-    # bs, zero points, m, n, k, prepack - one row over the repacked stream and over the caller's layout, the split-K kernel at 5
-    # rows, the tiled kernel at 40; each with K short (one wave / one slice) and long (several waves / K in slices)
+    # bs, zero points, m, n, k, prepack - one row and 5 / 16 rows over the repacked stream and over the caller's layout (the
+    # split-K kernel), the tiled kernel at 40; each with K short (one wave / one slice) and long (several waves / K in slices)
     (32, True, 1, 100, 32 * 11, True), (64, True, 1, 333, 64 * 37, True), (128, False, 1, 160, 128 * 40, True),
     (32, False, 1, 48, 32 * 9, False), (64, True, 1, 100, 64 * 50, False), (128, True, 1, 64, 128 * 24, False),
     (32, True, 5, 48, 32 * 9, True), (64, True, 5, 100, 64 * 50, True), (128, False, 5, 77, 128 * 33, True), (64, True, 16, 40, 200, True),
+    (32, True, 2, 100, 32 * 37, True), (128, True, 16, 33, 128 * 21, True),
+    (32, True, 5, 48, 32 * 9, False), (64, True, 5, 100, 64 * 50, False), (128, False, 5, 77, 128 * 33, False), (64, True, 16, 40, 200, False),
     (32, True, 40, 96, 32 * 35, True), (64, True, 40, 96, 64 * 17, True), (128, True, 130, 200, 128 * 20, True), (64, False, 40, 200, 64 * 3, True),
     (256, True, 40, 96, 256 * 3, True), (32, False, 33, 64, 200, True),
 ]
@@ -1155,7 +1157,7 @@ def test_production_kernels_block_accumulators_bit_exact(port, a_dt, bs, zero_po
     try:
         a = _tie_heavy_activation(m, k, bs, 300 + m, a_dt) if k % bs == 0 else synth.make_activation(m, k, 300 + m, a_dt)
         got, want, y32, y_want, variant = _production_block_acc(provider, port, a, a_dt, bs, zero_points, n, k, oracle.ROUND_HALF_EVEN, 310 + n)
-        assert variant == ("acc4_mfma_i8_packed" if prepack and m == 1 else "acc4_mfma_i8")
+        assert variant == ("acc4_mfma_i8_packed" if prepack and m <= 16 else "acc4_mfma_i8")
         assert not (got == 0x7FFFFFFF).any(), "an accumulator was never stored"
         assert np.array_equal(got, want)
         assert helpers.rel_l2(y32, y_want) <= TOL_F32
@@ -1220,9 +1222,9 @@ ACC4_CASES = [
 ]
 
 
-# every case under both rounding rules; one-row cases once more with the repacked path turned off
+# every case under both rounding rules; the cases of up to 16 rows once more with the repacked path turned off
 ACC4_RUNS = [case + (rounding, True) for case in ACC4_CASES for rounding in ("mlas", "native")] + \
-            [case + ("mlas", False) for case in ACC4_CASES if case[3] == 1]
+            [case + ("mlas", False) for case in ACC4_CASES if case[3] <= 16]
 
 
 @pytest.mark.parametrize("a_dt,bs,zero_points,m,n,k,rounding,prepack", ACC4_RUNS)
@@ -1235,7 +1237,7 @@ def test_acc4_outputs(port, ref, a_dt, bs, zero_points, m, n, k, rounding, prepa
         y32, variant = run_op(provider, a, a_dt, b, s, a_dt, zp, n, k, bs, accuracy_level=4, bias=bias, bias_dtype=a_dt, y_dtype=E.F32)
         on_matrix_cores = bs in (32, 64, 128) if m <= 16 else bs >= 32
         expected = "acc4_mfma_i8" if on_matrix_cores else "acc4_gemv_dot4"
-        if prepack and m == 1 and on_matrix_cores:
+        if prepack and m <= 16 and on_matrix_cores:
             expected = "acc4_mfma_i8_packed"                            # constant weights: the repacked stream
         assert variant == expected
         rnd = oracle.ROUND_HALF_EVEN if rounding == "mlas" else oracle.ROUND_HALF_AWAY
@@ -1279,7 +1281,7 @@ def test_acc4_decode_wave_counts_agree(port, waves, s_dt, prepack):
         for m in (1, 6):
             a = synth.make_activation(m, k, 95 + m, a_dt)
             y32, variant = run_op(provider, a, a_dt, b, s, s_dt, zp, n, k, bs, accuracy_level=4, y_dtype=E.F32)
-            assert variant == ("acc4_mfma_i8_packed" if prepack and m == 1 else "acc4_mfma_i8")
+            assert variant == ("acc4_mfma_i8_packed" if prepack else "acc4_mfma_i8")
             want = port.matmul_acc4_f32(synth.to_f32(a, a_dt), b, synth.to_f32(s, s_dt), zp, n, k, bs, oracle.ROUND_HALF_EVEN)
             assert helpers.rel_l2(y32, want) <= TOL_F32
     finally:
@@ -1292,7 +1294,7 @@ def test_acc4_power_of_two_scaling_at_full_70b_shape(ep):
     a_dt, bs, n, k = E.F16, 64, 10240, 8192
     b, s, zp = synth.make_weights(n, k, bs, 23, zero_points=True, scale_lo=0.002, scale_hi=0.01, scale_dtype=a_dt)
     ops = E.DeviceOperands(ep, b, s, a_dt, zp, n, k, bs, accuracy_level=4)
-    for m in (1, 40):
+    for m in (1, 8, 40):
         a = np.random.default_rng(m).uniform(-1.0, 1.0, size=(m, k)).astype(np.float16)
         ys = []
         for scale in (1.0, 2.0):
@@ -1301,7 +1303,7 @@ def test_acc4_power_of_two_scaling_at_full_70b_shape(ep):
             ys.append(ep.download(yb, (m, n), np.float32))
             ep.deallocate(ab)
             ep.deallocate(yb)
-        assert ops.kernel.last_variant() == ("acc4_mfma_i8_packed" if m == 1 else "acc4_mfma_i8")
+        assert ops.kernel.last_variant() == ("acc4_mfma_i8_packed" if m <= 16 else "acc4_mfma_i8")
         assert np.isfinite(ys[0]).all() and np.abs(ys[0]).max() > 0
         assert np.array_equal(ys[1], 2.0 * ys[0])
     ops.free()
