@@ -42,8 +42,12 @@ typedef struct NxrtRocmMatMulNBits NxrtRocmMatMulNBits;   /* one kernel = one Ma
  *             "dense_weights" = "transient" (default: one buffer per provider, refilled by every such call) |
  *             "resident" (a constant weight keeps its dense copy: 2 bytes per weight of HBM for a call that is the
  *             GEMM alone);
+ *             "rmsnorm_in_kernel_max_cols" = widest launch (columns; both projections of a gate/up node together) whose
+ *             decode kernel applies an RMS-normalization prologue itself at up to four rows; wider nodes and "0" normalize
+ *             in a launch of their own (default 8192: every workgroup repeats the row's normalization, which pays only
+ *             while there are few of them);
  *             "decode_waves", "decode_col_groups", "prefill_tile" = launch overrides (tests, tuning).
- * The same settings are read from NXRT_ROCM_ACC4_ROUNDING, NXRT_SQNBIT_DECODE_MIN, NXRT_ROCM_PREPACK,
+ * The same settings are read from NXRT_ROCM_RMSNORM_IN_KERNEL_MAX_COLS, NXRT_ROCM_ACC4_ROUNDING, NXRT_SQNBIT_DECODE_MIN, NXRT_ROCM_PREPACK,
  * NXRT_ROCM_DENSE_GEMM_MIN_ROWS, NXRT_ROCM_DENSE_GEMM_MAX_MB, NXRT_ROCM_DENSE_WEIGHTS, NXRT_ROCM_DECODE_WAVES,
  * NXRT_ROCM_DECODE_COL_GROUPS, NXRT_ROCM_PREFILL_TILE when the map does not give them. */
 NxrtStatus nxrt_rocm_ep_create(uint32_t device_ordinal, const char* const* config_keys,

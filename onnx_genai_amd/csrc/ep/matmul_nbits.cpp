@@ -405,8 +405,40 @@ bool f32_in_row_blocks(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& args,
     return true;
 }
 
+// The RMS-normalization prologue of a node on its way through the dispatch: the decode kernels over the repacked stream
+// apply it themselves (up to four rows); every other route first normalizes the rows into `owner`'s buffer with a
+// launch of its own.
+struct NormPrologue {
+    const void* gamma;
+    int gamma_dtype;
+    float epsilon;
+    NxrtRocmMatMulNBits* owner;     // the node that carries the prologue: its buffer holds the normalized rows
+    bool fused = false;             // out: the kernel applied it
+};
+
+// a -> round16((a * inv_std) * gamma), [rows, K] of a 16-bit type, into owner.norm; `a` is replaced by the buffer.
+NxrtStatus normalize_rows(const NormPrologue& np, const void*& a, int a_dtype, uint64_t rows, uint64_t k)
+{
+    NxrtRocmMatMulNBits& owner = *np.owner;
+    const uint64_t need = rows * k * 2;
+    if (owner.norm_bytes < need) {
+        if (frozen(owner))
+            return make_status(NXRT_INVALID_ARGUMENT, err("rmsnorm_prologue fusion under graph capture needs one eager call of this height first (the "
+                                                          "normalized activations live in a buffer the kernel may not allocate while a capture is open)"));
+        const int e = grow_buffer(owner.norm, owner.norm_bytes, need, owner.retired);
+        if (e != 0) return hip_status(e, "MatMulNBits: workspace hipMalloc");
+    }
+    if ((reinterpret_cast<uintptr_t>(a) & 7) != 0 || (reinterpret_cast<uintptr_t>(np.gamma) & 15) != 0)
+        return make_status(NXRT_INVALID_ARGUMENT, err("rmsnorm_prologue fusion needs A at an 8-byte and gamma at a 16-byte boundary (data pointer plus byte offset)"));
+    const int rc = rocm_launch_rmsnorm16(a, np.gamma, np.gamma_dtype, static_cast<int64_t>(rows), static_cast<int64_t>(k), np.epsilon, a_dtype, owner.norm, owner.ep->stream);
+    if (rc != 0) return hip_status(rc, "MatMulNBits: kernel launch");
+    owner.ep->launches.fetch_add(1);
+    a = owner.norm;
+    return ok();
+}
+
 NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, uint32_t n_in, NxrtRocmTensorView* out, uint32_t n_out,
-                        void* workspace, uint64_t workspace_bytes, bool no_alloc = false)
+                        void* workspace, uint64_t workspace_bytes, bool no_alloc = false, NormPrologue* norm = nullptr)
 {
     std::lock_guard<std::mutex> lock(kn.mu);
     struct Mode {
@@ -531,6 +563,9 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
     args.block_size = static_cast<int>(kn.block_size);
     args.g_idx = G ? static_cast<const int32_t*>(at(*G)) : nullptr;
     args.acc_probe = nullptr;
+    args.gamma = nullptr;
+    args.gamma_dtype = 0;
+    args.norm_epsilon = 0.f;
     if (kn.acc_probe) {
         if (kn.accuracy_level != 4) return make_status(NXRT_INVALID_ARGUMENT, err("the block-accumulator probe needs accuracy_level=4"));
         if (M * N * kb > kn.acc_probe_elems)
@@ -541,6 +576,22 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
 
     rocm_stream_t stream = kn.ep->stream;
     int rc = 0;
+    if (norm) {
+        // up to four rows over the repacked stream: the decode kernel normalizes the rows itself; otherwise a launch of its own
+        RocmMatMulNBitsArgs fused = args;
+        fused.gamma = norm->gamma;
+        fused.gamma_dtype = norm->gamma_dtype;
+        fused.norm_epsilon = norm->epsilon;
+        int pack_rc = 0;
+        if (kn.bits == 4 && !G && kn.accuracy_level != 4 && !kn.pair_member && kn.n <= kn.ep->rmsnorm_in_kernel_max_cols && rocm_decode_packed_fuses_norm(&fused) &&
+            use_packed(kn, args, pack_rc) && pack_rc == 0) {
+            args = fused;
+            norm->fused = true;
+        } else {
+            const NxrtStatus ns = normalize_rows(*norm, args.a, args.a_dtype, M, K);
+            if (ns.code != NXRT_OK) return ns;
+        }
+    }
     if (G && kn.g_idx_checked != args.g_idx) {
         // matmul_nbits.rs:3515-3521: every group must lie in 0..kb. Checked once per tensor (a device pass and a read-back).
         if (frozen(kn))
@@ -656,7 +707,7 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
 // inputs [x, W_gate, scales_gate, W_up, scales_up, (gamma), (zp_gate, zp_up)], output silu(gate) * up with both projections
 // rounded to the 16-bit type first. Here both projections run through the ordinary dispatch into scratch, then the epilogue.
 NxrtStatus execute_swiglu(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, uint32_t n_in, NxrtRocmTensorView* out, uint32_t n_out,
-                          void* workspace, uint64_t workspace_bytes)
+                          void* workspace, uint64_t workspace_bytes, NormPrologue* norm = nullptr)
 {
     std::lock_guard<std::mutex> lock(kn.mu);
     if (n_in < 5 || n_in > 8 || n_out != 1)
@@ -702,6 +753,7 @@ NxrtStatus execute_swiglu(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in,
     // tensor validated) by the projections' own first call below, so this path serves the calls after the first with the
     // same weight tensors; it sums each projection exactly as that first call did.
     // (accuracy_level 4 stays on its own int8 kernels for every call: the paired launch is the float path)
+    const void* normalized = nullptr;                    // the rows after a normalization launch of their own, once made
     if (M <= 4 && kn.accuracy_level != 4 && kn.gate->packed && kn.up->packed) {
         auto current = [&](const NxrtRocmMatMulNBits& child, const NxrtRocmTensorView& w, const NxrtRocmTensorView& s, const NxrtRocmTensorView* zp) {
             auto at = [](const NxrtRocmTensorView& v) { return static_cast<const void*>(static_cast<const uint8_t*>(v.data) + v.byte_offset); };
@@ -724,7 +776,20 @@ NxrtStatus execute_swiglu(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in,
             args.n = kn.n;
             args.k = kn.k;
             args.block_size = static_cast<int>(kn.block_size);
-            if (rocm_decode_packed_eligible(&args) && rocm_decode_packed_pair_fits(&args, kn.ep->decode_waves)) {
+            // (a prologue rides along where the pair is narrow enough for the in-kernel form to pay; a wider pair normalizes first)
+            const bool norm_inside = norm && 2 * kn.n <= kn.ep->rmsnorm_in_kernel_max_cols;
+            if (norm_inside) {
+                args.gamma = norm->gamma;
+                args.gamma_dtype = norm->gamma_dtype;
+                args.norm_epsilon = norm->epsilon;
+            } else if (norm) {
+                normalized = args.a;
+                const NxrtStatus ns = normalize_rows(*norm, normalized, args.a_dtype, M, K);
+                if (ns.code != NXRT_OK) return ns;
+                args.a = normalized;                     // whatever runs below sees these rows
+            }
+            if (rocm_decode_packed_eligible(&args) && (!norm_inside || rocm_decode_packed_fuses_norm(&args)) && rocm_decode_packed_pair_fits(&args, kn.ep->decode_waves)) {
+                if (norm_inside) norm->fused = true;
                 const int rc = rocm_launch_decode_packed_pair(&args, kn.gate->packed, kn.up->packed, kn.decomposed_silu ? 1 : 0, kn.ep->decode_waves, kn.ep->stream);
                 kn.ep->launches.fetch_add(1);
                 kn.variant = "gate_up_swiglu_packed";
@@ -746,9 +811,23 @@ NxrtStatus execute_swiglu(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in,
         }
         ws = static_cast<uint8_t*>(kn.scratch);
     }
+    // the children see normalized rows: one launch for both projections
+    NxrtRocmTensorView a_view = A;
+    if (norm) {
+        if (!normalized) {
+            if (!is_contiguous(A) || A.device_type != NXRT_DEVICE_ROCM || A.device_index != kn.ep->device)
+                return make_status(NXRT_INVALID_ARGUMENT, err("A must be contiguous and live on ROCm device " + std::to_string(kn.ep->device)));
+            normalized = static_cast<const uint8_t*>(A.data) + A.byte_offset;
+            const NxrtStatus ns = normalize_rows(*norm, normalized, static_cast<int>(A.dtype), M, K);
+            if (ns.code != NXRT_OK) return ns;
+        }
+        a_view.data = const_cast<void*>(normalized);
+        a_view.byte_offset = 0;
+        a_view.strides = nullptr;
+    }
     auto run = [&](NxrtRocmMatMulNBits& child, const NxrtRocmTensorView& w, const NxrtRocmTensorView& s, const NxrtRocmTensorView* zp, void* dst) {
         NxrtRocmTensorView cin[4];
-        cin[0] = A;
+        cin[0] = a_view;
         cin[1] = w;
         cin[2] = s;
         if (zp) cin[3] = *zp;
@@ -771,8 +850,9 @@ NxrtStatus execute_swiglu(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in,
 
 // A node with the RMS-normalization prologue (the CUDA provider's `_cuda_matmul_nbits_rmsnorm_prologue`,
 // onnx-runtime-ep-cuda/src/optimizer.rs:48-60; kernels/matmul_nbits.rs:7739-7745, 9042-9050): gamma [K] rides at input 6
-// (input 5 of the fused gate/up node). The activations are normalized into a buffer of the kernel's own, then the node runs
-// on them as it would without the prologue.
+// (input 5 of the fused gate/up node). Up to four rows over the repacked stream are normalized inside the decode kernel
+// (kernels/matmul_nbits.rs:3747-3783 does the same in its GEMV); on every other route the activations are normalized into a
+// buffer of the kernel's own, then the node runs on them as it would without the prologue.
 NxrtStatus execute_normalized(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, uint32_t n_in, NxrtRocmTensorView* out, uint32_t n_out,
                               void* workspace, uint64_t workspace_bytes)
 {
@@ -798,36 +878,19 @@ NxrtStatus execute_normalized(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView*
         if (t->device_type != NXRT_DEVICE_ROCM || t->device_index != kn.ep->device)
             return make_status(NXRT_INVALID_ARGUMENT, err(std::string(t == &A ? "A" : "gamma") + " must live on ROCm device " + std::to_string(kn.ep->device)));
     }
-    uint64_t M = 1;
-    for (uint32_t i = 0; i + 1 < A.ndim; ++i) M *= A.shape[i];
     std::vector<NxrtRocmTensorView> views(in, in + n_in);
     views[slot].data = nullptr;                                  // the node proper sees no gamma
     uint32_t n_views = n_in;
     if (!kn.gate_up_swiglu) n_views = n_in < 6 ? n_in : 6;
-    if (M > 0) {
-        NxrtStatus st = kn.ep->bind();
-        if (st.code != NXRT_OK) return st;
-        const uint64_t need = M * K * 2;
-        if (kn.norm_bytes < need) {
-            if (kn.ep->capturing)
-                return make_status(NXRT_INVALID_ARGUMENT, err("rmsnorm_prologue fusion under graph capture needs one eager call of this height first (the "
-                                                              "normalized activations live in a buffer the kernel may not allocate while a capture is open)"));
-            const int e = grow_buffer(kn.norm, kn.norm_bytes, need, kn.retired);
-            if (e != 0) return hip_status(e, "MatMulNBits: workspace hipMalloc");
-        }
-        const void* a = static_cast<const uint8_t*>(A.data) + A.byte_offset;
-        const void* g = static_cast<const uint8_t*>(G.data) + G.byte_offset;
-        const int rc = rocm_launch_rmsnorm16(a, g, static_cast<int>(G.dtype), static_cast<int64_t>(M), static_cast<int64_t>(K), kn.rmsnorm_epsilon,
-                                             static_cast<int>(A.dtype), kn.norm, kn.ep->stream);
-        if (rc != 0) return hip_status(rc, "MatMulNBits: kernel launch");
-        kn.ep->launches.fetch_add(1);
-        views[0].data = kn.norm;
-        views[0].byte_offset = 0;
-        views[0].strides = nullptr;
-    }
-    NxrtStatus st = kn.gate_up_swiglu ? execute_swiglu(kn, views.data(), n_views, out, n_out, workspace, workspace_bytes)
-                                      : execute_impl(kn, views.data(), n_views, out, n_out, workspace, workspace_bytes);
-    if (st.code == NXRT_OK) kn.variant = "rmsnorm+" + kn.variant;
+    NormPrologue np;
+    np.gamma = static_cast<const uint8_t*>(G.data) + G.byte_offset;
+    np.gamma_dtype = static_cast<int>(G.dtype);
+    np.epsilon = kn.rmsnorm_epsilon;
+    np.owner = &kn;
+    NxrtStatus st = kn.gate_up_swiglu ? execute_swiglu(kn, views.data(), n_views, out, n_out, workspace, workspace_bytes, &np)
+                                      : execute_impl(kn, views.data(), n_views, out, n_out, workspace, workspace_bytes, false, &np);
+    // "rmsnorm[...]": the kernel normalized the rows itself; "rmsnorm+...": a launch of its own did
+    if (st.code == NXRT_OK) kn.variant = np.fused ? "rmsnorm[" + kn.variant + "]" : "rmsnorm+" + kn.variant;
     return st;
 }
 

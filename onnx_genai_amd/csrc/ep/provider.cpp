@@ -86,6 +86,8 @@ NxrtStatus nxrt_rocm_ep_create(uint32_t device_ordinal, const char* const* keys,
         if ((it = ep->config.find("decode_col_groups")) != ep->config.end()) ep->decode_col_groups = parse_int(it->second, 0);
         if ((it = ep->config.find("prepack")) != ep->config.end()) ep->prepack = parse_int(it->second, 1);
         if ((it = ep->config.find("prefill_tile")) != ep->config.end()) ep->prefill_tile = parse_int(it->second, 0);
+        if (const char* env = std::getenv("NXRT_ROCM_RMSNORM_IN_KERNEL_MAX_COLS")) ep->config.emplace("rmsnorm_in_kernel_max_cols", env);
+        if ((it = ep->config.find("rmsnorm_in_kernel_max_cols")) != ep->config.end()) ep->rmsnorm_in_kernel_max_cols = parse_int(it->second, 8192);
         if ((it = ep->config.find("dense_gemm_max_mb")) != ep->config.end()) ep->dense_gemm_max_bytes = static_cast<uint64_t>(parse_int(it->second, 1024)) << 20;
         if ((it = ep->config.find("dense_weights")) != ep->config.end()) {
             if (it->second == "resident") ep->dense_resident = 1;

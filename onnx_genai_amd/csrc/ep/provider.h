@@ -22,6 +22,7 @@ struct NxrtRocmEp {
     int decode_col_groups = 0;
     int prefill_tile = 0;                         // 0 = chosen per shape; 1..3 force a tile (tests, tuning)
     int prepack = 1;                              // repack constant weights for the decode kernel on first use
+    int rmsnorm_in_kernel_max_cols = 8192;        // widest node (columns the launch covers) whose decode kernel applies an RMS-norm prologue itself; 0 = never
     int dense_gemm_min_rows = 0;                  // calls with at least this many rows expand the weights and run the library GEMM; 0 = never
     uint64_t dense_gemm_max_bytes = 1ull << 30;   // largest dense copy of one weight that route makes
     int dense_resident = 0;                       // 1: a constant weight keeps its dense copy (made once); 0: one shared buffer, refilled per call

@@ -73,6 +73,11 @@ typedef struct RocmMatMulNBitsArgs {
   int32_t* acc_probe;    /* accuracy_level 4, int8 matrix-core kernels only: int32 [M, N, kb], or NULL. When set, the kernel also
                             stores every block accumulator sum_k code * (q - zp) it flushes - the integer its f32 result is built
                             from - so that a test can compare the production kernels' integers bit for bit. */
+  const void* gamma;     /* RMS-normalization prologue inside the kernel: the weight [K], or NULL. Only rocm_launch_decode_packed and
+                            rocm_launch_decode_packed_pair read it, and only where rocm_decode_packed_fuses_norm() holds: the
+                            activations are then replaced by round16((a * inv_std) * gamma), inv_std = 1 / sqrt(mean(a^2) + eps). */
+  int gamma_dtype;       /* ROCM_DT_F32 or a_dtype */
+  float norm_epsilon;
 } RocmMatMulNBitsArgs;
 
 /* w[n,k] = (q - zp) * scale as f32 [N, K]. */
@@ -133,6 +138,9 @@ int rocm_decode_packed_eligible(const RocmMatMulNBitsArgs* args);
 uint64_t rocm_decode_packed_bytes(const RocmMatMulNBitsArgs* args);
 int rocm_launch_pack_decode(const RocmMatMulNBitsArgs* args, void* packed, rocm_stream_t stream);
 int rocm_launch_decode_packed(const RocmMatMulNBitsArgs* args, const void* packed, int waves, rocm_stream_t stream);
+/* 1 when the launch above (and the paired one below) applies args->gamma inside the kernel: up to 4 rows, K % 128 == 0, gamma f32 or
+ * of the activations' type and 16-byte aligned, and a shape the split-K kernel takes (not the shared-activation one). */
+int rocm_decode_packed_fuses_norm(const RocmMatMulNBitsArgs* args);
 /* The fused gate/up node at up to four rows: one launch over both projections' repacked copies; Y (the activations'
  * 16-bit type) = round16(silu(round16(gate)) * round16(up)), each projection summed exactly as its own launch would.
  * args names the shared operands (a, y, m, n, k, block_size, dtypes; b / scales / zp only for the eligibility checks).

@@ -109,6 +109,9 @@ struct PackedParams {
     int bias_dtype, y_dtype;
     uint32_t nibble_mask;   // 0x000F000F
     uint32_t magic;         // two 16-bit magic exponents; a kernel argument so that it stays in a scalar register
+    const void* gamma;      // NORM kernels: the RMS-normalization weight [k], f32 or the activations' type
+    int gamma_f32;
+    float norm_epsilon;
 };
 
 template <bool BF16>
@@ -118,11 +121,12 @@ __device__ __forceinline__ float4p_t mfma16p(const uint4& act, const uint4& wgt,
     else return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8p_t, act), __builtin_bit_cast(half8p_t, wgt), acc, 0, 0, 0);
 }
 
-template <int NR, int NA>
+template <int NR, int NA, int NG>
 struct PackedGroup {
     uint4 w[kGroupTiles];
     uint4 r[NR];
     uint4 a[NA];
+    uint4 gm[NG];     // NORM: the normalization weights of the activation pieces (two loads each: f32 weights are 32 bytes a piece)
 };
 
 // v + (v of the lane a DPP control selects): quad_perm [1,0,3,2] = 0xB1, [2,3,0,1] = 0x4E, row_half_mirror = 0x141,
@@ -184,11 +188,18 @@ __device__ __forceinline__ float block_sum(float s)
 // PAIR: the fused gate/up node. The first half of the workgroup's waves runs the gate projection's column group, the
 // second half the up projection's - each half exactly as a launch of its own would (same split of K, same order of
 // summation, so the same f32 totals) - and the epilogue writes round16(silu(round16(gate)) * round16(up)).
-template <bool BF16, int BS, int MR, typename ST, int SETS, bool PAIR>
+// NORM (up to 4 rows): the RMS-normalization prologue inside the kernel (the CUDA provider's form,
+// onnx-runtime-ep-cuda/src/kernels/matmul_nbits.rs:3747-3783). Every wave first sums the squares of the call's rows in
+// the reference's order (32 lanes, four running sums over 4-element chunks, (s0 + s1) + (s2 + s3), a shuffle tree over
+// 32 lanes: half a wavefront plays one warp, so a wave covers two rows per pass), then replaces each activation piece it
+// loads by round16((a * inv_std) * gamma) before the piece is staged - the values a separate normalization launch
+// would have written, bit for bit.
+template <bool BF16, int BS, int MR, typename ST, int SETS, bool PAIR, bool NORM = false>
 __global__ __launch_bounds__((BS == 128 && sizeof(ST) == 2 && (MR != 16 || BF16)) ? 1024 : 512)   // block 128, 16-bit scales, up to 4 rows: up to 16 waves split a long K
-__attribute__((amdgpu_waves_per_eu((BS == 128 && MR == 1 && sizeof(ST) == 2) ? (SETS == 1 ? 8 : 5) : 1)))
+__attribute__((amdgpu_waves_per_eu((BS == 128 && MR == 1 && sizeof(ST) == 2 && !NORM) ? (SETS == 1 ? 8 : 5) : 1)))
 void decode_packed_kernel(PackedParams p)
 {
+    static_assert(!NORM || MR <= 4, "the fused normalization covers up to four rows");
     constexpr int U = kGroupTiles;
     constexpr int NBT = 128 / BS;
     constexpr int NB = U * NBT;
@@ -196,6 +207,8 @@ void decode_packed_kernel(PackedParams p)
     constexpr int NR = R / 16;
     constexpr int RQ = MR == 1 ? 1 : MR / 4;       // loads per tile: each covers four rows (row g + 4 i, piece c)
     constexpr int NA = MR == 1 ? 1 : U * RQ;
+    constexpr int NGP = MR == 1 ? 1 : U;           // activation pieces with distinct elements per group (rows share them)
+    constexpr int NG = NORM ? 2 * NGP : 1;
     constexpr int kStageBytes = MR == 1 ? 1024 : MR * kRowPitchP;
     constexpr float kMagicF = BF16 ? 128.0f : 1024.0f;
     constexpr uint32_t kMagicNeg = BF16 ? 0xC300C300u : 0xE400E400u;
@@ -222,6 +235,7 @@ void decode_packed_kernel(PackedParams p)
 
     const __amdgpu_buffer_rsrc_t srd_p = make_srd((second ? p.packed_up : p.packed) + static_cast<int64_t>(blockIdx.x) * p.cg_stride, static_cast<uint64_t>(p.cg_stride));
     const __amdgpu_buffer_rsrc_t srd_a = make_srd(p.a, static_cast<uint64_t>(p.m * p.k) * 2);
+    const __amdgpu_buffer_rsrc_t srd_g = make_srd(NORM ? p.gamma : p.a, NORM ? static_cast<uint64_t>(p.k) * (p.gamma_f32 ? 4 : 2) : 0);
 
     const uint32_t w_off = static_cast<uint32_t>(lane * 16);
     const uint32_t r_off = static_cast<uint32_t>(kChunkWeights + c * R);
@@ -239,7 +253,7 @@ void decode_packed_kernel(PackedParams p)
     const int g_begin = split * p.groups_per_wave;
     const int g_end = min(g_begin + p.groups_per_wave, p.groups);
 
-    using Grp = PackedGroup<NR, NA>;
+    using Grp = PackedGroup<NR, NA, NG>;
     // No branch in here: a group past the wave's last one (the prefetch of the final iteration) gets every offset out of
     // range, which fetches nothing and returns zeros - weights 0, scale 0, activations 0: a group that adds nothing.
     // With a branch instead, the compiler waits for all loads in flight at the next use, the prefetch included.
@@ -258,6 +272,17 @@ void decode_packed_kernel(PackedParams p)
             // rows past M lie past the end of the activations' range and read as zeros
             a_voff[x] = (beyond ? kOutOfRange : a_off + static_cast<uint32_t>(4 * i) * static_cast<uint32_t>(p.k) * 2u) | oor;
         }
+        uint32_t g_voff[NG];
+        if constexpr (NORM) {
+#pragma unroll
+            for (int x = 0; x < NGP; ++x) {
+                const int tile = MR == 1 ? t0 + g : t0 + x;
+                const bool beyond = static_cast<int64_t>(tile) * 128 + c * 8 + 8 > p.k;
+                const uint32_t first = static_cast<uint32_t>(tile * 128 + c * 8) * (p.gamma_f32 ? 4u : 2u);
+                g_voff[2 * x] = (beyond ? kOutOfRange : first) | oor;
+                g_voff[2 * x + 1] = ((beyond || !p.gamma_f32) ? kOutOfRange : first + 16u) | oor;
+            }
+        }
         const uint32_t w_voff = w_off | oor, r_voff = r_off | oor;
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -266,14 +291,103 @@ void decode_packed_kernel(PackedParams p)
         for (int i = 0; i < NR; ++i) grp.r[i] = load16(srd_p, r_voff + static_cast<uint32_t>(i * 16), soff);
 #pragma unroll
         for (int x = 0; x < NA; ++x) grp.a[x] = load16(srd_a, a_voff[x], static_cast<uint32_t>(MR == 1 ? t0 : t0 + x / RQ) * 256u);
+        if constexpr (NORM) {
+#pragma unroll
+            for (int x = 0; x < NG; ++x) grp.gm[x] = load16(srd_g, g_voff[x], 0u);
+        }
         __builtin_amdgcn_sched_barrier(0);
+    };
+
+    // ---- NORM: 1 / sqrt(mean(a^2) + eps) of this lane's row (row 0, or row g of up to four) ----
+    // With one row the wave's first group is requested before, so that its trip to memory overlaps the sums (with four
+    // rows the compiler would keep the group in scratch memory across the passes).
+    constexpr bool kEarly = NORM && MR == 1;
+    Grp ga;
+    if constexpr (kEarly || SETS == 2) fetch_group(ga, g_begin);
+    float inv_std = 1.0f;
+    if constexpr (NORM) {
+        // One wave per pair of rows does the sums (every wave doing them would re-read the rows once per wave: at 3584 ->
+        // 2 x 18944 three times the bytes of the weights) and leaves the results in LDS behind the staging buffers.
+        float* inv_shared = reinterpret_cast<float*>(smem + (blockDim.x >> 6) * (2 * kStageBytes));
+        const int all_waves = static_cast<int>(blockDim.x >> 6);
+        const int l32 = lane & 31;
+        const int items = static_cast<int>(p.k >> 7);
+#pragma unroll
+        for (int pass = 0; pass < (MR == 1 ? 1 : 2); ++pass) {
+            if (wave != pass % all_waves) continue;              // (wave-uniform)
+            const int row = 2 * pass + (lane >> 5);              // rows past M lie past the range and read as zeros
+            const uint32_t base = static_cast<uint32_t>(row) * static_cast<uint32_t>(p.k) * 2u + static_cast<uint32_t>(l32 * 8);
+            float inv = 1.0f;
+            if (MR == 1 || 2 * pass < p.m) {                     // (wave-uniform) rows 2 and 3 only where the call has them
+                float ss0 = 0.f, ss1 = 0.f, ss2 = 0.f, ss3 = 0.f;
+                // sixteen loads in flight at a time: one after the other they would cost a trip to the cache each. A chunk past
+                // the row reads as zeros, and fma(0, 0, s) = s.
+                constexpr int kBatch = 16;
+                for (int first = 0; first < items; first += kBatch) {
+                    uint32_t d0[kBatch], d1[kBatch];
+#pragma unroll
+                    for (int i = 0; i < kBatch; ++i) {
+                        const auto raw = __builtin_amdgcn_raw_buffer_load_b64(srd_a, static_cast<int>(first + i < items ? base : kOutOfRange), (first + i) * 256, 0);
+                        d0[i] = raw[0];
+                        d1[i] = raw[1];
+                    }
+#pragma unroll
+                    for (int i = 0; i < kBatch; ++i) {
+                        const float v0 = BF16 ? __uint_as_float(d0[i] << 16) : f16_bits_to_f32(static_cast<uint16_t>(d0[i]));
+                        const float v1 = BF16 ? __uint_as_float(d0[i] & 0xffff0000u) : f16_bits_to_f32(static_cast<uint16_t>(d0[i] >> 16));
+                        const float v2 = BF16 ? __uint_as_float(d1[i] << 16) : f16_bits_to_f32(static_cast<uint16_t>(d1[i]));
+                        const float v3 = BF16 ? __uint_as_float(d1[i] & 0xffff0000u) : f16_bits_to_f32(static_cast<uint16_t>(d1[i] >> 16));
+                        ss0 = __fmaf_rn(v0, v0, ss0);
+                        ss1 = __fmaf_rn(v1, v1, ss1);
+                        ss2 = __fmaf_rn(v2, v2, ss2);
+                        ss3 = __fmaf_rn(v3, v3, ss3);
+                    }
+                }
+                float ss = __fadd_rn(__fadd_rn(ss0, ss1), __fadd_rn(ss2, ss3));
+#pragma unroll
+                for (int off = 16; off > 0; off >>= 1) ss = __fadd_rn(ss, __shfl_down(ss, off, 32));
+                // sqrtf and the divisions are correctly rounded (the compiler's default for f32)
+                inv = __fdiv_rn(1.0f, sqrtf(__fadd_rn(__fdiv_rn(ss, static_cast<float>(p.k)), p.norm_epsilon)));
+            }
+            if (l32 == 0) inv_shared[row] = inv;
+        }
+        __syncthreads();
+        inv_std = inv_shared[MR == 1 ? 0 : g];
+    }
+    // round16((a * inv_std) * gamma) of one 16-byte piece; g0 / g1: the piece's weights (16-bit: all eight in g0)
+    auto normalized = [&](const uint4& a, const uint4& g0, const uint4& g1) -> uint4 {
+        const uint32_t ad[4] = {a.x, a.y, a.z, a.w};
+        const uint32_t gd[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
+        uint32_t out[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float v0 = BF16 ? __uint_as_float(ad[i] << 16) : f16_bits_to_f32(static_cast<uint16_t>(ad[i]));
+            const float v1 = BF16 ? __uint_as_float(ad[i] & 0xffff0000u) : f16_bits_to_f32(static_cast<uint16_t>(ad[i] >> 16));
+            float w0, w1;
+            if (p.gamma_f32) {
+                w0 = __uint_as_float(gd[2 * i]);
+                w1 = __uint_as_float(gd[2 * i + 1]);
+            } else {
+                w0 = BF16 ? __uint_as_float(gd[i] << 16) : f16_bits_to_f32(static_cast<uint16_t>(gd[i]));
+                w1 = BF16 ? __uint_as_float(gd[i] & 0xffff0000u) : f16_bits_to_f32(static_cast<uint16_t>(gd[i] >> 16));
+            }
+            // (as_f32: the product is rounded to f32 before the 16-bit conversion sees it, never folded into one mixed-precision multiply)
+            const float y0 = as_f32(__fmul_rn(__fmul_rn(v0, inv_std), w0)), y1 = as_f32(__fmul_rn(__fmul_rn(v1, inv_std), w1));
+            const uint32_t lo = BF16 ? f32_to_bf16_bits(y0) : f32_to_f16_bits(y0);
+            const uint32_t hi = BF16 ? f32_to_bf16_bits(y1) : f32_to_f16_bits(y1);
+            out[i] = lo | (hi << 16);
+        }
+        return make_uint4(out[0], out[1], out[2], out[3]);
     };
     // `asum` (with SUMS): this lane's block sum of the group's tile lane / 16 (one load covers the group's four tiles).
     auto compute_tile = [&](const Grp& grp, int u, int parity, float asum) {
         unsigned char* st = stage + (MR == 1 ? parity : (u & 1)) * kStageBytes;
         if constexpr (MR != 1) {
 #pragma unroll
-            for (int i = 0; i < RQ; ++i) *reinterpret_cast<uint4*>(st + st_write + i * 4 * kRowPitchP) = grp.a[u * RQ + i];
+            for (int i = 0; i < RQ; ++i) {
+                if constexpr (NORM) *reinterpret_cast<uint4*>(st + st_write + i * 4 * kRowPitchP) = normalized(grp.a[u * RQ + i], grp.gm[2 * u], grp.gm[2 * u + 1]);
+                else *reinterpret_cast<uint4*>(st + st_write + i * 4 * kRowPitchP) = grp.a[u * RQ + i];
+            }
             lds_order();
         }
         uint4 av[4];
@@ -342,7 +456,8 @@ void decode_packed_kernel(PackedParams p)
         __builtin_amdgcn_sched_barrier(0);
         if (prefetch) fetch_group(next, gi + 1);
         if constexpr (MR == 1) {
-            *reinterpret_cast<uint4*>(stage + parity * kStageBytes + st_write) = cur.a[0];
+            if constexpr (NORM) *reinterpret_cast<uint4*>(stage + parity * kStageBytes + st_write) = normalized(cur.a[0], cur.gm[0], cur.gm[1]);
+            else *reinterpret_cast<uint4*>(stage + parity * kStageBytes + st_write) = cur.a[0];
             lds_order();
         }
 #pragma unroll
@@ -350,8 +465,7 @@ void decode_packed_kernel(PackedParams p)
     };
 
     if constexpr (SETS == 2) {
-        Grp ga, gb;
-        fetch_group(ga, g_begin);
+        Grp gb;
         int gi = g_begin;
         for (; gi + 1 < g_end; gi += 2) {                      // whole pairs, no branch inside: every wait counts loads exactly
             run_group(ga, gb, gi, 0, true);
@@ -360,17 +474,26 @@ void decode_packed_kernel(PackedParams p)
         if (gi < g_end) run_group(ga, gb, gi, 0, false);       // an odd group out
 
     } else {
-        Grp ga;
-        for (int gi = g_begin; gi < g_end; ++gi) {
-            fetch_group(ga, gi);
+        auto multiply = [&]() {
             float asum = 0.f;
             if constexpr (MR == 1) {
-                *reinterpret_cast<uint4*>(stage + st_write) = ga.a[0];
+                uint4 piece = ga.a[0];
+                if constexpr (NORM) piece = normalized(ga.a[0], ga.gm[0], ga.gm[1]);
+                *reinterpret_cast<uint4*>(stage + st_write) = piece;
                 lds_order();
-                if constexpr (SUMS) asum = block_sum<BS>(sum_piece<BF16>(ga.a[0]));
+                if constexpr (SUMS) asum = block_sum<BS>(sum_piece<BF16>(piece));
             }
 #pragma unroll
             for (int u = 0; u < U; ++u) compute_tile(ga, u, 0, asum);
+        };
+        int gi = g_begin;
+        if constexpr (kEarly) {                                // the first group is already on its way
+            if (gi < g_end) multiply();
+            ++gi;
+        }
+        for (; gi < g_end; ++gi) {
+            fetch_group(ga, gi);
+            multiply();
         }
     }
 
@@ -411,7 +534,14 @@ static int launch_packed_cfg(const PackedParams& p, int waves, hipStream_t strea
     const int all = pair ? 2 * waves : waves;
     const size_t stage = static_cast<size_t>(all) * 2 * (MR == 1 ? 1024 : MR * kRowPitchP);
     const size_t red = static_cast<size_t>(all) * 1024;
-    const size_t lds = stage > red ? stage : red;
+    const size_t lds = (stage > red ? stage : red) + (p.gamma ? 16 : 0);      // + the rows' 1 / rms of a launch with the normalization prologue
+    if constexpr (MR == 1 || (MR == 4 && SETS == 1)) {       // (four rows with a second register set and the weights of the prologue would spill)
+        if (p.gamma) {
+            if (pair) hipLaunchKernelGGL((decode_packed_kernel<BF16, BS, MR, ST, SETS, true, true>), dim3(grid), dim3(all * 64), lds, stream, p);
+            else hipLaunchKernelGGL((decode_packed_kernel<BF16, BS, MR, ST, SETS, false, true>), dim3(grid), dim3(all * 64), lds, stream, p);
+            return static_cast<int>(hipGetLastError());
+        }
+    }
     if constexpr (MR == 16) {
         // sixteen staged rows of sixteen waves outgrow the 64 KiB a kernel gets without asking
         if (lds > 65536) {
@@ -431,7 +561,7 @@ template <bool BF16, int BS, typename ST>
 static int launch_packed_mr(const PackedParams& p, int waves, bool single_set, hipStream_t stream)
 {
     if (p.m <= 1) return single_set ? launch_packed_cfg<BF16, BS, 1, ST, 1>(p, waves, stream) : launch_packed_cfg<BF16, BS, 1, ST, 2>(p, waves, stream);
-    if (p.m <= 4) return single_set ? launch_packed_cfg<BF16, BS, 4, ST, 1>(p, waves, stream) : launch_packed_cfg<BF16, BS, 4, ST, 2>(p, waves, stream);
+    if (p.m <= 4) return (single_set || p.gamma) ? launch_packed_cfg<BF16, BS, 4, ST, 1>(p, waves, stream) : launch_packed_cfg<BF16, BS, 4, ST, 2>(p, waves, stream);
     // 5 .. 16 rows: one register set (64 registers of activations per group; a second set in flight measured slower)
     return launch_packed_cfg<BF16, BS, 16, ST, 1>(p, waves, stream);
 }
@@ -1176,6 +1306,13 @@ extern "C" int rocm_launch_pack_decode(const RocmMatMulNBitsArgs* a, void* packe
 // the return value says whether a paired launch with this split of K fits a workgroup (1) or not (0).
 // `pair_member`: the launch is one projection of a gate/up pair (or the paired launch itself): the split of K is chosen
 // for the pair's column groups together, so that the separate launches and the paired one add up in the same order.
+extern "C" int rocm_decode_packed_fuses_norm(const RocmMatMulNBitsArgs* a)
+{
+    if (!a->gamma || a->m > 4 || a->k % 128 != 0 || wide_shape(a) || !rocm_decode_packed_eligible(a)) return 0;
+    if (a->gamma_dtype != ROCM_DT_F32 && a->gamma_dtype != a->a_dtype) return 0;
+    return (reinterpret_cast<uintptr_t>(a->gamma) & 15) == 0;
+}
+
 static int launch_decode_packed(const RocmMatMulNBitsArgs* a, const void* packed, const void* packed_up, int decomposed, int waves, bool probe_only,
                                 bool pair_member, rocm_stream_t stream)
 {
@@ -1198,6 +1335,15 @@ static int launch_decode_packed(const RocmMatMulNBitsArgs* a, const void* packed
     p.nibble_mask = 0x000F000Fu;
     const bool bf16 = a->a_dtype == ROCM_DT_BF16;
     p.magic = bf16 ? 0x43004300u : 0x64006400u;
+    p.gamma = nullptr;
+    p.gamma_f32 = 0;
+    p.norm_epsilon = 0.f;
+    if (a->gamma) {
+        if (!rocm_decode_packed_fuses_norm(a)) return probe_only ? 0 : -1;
+        p.gamma = a->gamma;
+        p.gamma_f32 = a->gamma_dtype == ROCM_DT_F32;
+        p.norm_epsilon = a->norm_epsilon;
+    }
 
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool f32_scales = a->scale_dtype == ROCM_DT_F32;
@@ -1214,12 +1360,13 @@ static int launch_decode_packed(const RocmMatMulNBitsArgs* a, const void* packed
     const int64_t wgs = (a->n + 15) / 16 * (pair_member ? 2 : 1);
     int w = waves;
     bool single_set = wgs * 4 >= 6144;
-    // One row (not a member of a gate/up pair, whose split of K is fixed by the paired launch): one tile group per wave where
+    // One row: one tile group per wave where
     // the workgroup can hold that many waves, no prefetch, offset and zero point through the activation sums. Every byte
     // of the call is then requested as soon as its wave starts, and what a wave computes between its loads and the
     // reduction is the least any variant here does. Measured against the few-wave prefetching build it replaced on the
     // small shapes (bf16, block 128): 3584 -> 4608 5.06 -> 4.78 us, 3584 -> 3584 4.17 -> 3.97, 18944 -> 3584 9.94 -> 9.41,
     // 3584 -> 37888 15.81 -> 15.48.
+    // (a gate/up pair keeps the few-wave split: with fourteen waves a workgroup the paired launch measured 17.8 us against 15.5)
     const bool one_row = a->m <= 1 && !pair_member;
     if (one_row && w <= 0) {
         single_set = true;

@@ -840,6 +840,15 @@ RMSNORM_CASES = [
     (E.BF16, E.BF16, 128, 1, 520, 3584, 1e-6),
     (E.BF16, E.F32, 128, 16, 200, 1024, 1e-5),
     (E.F16, E.F16, 64, 100, 136, 512, 1e-5),
+    # up to four rows over constant weights: normalized inside the decode kernel - one row and four, both gamma types, every
+    # block size, K over several waves, few and many workgroups (with and without the second register set)
+    (E.BF16, E.F32, 128, 1, 4608, 3584, 1e-6),
+    (E.BF16, E.BF16, 128, 4, 520, 3584, 1e-6),
+    (E.F16, E.F32, 64, 2, 333, 2048, 1e-5),
+    (E.F16, E.F16, 64, 1, 24576, 512, 1e-5),
+    (E.F16, E.F16, 32, 4, 24576, 512, 1e-6),
+    (E.BF16, E.F32, 32, 3, 100, 128 * 9, 1e-5),
+    (E.F16, E.F32, 128, 4, 77, 128 * 40, 1e-5),
 ]
 
 
@@ -867,7 +876,7 @@ def test_gate_up_swiglu_at_accuracy_level_4_stays_on_the_int8_kernels(ep):
 
 
 @pytest.mark.parametrize("a_dt,g_dt,bs,m,n,k,eps", RMSNORM_CASES)
-def test_rmsnorm_prologue(ep, port, a_dt, g_dt, bs, m, n, k, eps):
+def test_rmsnorm_prologue(ep, ep_unpacked, port, a_dt, g_dt, bs, m, n, k, eps):
     """A node with the RMS-normalization prologue gives, bit for bit, what the same node without it gives on activations the
     oracle normalized: the prologue's kernel equals the oracle's restatement (sums in the reference's order) on every element
     that matters to the product."""
@@ -879,8 +888,24 @@ def test_rmsnorm_prologue(ep, port, a_dt, g_dt, bs, m, n, k, eps):
     normalized = port.rmsnorm16(np.asarray(a).reshape(m, k), gamma, g_code, eps, o_dt)
     y, variant = run_op(ep, a, a_dt, b, s, a_dt, zp, n, k, bs, gamma=gamma, gamma_dtype=g_dt, rmsnorm_epsilon=eps)
     want, plain_variant = run_op(ep, normalized, a_dt, b, s, a_dt, zp, n, k, bs)
-    assert variant == "rmsnorm+" + plain_variant
+    # up to four rows over the repacked stream, up to 8192 columns: the decode kernel normalizes the rows itself; otherwise a
+    # launch of its own does
+    assert variant == ("rmsnorm[decode_mfma_packed]" if m <= 4 and n <= 8192 else "rmsnorm+" + plain_variant)
     assert np.array_equal(np.asarray(y).view(np.uint16), np.asarray(want).view(np.uint16))
+    if m <= 4 and n > 8192:
+        # the in-kernel form at this width too, where the setting allows it
+        wide = E.RocmExecutionProvider(0, {"rmsnorm_in_kernel_max_cols": str(n)})
+        try:
+            y3, variant3 = run_op(wide, a, a_dt, b, s, a_dt, zp, n, k, bs, gamma=gamma, gamma_dtype=g_dt, rmsnorm_epsilon=eps)
+        finally:
+            wide.shutdown()
+        assert variant3 == "rmsnorm[decode_mfma_packed]"
+        assert np.array_equal(np.asarray(y3).view(np.uint16), np.asarray(want).view(np.uint16))
+    if m <= 4:
+        # the same node where nothing is repacked: the separate normalization launch, the same bits
+        y2, variant2 = run_op(ep_unpacked, a, a_dt, b, s, a_dt, zp, n, k, bs, gamma=gamma, gamma_dtype=g_dt, rmsnorm_epsilon=eps)
+        assert variant2 == "rmsnorm+decode_mfma_splitk"
+        assert helpers.rel_l2(synth.to_f32(y2, a_dt), synth.to_f32(want, a_dt)) <= TOL_HALF
     # and the normalization is one: mean square of the normalized row over gamma^2 is 1 within the 16-bit roundings
     nf = synth.to_f32(normalized, a_dt) / synth.to_f32(gamma, g_dt)[None, :]
     assert np.allclose(np.mean(nf.astype(np.float64) ** 2, axis=1), 1.0, rtol=2e-2)
@@ -897,6 +922,38 @@ def test_rmsnorm_prologue_on_the_fused_gate_up_node(ep, port):
     want, _ = E.gate_up_swiglu(ep, normalized, a_dt, gate, up, a_dt, n, k, bs)
     assert variant.startswith("rmsnorm+gate_up_swiglu")
     assert np.array_equal(np.asarray(y).view(np.uint16), np.asarray(want).view(np.uint16))
+
+
+@pytest.mark.parametrize("a_dt,g_dt,bs,m,n,k", [(E.F16, E.F32, 32, 2, 200, 1024), (E.BF16, E.BF16, 128, 1, 2368, 3584), (E.BF16, E.F32, 128, 4, 300, 3584),
+                                                (E.F16, E.F16, 64, 3, 100, 512)])
+def test_rmsnorm_prologue_inside_the_single_launch_gate_up_node(ep, port, a_dt, g_dt, bs, m, n, k):
+    """Calls after the first (which repacks both projections) run normalization, both projections and the SwiGLU epilogue as
+    one launch; the result equals, bit for bit, the first call's (separate normalization launch, separate projections) and
+    the node without the prologue on rows the oracle normalized."""
+    eps = 1e-6
+    gate = synth.make_weights(n, k, bs, 840, zero_points=True, scale_lo=0.004, scale_hi=0.02, scale_dtype=a_dt)
+    up = synth.make_weights(n, k, bs, 841, zero_points=True, scale_lo=0.004, scale_hi=0.02, scale_dtype=a_dt)
+    a = synth.make_activation(m, k, 842, a_dt)
+    gamma = synth.to_dtype((1.0 + 0.25 * np.random.default_rng(8).standard_normal(k)).astype(np.float32), g_dt)
+    o_dt = oracle.F16 if a_dt == E.F16 else oracle.BF16
+    normalized = port.rmsnorm16(np.asarray(a).reshape(m, k), gamma, oracle.F32 if g_dt == E.F32 else o_dt, eps, o_dt)
+    want, _ = E.gate_up_swiglu(ep, normalized, a_dt, gate, up, a_dt, n, k, bs)
+    ops = E.GateUpOperands(ep, gate, up, a_dt, n, k, bs, gamma=gamma, gamma_dtype=g_dt, rmsnorm_epsilon=eps)
+    ab, yb = ep.upload(a), ep.allocate(m * n * 2)
+    try:
+        outs, variants = [], []
+        for _ in range(3):
+            ops.run(ab, a_dt, m, yb)
+            outs.append(ep.download(yb, (m, n), np.uint16).copy())
+            variants.append(ops.kernel.last_variant())
+        assert variants[0].startswith("rmsnorm+gate_up_swiglu[")
+        assert variants[1] == variants[2] == "rmsnorm[gate_up_swiglu_packed]", variants
+        for got in outs:
+            assert np.array_equal(got, np.asarray(want).view(np.uint16))
+    finally:
+        ep.deallocate(ab)
+        ep.deallocate(yb)
+        ops.free()
 
 
 def test_rmsnorm_prologue_validation(ep):
