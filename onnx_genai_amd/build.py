@@ -27,7 +27,7 @@ HIP_SOURCES = [
     "kernels/acc4.hip",
     "kernels/acc4_mfma.hip",
 ]
-HOST_SOURCES = ["ep/provider.cpp", "ep/matmul_nbits.cpp", "ep/nxrt_plugin.cpp", "ep/nxmem_plugin.cpp"]
+HOST_SOURCES = ["ep/provider.cpp", "ep/matmul_nbits.cpp", "ep/nxrt_plugin.cpp", "ep/nxmem_plugin.cpp", "ep/ort_plugin.cpp"]
 
 # packed-fp32 VALU forms are kept off for all device code
 DEVICE_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]

@@ -25,7 +25,7 @@ def declared_symbols():
     for header in sorted(os.listdir(INCLUDE)):
         text = open(os.path.join(INCLUDE, header)).read()
         text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-        for m in re.finditer(r"^[A-Za-z_][\w\s\*]*?\b((?:nxrt_rocm_|Nxrt|Nxmem)\w+)\s*\(", text, flags=re.M):
+        for m in re.finditer(r"^[A-Za-z_][\w\s\*]*?\b((?:nxrt_rocm_|Nxrt|Nxmem)\w+|CreateEpFactories|ReleaseEpFactory)\s*\(", text, flags=re.M):
             line_start = text.rfind("\n", 0, m.start()) + 1
             if text[line_start:m.start()].strip().startswith("typedef"):
                 continue
@@ -36,6 +36,7 @@ def declared_symbols():
 def test_every_declared_symbol_is_exported(lib):
     names = declared_symbols()
     assert len(names) >= 40 and "NxrtNegotiate" in names and "nxrt_rocm_matmul_nbits_execute" in names and "NxmemQueryUnloadReadiness" in names
+    assert "CreateEpFactories" in names and "ReleaseEpFactory" in names               # the ORT plugin-EP export
     missing = [n for n in names if not hasattr(lib, n)]
     assert not missing, missing
 
@@ -43,7 +44,8 @@ def test_every_declared_symbol_is_exported(lib):
 def test_headers_compile_as_c_and_cxx():
     import subprocess
     for lang, std in (("c", "-std=c11"), ("c++", "-std=c++17")):
-        subprocess.run(["gcc", "-fsyntax-only", "-x", lang, std, "-Wall", "-Werror", os.path.join(INCLUDE, "nxrt_ep_rocm.h")], check=True)
+        for header in ("nxrt_ep_rocm.h", "nxrt_ort_plugin.h", "ort_plugin_ep_subset.h"):
+            subprocess.run(["gcc", "-fsyntax-only", "-x", lang, std, "-Wall", "-Werror", os.path.join(INCLUDE, header)], check=True)
 
 
 class VersionRange(C.Structure):
