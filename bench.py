@@ -45,7 +45,7 @@ A_DT = E.BF16
 # (FETCH_SIZE, then WRITE_SIZE, each scaled by what the same counter reads for the 256 MiB copy that run ends with).
 # `bench.py --traffic-from <fetch csv> <write csv>` turns the two counter files into this tracked JSON; the benchmark line
 # reports its figure only while the kernel variant it was taken on is still the one that runs.
-TRAFFIC_JSON = os.path.join(ROOT, "profiles", "decode_gate_up_m1_traffic.json")
+TRAFFIC_JSON = os.path.join(ROOT, "profiles", "decode_gate_up_m1_traffic.txt")
 
 
 def traffic_from_counters(fetch_csv, write_csv):
@@ -78,6 +78,35 @@ def traffic_from_counters(fetch_csv, write_csv):
     with open(TRAFFIC_JSON, "w") as f:
         json.dump(out, f, indent=1)
         f.write("\n")
+    return out
+
+
+def trace_summary(kernel_trace_csv):
+    """Per kernel and launch shape of a rocprofv3 `--kernel-trace` file of this benchmark: launches, average and shortest
+    duration, and the average distance from one launch's start to the next launch's start inside a graph replay (what a
+    call costs the step, launch overhead included). No GPU work."""
+    import collections
+    import csv
+    rows = sorted(csv.DictReader(open(kernel_trace_csv)), key=lambda r: int(r["Start_Timestamp"]))
+
+    def key(r):
+        grid = int(r.get("Grid_Size_X") or r.get("Grid_Size") or 0)
+        wg = int(r.get("Workgroup_Size_X") or r.get("Workgroup_Size") or 0)
+        return r["Kernel_Name"].split("(")[0][:90], grid // max(wg, 1), wg
+
+    stats = collections.defaultdict(lambda: {"dur": [], "s2s": []})
+    prev = None
+    for r in rows:
+        start, end = int(r["Start_Timestamp"]), int(r["End_Timestamp"])
+        k = key(r)
+        stats[k]["dur"].append(end - start)
+        if prev is not None and start - prev[1] < 20000:          # the same replay
+            stats[prev[2]]["s2s"].append(start - prev[0])
+        prev = (start, end, k)
+    out = []
+    for (name, wgs, wg), v in sorted(stats.items(), key=lambda kv: -sum(kv[1]["dur"])):
+        out.append({"kernel": name, "workgroups": wgs, "threads": wg, "launches": len(v["dur"]), "avg_ns": round(sum(v["dur"]) / len(v["dur"])),
+                    "min_ns": min(v["dur"]), "avg_start_to_start_ns": round(sum(v["s2s"]) / len(v["s2s"])) if v["s2s"] else None})
     return out
 
 
@@ -351,7 +380,11 @@ def main():
     ap.add_argument("--only-tables", action="store_true",
                     help="run only the prefill and accuracy_level=4 tables, one JSON line per row (the command their profiles are taken from)")
     ap.add_argument("--traffic-from", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
-                    help="no GPU work: turn two rocprofv3 counter files of --only-roofline runs (FETCH_SIZE, WRITE_SIZE) into profiles/decode_gate_up_m1_traffic.json")
+                    help="no GPU work: turn two rocprofv3 counter files of --only-roofline runs (FETCH_SIZE, WRITE_SIZE) into profiles/decode_gate_up_m1_traffic.txt")
+    ap.add_argument("--trace-summary", metavar="KERNEL_TRACE_CSV",
+                    help="no GPU work: per kernel and launch shape of a rocprofv3 --kernel-trace file of this benchmark, one JSON line each")
+    ap.add_argument("--read-floor", action="store_true",
+                    help="run only the yardstick: a plain read of each decode shape's bytes, one launch per layer buffer in a graph, beside the decode kernel's time on the same buffers")
     ap.add_argument("--row-sweep", action="store_true",
                     help="run only a sweep of the row count M across the dispatch boundaries (1 .. 2048), one JSON line per call shape")
     args = ap.parse_args()
@@ -360,11 +393,19 @@ def main():
     if args.traffic_from:
         print(json.dumps(traffic_from_counters(*args.traffic_from)), flush=True)
         return
+    if args.trace_summary:
+        for row in trace_summary(args.trace_summary):
+            print(json.dumps(row), flush=True)
+        return
 
     ep = E.RocmExecutionProvider(0)
     info = ep.device_info()
     if args.only_roofline:
         return roofline_only(ep, args)
+    if args.read_floor:
+        for row in read_floor(ep, args):
+            print(json.dumps(row), flush=True)
+        return
     if args.row_sweep:
         for row in row_sweep(ep):
             print(json.dumps(row), flush=True)
@@ -467,6 +508,51 @@ def roofline_only(ep, args):
     print(json.dumps({"kernel": nodes[0].ops.kernel.last_variant() + " on gate_up 3584->37888", "m": args.m, "launches": len(nodes) * (args.steps + args.warmup) + 1,
                       "us_per_launch": round(us, 2), "bytes_per_launch": nodes[0].bytes, "achieved_gbs": round(nodes[0].bytes / us / 1e3, 1),
                       "copy_kernel_bytes_read": copy_bytes, "copy_kernel_bytes_written": copy_bytes}), flush=True)
+
+
+def read_floor(ep, args):
+    """What the chain of dependent launches allows at best: for every decode shape, `layers` launches of a kernel that only
+    reads the shape's algorithmic bytes (distinct buffers, one HIP graph, the same timing as the decode sweep), beside the
+    decode kernel itself over its own `layers` weight buffers. A launch that does nothing but read cannot be beaten, so
+    `floor_us` bounds the shape's share of the step; the step's bound is their sum."""
+    rows, a_bufs = [], {k: ep.upload(synth.make_activation(args.m, k, 5, A_DT)) for k in (HIDDEN, INTER)}
+    for name, k, n in LAYER_SHAPES + [LM_HEAD]:
+        copies = args.layers if name != LM_HEAD[0] else 3
+        nodes, reuse = [], None
+        for i in range(copies):
+            node = Node(ep, f"{name}.{i}", k, n, BS, 50 + i, A_DT, args.m, reuse=reuse)
+            reuse = node.host_b if reuse is None else reuse
+            nodes.append(node)
+        for node in nodes:
+            node.run(a_bufs[k])
+        ep.sync()
+        graph = capture(ep, lambda: [node.run(a_bufs[k]) for node in nodes])
+        kernel_us = time_graph(ep, graph, args.steps, args.warmup) * 1e3 / copies
+        graph.release()
+        nbytes = nodes[0].bytes
+        bufs = [ep.allocate(nbytes) for _ in range(copies)]
+        for b in bufs:
+            ep.read_probe(b, nbytes)
+        ep.sync()
+        graph = capture(ep, lambda: [ep.read_probe(b, nbytes) for b in bufs])
+        floor_us = time_graph(ep, graph, args.steps, args.warmup) * 1e3 / copies
+        graph.release()
+        rows.append({"shape": name, "k": k, "n": n, "m": args.m, "bytes": nbytes, "launches_per_graph": copies, "read_only_us": round(floor_us, 2),
+                     "read_only_gbs": round(nbytes / floor_us / 1e3, 1), "decode_kernel_us": round(kernel_us, 2), "decode_over_read_only": round(kernel_us / floor_us, 3),
+                     "variant": nodes[0].ops.kernel.last_variant()})
+        for b in bufs:
+            ep.deallocate(b)
+        for node in nodes:
+            node.free(ep)
+    per_layer = [r for r in rows if r["shape"] != LM_HEAD[0]]
+    lm = rows[-1]
+    step_floor = args.layers * sum(r["read_only_us"] for r in per_layer) + lm["read_only_us"]
+    step_now = args.layers * sum(r["decode_kernel_us"] for r in per_layer) + lm["decode_kernel_us"]
+    step_bytes = args.layers * sum(r["bytes"] for r in per_layer) + lm["bytes"]
+    rows.append({"step": "%d layers + lm_head" % args.layers, "bytes": step_bytes, "read_only_us": round(step_floor, 1), "read_only_gbs": round(step_bytes / step_floor / 1e3, 1),
+                 "read_only_hbm_frac": round(step_bytes / step_floor / 1e3 / HBM_PEAK_GBS, 4), "decode_kernels_us": round(step_now, 1),
+                 "decode_hbm_frac": round(step_bytes / step_now / 1e3 / HBM_PEAK_GBS, 4)})
+    return rows
 
 
 def sweep(ep, nodes, a_bufs, args):

@@ -71,6 +71,10 @@ NxrtStatus nxrt_rocm_ep_copy_from_host(NxrtRocmEp* ep, void* dst_device, const v
 NxrtStatus nxrt_rocm_ep_copy_to_host(NxrtRocmEp* ep, void* dst_host, const void* src_device, size_t bytes);
 NxrtStatus nxrt_rocm_ep_copy(NxrtRocmEp* ep, void* dst_device, const void* src_device, size_t bytes);
 NxrtStatus nxrt_rocm_ep_sync(NxrtRocmEp* ep);
+/* A benchmark's yardstick, not part of the reference's interface: enqueues a kernel that reads `bytes` of device memory (16-byte
+ * loads, four in flight per lane, one workgroup per 16 KiB) and keeps nothing. Its time is the least any kernel can spend
+ * pulling that many bytes from HBM; bench.py --read-floor reports it beside the decode kernels' times. */
+NxrtStatus nxrt_rocm_ep_read_probe(NxrtRocmEp* ep, const void* src_device, size_t bytes);
 /* The nxrt EP vtable whose ctx is this provider (what NxrtEpFactoryVtable.create_ep hands out);
  * the inverse recovers the provider from a vtable obtained through the plugin exports. */
 NxrtRocmEp* nxrt_rocm_ep_from_vtable(const NxrtEpVtable* vtable);

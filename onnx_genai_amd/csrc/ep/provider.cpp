@@ -209,6 +209,16 @@ NxrtStatus nxrt_rocm_ep_copy(NxrtRocmEp* ep, void* dst, const void* src, size_t 
     });
 }
 
+NxrtStatus nxrt_rocm_ep_read_probe(NxrtRocmEp* ep, const void* src, size_t bytes)
+{
+    return fenced([&]() -> NxrtStatus {
+        if (!ep || (bytes && !src)) return make_status(NXRT_INVALID_ARGUMENT, "read_probe: null pointer");
+        NxrtStatus st = ep->bind();
+        if (st.code != NXRT_OK) return st;
+        return hip_status(rocm_ffi_read_probe(src, bytes, nullptr, ep->stream), "read probe launch");
+    });
+}
+
 NxrtStatus nxrt_rocm_ep_sync(NxrtRocmEp* ep)
 {
     return fenced([&]() -> NxrtStatus {

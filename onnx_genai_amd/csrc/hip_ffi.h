@@ -40,6 +40,9 @@ uint64_t rocm_ffi_malloc_calls(void);
 int rocm_ffi_static_scratch(int device, void** ptr, size_t* bytes);
 int rocm_ffi_memcpy_h2d(void* dst, const void* src, size_t bytes, rocm_stream_t stream);
 int rocm_ffi_memcpy_d2h(void* dst, const void* src, size_t bytes, rocm_stream_t stream);
+/* Reads `bytes` (a multiple of 16 is read) of device memory and keeps nothing: the time of the plainest kernel that pulls
+ * that many bytes, for benchmarks to hold other kernels against. `sink`: 4 writable bytes, or NULL. */
+int rocm_ffi_read_probe(const void* src, size_t bytes, void* sink, rocm_stream_t stream);
 int rocm_ffi_memcpy_d2d(void* dst, const void* src, size_t bytes, rocm_stream_t stream);
 int rocm_ffi_stream_create(rocm_stream_t* stream);
 int rocm_ffi_stream_destroy(rocm_stream_t stream);

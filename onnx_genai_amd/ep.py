@@ -97,6 +97,8 @@ def load_library() -> C.CDLL:
     L.nxrt_rocm_ep_copy_to_host.argtypes = [v, v, v, sz]
     L.nxrt_rocm_ep_copy.restype = S
     L.nxrt_rocm_ep_copy.argtypes = [v, v, v, sz]
+    L.nxrt_rocm_ep_read_probe.restype = S
+    L.nxrt_rocm_ep_read_probe.argtypes = [v, v, sz]
     L.nxrt_rocm_ep_sync.restype = S
     L.nxrt_rocm_ep_sync.argtypes = [v]
     L.nxrt_rocm_ep_from_vtable.restype = v
@@ -286,6 +288,10 @@ class RocmExecutionProvider:
 
     def copy(self, dst: DeviceBuffer, src: DeviceBuffer, nbytes: int) -> None:
         self.lib.nxrt_rocm_ep_copy(self.handle, dst.ptr, src.ptr, nbytes).check()
+
+    def read_probe(self, src: DeviceBuffer, nbytes: int) -> None:
+        """Enqueues a plain read of `nbytes` of `src` (a benchmark's yardstick: the least time a kernel can take to pull them)."""
+        self.lib.nxrt_rocm_ep_read_probe(self.handle, src.ptr, nbytes).check()
 
     def sync(self) -> None:
         self.lib.nxrt_rocm_ep_sync(self.handle).check()
