@@ -749,12 +749,13 @@ NxrtStatus execute_swiglu(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in,
     NxrtStatus st = kn.ep->bind();
     if (st.code != NXRT_OK) return st;
 
-    // Up to four rows over constant weights: one launch over both repacked copies. The copies are made (and every weight
-    // tensor validated) by the projections' own first call below, so this path serves the calls after the first with the
-    // same weight tensors; it sums each projection exactly as that first call did.
+    // Up to four rows over constant weights (up to sixteen where the projections are wide enough for the shared-activation
+    // kernel): one launch over both repacked copies. The copies are made (and every weight tensor validated) by the
+    // projections' own first call below, so this path serves the calls after the first with the same weight tensors; it
+    // sums each projection exactly as that first call did.
     // (accuracy_level 4 stays on its own int8 kernels for every call: the paired launch is the float path)
     const void* normalized = nullptr;                    // the rows after a normalization launch of their own, once made
-    if (M <= 4 && kn.accuracy_level != 4 && kn.gate->packed && kn.up->packed) {
+    if (M <= 16 && kn.accuracy_level != 4 && kn.gate->packed && kn.up->packed) {
         auto current = [&](const NxrtRocmMatMulNBits& child, const NxrtRocmTensorView& w, const NxrtRocmTensorView& s, const NxrtRocmTensorView* zp) {
             auto at = [](const NxrtRocmTensorView& v) { return static_cast<const void*>(static_cast<const uint8_t*>(v.data) + v.byte_offset); };
             return child.packed_from[0] == at(w) && child.packed_from[1] == at(s) && child.packed_from[2] == (zp ? at(*zp) : nullptr) &&
@@ -777,7 +778,7 @@ NxrtStatus execute_swiglu(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in,
             args.k = kn.k;
             args.block_size = static_cast<int>(kn.block_size);
             // (a prologue rides along where the pair is narrow enough for the in-kernel form to pay; a wider pair normalizes first)
-            const bool norm_inside = norm && 2 * kn.n <= kn.ep->rmsnorm_in_kernel_max_cols;
+            const bool norm_inside = norm && M <= 4 && 2 * kn.n <= kn.ep->rmsnorm_in_kernel_max_cols;
             if (norm_inside) {
                 args.gamma = norm->gamma;
                 args.gamma_dtype = norm->gamma_dtype;

@@ -602,11 +602,16 @@ constexpr int kWideWaves = 8;
 // PF (with DEEP only): the next group's weights travel while the current one is multiplied (a second register set):
 // for grids with fewer workgroups than CUs, where no other workgroup covers a wave's memory latency.
 // DEEP: the activation windows travel two ahead instead of one (a second set of window registers; RB <= 2).
-template <bool BF16, int BS, typename ST, int RB, bool SUMS, bool PF, bool DEEP>
+// PAIR (RB = 1): the fused gate/up node at 5 .. 16 rows. Waves 0 .. 3 own four column groups of the gate projection,
+// waves 4 .. 7 the same four of the up projection - each wave exactly as in a launch of its projection alone (the whole
+// of K, the same order of summation) - and the epilogue writes round16(silu(round16(gate)) * round16(up)).
+template <bool BF16, int BS, typename ST, int RB, bool SUMS, bool PF, bool DEEP, bool PAIR = false>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu((BS == 128 && sizeof(ST) == 2 && RB == 1) ? (PF ? (SUMS ? 3 : 4) : SUMS ? (DEEP ? 4 : 5) : (DEEP ? 5 : 6)) : 1)))
 void decode_wide_kernel(PackedParams p)
 {
     static_assert(DEEP || !PF, "weights ahead only together with deep windows");
+    static_assert(!PAIR || RB == 1, "the paired form takes up to 16 rows");
+    constexpr int kTileWaves = PAIR ? kWideWaves / 2 : kWideWaves;      // column groups per workgroup (and projection)
     constexpr int U = kGroupTiles;
     constexpr int NBT = 128 / BS;
     constexpr int NB = U * NBT;
@@ -635,11 +640,12 @@ void decode_wide_kernel(PackedParams p)
     const int c = lane & 15;
     const int g = lane >> 4;
     const int64_t col_groups = (p.n + 15) / 16;
-    const int64_t cgi = static_cast<int64_t>(blockIdx.x) * kWideWaves + wave;
+    const bool second = PAIR && wave >= kTileWaves;       // (wave-uniform) the up projection's half
+    const int64_t cgi = static_cast<int64_t>(blockIdx.x) * kTileWaves + (second ? wave - kTileWaves : wave);
     const bool active = cgi < col_groups;                 // a wave beyond the last column group still helps with the windows
     const int64_t n_base = cgi * 16;
 
-    const __amdgpu_buffer_rsrc_t srd_p = make_srd(p.packed + (active ? cgi : 0) * p.cg_stride, active ? static_cast<uint64_t>(p.cg_stride) : 0);
+    const __amdgpu_buffer_rsrc_t srd_p = make_srd((second ? p.packed_up : p.packed) + (active ? cgi : 0) * p.cg_stride, active ? static_cast<uint64_t>(p.cg_stride) : 0);
     const __amdgpu_buffer_rsrc_t srd_a = make_srd(p.a, static_cast<uint64_t>(p.m * p.k) * 2);
 
     const uint32_t w_off = static_cast<uint32_t>(lane * 16);
@@ -811,6 +817,28 @@ void decode_wide_kernel(PackedParams p)
         }
     }
 
+    if constexpr (PAIR) {
+        // every window has been read (the loop ends on a barrier): the up half leaves its totals where the windows were
+        float* up_totals = reinterpret_cast<float*>(smem);            // [kTileWaves][4][64]
+        if (second) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) up_totals[((wave - kTileWaves) * 4 + r) * 64 + lane] = y[0][r];
+        }
+        __syncthreads();
+        const int64_t col = n_base + c;
+        if (!second && active && col < p.n) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int row = 4 * g + r;
+                if (row < p.m) {
+                    const float up = up_totals[(wave * 4 + r) * 64 + lane];
+                    const uint16_t gate16 = BF16 ? f32_to_bf16_bits(y[0][r]) : f32_to_f16_bits(y[0][r]);
+                    const uint16_t up16 = BF16 ? f32_to_bf16_bits(up) : f32_to_f16_bits(up);
+                    static_cast<uint16_t*>(p.y)[static_cast<int64_t>(row) * p.n + col] = swiglu16<BF16>(gate16, up16, p.decomposed_silu != 0);
+                }
+            }
+        }
+    } else
     if (active) {
         const int64_t col = n_base + c;
         if (col < p.n) {
@@ -832,7 +860,11 @@ template <bool BF16, typename ST>
 static int launch_wide_bs(const PackedParams& p, int bs, hipStream_t stream)
 {
     const int64_t col_groups = (p.n + 15) / 16;
-    const dim3 grid(static_cast<unsigned>((col_groups + kWideWaves - 1) / kWideWaves));
+    const bool pair = p.packed_up != nullptr;
+    // a paired launch holds four column groups of each projection per workgroup; which build runs is decided as for a launch
+    // of one projection alone (the builds differ in how offset and zero point leave the accumulator, so in the last bits)
+    const dim3 grid(static_cast<unsigned>(pair ? (col_groups + kWideWaves / 2 - 1) / (kWideWaves / 2) : (col_groups + kWideWaves - 1) / kWideWaves));
+    const unsigned alone = static_cast<unsigned>((col_groups + kWideWaves - 1) / kWideWaves);
     auto go = [&](auto kernel, size_t lds) {
         if (lds > 65536) {
             const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
@@ -847,6 +879,14 @@ static int launch_wide_bs(const PackedParams& p, int bs, hipStream_t stream)
         constexpr int NBT = 128 / BS;
         constexpr size_t lds16 = 2 * 16 * (4 * 256 + 16), sums16 = 2 * 4 * NBT * 16 * 4;
         if (p.m <= 16) {
+            if (pair) {
+                // the sums build unless a projection alone would run the other one; prefetch as the pair's own grid wants it
+                if (alone >= 768) return go(decode_wide_kernel<BF16, BS, ST, 1, false, false, true, true>, lds16);
+                if constexpr (BS != 32) {
+                    if (grid.x < 256) return go(decode_wide_kernel<BF16, BS, ST, 1, true, true, true, true>, lds16 + sums16);
+                }
+                return go(decode_wide_kernel<BF16, BS, ST, 1, true, false, false, true>, lds16 + sums16);
+            }
             // Measured at 8 / 16 rows (3584 -> 152064, 3584 -> 37888, 4096 -> 16384): three or more workgroups per CU run
             // best without the sums and with the windows two ahead (68 -> 64 us); fewer workgroups than CUs with weights
             // and windows both ahead (17.2 -> 14.5 us); in between neither helps (20.6 us either way).
@@ -857,6 +897,7 @@ static int launch_wide_bs(const PackedParams& p, int bs, hipStream_t stream)
             }
             return go(decode_wide_kernel<BF16, BS, ST, 1, true, false, false>, lds16 + sums16);
         }
+        if (pair) return -1;                               // the paired form takes up to 16 rows
         // More row blocks per wave only where they fit the register file: two from block size 64, four at 128. The
         // spilling forms ran several times slower than the routes that take those calls instead (3584 -> 37888: 153 us
         // at block 32 and 32 rows against 2 x 37 us in blocks of 16 rows; 258 us at block 64 and 64 rows against 83 us
@@ -1348,7 +1389,9 @@ static int launch_decode_packed(const RocmMatMulNBitsArgs* a, const void* packed
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool f32_scales = a->scale_dtype == ROCM_DT_F32;
     if (wide_shape(a)) {
-        if (probe_only || packed_up) return probe_only ? 0 : -1;          // the shared-activation kernel has no paired form
+        // the shared-activation kernel's paired form takes up to 16 rows (one block of rows per wave)
+        if (probe_only) return a->m <= 16 ? 1 : 0;
+        if (packed_up && a->m > 16) return -1;
         p.groups_per_wave = p.groups;
         if (bf16) return f32_scales ? mnb::launch_wide_bs<true, float>(p, a->block_size, s) : mnb::launch_wide_bs<true, uint16_t>(p, a->block_size, s);
         return f32_scales ? mnb::launch_wide_bs<false, float>(p, a->block_size, s) : mnb::launch_wide_bs<false, uint16_t>(p, a->block_size, s);

@@ -833,6 +833,60 @@ def test_gate_up_swiglu_single_launch(ep, port, a_dt, s_dt, bs, zero_points, m, 
         ops.free()
 
 
+@pytest.mark.parametrize("a_dt,s_dt,bs,m,n,k,decomposed", [
+    (E.BF16, E.BF16, 128, 16, 18944, 3584, False),    # the 7B pair: fewer workgroups than CUs per projection alone (weights and windows ahead)
+    (E.BF16, E.BF16, 128, 5, 14336, 512, True),
+    (E.F16, E.F16, 64, 9, 14400, 640, False),         # ragged: the last workgroup's waves run out of column groups
+    (E.F16, E.F32, 32, 16, 14336, 256, False),
+    (E.BF16, E.BF16, 128, 8, 98400, 256, False),      # three or more workgroups per CU: the build with the second MFMA
+])
+def test_gate_up_swiglu_single_launch_at_5_to_16_rows(ep, port, a_dt, s_dt, bs, m, n, k, decomposed):
+    """5 to 16 rows where both projections are wide enough for the shared-activation kernel: from the second call on one
+    launch whose workgroups hold four column groups of each projection; the result of the first call (two launches and the
+    epilogue) bit for bit, also replayed from a HIP graph, and the oracle's SwiGLU of the two projections rounded to 16 bits."""
+    gate = synth.make_weights(n, k, bs, 850 + m, zero_points=True, scale_lo=0.004, scale_hi=0.02, scale_dtype=s_dt)
+    up = synth.make_weights(n, k, bs, 851 + m, zero_points=True, scale_lo=0.004, scale_hi=0.02, scale_dtype=s_dt)
+    a = synth.make_activation(m, k, 852 + m, a_dt)
+    ops = E.GateUpOperands(ep, gate, up, s_dt, n, k, bs, decomposed=decomposed)
+    ab, yb = ep.upload(a), ep.allocate(m * n * 2)
+    try:
+        ops.run(ab, a_dt, m, yb)
+        first = ep.download(yb, (m, n), np.uint16).copy()
+        assert ops.kernel.last_variant() == "gate_up_swiglu[decode_mfma_packed]"
+        ep.copy_from_host(yb, np.full(m * n * 2, 0xFF, np.uint8))
+        ops.run(ab, a_dt, m, yb)
+        assert ops.kernel.last_variant() == "gate_up_swiglu_packed"
+        assert np.array_equal(ep.download(yb, (m, n), np.uint16), first)
+        ep.sync()
+        ep.capture_begin()
+        try:
+            ops.run(ab, a_dt, m, yb)
+        finally:
+            graph = ep.capture_end()
+        ep.copy_from_host(yb, np.full(m * n * 2, 0xFF, np.uint8))
+        graph.replay()
+        assert np.array_equal(ep.download(yb, (m, n), np.uint16), first)
+        graph.release()
+        # against the oracle on a sample of columns (the last 16 included): each projection rounded to 16 bits, then the epilogue
+        cols = np.unique(np.concatenate([np.linspace(0, n - 1, 64).astype(np.int64), np.arange(n - 16, n)]))
+        o_dt = oracle.F16 if a_dt == E.F16 else oracle.BF16
+        sub = lambda w: (np.ascontiguousarray(w[0][cols]), np.ascontiguousarray(w[1][cols]), np.ascontiguousarray(w[2][cols]))
+        g16, _ = run_op(ep, a, a_dt, *sub(gate)[:2], s_dt, sub(gate)[2], len(cols), k, bs)
+        u16, _ = run_op(ep, a, a_dt, *sub(up)[:2], s_dt, sub(up)[2], len(cols), k, bs)
+        want = port.swiglu(g16, u16, o_dt, decomposed)
+        got = first.reshape(m, n)[:, cols]
+        # the narrow sub-problem runs another kernel (other summation order): compare in value, not in bits
+        assert helpers.rel_l2(synth.to_f32(got.view(NPDT[a_dt]), a_dt), synth.to_f32(np.asarray(want), a_dt)) <= 2 * TOL_HALF
+        g64 = oracle_f64(port, a, a_dt, *sub(gate)[:2], s_dt, sub(gate)[2], len(cols), k, bs)
+        u64 = oracle_f64(port, a, a_dt, *sub(up)[:2], s_dt, sub(up)[2], len(cols), k, bs)
+        ideal = g64 / (1.0 + np.exp(-g64)) * u64
+        assert helpers.rel_l2(synth.to_f32(got.view(NPDT[a_dt]), a_dt), ideal) <= 2 * TOL_HALF
+    finally:
+        ep.deallocate(ab)
+        ep.deallocate(yb)
+        ops.free()
+
+
 RMSNORM_CASES = [
     # a_dt, gamma dtype, bs, m, n, k, epsilon
     (E.F16, E.F16, 32, 1, 300, 896, 1e-6),
