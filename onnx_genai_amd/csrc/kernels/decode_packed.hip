@@ -591,7 +591,8 @@ static int launch_packed_bs(const PackedParams& p, int bs, int waves, bool singl
 // accumulators, share every unpacked weight operand - up to that height the call still costs what streaming the
 // weights costs, which the tiled kernel cannot offer below a few hundred rows.
 
-constexpr int kWideWaves = 8;
+constexpr int kWideWaves = 8;        // waves that fill the activation windows; a workgroup has 8 .. kWideWavesMax waves
+constexpr int kWideWavesMax = 12;    // (a launch picks the count that spreads its column groups evenly over the CUs)
 
 // RB: blocks of 16 rows (1, 2 or 4). A window is WT tiles of 128 k: a whole tile group for RB <= 2, half of one for
 // RB = 4, so that two buffers of RB * 16 rows stay within 66 KB.
@@ -605,13 +606,18 @@ constexpr int kWideWaves = 8;
 // PAIR (RB = 1): the fused gate/up node at 5 .. 16 rows. Waves 0 .. 3 own four column groups of the gate projection,
 // waves 4 .. 7 the same four of the up projection - each wave exactly as in a launch of its projection alone (the whole
 // of K, the same order of summation) - and the epilogue writes round16(silu(round16(gate)) * round16(up)).
-template <bool BF16, int BS, typename ST, int RB, bool SUMS, bool PF, bool DEEP, bool PAIR = false>
-__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu((BS == 128 && sizeof(ST) == 2 && RB == 1) ? (PF ? (SUMS ? 3 : 4) : SUMS ? (DEEP ? 4 : 5) : (DEEP ? 5 : 6)) : 1)))
+// WMAX: the most waves a workgroup of this build may have (8, or 12 for the builds that balanced grids launch).
+template <bool BF16, int BS, typename ST, int RB, bool SUMS, bool PF, bool DEEP, bool PAIR = false, int WMAX = kWideWaves>
+__global__ __launch_bounds__(WMAX * 64)
+__attribute__((amdgpu_waves_per_eu((BS == 128 && sizeof(ST) == 2 && RB == 1) ? (PF ? (SUMS ? 3 : 4) : SUMS ? (DEEP || WMAX > kWideWaves ? 4 : 5) : (DEEP ? 5 : 6)) : 1)))
 void decode_wide_kernel(PackedParams p)
 {
+    static_assert(WMAX == kWideWaves || (WMAX == kWideWavesMax && RB == 1 && SUMS), "twelve waves: the one-block sums builds only");
     static_assert(DEEP || !PF, "weights ahead only together with deep windows");
     static_assert(!PAIR || RB == 1, "the paired form takes up to 16 rows");
-    constexpr int kTileWaves = PAIR ? kWideWaves / 2 : kWideWaves;      // column groups per workgroup (and projection)
+    // column groups per workgroup (and projection): one per wave. The first eight waves also fill the windows.
+    // (a build for eight waves knows both at compile time)
+    const int tile_waves = WMAX == kWideWaves ? (PAIR ? kWideWaves / 2 : kWideWaves) : (PAIR ? static_cast<int>(blockDim.x >> 7) : static_cast<int>(blockDim.x >> 6));
     constexpr int U = kGroupTiles;
     constexpr int NBT = 128 / BS;
     constexpr int NB = U * NBT;
@@ -640,8 +646,9 @@ void decode_wide_kernel(PackedParams p)
     const int c = lane & 15;
     const int g = lane >> 4;
     const int64_t col_groups = (p.n + 15) / 16;
-    const bool second = PAIR && wave >= kTileWaves;       // (wave-uniform) the up projection's half
-    const int64_t cgi = static_cast<int64_t>(blockIdx.x) * kTileWaves + (second ? wave - kTileWaves : wave);
+    const bool filler = WMAX == kWideWaves || wave < kWideWaves;      // (wave-uniform)
+    const bool second = PAIR && wave >= tile_waves;       // (wave-uniform) the up projection's half
+    const int64_t cgi = static_cast<int64_t>(blockIdx.x) * tile_waves + (second ? wave - tile_waves : wave);
     const bool active = cgi < col_groups;                 // a wave beyond the last column group still helps with the windows
     const int64_t n_base = cgi * 16;
 
@@ -683,12 +690,13 @@ void decode_wide_kernel(PackedParams p)
             const int row = q / kPieces, piece = q % kPieces;
             const int64_t k0 = static_cast<int64_t>(win) * (WT * 128) + piece * 8;
             uint32_t off = static_cast<uint32_t>(row) * static_cast<uint32_t>(p.k) * 2u + static_cast<uint32_t>(piece * 16);
-            if (row >= p.m || k0 >= p.k) off = kOutOfRange;       // K is a multiple of 8: a piece is all inside or all outside
+            if (row >= p.m || k0 >= p.k || !filler) off = kOutOfRange;       // K is a multiple of 8: a piece is all inside or all outside
             dst[i] = load16(srd_a, off, static_cast<uint32_t>(win) * (WT * 256u));
         }
     };
     auto load_window = [&](int win) { load_window_into(wa, win); };
     auto store_window_from = [&](const uint4* src, int buf) {
+        if (!filler) return;
 #pragma unroll
         for (int i = 0; i < NW; ++i) {
             const int q = t + 512 * i;
@@ -819,10 +827,10 @@ void decode_wide_kernel(PackedParams p)
 
     if constexpr (PAIR) {
         // every window has been read (the loop ends on a barrier): the up half leaves its totals where the windows were
-        float* up_totals = reinterpret_cast<float*>(smem);            // [kTileWaves][4][64]
+        float* up_totals = reinterpret_cast<float*>(smem);            // [tile_waves][4][64]
         if (second) {
 #pragma unroll
-            for (int r = 0; r < 4; ++r) up_totals[((wave - kTileWaves) * 4 + r) * 64 + lane] = y[0][r];
+            for (int r = 0; r < 4; ++r) up_totals[((wave - tile_waves) * 4 + r) * 64 + lane] = y[0][r];
         }
         __syncthreads();
         const int64_t col = n_base + c;
@@ -861,16 +869,31 @@ static int launch_wide_bs(const PackedParams& p, int bs, hipStream_t stream)
 {
     const int64_t col_groups = (p.n + 15) / 16;
     const bool pair = p.packed_up != nullptr;
-    // a paired launch holds four column groups of each projection per workgroup; which build runs is decided as for a launch
-    // of one projection alone (the builds differ in how offset and zero point leave the accumulator, so in the last bits)
-    const dim3 grid(static_cast<unsigned>(pair ? (col_groups + kWideWaves / 2 - 1) / (kWideWaves / 2) : (col_groups + kWideWaves - 1) / kWideWaves));
+    // Waves (= column groups) per workgroup: eight, unless that leaves the grid between one and one and a half workgroups
+    // per CU - then some CUs run two workgroups while the others run one, and the launch lasts as long as the doubly
+    // loaded ones (3584 -> 37888: 296 workgroups on 256 CUs, 22.6 us; with ten waves, 237 workgroups, 19.2 us at 8 rows).
+    // Such a launch takes as many waves as spread its column groups over one workgroup per CU, up to twelve. (Larger
+    // workgroups lose where the grid is several times the CUs: 3584 -> 152064 65 -> 80 us with ten.) A paired launch holds
+    // half of its waves' column groups from each projection.
+    constexpr int64_t kCus = 256;
+    const int64_t all_groups = pair ? 2 * col_groups : col_groups;
+    int ww = kWideWaves;
+    if (p.m <= 16 && bs == 128 && sizeof(ST) == 2 && all_groups > kCus * kWideWaves && all_groups <= kCus * kWideWavesMax) {   // (the builds compiled for up to twelve waves)
+        ww = static_cast<int>((all_groups + kCus - 1) / kCus);
+        if (pair && (ww & 1)) ++ww;
+        if (ww > kWideWavesMax) ww = kWideWaves;
+    }
+    const int per_wg = pair ? ww / 2 : ww;
+    // which build runs is decided as for a launch of one projection alone (the builds differ in how offset and zero point
+    // leave the accumulator, so in the last bits)
+    const dim3 grid(static_cast<unsigned>((col_groups + per_wg - 1) / per_wg));
     const unsigned alone = static_cast<unsigned>((col_groups + kWideWaves - 1) / kWideWaves);
     auto go = [&](auto kernel, size_t lds) {
         if (lds > 65536) {
             const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
             if (e != hipSuccess) return static_cast<int>(e);
         }
-        hipLaunchKernelGGL(kernel, grid, dim3(kWideWaves * 64), lds, stream, p);
+        hipLaunchKernelGGL(kernel, grid, dim3(ww * 64), lds, stream, p);
         return static_cast<int>(hipGetLastError());
     };
     auto by_rows = [&](auto bs_tag) {
@@ -879,6 +902,18 @@ static int launch_wide_bs(const PackedParams& p, int bs, hipStream_t stream)
         constexpr int NBT = 128 / BS;
         constexpr size_t lds16 = 2 * 16 * (4 * 256 + 16), sums16 = 2 * 4 * NBT * 16 * 4;
         if (p.m <= 16) {
+            if (ww > kWideWaves) {
+                // a balanced grid has at most one workgroup per CU: the builds for few workgroups, compiled for twelve waves
+                if constexpr (BS == 128 && sizeof(ST) == 2) {
+                    if (pair) {
+                        if (grid.x < 256) return go(decode_wide_kernel<BF16, BS, ST, 1, true, true, true, true, kWideWavesMax>, lds16 + sums16);
+                        return go(decode_wide_kernel<BF16, BS, ST, 1, true, false, false, true, kWideWavesMax>, lds16 + sums16);
+                    }
+                    if (grid.x < 256) return go(decode_wide_kernel<BF16, BS, ST, 1, true, true, true, false, kWideWavesMax>, lds16 + sums16);
+                    return go(decode_wide_kernel<BF16, BS, ST, 1, true, false, false, false, kWideWavesMax>, lds16 + sums16);
+                }
+                return -1;
+            }
             if (pair) {
                 // the sums build unless a projection alone would run the other one; prefetch as the pair's own grid wants it
                 if (alone >= 768) return go(decode_wide_kernel<BF16, BS, ST, 1, false, false, true, true>, lds16);
