@@ -609,10 +609,10 @@ constexpr int kWideWavesMax = 12;    // (a launch picks the count that spreads i
 // WMAX: the most waves a workgroup of this build may have (8, or 12 for the builds that balanced grids launch).
 template <bool BF16, int BS, typename ST, int RB, bool SUMS, bool PF, bool DEEP, bool PAIR = false, int WMAX = kWideWaves>
 __global__ __launch_bounds__(WMAX * 64)
-__attribute__((amdgpu_waves_per_eu((BS == 128 && sizeof(ST) == 2 && RB == 1) ? (PF ? (SUMS ? 3 : 4) : SUMS ? (DEEP || WMAX > kWideWaves ? 4 : 5) : (DEEP ? 5 : 6)) : 1)))
+__attribute__((amdgpu_waves_per_eu((BS == 128 && sizeof(ST) == 2 && RB == 1) ? (PF ? (SUMS ? 3 : 4) : SUMS ? (DEEP || WMAX > kWideWaves ? 4 : 5) : (DEEP ? 5 : 6)) : (WMAX > kWideWaves ? 3 : 1))))
 void decode_wide_kernel(PackedParams p)
 {
-    static_assert(WMAX == kWideWaves || (WMAX == kWideWavesMax && RB == 1 && SUMS), "twelve waves: the one-block sums builds only");
+    static_assert(WMAX == kWideWaves || (WMAX == kWideWavesMax && RB == 1), "twelve waves: the one-block builds only");
     static_assert(DEEP || !PF, "weights ahead only together with deep windows");
     static_assert(!PAIR || RB == 1, "the paired form takes up to 16 rows");
     // column groups per workgroup (and projection): one per wave. The first eight waves also fill the windows.
@@ -869,25 +869,34 @@ static int launch_wide_bs(const PackedParams& p, int bs, hipStream_t stream)
 {
     const int64_t col_groups = (p.n + 15) / 16;
     const bool pair = p.packed_up != nullptr;
-    // Waves (= column groups) per workgroup: eight, unless that leaves the grid between one and one and a half workgroups
-    // per CU - then some CUs run two workgroups while the others run one, and the launch lasts as long as the doubly
-    // loaded ones (3584 -> 37888: 296 workgroups on 256 CUs, 22.6 us; with ten waves, 237 workgroups, 19.2 us at 8 rows).
-    // Such a launch takes as many waves as spread its column groups over one workgroup per CU, up to twelve. (Larger
-    // workgroups lose where the grid is several times the CUs: 3584 -> 152064 65 -> 80 us with ten.) A paired launch holds
-    // half of its waves' column groups from each projection.
     constexpr int64_t kCus = 256;
     const int64_t all_groups = pair ? 2 * col_groups : col_groups;
+    // A grid between one and one and a half workgroups of eight waves per CU (3584 -> 37888: 296 workgroups on 256 CUs)
+    // leaves some CUs with two workgroups while the others run one, and the launch lasts as long as the doubly loaded ones.
+    const bool in_between = all_groups > kCus * kWideWaves && all_groups <= kCus * kWideWavesMax;
+    const unsigned alone = static_cast<unsigned>((col_groups + kWideWaves - 1) / kWideWaves);
+    // How offset and zero point leave the accumulator (it shows in the last bits, so it is decided as for a launch of one
+    // projection alone, and a pair follows its projections). Through the block activation sums, except:
+    //  * grids of three or more workgroups per CU (3584 -> 152064 at 16 rows: 59 against 64 us);
+    //  * block size 32: the sums build takes 185-196 registers there, one workgroup per CU, and a grid above 256
+    //    workgroups runs in two rounds (3584 -> 37888 at 8 rows: 37.8 us; the second-MFMA build with the next group's
+    //    weights in flight 26.2, 4096 -> 14336 21.6 -> 17.2, 4096 -> 28672 24.0 -> 20.2);
+    //  * block size 64 where a launch of the projection gets a balanced grid (below): the sums build with weights ahead
+    //    takes 218 registers, too many for more than eight waves a workgroup.
+    const bool sums = alone < 768 && bs != 32 && !(bs == 64 && sizeof(ST) == 2 && col_groups > kCus * kWideWaves && col_groups <= kCus * kWideWavesMax);
+    // Waves (= column groups) per workgroup: eight, unless the grid is in between and a build for more waves exists - then
+    // as many as spread the column groups over one workgroup per CU, up to twelve (3584 -> 37888 at block 128: ten waves,
+    // 237 workgroups, 22.6 -> 18.0 us at 8 rows; at block 64 23.7 -> 21.2). Larger workgroups lose where the grid is several
+    // times the CUs (3584 -> 152064 65 -> 80 us with ten). A paired launch holds half of its waves' column groups from each
+    // projection. The builds for twelve waves: block 128 with the sums, block 64 without (16-bit scales).
     int ww = kWideWaves;
-    if (p.m <= 16 && bs == 128 && sizeof(ST) == 2 && all_groups > kCus * kWideWaves && all_groups <= kCus * kWideWavesMax) {   // (the builds compiled for up to twelve waves)
+    if (p.m <= 16 && sizeof(ST) == 2 && in_between && ((bs == 128 && sums) || (bs == 64 && !sums && !pair))) {
         ww = static_cast<int>((all_groups + kCus - 1) / kCus);
         if (pair && (ww & 1)) ++ww;
         if (ww > kWideWavesMax) ww = kWideWaves;
     }
     const int per_wg = pair ? ww / 2 : ww;
-    // which build runs is decided as for a launch of one projection alone (the builds differ in how offset and zero point
-    // leave the accumulator, so in the last bits)
     const dim3 grid(static_cast<unsigned>((col_groups + per_wg - 1) / per_wg));
-    const unsigned alone = static_cast<unsigned>((col_groups + kWideWaves - 1) / kWideWaves);
     auto go = [&](auto kernel, size_t lds) {
         if (lds > 65536) {
             const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
@@ -901,37 +910,35 @@ static int launch_wide_bs(const PackedParams& p, int bs, hipStream_t stream)
         // two window buffers of rows x (tiles x 256 + 16) bytes, then two tables of (blocks per window) x rows f32 sums
         constexpr int NBT = 128 / BS;
         constexpr size_t lds16 = 2 * 16 * (4 * 256 + 16), sums16 = 2 * 4 * NBT * 16 * 4;
-        if (p.m <= 16) {
+        // up to 16 rows, PAIR or not: the build by grid size. Measured at 8 / 16 rows (3584 -> 152064, 3584 -> 37888,
+        // 4096 -> 16384): three or more workgroups per CU run best with the windows two ahead (68 -> 64 us); fewer
+        // workgroups than CUs with weights and windows both ahead (17.2 -> 14.5 us); in between neither helps the sums build
+        // (20.6 us either way; with both ahead it spills at block size 32).
+        auto upto16 = [&](auto pair_tag) {
+            constexpr bool P = decltype(pair_tag)::value;
             if (ww > kWideWaves) {
                 // a balanced grid has at most one workgroup per CU: the builds for few workgroups, compiled for twelve waves
                 if constexpr (BS == 128 && sizeof(ST) == 2) {
-                    if (pair) {
-                        if (grid.x < 256) return go(decode_wide_kernel<BF16, BS, ST, 1, true, true, true, true, kWideWavesMax>, lds16 + sums16);
-                        return go(decode_wide_kernel<BF16, BS, ST, 1, true, false, false, true, kWideWavesMax>, lds16 + sums16);
-                    }
-                    if (grid.x < 256) return go(decode_wide_kernel<BF16, BS, ST, 1, true, true, true, false, kWideWavesMax>, lds16 + sums16);
-                    return go(decode_wide_kernel<BF16, BS, ST, 1, true, false, false, false, kWideWavesMax>, lds16 + sums16);
+                    if (grid.x < 256) return go(decode_wide_kernel<BF16, BS, ST, 1, true, true, true, P, kWideWavesMax>, lds16 + sums16);
+                    return go(decode_wide_kernel<BF16, BS, ST, 1, true, false, false, P, kWideWavesMax>, lds16 + sums16);
+                } else if constexpr (BS == 64 && sizeof(ST) == 2 && !P) {
+                    return go(decode_wide_kernel<BF16, BS, ST, 1, false, true, true, false, kWideWavesMax>, lds16);
+                } else {
+                    return -1;
                 }
-                return -1;
             }
-            if (pair) {
-                // the sums build unless a projection alone would run the other one; prefetch as the pair's own grid wants it
-                if (alone >= 768) return go(decode_wide_kernel<BF16, BS, ST, 1, false, false, true, true>, lds16);
-                if constexpr (BS != 32) {
-                    if (grid.x < 256) return go(decode_wide_kernel<BF16, BS, ST, 1, true, true, true, true>, lds16 + sums16);
-                }
-                return go(decode_wide_kernel<BF16, BS, ST, 1, true, false, false, true>, lds16 + sums16);
+            if (!sums) {
+                if (alone >= 768 && bs != 32) return go(decode_wide_kernel<BF16, BS, ST, 1, false, false, true, P>, lds16);
+                return go(decode_wide_kernel<BF16, BS, ST, 1, false, true, true, P>, lds16);
             }
-            // Measured at 8 / 16 rows (3584 -> 152064, 3584 -> 37888, 4096 -> 16384): three or more workgroups per CU run
-            // best without the sums and with the windows two ahead (68 -> 64 us); fewer workgroups than CUs with weights
-            // and windows both ahead (17.2 -> 14.5 us); in between neither helps (20.6 us either way).
-            if (grid.x >= 768) return go(decode_wide_kernel<BF16, BS, ST, 1, false, false, true>, lds16);
-            // (block size 32 carries four times the scales per window: with both ahead it spills)
             if constexpr (BS != 32) {
-                if (grid.x < 256) return go(decode_wide_kernel<BF16, BS, ST, 1, true, true, true>, lds16 + sums16);
+                if (grid.x < 256) return go(decode_wide_kernel<BF16, BS, ST, 1, true, true, true, P>, lds16 + sums16);
+                return go(decode_wide_kernel<BF16, BS, ST, 1, true, false, false, P>, lds16 + sums16);
+            } else {
+                return -1;                                 // (block size 32 never takes the sums)
             }
-            return go(decode_wide_kernel<BF16, BS, ST, 1, true, false, false>, lds16 + sums16);
-        }
+        };
+        if (p.m <= 16) return pair ? upto16(std::true_type{}) : upto16(std::false_type{});
         if (pair) return -1;                               // the paired form takes up to 16 rows
         // More row blocks per wave only where they fit the register file: two from block size 64, four at 128. The
         // spilling forms ran several times slower than the routes that take those calls instead (3584 -> 37888: 153 us

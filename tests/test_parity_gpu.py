@@ -209,6 +209,10 @@ DECODE_CASES = [
     (E.BF16, E.BF16, 128, True, 16, 14336, 1024),       # the narrowest shape the shared-activation kernel takes (fewer workgroups than CUs)
     (E.F16, E.F16, 64, True, 11, 14400, 512),
     (E.F16, E.F16, 32, True, 9, 14336, 512),
+    (E.BF16, E.BF16, 64, True, 8, 37888, 1024 + 64),    # block 64, between one and 1.5 workgroups per CU: ten waves a workgroup, second-MFMA build with weights ahead
+    (E.F16, E.F16, 64, True, 16, 32784, 512),           # the same with nine waves and a ragged last workgroup
+    (E.F16, E.F16, 32, True, 12, 37888, 512),           # block 32 never takes the sums build (here: 296 workgroups of eight waves)
+    (E.BF16, E.F32, 32, True, 7, 20000, 32 * 19),       # ... nor with f32 scales; a partial last tile group
     (E.BF16, E.BF16, 128, True, 17, 16400, 3584),       # up to 64 rows ride on one pass over the weights
     (E.F16, E.F16, 64, True, 40, 16384, 1024 + 64),     # block size 64 stops at 32 rows per pass: the tiled kernel takes this one
     (E.F16, E.F16, 64, True, 25, 16384, 1024 + 64),
@@ -839,6 +843,8 @@ def test_gate_up_swiglu_single_launch(ep, port, a_dt, s_dt, bs, zero_points, m, 
     (E.F16, E.F16, 64, 9, 14400, 640, False),         # ragged: the last workgroup's waves run out of column groups
     (E.F16, E.F32, 32, 16, 14336, 256, False),
     (E.BF16, E.BF16, 128, 8, 98400, 256, False),      # three or more workgroups per CU: the build with the second MFMA
+    (E.BF16, E.BF16, 32, 6, 18944, 512, False),       # block 32: the second-MFMA build with weights ahead, in both projections and in the pair
+    (E.F16, E.F16, 64, 8, 37888, 256, True),          # block 64 where one projection alone gets a balanced grid (second MFMA): the pair follows it
 ])
 def test_gate_up_swiglu_single_launch_at_5_to_16_rows(ep, port, a_dt, s_dt, bs, m, n, k, decomposed):
     """5 to 16 rows where both projections are wide enough for the shared-activation kernel: from the second call on one
