@@ -1475,6 +1475,11 @@ static int launch_decode_packed(const RocmMatMulNBitsArgs* a, const void* packed
     const int gpw = (p.groups + w - 1) / w;
     w = (p.groups + gpw - 1) / gpw;
     p.groups_per_wave = gpw;
+    // Two to four rows with one group per wave: the second register set has nothing to fetch ahead and only costs waves
+    // per SIMD, which shows once the grid is a few workgroups per CU (4 rows, one set against two: 4096 -> 14336 10.5 ->
+    // 9.6 us at block 128, 11.4 -> 10.6 at 64, 15.3 -> 11.6 at 32; 3584 -> 4608 at block 32 7.9 -> 6.7). Smaller grids keep
+    // the two-set build, whose first fetch is issued before anything else (3584 -> 4608 at block 128: 5.56 against 5.72 us).
+    if (!one_row && gpw == 1 && wgs >= (a->block_size == 32 ? 256 : 640)) single_set = true;
     // a paired launch keeps each projection's own split of K (so that it adds up in the same order) and needs twice the waves
     if (probe_only) return a->m <= 4 && 2 * w <= w_max ? 1 : 0;
     if (packed_up && (a->m > 4 || 2 * w > w_max)) return -1;
@@ -1567,6 +1572,9 @@ extern "C" int rocm_launch_acc4_packed(const RocmMatMulNBitsArgs* a, const void*
     const int gpw = (p.groups + w - 1) / w;
     w = (p.groups + gpw - 1) / gpw;
     p.groups_per_wave = gpw;
+    // one group per wave: a second register set has nothing to fetch ahead (one row, 4096 -> 14336: 14.3 -> 9.8 us at block
+    // 32, 9.7 -> 8.8 at 64, 9.2 -> 8.4 at 128; never slower on the smaller grids)
+    if (gpw == 1) single_set = true;
 
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool f32_scales = a->scale_dtype == ROCM_DT_F32;
