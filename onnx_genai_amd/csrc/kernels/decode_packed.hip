@@ -1396,6 +1396,12 @@ extern "C" int rocm_decode_packed_fuses_norm(const RocmMatMulNBitsArgs* a)
     return (reinterpret_cast<uintptr_t>(a->gamma) & 15) == 0;
 }
 
+// the most waves a workgroup of decode_packed_kernel may have (see the kernel's launch bounds)
+static int w_max_of(const RocmMatMulNBitsArgs* a, bool f32_scales)
+{
+    return (a->block_size == 128 && !f32_scales && (a->m <= 4 || a->a_dtype == ROCM_DT_BF16)) ? 16 : 8;
+}
+
 static int launch_decode_packed(const RocmMatMulNBitsArgs* a, const void* packed, const void* packed_up, int decomposed, int waves, bool probe_only,
                                 bool pair_member, rocm_stream_t stream)
 {
@@ -1468,8 +1474,11 @@ static int launch_decode_packed(const RocmMatMulNBitsArgs* a, const void* packed
     } else {
         single_set = wgs * w >= 6144;
     }
-    if (one_row) single_set = true;
-    const int w_max = (a->block_size == 128 && !f32_scales && (a->m <= 4 || a->a_dtype == ROCM_DT_BF16)) ? 16 : 8;      // see the kernel's launch bounds
+    // (block size 32 with several groups per wave: sixteen scale steps per group leave enough arithmetic between a wave's
+    // loads that fetching the next group ahead pays - 18944 -> 3584 12.4 -> 11.8 us, 14336 -> 4096 10.9 -> 10.6; at block
+    // 128 the one-set build stays ahead, 9.5 against 9.9 us)
+    if (one_row) single_set = !(a->block_size == 32 && p.groups > w_max_of(a, f32_scales));
+    const int w_max = w_max_of(a, f32_scales);
     if (w > w_max) w = w_max;
     if (w > p.groups) w = p.groups;
     const int gpw = (p.groups + w - 1) / w;
