@@ -608,13 +608,14 @@ ROW_SWEEP_SHAPES = (   # block size, K, N, accuracy_level
 
 def row_sweep(ep):
     """Time per call against the row count M, bf16 with zero points, on the default dispatch: each step in the table should
-    cost no more than the rows it adds (a step that does marks a kernel boundary placed at the wrong M). Two copies of the
-    weights per graph, replayed after a warm-up."""
+    cost no more than the rows it adds (a step that does marks a kernel boundary placed at the wrong M). Per graph four
+    copies of the weights up to 64 rows (with two, the graph's own launch cost shows in a 10 us call and the figures
+    scatter by 10-30 %), two above; replayed after a warm-up."""
     out = []
     for bs, k, n, acc in ROW_SWEEP_SHAPES:
         shape_rows = []
         for m in reversed(ROW_SWEEP_ROWS):      # tallest first: the short calls then follow light work, not 2048-row GEMMs
-            nodes = [Node(ep, f"w{i}", k, n, bs, i, E.BF16, m, accuracy_level=acc) for i in range(2)]
+            nodes = [Node(ep, f"w{i}", k, n, bs, i, E.BF16, m, accuracy_level=acc) for i in range(4 if m <= 64 else 2)]
             a = ep.upload(synth.make_activation(m, k, 5, E.BF16))
             for nd in nodes:
                 nd.run(a)

@@ -668,7 +668,7 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
             }
         }
     } else if (M <= 64 && use_packed(kn, args, rc)) {
-        if (rc == 0) rc = (kn.pair_member && M <= 4) ? rocm_launch_decode_packed_pair_member(&args, kn.packed, kn.ep->decode_waves, stream)
+        if (rc == 0) rc = (kn.pair_member && M <= 16) ? rocm_launch_decode_packed_pair_member(&args, kn.packed, kn.ep->decode_waves, stream)
                                                       : rocm_launch_decode_packed(&args, kn.packed, kn.ep->decode_waves, stream);
         kn.variant = "decode_mfma_packed";
     } else if (M <= 16 && rocm_decode_mfma_eligible(&args)) {

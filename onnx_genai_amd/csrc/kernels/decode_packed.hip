@@ -1337,15 +1337,21 @@ static int packed_chunk_bytes(const RocmMatMulNBitsArgs* a)
 
 // Rows 5..64 only run from the repacked copy in the shared-activation kernel, which wants many column groups.
 // (16 rows at block size 32, 32 at 64, 64 at 128: more row blocks than that do not fit the register file)
-static bool wide_shape(const RocmMatMulNBitsArgs* a)
+// `pair`: the call is the fused gate/up launch or one of its two projections - both projections' columns count, since the
+// paired launch streams both, and a projection launched on its own must add up the way the paired launch does.
+static bool wide_shape(const RocmMatMulNBitsArgs* a, bool pair)
 {
     const int64_t max_rows = a->block_size == 32 ? 16 : a->block_size == 64 ? 32 : 64;
-    // Columns from which it beats the split-K and tiled kernels (bf16, 4096 -> 14336: 19.9 -> 14.6 us at 16 rows and
-    // 30.6 -> 24.4 at 32 with block 128, 20-24 -> 16 and 31.5 -> 25.7 with block 64; at 12288 columns it ties at 16 rows
-    // and loses 2 us at 5-8; at 9216 and below it loses throughout, and so do 33-64 rows below 16384 columns:
-    // 32.9 -> 38.7 us). Block size 32: 20.7 -> 20.3 us at 5-8 rows, 26.1 -> 20.4 at 16 (one pass of 16 rows is all it takes).
-    const int64_t min_cols = a->m > 32 ? 16384 : 14336;
-    return a->m >= 5 && a->m <= max_rows && a->n >= min_cols;
+    // Columns from which it beats the other kernels. 17 rows and more (against the tiled kernel and two passes of the
+    // split-K kernel; bf16, 4096 -> 14336: 30.6 -> 24.4 us at 32 rows with block 128, 31.5 -> 25.7 with block 64; 33-64 rows
+    // lose below 16384 columns: 32.9 -> 38.7 us). Up to 16 rows the 16-row split-K kernel over the same repacked stream is
+    // the alternative, and with 4096 rows of K it stays ahead up to 16384 columns at block 128 (5 / 8 / 16 rows, 14336
+    // columns: 12.0 / 12.1 / 13.8 against 13.2 / 13.3 / 14.2 us; 16384: 12.5 / 12.8 / 14.4 against 13.4 / 13.5 / 14.5; at 20480
+    // it loses, 14.9-17.3 against 14.1-15.3) and up to 20480 at block 32 (14336: 13.2 / 13.2 / 14.7 against 17.1 / 17.2 / 17.7;
+    // 20480: 16.9 / 17.2 / 18.6 against 17.8 / 17.9 / 18.4; at 28672 it loses, 22-25 against 20-21).
+    // (block 64: 12.3 / 12.6 / 14.4 us at 14336 and 13.2 / 13.7 / 15.2 at 16384 against 15.4-16.0 in the shared-activation kernel)
+    const int64_t min_cols = a->m > 32 ? 16384 : a->m > 16 ? 14336 : a->block_size == 32 ? 22528 : a->block_size == 64 ? 20480 : 18432;
+    return a->m >= 5 && a->m <= max_rows && a->n * (pair ? 2 : 1) >= min_cols;
 }
 
 extern "C" int rocm_decode_packed_eligible(const RocmMatMulNBitsArgs* a)
@@ -1354,7 +1360,7 @@ extern "C" int rocm_decode_packed_eligible(const RocmMatMulNBitsArgs* a)
     if (base.m > 16) base.m = 16;                         // the shared-activation kernel takes up to 64 rows
     if (!rocm_decode_mfma_eligible(&base)) return 0;
     if (a->m * a->k * 2 >= 0x7ffffff0) return 0;
-    if (a->m > 16 && !wide_shape(a)) return 0;           // up to 16 rows the split-K kernel stages the rows per wave
+    if (a->m > 16 && !wide_shape(a, false)) return 0;    // up to 16 rows the split-K kernel stages the rows per wave
     return static_cast<int64_t>(mnb::packed_groups(a)) * mnb::packed_chunk_bytes(a) < 0x7fffffff;
 }
 
@@ -1391,7 +1397,7 @@ extern "C" int rocm_launch_pack_decode(const RocmMatMulNBitsArgs* a, void* packe
 // for the pair's column groups together, so that the separate launches and the paired one add up in the same order.
 extern "C" int rocm_decode_packed_fuses_norm(const RocmMatMulNBitsArgs* a)
 {
-    if (!a->gamma || a->m > 4 || a->k % 128 != 0 || wide_shape(a) || !rocm_decode_packed_eligible(a)) return 0;
+    if (!a->gamma || a->m > 4 || a->k % 128 != 0 || !rocm_decode_packed_eligible(a)) return 0;      // (up to four rows: never the shared-activation kernel)
     if (a->gamma_dtype != ROCM_DT_F32 && a->gamma_dtype != a->a_dtype) return 0;
     return (reinterpret_cast<uintptr_t>(a->gamma) & 15) == 0;
 }
@@ -1436,7 +1442,7 @@ static int launch_decode_packed(const RocmMatMulNBitsArgs* a, const void* packed
 
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool f32_scales = a->scale_dtype == ROCM_DT_F32;
-    if (wide_shape(a)) {
+    if (wide_shape(a, pair_member)) {
         // the shared-activation kernel's paired form takes up to 16 rows (one block of rows per wave)
         if (probe_only) return a->m <= 16 ? 1 : 0;
         if (packed_up && a->m > 16) return -1;
@@ -1448,7 +1454,7 @@ static int launch_decode_packed(const RocmMatMulNBitsArgs* a, const void* packed
     // Waves per workgroup. Many column groups (thousands of waves even at four per group): short waves of at most two
     // tile groups and no prefetch, so that eight of them fit a SIMD and cover each other's memory latency. Few column
     // groups: enough waves per group to reach about 8k in flight, each prefetching its next group.
-    const int64_t wgs = (a->n + 15) / 16 * (pair_member ? 2 : 1);
+    const int64_t wgs = (a->n + 15) / 16 * ((pair_member && a->m <= 4) ? 2 : 1);      // (a pair shares a launch up to four rows here)
     int w = waves;
     bool single_set = wgs * 4 >= 6144;
     // One row: one tile group per wave where
