@@ -542,7 +542,7 @@ static int launch_packed_cfg(const PackedParams& p, int waves, hipStream_t strea
             return static_cast<int>(hipGetLastError());
         }
     }
-    if constexpr (MR == 16) {
+    if constexpr (MR >= 8) {
         // sixteen staged rows of sixteen waves outgrow the 64 KiB a kernel gets without asking
         if (lds > 65536) {
             const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(decode_packed_kernel<BF16, BS, MR, ST, SETS, false>),
@@ -562,7 +562,9 @@ static int launch_packed_mr(const PackedParams& p, int waves, bool single_set, h
 {
     if (p.m <= 1) return single_set ? launch_packed_cfg<BF16, BS, 1, ST, 1>(p, waves, stream) : launch_packed_cfg<BF16, BS, 1, ST, 2>(p, waves, stream);
     if (p.m <= 4) return (single_set || p.gamma) ? launch_packed_cfg<BF16, BS, 4, ST, 1>(p, waves, stream) : launch_packed_cfg<BF16, BS, 4, ST, 2>(p, waves, stream);
-    // 5 .. 16 rows: one register set (64 registers of activations per group; a second set in flight measured slower)
+    // 5 .. 16 rows: one register set (64 registers of activations per group at 16 rows; a second set in flight measured
+    // slower). Up to 8 rows a build that stages eight: half the activation bytes per wave and group.
+    if (p.m <= 8) return launch_packed_cfg<BF16, BS, 8, ST, 1>(p, waves, stream);
     return launch_packed_cfg<BF16, BS, 16, ST, 1>(p, waves, stream);
 }
 
@@ -1405,7 +1407,7 @@ extern "C" int rocm_decode_packed_fuses_norm(const RocmMatMulNBitsArgs* a)
 // the most waves a workgroup of decode_packed_kernel may have (see the kernel's launch bounds)
 static int w_max_of(const RocmMatMulNBitsArgs* a, bool f32_scales)
 {
-    return (a->block_size == 128 && !f32_scales && (a->m <= 4 || a->a_dtype == ROCM_DT_BF16)) ? 16 : 8;
+    return (a->block_size == 128 && !f32_scales && (a->m <= 8 || a->a_dtype == ROCM_DT_BF16)) ? 16 : 8;
 }
 
 static int launch_decode_packed(const RocmMatMulNBitsArgs* a, const void* packed, const void* packed_up, int decomposed, int waves, bool probe_only,
