@@ -1489,6 +1489,16 @@ static int launch_decode_packed(const RocmMatMulNBitsArgs* a, const void* packed
     const int w_max = w_max_of(a, f32_scales);
     if (w > w_max) w = w_max;
     if (w > p.groups) w = p.groups;
+    if (a->m > 4 && waves <= 0 && w != 8) {
+        // 5 .. 16 rows: these builds hold three to five waves per SIMD. A launch whose waves do not all fit the chip at once
+        // queues workgroups behind each other, and workgroups of 6, 10 or 12 waves leave slots of a CU empty on top; fewer
+        // waves of more groups each run it faster (16 rows, block 128: 3072 -> 16384 13.8 -> 12.2 us, 5120 -> 13824 21.0 -> 17.6,
+        // 6144 -> 16384 24.6 -> 21.1, 5120 -> 17920 24.1 -> 21.7; 8 rows: 16.2 -> 13.9 on 5120 -> 13824). Workgroups of eight waves
+        // fill a CU's slots exactly and stay (K = 4096: 14336 columns 13.9 against 14.9 us with four waves, 11008 11.3 against 11.6).
+        const int per_simd = a->m <= 8 ? (a->block_size == 32 ? 4 : 5) : (f32_scales ? 3 : 4);
+        const int64_t fit = 256 * 4 * per_simd / wgs;
+        if (fit >= 1 && w > fit) w = static_cast<int>(fit);
+    }
     const int gpw = (p.groups + w - 1) / w;
     w = (p.groups + gpw - 1) / gpw;
     p.groups_per_wave = gpw;
