@@ -1404,6 +1404,17 @@ extern "C" int rocm_decode_packed_fuses_norm(const RocmMatMulNBitsArgs* a)
     return (reinterpret_cast<uintptr_t>(a->gamma) & 15) == 0;
 }
 
+// waves per SIMD of the one-set builds (from their register counts: 59-76 registers with one row, 71-102 with four, 84-112
+// with eight, 110-134 with sixteen)
+static int waves_per_simd(const RocmMatMulNBitsArgs* a, bool f32_scales)
+{
+    const int bs = a->block_size;
+    if (a->m <= 1) return bs == 128 ? 8 : bs == 64 ? (f32_scales ? 7 : 8) : (f32_scales ? 6 : 7);
+    if (a->m <= 4) return bs == 128 ? (f32_scales ? 6 : 7) : bs == 64 ? 6 : (f32_scales ? 4 : 5);
+    if (a->m <= 8) return bs == 32 ? 4 : 5;
+    return f32_scales ? 3 : 4;
+}
+
 // the most waves a workgroup of decode_packed_kernel may have (see the kernel's launch bounds)
 static int w_max_of(const RocmMatMulNBitsArgs* a, bool f32_scales)
 {
@@ -1458,55 +1469,77 @@ static int launch_decode_packed(const RocmMatMulNBitsArgs* a, const void* packed
     // groups: enough waves per group to reach about 8k in flight, each prefetching its next group.
     const int64_t wgs = (a->n + 15) / 16 * ((pair_member && a->m <= 4) ? 2 : 1);      // (a pair shares a launch up to four rows here)
     int w = waves;
-    bool single_set = wgs * 4 >= 6144;
-    // One row: one tile group per wave where
-    // the workgroup can hold that many waves, no prefetch, offset and zero point through the activation sums. Every byte
-    // of the call is then requested as soon as its wave starts, and what a wave computes between its loads and the
-    // reduction is the least any variant here does. Measured against the few-wave prefetching build it replaced on the
-    // small shapes (bf16, block 128): 3584 -> 4608 5.06 -> 4.78 us, 3584 -> 3584 4.17 -> 3.97, 18944 -> 3584 9.94 -> 9.41,
-    // 3584 -> 37888 15.81 -> 15.48.
+    const int w_max = w_max_of(a, f32_scales);
+    // One row: one tile group per wave where the workgroup can hold that many waves, no prefetch, offset and zero point
+    // through the activation sums. Every byte of the call is then requested as soon as its wave starts, and what a wave
+    // computes between its loads and the reduction is the least any variant here does. Measured against the few-wave
+    // prefetching build it replaced on the small shapes (bf16, block 128): 3584 -> 4608 5.06 -> 4.78 us, 3584 -> 3584
+    // 4.17 -> 3.97, 18944 -> 3584 9.94 -> 9.41, 3584 -> 37888 15.81 -> 15.48.
     // (a gate/up pair keeps the few-wave split: with fourteen waves a workgroup the paired launch measured 17.8 us against 15.5)
     const bool one_row = a->m <= 1 && !pair_member;
-    if (one_row && w <= 0) {
-        single_set = true;
-        w = p.groups;
-    } else
+    const bool large_grid = wgs * 4 >= 6144;
     if (w <= 0) {
-        if (single_set) {
+        if (one_row) {
+            w = p.groups;
+        } else if (large_grid) {
             w = (p.groups + 1) / 2;
         } else {
             const int want = static_cast<int>((8192 + wgs - 1) / wgs);
             w = want < p.groups ? want : p.groups;               // at least one group per wave
         }
         if (w < 1) w = 1;
-    } else {
-        single_set = wgs * w >= 6144;
     }
-    // (block size 32 with several groups per wave: sixteen scale steps per group leave enough arithmetic between a wave's
-    // loads that fetching the next group ahead pays - 18944 -> 3584 12.4 -> 11.8 us, 14336 -> 4096 10.9 -> 10.6; at block
-    // 128 the one-set build stays ahead, 9.5 against 9.9 us)
-    if (one_row) single_set = !(a->block_size == 32 && p.groups > w_max_of(a, f32_scales));
-    const int w_max = w_max_of(a, f32_scales);
+    // One register set or two (the second holds the next group's loads while the current one is multiplied, at the price
+    // of waves per SIMD). Swept over 384 .. 1024 column groups x K = 3584 .. 8192 x 1 / 2 / 4 rows x block 32 / 128: one set is
+    // ahead or level nearly everywhere, by up to 30 % from K = 5120 (block 128, 4 rows, 5120 -> 16384: 12.4 against 16.5 us;
+    // block 32: 15.8 against 21.7). Two sets keep:
+    //  * two to four rows on small grids, where the second set's first fetch, issued before anything else, is worth 1-3 %
+    //    (block 128, 3584 -> 4608: 5.56 against 5.72 us; 18944 -> 3584 at block 32: 13.3 against 13.9) - below 256 column groups at
+    //    block 32, else below 640, or below 320 when K is more than eight groups;
+    //  * one row at block size 32 with more groups than a workgroup has waves, on small grids: sixteen scale steps per group
+    //    leave enough arithmetic between a wave's loads that fetching ahead pays (18944 -> 3584 12.4 -> 11.8 us; with 1024
+    //    column groups it loses, 5120 -> 16384: 17.3 against 12.2; at block 128 one set stays ahead, 9.5 against 9.9 us).
+    bool single_set;
+    if (one_row) single_set = !(a->block_size == 32 && p.groups > w_max && wgs <= 256);
+    else if (a->block_size == 32) single_set = wgs >= 256;
+    else single_set = wgs >= 640 || (wgs >= 320 && p.groups > 8);
     if (w > w_max) w = w_max;
     if (w > p.groups) w = p.groups;
-    if (a->m > 4 && waves <= 0 && w != 8) {
-        // 5 .. 16 rows: these builds hold three to five waves per SIMD. A launch whose waves do not all fit the chip at once
-        // queues workgroups behind each other, and workgroups of 6, 10 or 12 waves leave slots of a CU empty on top; fewer
-        // waves of more groups each run it faster (16 rows, block 128: 3072 -> 16384 13.8 -> 12.2 us, 5120 -> 13824 21.0 -> 17.6,
-        // 6144 -> 16384 24.6 -> 21.1, 5120 -> 17920 24.1 -> 21.7; 8 rows: 16.2 -> 13.9 on 5120 -> 13824). Workgroups of eight waves
-        // fill a CU's slots exactly and stay (K = 4096: 14336 columns 13.9 against 14.9 us with four waves, 11008 11.3 against 11.6).
-        const int per_simd = a->m <= 8 ? (a->block_size == 32 ? 4 : 5) : (f32_scales ? 3 : 4);
+    // Mid-size grids: a launch whose waves do not all fit the chip at once queues workgroups behind each other, and
+    // workgroups of 6, 10 or 12 waves leave slots of a CU empty on top; fewer waves of more groups each run it faster
+    // (16 rows, block 128: 3072 -> 16384 13.8 -> 12.2 us, 5120 -> 13824 21.0 -> 17.6, 6144 -> 16384 24.6 -> 21.1, 5120 -> 17920
+    // 24.1 -> 21.7; 8 rows: 16.2 -> 13.9 on 5120 -> 13824; one row: 7168 -> 16384 16.2 -> 14.3; 4 rows at block 32: 3584 -> 16384
+    // 12.5 -> 11.4). Workgroups of eight waves of one group each fill a CU's slots exactly and stay (K = 4096, 16 rows: 14336
+    // columns 13.9 against 14.9 us with four waves, 11008 11.3 against 11.6), and so do the large grids, whose waves are
+    // short enough for the queue not to show (one row, 3584 -> 37888: seven waves of one group, 15.5 against 15.8 us).
+    // Which of the wave counts that fit: a workgroup's waves go round the four SIMDs, so k workgroups of w waves put
+    // k * ceil(w / 4) of them on the first SIMD, and with three to five waves per SIMD a workgroup of 5, 6 or 10 waves keeps
+    // a CU from filling up (16 rows, 5120 -> 13824: five waves 21.4 us, four 17.5, ten 21.0; 2 rows at block 32, 8192 -> 12288:
+    // six waves 18.9 us, four 16.6). Builds of up to five waves per SIMD take the count that holds the most waves per CU that way.
+    if (waves <= 0 && !(w == 8 && p.groups == 8)) {
+        const int per_simd = waves_per_simd(a, f32_scales);
         const int64_t fit = 256 * 4 * per_simd / wgs;
-        if (fit >= 1 && w > fit) w = static_cast<int>(fit);
+        const int64_t least = a->m <= 1 ? 6 : a->m <= 4 ? 4 : 1;
+        if (fit >= least && w > fit) {
+            w = static_cast<int>(fit);
+            if (per_simd <= 5) {                       // (with six or more waves per SIMD the plain count is as good or better: 4 rows at block 128, 6144 -> 16384: six waves 14.2 us, four 15.4)
+                int best = -1;
+                for (int g = 1; g <= p.groups; ++g) {
+                    const int cand = (p.groups + g - 1) / g;
+                    if (cand > fit) continue;
+                    const int held = per_simd / ((cand + 3) / 4) * cand;
+                    if (held > best) {                 // (ties: the first found, which has the most waves)
+                        best = held;
+                        w = cand;
+                    }
+                    if (cand == 1) break;
+                }
+            }
+        }
     }
     const int gpw = (p.groups + w - 1) / w;
     w = (p.groups + gpw - 1) / gpw;
     p.groups_per_wave = gpw;
-    // Two to four rows with one group per wave: the second register set has nothing to fetch ahead and only costs waves
-    // per SIMD, which shows once the grid is a few workgroups per CU (4 rows, one set against two: 4096 -> 14336 10.5 ->
-    // 9.6 us at block 128, 11.4 -> 10.6 at 64, 15.3 -> 11.6 at 32; 3584 -> 4608 at block 32 7.9 -> 6.7). Smaller grids keep
-    // the two-set build, whose first fetch is issued before anything else (3584 -> 4608 at block 128: 5.56 against 5.72 us).
-    if (!one_row && gpw == 1 && wgs >= (a->block_size == 32 ? 256 : 640)) single_set = true;
     // a paired launch keeps each projection's own split of K (so that it adds up in the same order) and needs twice the waves
     if (probe_only) return a->m <= 4 && 2 * w <= w_max ? 1 : 0;
     if (packed_up && (a->m > 4 || 2 * w > w_max)) return -1;
