@@ -387,6 +387,9 @@ def main():
                     help="run only the yardstick: a plain read of each decode shape's bytes, one launch per layer buffer in a graph, beside the decode kernel's time on the same buffers")
     ap.add_argument("--row-sweep", action="store_true",
                     help="run only a sweep of the row count M across the dispatch boundaries (1 .. 2048), one JSON line per call shape")
+    ap.add_argument("--model-sweep", action="store_true",
+                    help="run only a sweep of decoder-model call shapes (Qwen2.5-7B / 0.5B, Llama-3-8B, Phi-3-mini projections) over 1 .. 16 rows, "
+                         "block size 32 and 128, accuracy_level 0 and 4; one JSON line per shape and block size")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (no collectives exist on the MatMulNBits path); use --gpus 1")
@@ -408,6 +411,10 @@ def main():
         return
     if args.row_sweep:
         for row in row_sweep(ep):
+            print(json.dumps(row), flush=True)
+        return
+    if args.model_sweep:
+        for row in model_sweep(ep):
             print(json.dumps(row), flush=True)
         return
     if args.only_tables:
@@ -629,6 +636,48 @@ def row_sweep(ep):
                 nd.free(ep)
             ep.deallocate(a)
         out += reversed(shape_rows)
+    return out
+
+
+MODEL_SWEEP_SHAPES = (   # name, K, N
+    ("qwen2.5-7b qkv", 3584, 4608), ("qwen2.5-7b o", 3584, 3584), ("qwen2.5-7b gate/up", 3584, 37888), ("qwen2.5-7b down", 18944, 3584),
+    ("qwen2.5-7b lm_head", 3584, 152064),
+    ("llama-3-8b qkv", 4096, 6144), ("llama-3-8b o", 4096, 4096), ("llama-3-8b gate/up", 4096, 28672), ("llama-3-8b gate", 4096, 14336),
+    ("llama-3-8b down", 14336, 4096), ("llama-3-8b lm_head", 4096, 128256),
+    ("qwen2.5-0.5b q", 896, 896), ("qwen2.5-0.5b gate/up", 896, 4864), ("qwen2.5-0.5b down", 4864, 896), ("qwen2.5-0.5b lm_head", 896, 151936),
+    ("phi-3-mini qkv", 3072, 9216), ("phi-3-mini o", 3072, 3072), ("phi-3-mini gate/up", 3072, 16384), ("phi-3-mini down", 8192, 3072),
+    ("phi-3-mini lm_head", 3072, 32064),
+    ("qwen2.5-14b gate", 5120, 13824), ("qwen2.5-14b down", 13824, 5120),
+)
+MODEL_SWEEP_ROWS = (1, 2, 4, 5, 8, 16)
+
+
+def model_sweep(ep):
+    """Time per call (us) of decoder-model projections at 1 .. 16 rows, bf16 with zero points, block size 32 and 128, float and
+    accuracy_level = 4, on the default dispatch: the table that calls costing more than a taller or coarser-blocked neighbour
+    are read off. Per graph as many weight copies as 600 MB hold (2 .. 8), replayed after a warm-up."""
+    out = []
+    for acc in (0, 4):
+        for name, k, n in MODEL_SWEEP_SHAPES:
+            for bs in (32, 128):
+                wbytes = n * k // 2 + n * (k // bs) * 2 + n * ((k // bs + 1) // 2)
+                copies = max(2, min(8, int(600e6 // wbytes)))
+                us = {}
+                for m in MODEL_SWEEP_ROWS:
+                    nodes = [Node(ep, f"w{i}", k, n, bs, i, E.BF16, m, accuracy_level=acc) for i in range(copies)]
+                    a = ep.upload(synth.make_activation(m, k, 5, E.BF16))
+                    for nd in nodes:
+                        nd.run(a)
+                    ep.sync()
+                    graph = capture(ep, lambda: [nd.run(a) for nd in nodes])
+                    us[m] = round(time_graph(ep, graph, 10, 3) / len(nodes) * 1e3, 2)
+                    variant = nodes[0].ops.kernel.last_variant()
+                    graph.release()
+                    for nd in nodes:
+                        nd.free(ep)
+                    ep.deallocate(a)
+                out.append({"accuracy_level": acc, "shape": name, "k": k, "n": n, "block_size": bs, "us": us,
+                            "gbs_one_row": round(wbytes / us[1] / 1e3, 0), "variant_16_rows": variant})
     return out
 
 

@@ -1632,9 +1632,13 @@ extern "C" int rocm_launch_acc4_packed(const RocmMatMulNBitsArgs* a, const void*
     const int gpw = (p.groups + w - 1) / w;
     w = (p.groups + gpw - 1) / gpw;
     p.groups_per_wave = gpw;
-    // one group per wave: a second register set has nothing to fetch ahead (one row, 4096 -> 14336: 14.3 -> 9.8 us at block
-    // 32, 9.7 -> 8.8 at 64, 9.2 -> 8.4 at 128; never slower on the smaller grids)
-    if (gpw == 1) single_set = true;
+    // One register set (one-row launches; the builds for several rows have no other): with one group per wave a second set
+    // has nothing to fetch ahead (4096 -> 14336: 14.3 -> 9.8 us at block 32, 9.7 -> 8.8 at 64, 9.2 -> 8.4 at 128); at block 32 the
+    // two-set build holds three waves per SIMD against eight (5120 -> 13824 21.4 -> 11.6 us, 6144 -> 16384 23.8 -> 14.4,
+    // 8192 -> 8192 14.1 -> 10.5); and from a few hundred column groups on the other block sizes are level or ahead with one
+    // (13824 -> 5120 at block 128: 12.3 -> 11.2; 8192 -> 10240 at 64: 12.3 -> 11.5). Small K-heavy grids keep two (18944 -> 3584 at
+    // block 128: 9.3 against 10.2 us).
+    if (gpw == 1 || a->block_size == 32 || wgs > 256) single_set = true;
 
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool f32_scales = a->scale_dtype == ROCM_DT_F32;
