@@ -144,6 +144,9 @@ int rocm_launch_decode_packed(const RocmMatMulNBitsArgs* args, const void* packe
 /* 1 when the launch above (and the paired one below) applies args->gamma inside the kernel: up to 4 rows, K % 128 == 0, gamma f32 or
  * of the activations' type and 16-byte aligned, and a shape the split-K kernel takes (not the shared-activation one). */
 int rocm_decode_packed_fuses_norm(const RocmMatMulNBitsArgs* args);
+/* Waves per SIMD that the launcher assumes for the one-register-set build serving `m` rows (1, 2-4, 5-8, 9-16) when it sizes
+ * a launch to the chip; a test holds it against the registers the build reported. */
+int rocm_decode_packed_waves_per_simd(int block_size, int m, int f32_scales, int bf16);
 /* The fused gate/up node at up to four rows: one launch over both projections' repacked copies; Y (the activations'
  * 16-bit type) = round16(silu(round16(gate)) * round16(up)), each projection summed exactly as its own launch would.
  * args names the shared operands (a, y, m, n, k, block_size, dtypes; b / scales / zp only for the eligibility checks).

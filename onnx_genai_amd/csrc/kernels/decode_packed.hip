@@ -1404,15 +1404,27 @@ extern "C" int rocm_decode_packed_fuses_norm(const RocmMatMulNBitsArgs* a)
     return (reinterpret_cast<uintptr_t>(a->gamma) & 15) == 0;
 }
 
-// waves per SIMD of the one-set builds (from their register counts: 59-76 registers with one row, 71-102 with four, 84-112
-// with eight, 110-134 with sixteen)
+// Waves per SIMD of the one-set builds, from the registers the compiler reported for them (59-76 with one row, 71-102 with
+// four, 84-112 with eight, 110-134 with sixteen); a test holds the table against the build's report.
 static int waves_per_simd(const RocmMatMulNBitsArgs* a, bool f32_scales)
 {
-    const int bs = a->block_size;
-    if (a->m <= 1) return bs == 128 ? 8 : bs == 64 ? (f32_scales ? 7 : 8) : (f32_scales ? 6 : 7);
-    if (a->m <= 4) return bs == 128 ? (f32_scales ? 6 : 7) : bs == 64 ? 6 : (f32_scales ? 4 : 5);
-    if (a->m <= 8) return bs == 32 ? 4 : 5;
-    return f32_scales ? 3 : 4;
+    // [f16 / bf16][rows: 1, 2-4, 5-8, 9-16][block 32, 64, 128][16-bit / f32 scales]
+    static const unsigned char table[2][4][3][2] = {
+        {{{5, 6}, {7, 7}, {8, 8}}, {{5, 4}, {5, 6}, {6, 6}}, {{4, 4}, {5, 5}, {5, 5}}, {{4, 3}, {4, 4}, {3, 4}}},
+        {{{7, 6}, {8, 7}, {8, 8}}, {{5, 4}, {6, 6}, {7, 6}}, {{4, 4}, {5, 5}, {5, 5}}, {{4, 3}, {4, 4}, {4, 4}}},
+    };
+    const int rows = a->m <= 1 ? 0 : a->m <= 4 ? 1 : a->m <= 8 ? 2 : 3;
+    const int block = a->block_size == 32 ? 0 : a->block_size == 64 ? 1 : 2;
+    return table[a->a_dtype == ROCM_DT_BF16][rows][block][f32_scales];
+}
+
+extern "C" int rocm_decode_packed_waves_per_simd(int block_size, int m, int f32_scales, int bf16)
+{
+    RocmMatMulNBitsArgs a{};
+    a.block_size = block_size;
+    a.m = m;
+    a.a_dtype = bf16 ? ROCM_DT_BF16 : ROCM_DT_F16;
+    return waves_per_simd(&a, f32_scales != 0);
 }
 
 // the most waves a workgroup of decode_packed_kernel may have (see the kernel's launch bounds)

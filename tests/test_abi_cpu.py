@@ -261,6 +261,28 @@ def test_build_reads_kernel_resource_remarks():
     assert build._diagnostics(err) == "k.hip:3:1: warning: unused variable 'x'\n    3 | int x;\n      | ^"
 
 
+def test_launcher_occupancy_table_matches_the_build():
+    """The split-K launcher sizes mid-size launches by the waves per SIMD of the one-set builds: the figures it assumes are
+    the ones the build reported for those kernels."""
+    from onnx_genai_amd import build
+    report = os.path.join(build.OBJ, "kernel_resources.txt")
+    if not os.path.exists(report):
+        pytest.skip("no build report in this tree")
+    lib = C.CDLL(build.LIB)
+    lib.rocm_decode_packed_waves_per_simd.restype = C.c_int
+    lib.rocm_decode_packed_waves_per_simd.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int]
+    # _ZN3mnb20decode_packed_kernelILb<bf16>ELi<block>ELi<rows staged>E<t|f: scale type>Li<sets>ELb<pair>ELb<norm>EEEv...
+    pat = re.compile(r"decode_packed_kernelILb([01])ELi(\d+)ELi(\d+)E([tf])Li1ELb0ELb0EEE\S* .*Occupancy \[waves/SIMD\]=(\d+)")
+    seen = 0
+    for line in open(report).read().splitlines():
+        m = pat.search(line)
+        if m:
+            bf16, bs, rows, f32, built = int(m.group(1)), int(m.group(2)), int(m.group(3)), m.group(4) == "f", int(m.group(5))
+            assert lib.rocm_decode_packed_waves_per_simd(bs, rows, int(f32), bf16) == built, line
+            seen += 1
+    assert seen == 2 * 3 * 4 * 2
+
+
 def test_built_kernels_use_no_scratch():
     """The report the last build wrote lists every kernel with zero scratch bytes and zero spilled registers."""
     from onnx_genai_amd import build
