@@ -164,6 +164,9 @@ int rocm_prefill_mfma_eligible(const RocmMatMulNBitsArgs* args);
  * by a second kernel; rocm_prefill_mfma_scratch_bytes says how much the preferred plan wants (0 = no slicing). With less
  * scratch the launcher uses fewer slices, with none it does not slice. */
 uint64_t rocm_prefill_mfma_scratch_bytes(const RocmMatMulNBitsArgs* args, int tile_choice);
+/* The plan rocm_launch_prefill_mfma would follow with `scratch_bytes` of scratch: the tile and the slices of K (no GPU work;
+ * only the shape, dtype and pointer alignment of `args` are read). -1: shape not eligible. */
+int rocm_prefill_mfma_plan(const RocmMatMulNBitsArgs* args, int tile_choice, uint64_t scratch_bytes, int* tile_rows, int* tile_cols, int* slices);
 /* Y = sum over `slices` of partial[slice][M][N] (f32), in slice order, + bias. */
 int rocm_launch_slice_reduce(const float* partial, int slices, int64_t m, int64_t n, const void* bias, int bias_dtype, void* y, int y_dtype,
                              rocm_stream_t stream);

@@ -283,6 +283,43 @@ def test_launcher_occupancy_table_matches_the_build():
     assert seen == 2 * 3 * 4 * 2
 
 
+class _FfiArgs(C.Structure):
+    """RocmMatMulNBitsArgs of csrc/hip_ffi.h (the internal kernel-launch interface), for the calls below that do no GPU work."""
+    _fields_ = [("a", C.c_void_p), ("b", C.c_void_p), ("scales", C.c_void_p), ("zp", C.c_void_p), ("bias", C.c_void_p), ("y", C.c_void_p),
+                ("a_dtype", C.c_int), ("scale_dtype", C.c_int), ("bias_dtype", C.c_int), ("y_dtype", C.c_int),
+                ("m", C.c_int64), ("n", C.c_int64), ("k", C.c_int64), ("block_size", C.c_int),
+                ("g_idx", C.c_void_p), ("acc_probe", C.c_void_p), ("gamma", C.c_void_p), ("gamma_dtype", C.c_int), ("norm_epsilon", C.c_float)]
+
+
+def _prefill_plan(lib, m, n, k, bf16=True, scratch=1 << 40):
+    args = _FfiArgs()
+    args.a, args.b, args.scales, args.y = 0x10000, 0x20000, 0x30000, 0x40000         # never dereferenced: alignment only
+    args.a_dtype = args.scale_dtype = args.y_dtype = 16 if bf16 else 10
+    args.m, args.n, args.k, args.block_size = m, n, k, 128
+    rows, cols, slices = C.c_int(), C.c_int(), C.c_int()
+    assert lib.rocm_prefill_mfma_plan(C.byref(args), 0, C.c_uint64(scratch), C.byref(rows), C.byref(cols), C.byref(slices)) == 0
+    return rows.value, cols.value, slices.value
+
+
+def test_prefill_plan_slices_long_k_on_short_grids():
+    """The tiled prefill kernel's planner: tall calls on wide shapes take whole 256 x 256 tiles; a long K on a short grid takes
+    the larger tiles over slices of K instead of small unsliced ones; without scratch nothing is sliced."""
+    from onnx_genai_amd import build
+    lib = C.CDLL(build.LIB)
+    lib.rocm_prefill_mfma_plan.restype = C.c_int
+    lib.rocm_prefill_mfma_plan.argtypes = [C.c_void_p, C.c_int, C.c_uint64, C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int)]
+    assert _prefill_plan(lib, 8192, 14336, 4096) == (256, 256, 1)
+    assert _prefill_plan(lib, 4096, 37888, 3584) == (256, 256, 1)
+    rows, cols, slices = _prefill_plan(lib, 1536, 3584, 18944)            # 336 tiles of 128 x 128 would run in two rounds on 256 CUs
+    assert rows == 256 and slices >= 3
+    rows, cols, slices = _prefill_plan(lib, 1536, 3584, 18944, scratch=0)
+    assert slices == 1
+    # every plan covers K: the slices are whole 64-element steps
+    for m, n, k in [(256, 4096, 14336), (512, 3584, 18944), (3072, 4096, 14336), (300, 1000, 4160)]:
+        rows, cols, slices = _prefill_plan(lib, m, n, k)
+        assert rows in (128, 256) and cols in (64, 128, 256) and 1 <= slices <= 16 and slices <= k // 64
+
+
 def test_built_kernels_use_no_scratch():
     """The report the last build wrote lists every kernel with zero scratch bytes and zero spilled registers."""
     from onnx_genai_amd import build
