@@ -469,7 +469,7 @@ PrefillPlan plan_prefill(const RocmMatMulNBitsArgs* a, int tile_choice, uint64_t
         };
         double best = modelled(plan.tile, plan.splits) * 0.97;
         const PrefillPlan base = plan;
-        for (int tile = 0; tile <= 3; ++tile) {
+        for (int tile = 0; tile <= 2; ++tile) {            // (128 x 64 only where the rule above chose it: few timings back its figure)
             for (int pass = 0; pass < 2; ++pass) {
                 const int sl = pass == 0 ? 1 : slices(tile);
                 if ((pass == 1 && sl == 1) || (tile == base.tile && sl == base.splits)) continue;
