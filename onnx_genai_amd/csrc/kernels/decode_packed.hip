@@ -1013,6 +1013,13 @@ struct Acc4PackedGroup {
 // the activation-side (scale, sum) pairs of the group's blocks are staged once per group and read when a block ends.
 // With 4 (8), call row r sits in matrix row 4 r (2 r) and the rows between stay zero, so that a lane finds its rows in
 // component 0 (0 and 2) of its accumulator and a block's end scales one (two) values per lane instead of four.
+// ST: float, uint16_t, or Bf16Scale for the several-row builds when the 16-bit scales are bf16 - there the scale type is
+// known at compile time (a run-time choice between the two conversions made the compiler prepare both for all of a
+// group's blocks up front: 220 registers instead of 94 at block size 32 and 16 rows, two waves per SIMD instead of five).
+struct Bf16Scale {
+    uint16_t bits;
+};
+
 template <int BS, typename ST, int SETS, int FUSE, bool PROBE, int MR = 1>
 __global__ __launch_bounds__(512) void acc4_packed_kernel(Acc4PackedParams p)
 {
@@ -1036,7 +1043,7 @@ __global__ __launch_bounds__(512) void acc4_packed_kernel(Acc4PackedParams p)
     const int c = lane & 15;
     const int g = lane >> 4;
     const int64_t n_base = static_cast<int64_t>(blockIdx.x) * 16;
-    const bool bf16_scales = p.scales_bf16 != 0;
+    const bool bf16_scales = std::is_same<ST, Bf16Scale>::value || (MR == 1 && p.scales_bf16 != 0);
 
     const __amdgpu_buffer_rsrc_t srd_p = make_srd(p.packed + static_cast<int64_t>(blockIdx.x) * p.cg_stride, static_cast<uint64_t>(p.cg_stride));
     const __amdgpu_buffer_rsrc_t srd_a = FUSE ? make_srd(p.a, static_cast<uint64_t>(p.k) * 2) : make_srd(p.qa, static_cast<uint64_t>(p.m * p.padded_k));
@@ -1296,6 +1303,9 @@ static int launch_acc4_packed(const Acc4PackedParams& p, int waves, bool single_
 {
     const unsigned grid = static_cast<unsigned>((p.n + 15) / 16);
     if (p.m > 1) {
+        if constexpr (std::is_same<ST, uint16_t>::value) {
+            if (p.scales_bf16) return launch_acc4_packed<BS, Bf16Scale>(p, waves, single_set, fuse, stream);
+        }
         // two tiles of codes in turn + the group's pairs per wave; the reduction reuses the space (1 KiB per wave)
         const size_t lds16 = static_cast<size_t>(waves) * (2 * 16 * kCodePitchP + kGroupTiles * (128 / BS) * 128);
         if (p.m <= 4) {
@@ -1308,6 +1318,9 @@ static int launch_acc4_packed(const Acc4PackedParams& p, int waves, bool single_
         else hipLaunchKernelGGL((acc4_packed_kernel<BS, ST, 1, 0, false, 16>), dim3(grid), dim3(waves * 64), lds16, stream, p);
         return static_cast<int>(hipGetLastError());
     }
+    if constexpr (std::is_same<ST, Bf16Scale>::value) {
+        return -1;                                         // (several rows only)
+    } else {
     const size_t lds = static_cast<size_t>(waves) * 1024;
     auto go = [&](auto fuse) {
         constexpr int F = decltype(fuse)::value;
@@ -1321,6 +1334,7 @@ static int launch_acc4_packed(const Acc4PackedParams& p, int waves, bool single_
     else if (fuse == 2) go(std::integral_constant<int, 2>{});
     else go(std::integral_constant<int, 0>{});
     return static_cast<int>(hipGetLastError());
+    }
 }
 
 static int packed_groups(const RocmMatMulNBitsArgs* a)
