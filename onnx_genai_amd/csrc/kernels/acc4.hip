@@ -152,6 +152,69 @@ __global__ __launch_bounds__(256) void acc4_gemv_kernel(RocmMatMulNBitsArgs p, c
     }
 }
 
+// The same quantizer for f16 / bf16 rows with K a multiple of 8 and block size 32, 64 or 128: a lane owns eight consecutive
+// elements (one 16-byte load, one 8-byte store of codes - the orders above only permute inside such a run), the BS / 8
+// lanes of a block find its maximum and code sum with shuffles. Every arithmetic step is the one above (a maximum and an
+// integer sum do not depend on the order), so the codes, scales and sums are the same bits; what changes is the traffic:
+// one wave per block of 64 elements moved 2 bytes per lane per load and a byte per store (M = 4096, K = 28672: 622 us,
+// 0.57 TB/s).
+template <int BS>
+__global__ __launch_bounds__(256) void quantize_a16_kernel(
+    const uint16_t* __restrict__ a, int bf16, int64_t m, int64_t k, int64_t kb, int rounding, int interleave,
+    int8_t* __restrict__ qa, float* __restrict__ qscale, int32_t* __restrict__ qsum, float* __restrict__ aq, float* __restrict__ aux16, float* __restrict__ sa_t)
+{
+    constexpr int L = BS / 8;                                    // lanes per block
+    const int64_t row_pieces = kb * L;                           // 16-byte pieces of a padded row
+    const int64_t piece = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    const bool inside = piece < m * row_pieces;                  // (lanes past the end still take part in the shuffles)
+    const int64_t row = inside ? piece / row_pieces : 0;
+    const int64_t in_row = inside ? piece - row * row_pieces : 0;
+    const int64_t blk = in_row / L;
+    const int64_t k0 = in_row * 8;
+    uint4 raw = make_uint4(0u, 0u, 0u, 0u);
+    if (inside && k0 < k) raw = *reinterpret_cast<const uint4*>(a + row * k + k0);      // K % 8 = 0: a piece is all inside or all outside
+    const uint32_t d[4] = {raw.x, raw.y, raw.z, raw.w};
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        v[2 * i] = bf16 ? __uint_as_float(d[i] << 16) : f16_bits_to_f32(static_cast<uint16_t>(d[i]));
+        v[2 * i + 1] = bf16 ? __uint_as_float(d[i] & 0xffff0000u) : f16_bits_to_f32(static_cast<uint16_t>(d[i] >> 16));
+    }
+    float vmax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) vmax = fmaxf(vmax, fabsf(v[i]));
+#pragma unroll
+    for (int off = L / 2; off > 0; off >>= 1) vmax = fmaxf(vmax, __shfl_xor(vmax, off, 64));
+    const float scale = __fdiv_rn(vmax, 127.0f);
+    const float inv = vmax != 0.0f ? __fdiv_rn(127.0f, vmax) : 0.0f;
+    int sum = 0;
+    uint32_t lo = 0, hi = 0;                                      // the run's eight code bytes, in storage order
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const float scaled = __fmul_rn(v[e], inv);
+        float r = rounding == 1 ? roundf(scaled) : rintf(scaled);
+        r = fminf(fmaxf(r, -127.0f), 127.0f);
+        const int code = static_cast<int>(r);
+        sum += code;
+        // inside every run of 8: as is (0), elements 0,2,4,6,1,3,5,7 (1), or 0,4,1,5,2,6,3,7 (2)
+        const int pos = interleave == 1 ? (((e & 1) << 2) | (e >> 1)) : interleave == 2 ? (((e & 3) << 1) | (e >> 2)) : e;
+        const uint32_t byte = static_cast<uint32_t>(code) & 0xffu;
+        if (pos < 4) lo |= byte << (8 * pos);
+        else hi |= byte << (8 * (pos - 4));
+    }
+#pragma unroll
+    for (int off = L / 2; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    if (!inside) return;
+    *reinterpret_cast<uint2*>(qa + row * kb * BS + k0) = make_uint2(lo, hi);
+    if (in_row % L == 0) {
+        if (qscale) qscale[row * kb + blk] = scale;
+        if (qsum) qsum[row * kb + blk] = sum;
+        if (aq) *reinterpret_cast<float2*>(aq + (row * kb + blk) * 2) = make_float2(scale, static_cast<float>(sum));   // |sum| <= 127 * bs: exact
+        if (sa_t) sa_t[blk * m + row] = scale;
+        if (aux16 && row < 16) *reinterpret_cast<float2*>(aux16 + (blk * 16 + row) * 2) = make_float2(scale, static_cast<float>(sum));
+    }
+}
+
 }  // namespace mnb
 
 static int launch_quantize(const void* a, int a_dtype, int64_t m, int64_t k, int block_size, int rounding, int interleave,
@@ -160,6 +223,19 @@ static int launch_quantize(const void* a, int a_dtype, int64_t m, int64_t k, int
     if (m <= 0 || k <= 0) return 0;
     const int64_t kb = (k + block_size - 1) / block_size;
     const int64_t items = m * kb;
+    const bool half = a_dtype == ROCM_DT_F16 || a_dtype == ROCM_DT_BF16;
+    if (half && k % 8 == 0 && (block_size == 32 || block_size == 64 || block_size == 128) && (reinterpret_cast<uintptr_t>(a) & 15) == 0 &&
+        (reinterpret_cast<uintptr_t>(qa) & 7) == 0 && (!aq || (reinterpret_cast<uintptr_t>(aq) & 7) == 0) && (!aux16 || (reinterpret_cast<uintptr_t>(aux16) & 7) == 0)) {
+        const int64_t pieces = items * (block_size / 8);
+        const dim3 grid(static_cast<unsigned>((pieces + 255) / 256));
+        const int bf16 = a_dtype == ROCM_DT_BF16;
+        const uint16_t* a16 = static_cast<const uint16_t*>(a);
+        hipStream_t s = static_cast<hipStream_t>(stream);
+        if (block_size == 32) hipLaunchKernelGGL(mnb::quantize_a16_kernel<32>, grid, dim3(256), 0, s, a16, bf16, m, k, kb, rounding, interleave, qa, qscale, qsum, aq, aux16, sa_t);
+        else if (block_size == 64) hipLaunchKernelGGL(mnb::quantize_a16_kernel<64>, grid, dim3(256), 0, s, a16, bf16, m, k, kb, rounding, interleave, qa, qscale, qsum, aq, aux16, sa_t);
+        else hipLaunchKernelGGL(mnb::quantize_a16_kernel<128>, grid, dim3(256), 0, s, a16, bf16, m, k, kb, rounding, interleave, qa, qscale, qsum, aq, aux16, sa_t);
+        return static_cast<int>(hipGetLastError());
+    }
     hipLaunchKernelGGL(mnb::quantize_a_kernel, dim3(static_cast<unsigned>((items + 3) / 4)), dim3(256), 0, static_cast<hipStream_t>(stream),
                        a, a_dtype, m, k, block_size, kb, rounding, interleave, qa, qscale, qsum, aq, aux16, sa_t);
     return static_cast<int>(hipGetLastError());
