@@ -1023,7 +1023,8 @@ struct Bf16Scale {
 template <int BS, typename ST, int SETS, int FUSE, bool PROBE, int MR = 1>
 __global__ __launch_bounds__(512) void acc4_packed_kernel(Acc4PackedParams p)
 {
-    static_assert(MR == 1 || ((MR == 4 || MR == 8 || MR == 16) && FUSE == 0 && SETS == 1), "several rows: codes from the workspace, one register set");
+    static_assert(MR == 1 || ((MR == 4 || MR == 8 || MR == 16) && (FUSE == 0 || MR == 4) && SETS == 1),
+                  "several rows: one register set; codes from the workspace, or up to four rows quantized here");
     constexpr int U = kGroupTiles;
     constexpr int NBT = 128 / BS;
     constexpr int NB = U * NBT;
@@ -1046,7 +1047,7 @@ __global__ __launch_bounds__(512) void acc4_packed_kernel(Acc4PackedParams p)
     const bool bf16_scales = std::is_same<ST, Bf16Scale>::value || (MR == 1 && p.scales_bf16 != 0);
 
     const __amdgpu_buffer_rsrc_t srd_p = make_srd(p.packed + static_cast<int64_t>(blockIdx.x) * p.cg_stride, static_cast<uint64_t>(p.cg_stride));
-    const __amdgpu_buffer_rsrc_t srd_a = FUSE ? make_srd(p.a, static_cast<uint64_t>(p.k) * 2) : make_srd(p.qa, static_cast<uint64_t>(p.m * p.padded_k));
+    const __amdgpu_buffer_rsrc_t srd_a = FUSE ? make_srd(p.a, static_cast<uint64_t>(p.m * p.k) * 2) : make_srd(p.qa, static_cast<uint64_t>(p.m * p.padded_k));
     const __amdgpu_buffer_rsrc_t srd_x = MR == 1 ? make_srd(p.aq, FUSE ? 0 : static_cast<uint64_t>(p.kb) * 8) : make_srd(p.aux16, static_cast<uint64_t>(p.kb) * 128);
     constexpr int kBlockLanes = BS / 8;
 
@@ -1083,7 +1084,16 @@ __global__ __launch_bounds__(512) void acc4_packed_kernel(Acc4PackedParams p)
         for (int u = 0; u < U; ++u) grp.w[u] = load16(srd_p, (w_off + static_cast<uint32_t>(u * 1024)) | oor, soff);
 #pragma unroll
         for (int i = 0; i < NR; ++i) grp.r[i] = load16(srd_p, (r_off + static_cast<uint32_t>(i * 16)) | oor, soff);
-        if constexpr (MR != 1) {
+        if constexpr (MR != 1 && FUSE != 0) {
+            // up to four rows quantized here: a[r] = 8 activations of row r (lane * 8 of the group's 512); a row past M lies past
+            // the range and reads as zeros, a piece past K would be the next row's and is kept out
+            const bool beyond = static_cast<int64_t>(gi) * 512 + lane * 8 >= p.k;
+#pragma unroll
+            for (int r = 0; r < NA; ++r) {
+                const uint32_t off = beyond ? kOutOfRange : static_cast<uint32_t>(r) * static_cast<uint32_t>(p.k) * 2u + static_cast<uint32_t>(lane * 16);
+                grp.a[r] = load16(srd_a, off | oor, static_cast<uint32_t>(gi) * 1024u);
+            }
+        } else if constexpr (MR != 1) {
 #pragma unroll
             for (int x = 0; x < NA; ++x) {
                 const int u = MR == 16 ? x / 2 : x, i = MR == 16 ? x % 2 : 0;
@@ -1107,12 +1117,11 @@ __global__ __launch_bounds__(512) void acc4_packed_kernel(Acc4PackedParams p)
     auto compute_group = [&](const Grp& grp, int gi, int slot) {
         unsigned char* st = stage + slot * 512;
         float sa_lane = 0.f, qs_lane = 0.f;          // FUSE: scale and f32(code sum) of the block this lane's activations lie in
-        if constexpr (MR != 1) {
-#pragma unroll
-            for (int x = 0; x < NX; ++x)
-                if (lane + 64 * x < NB * 8) *reinterpret_cast<uint4*>(aux_stage + (lane + 64 * x) * 16) = grp.x[x];
-        } else if constexpr (FUSE) {
-            const uint32_t d[4] = {grp.a[0].x, grp.a[0].y, grp.a[0].z, grp.a[0].w};
+        uint2 fused_codes[MR != 1 && FUSE != 0 ? MR : 1];
+        // FUSE: the quantizer's arithmetic on one 16-byte piece (8 activations); the block's lanes share maximum and code sum.
+        // Returns the eight codes in the byte order the repacked weights unpack to, elements 0,4,1,5 | 2,6,3,7.
+        auto quantize_piece = [&](const uint4& piece) -> uint2 {
+            const uint32_t d[4] = {piece.x, piece.y, piece.z, piece.w};
             float v[8];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
@@ -1152,10 +1161,24 @@ __global__ __launch_bounds__(512) void acc4_packed_kernel(Acc4PackedParams p)
             if constexpr (BS >= 64) sum = dpp_addi<0x141>(sum);
             if constexpr (BS >= 128) sum = dpp_addi<0x140>(sum);
             qs_lane = static_cast<float>(sum);                     // |sum| <= 127 * BS: exact
-            // the byte order the repacked weights unpack to: elements 0,4,1,5 | 2,6,3,7
             const uint32_t lo = (q[0] & 0xff) | ((q[4] & 0xff) << 8) | ((q[1] & 0xff) << 16) | (static_cast<uint32_t>(q[5]) << 24);
             const uint32_t hi = (q[2] & 0xff) | ((q[6] & 0xff) << 8) | ((q[3] & 0xff) << 16) | (static_cast<uint32_t>(q[7]) << 24);
-            *reinterpret_cast<uint2*>(st + lane * 8) = make_uint2(lo, hi);
+            return make_uint2(lo, hi);
+        };
+        if constexpr (MR != 1 && FUSE != 0) {
+            // every row's piece is quantized; the first lane of a block leaves the row's (scale, code sum) where a block's end
+            // reads it: pair [block][row] of the group
+#pragma unroll
+            for (int r = 0; r < MR; ++r) {
+                fused_codes[r] = quantize_piece(grp.a[r]);
+                if (lane % kBlockLanes == 0) *reinterpret_cast<float2*>(aux_stage + (lane / kBlockLanes) * 128 + r * 8) = make_float2(sa_lane, qs_lane);
+            }
+        } else if constexpr (MR != 1) {
+#pragma unroll
+            for (int x = 0; x < NX; ++x)
+                if (lane + 64 * x < NB * 8) *reinterpret_cast<uint4*>(aux_stage + (lane + 64 * x) * 16) = grp.x[x];
+        } else if constexpr (FUSE) {
+            *reinterpret_cast<uint2*>(st + lane * 8) = quantize_piece(grp.a[0]);
         } else {
             if (lane < 32) *reinterpret_cast<uint4*>(st + lane * 16) = grp.a[0];
         }
@@ -1177,7 +1200,13 @@ __global__ __launch_bounds__(512) void acc4_packed_kernel(Acc4PackedParams p)
             long av[4];
             if constexpr (MR != 1) {
                 unsigned char* tile = stage + (u & 1) * kCodeStage;
-                if constexpr (MR != 16) {
+                if constexpr (FUSE != 0) {
+                    // the lanes that hold this tile's elements (lane / 16 = u) write each row's eight codes into its matrix row
+                    if ((lane >> 4) == u) {
+#pragma unroll
+                        for (int r = 0; r < MR; ++r) *reinterpret_cast<uint2*>(tile + r * SP * kCodePitchP + (lane & 15) * 8) = fused_codes[r];
+                    }
+                } else if constexpr (MR != 16) {
                     if (MR == 8 || lane < 32) *reinterpret_cast<uint4*>(tile + st_write16) = grp.a[u];
                 } else {
 #pragma unroll
@@ -1308,6 +1337,13 @@ static int launch_acc4_packed(const Acc4PackedParams& p, int waves, bool single_
         }
         // two tiles of codes in turn + the group's pairs per wave; the reduction reuses the space (1 KiB per wave)
         const size_t lds16 = static_cast<size_t>(waves) * (2 * 16 * kCodePitchP + kGroupTiles * (128 / BS) * 128);
+        if (fuse != 0) {
+            // up to four f16 / bf16 rows: the kernel quantizes them itself (no codes, no pairs, no launch before this one)
+            if (p.m > 4 || p.acc_probe) return -1;
+            if (fuse == 2) hipLaunchKernelGGL((acc4_packed_kernel<BS, ST, 1, 2, false, 4>), dim3(grid), dim3(waves * 64), lds16, stream, p);
+            else hipLaunchKernelGGL((acc4_packed_kernel<BS, ST, 1, 1, false, 4>), dim3(grid), dim3(waves * 64), lds16, stream, p);
+            return static_cast<int>(hipGetLastError());
+        }
         if (p.m <= 4) {
             if (p.acc_probe) hipLaunchKernelGGL((acc4_packed_kernel<BS, ST, 1, 0, true, 4>), dim3(grid), dim3(waves * 64), lds16, stream, p);
             else hipLaunchKernelGGL((acc4_packed_kernel<BS, ST, 1, 0, false, 4>), dim3(grid), dim3(waves * 64), lds16, stream, p);
@@ -1608,8 +1644,15 @@ extern "C" int rocm_acc4_packed_eligible(const RocmMatMulNBitsArgs* a)
 
 extern "C" int rocm_acc4_packed_fuses_quantizer(const RocmMatMulNBitsArgs* a)
 {
-    return rocm_acc4_packed_eligible(a) && a->m == 1 && (a->a_dtype == ROCM_DT_F16 || a->a_dtype == ROCM_DT_BF16) && a->k % 8 == 0 &&
-           (reinterpret_cast<uintptr_t>(a->a) & 15) == 0;
+    if (!(rocm_acc4_packed_eligible(a) && (a->a_dtype == ROCM_DT_F16 || a->a_dtype == ROCM_DT_BF16) && a->k % 8 == 0 && (reinterpret_cast<uintptr_t>(a->a) & 15) == 0))
+        return 0;
+    if (a->m == 1) return 1;
+    // Two to four rows: every workgroup quantizes the rows again, which more than doubles what a wave computes per tile
+    // group - worth it only where the call is short enough for the quantizer's own launch (about 3 us) to weigh more:
+    // 3584 -> 3584 8.2 -> 6.3 us, 3584 -> 4608 8.9 -> 8.0; 4096 -> 14336 level; 18944 -> 3584 14.5 -> 16.6 and 3584 -> 37888 19.6 -> 22.4
+    // the wrong way. (The builds that probe block accumulators read the workspace's codes.)
+    const int64_t work = (a->n + 15) / 16 * mnb::packed_groups(a);            // column groups x tile groups
+    return a->m <= 4 && !a->acc_probe && work <= 4096;
 }
 
 extern "C" int rocm_launch_acc4_packed(const RocmMatMulNBitsArgs* a, const void* packed, const RocmAcc4Workspace* ws, int rounding, int waves, rocm_stream_t stream)

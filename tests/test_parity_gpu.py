@@ -1257,6 +1257,8 @@ PRODUCTION_ACC_CASES = [
     (32, False, 1, 48, 32 * 9, False), (64, True, 1, 100, 64 * 50, False), (128, True, 1, 64, 128 * 24, False),
     (32, True, 5, 48, 32 * 9, True), (64, True, 5, 100, 64 * 50, True), (128, False, 5, 77, 128 * 33, True), (64, True, 16, 40, 200, True),
     (32, True, 2, 100, 32 * 37, True), (128, True, 16, 33, 128 * 21, True),
+    # two to four 16-bit rows on a short call: quantized inside the kernel when no probe is set (the helper compares that run with the probing one bit for bit)
+    (64, True, 3, 100, 64 * 50, True), (128, False, 4, 77, 128 * 33, True), (32, True, 4, 130, 32 * 21 + 8, True),
     (32, True, 5, 48, 32 * 9, False), (64, True, 5, 100, 64 * 50, False), (128, False, 5, 77, 128 * 33, False), (64, True, 16, 40, 200, False),
     (32, True, 40, 96, 32 * 35, True), (64, True, 40, 96, 64 * 17, True), (128, True, 130, 200, 128 * 20, True), (64, False, 40, 200, 64 * 3, True),
     (256, True, 40, 96, 256 * 3, True), (32, False, 33, 64, 200, True),
