@@ -1526,9 +1526,9 @@ static int launch_decode_packed(const RocmMatMulNBitsArgs* a, const void* packed
         return f32_scales ? mnb::launch_wide_bs<false, float>(p, a->block_size, s) : mnb::launch_wide_bs<false, uint16_t>(p, a->block_size, s);
     }
 
-    // Waves per workgroup. Many column groups (thousands of waves even at four per group): short waves of at most two
-    // tile groups and no prefetch, so that eight of them fit a SIMD and cover each other's memory latency. Few column
-    // groups: enough waves per group to reach about 8k in flight, each prefetching its next group.
+    // Waves per workgroup (they split K in whole tile groups). Many column groups (thousands of waves even at four per
+    // group): short waves of at most two tile groups. Few column groups: enough waves per group to reach about 8k in
+    // flight. Then the adjustments below: register sets, and wave counts that fit the chip.
     const int64_t wgs = (a->n + 15) / 16 * ((pair_member && a->m <= 4) ? 2 : 1);      // (a pair shares a launch up to four rows here)
     int w = waves;
     const int w_max = w_max_of(a, f32_scales);
