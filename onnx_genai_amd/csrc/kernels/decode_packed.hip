@@ -1403,6 +1403,11 @@ static bool wide_shape(const RocmMatMulNBitsArgs* a, bool pair)
     // 20480: 16.9 / 17.2 / 18.6 against 17.8 / 17.9 / 18.4; at 28672 it loses, 22-25 against 20-21).
     // (block 64: 12.3 / 12.6 / 14.4 us at 14336 and 13.2 / 13.7 / 15.2 at 16384 against 15.4-16.0 in the shared-activation kernel)
     const int64_t min_cols = a->m > 32 ? 16384 : a->m > 16 ? 14336 : a->block_size == 32 ? 22528 : a->block_size == 64 ? 20480 : 18432;
+    // Four rows of a plain call on 18432 .. 49151 columns at block 128 run here as well: level with the four-row split-K build
+    // on a GPU that runs it well (3584 -> 37888 18.1 -> 17.6 us, 4096 -> 28672 16.0 -> 16.2, 3072 -> 32064 13.8 -> 13.5), and this kernel
+    // moved far less from one GPU to the next (on two others the same three calls took 21-22.5 / 18.0-18.3 / 16.8-17.0 us there
+    // against 18.8 / 16.5 / 14.9-15.4 at five rows here). More columns lose (4096 -> 128256: 56.4 -> 62.3), and so do three rows.
+    if (a->m == 4 && !pair && a->gamma == nullptr && a->block_size == 128) return a->n >= 18432 && a->n < 49152;
     return a->m >= 5 && a->m <= max_rows && a->n * (pair ? 2 : 1) >= min_cols;
 }
 
@@ -1449,7 +1454,7 @@ extern "C" int rocm_launch_pack_decode(const RocmMatMulNBitsArgs* a, void* packe
 // for the pair's column groups together, so that the separate launches and the paired one add up in the same order.
 extern "C" int rocm_decode_packed_fuses_norm(const RocmMatMulNBitsArgs* a)
 {
-    if (!a->gamma || a->m > 4 || a->k % 128 != 0 || !rocm_decode_packed_eligible(a)) return 0;      // (up to four rows: never the shared-activation kernel)
+    if (!a->gamma || a->m > 4 || a->k % 128 != 0 || !rocm_decode_packed_eligible(a)) return 0;      // (with gamma, up to four rows never take the shared-activation kernel)
     if (a->gamma_dtype != ROCM_DT_F32 && a->gamma_dtype != a->a_dtype) return 0;
     return (reinterpret_cast<uintptr_t>(a->gamma) & 15) == 0;
 }
