@@ -213,6 +213,9 @@ DECODE_CASES = [
     (E.F16, E.F16, 64, True, 16, 32784, 512),           # the same with nine waves and a ragged last workgroup
     (E.F16, E.F16, 32, True, 12, 37888, 512),           # block 32 never takes the sums build (here: 296 workgroups of eight waves)
     (E.BF16, E.F32, 32, True, 7, 20000, 32 * 19),       # ... nor with f32 scales; a partial last tile group
+    (E.F16, E.F32, 128, True, 4, 18432, 512),           # four rows at block 128 from 18432 columns: the shared-activation kernel with one block of rows
+    (E.BF16, E.BF16, 128, False, 4, 18450, 1024 + 128),  # ... a ragged last workgroup
+    (E.BF16, E.BF16, 128, True, 4, 18431, 512),         # one column short of it: the four-row split-K build
     (E.BF16, E.BF16, 128, True, 17, 16400, 3584),       # up to 64 rows ride on one pass over the weights
     (E.F16, E.F16, 64, True, 40, 16384, 1024 + 64),     # block size 64 stops at 32 rows per pass: the tiled kernel takes this one
     (E.F16, E.F16, 64, True, 25, 16384, 1024 + 64),
