@@ -140,3 +140,59 @@ def test_acc4_configs_at_full_size(ep, port, k, n, m):
                                 len(cols), k, bs, oracle.ROUND_HALF_EVEN)
     assert np.isfinite(y).all()
     assert helpers.rel_l2(y[np.ix_(rows, cols)], want) <= TOL_F32
+
+
+def _random_decode_cases(count, seed):
+    """Seeded decode calls at model widths: 64 .. 3200 column groups (some ragged), 1 .. 37 tile groups of K (some ending inside a
+    tile group), 1 .. 16 rows, block 32 / 64 / 128, f16 / bf16 with 16-bit or f32 scales, float and accuracy_level 4 - the ranges
+    over which the launchers pick wave counts, register sets, row builds and kernels."""
+    rng = np.random.default_rng(seed)
+    cases = []
+    for _ in range(count):
+        a_dt = int(rng.choice([E.F16, E.BF16]))
+        s_dt = a_dt if rng.random() < 0.8 else E.F32
+        bs = int(rng.choice([32, 64, 128]))
+        zero_points = bool(rng.random() < 0.6)
+        m = int(rng.choice([1, 1, 2, 3, 4, 4, 5, 6, 8, 9, 12, 16]))
+        k = int(rng.integers(1, 38)) * 512 - (int(rng.integers(0, 512 // bs)) * bs if rng.random() < 0.4 else 0)
+        k = max(k, bs)
+        n = int(np.exp(rng.uniform(np.log(64), np.log(3200)))) * 16 - (int(rng.integers(0, 16)) if rng.random() < 0.4 else 0)
+        while n * k > 3.0e8:
+            n //= 2
+        cases.append((a_dt, s_dt, bs, zero_points, m, max(n, 17), k, 4 if rng.random() < 0.35 else 0, bool(rng.random() < 0.5)))
+    return cases
+
+
+@pytest.mark.parametrize("a_dt,s_dt,bs,zero_points,m,n,k,acc,with_bias", _random_decode_cases(80, 20260214))
+def test_random_decode_shapes_at_model_widths(ep, port, a_dt, s_dt, bs, zero_points, m, n, k, acc, with_bias):
+    """Whatever wave count, register-set build, row build or kernel the launcher picks for the shape: f32 output against the
+    oracle on a column sample, and the second call (what a graph replays) equal to the first (which repacks) bit for bit."""
+    b, s, zp = random_weights(n, k, bs, 900 + n + k, zero_points, s_dt, 0.002, 0.01)
+    a = synth.make_activation(m, k, 900 + m, a_dt)
+    bias = synth.to_dtype(np.random.default_rng(n).standard_normal(n).astype(np.float32), a_dt) if with_bias else None
+    cols = spread(n, 160)
+    ops = E.DeviceOperands(ep, b, s, s_dt, zp, n, k, bs, accuracy_level=acc, bias=bias, bias_dtype=a_dt)
+    ab, yb = ep.upload(a), ep.allocate(m * n * 4)
+    try:
+        ys = []
+        for _ in range(2):
+            ops.run(ab, a_dt, m, yb, E.F32)
+            ys.append(ep.download(yb, (m, n), np.float32).copy())
+        variant = ops.kernel.last_variant()
+    finally:
+        ep.deallocate(ab)
+        ep.deallocate(yb)
+        ops.free()
+    assert variant == ("acc4_mfma_i8_packed" if acc == 4 else "decode_mfma_packed")
+    assert np.isfinite(ys[1]).all()
+    assert np.array_equal(ys[0], ys[1])
+    af, sf = synth.to_f32(a, a_dt), synth.to_f32(s, s_dt)
+    bc, sc = np.ascontiguousarray(b[cols]), np.ascontiguousarray(sf[cols])
+    zc = np.ascontiguousarray(zp[cols]) if zp is not None else None
+    bf = None if bias is None else np.ascontiguousarray(synth.to_f32(bias, a_dt)[cols])
+    if acc == 4:
+        want = port.matmul_acc4_f32(af, bc, sc, zc, len(cols), k, bs, oracle.ROUND_HALF_EVEN, bias=bf)
+        assert helpers.rel_l2(ys[1][:, cols], want) <= TOL_F32
+    else:
+        want = port.matmul_f64(af, bc, sc, zc, len(cols), k, bs, bias=bf)
+        assert helpers.rel_l2(ys[1][:, cols], want) <= 1e-4
