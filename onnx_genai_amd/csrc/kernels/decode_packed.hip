@@ -1391,6 +1391,12 @@ static int packed_chunk_bytes(const RocmMatMulNBitsArgs* a)
 // (16 rows at block size 32, 32 at 64, 64 at 128: more row blocks than that do not fit the register file)
 // `pair`: the call is the fused gate/up launch or one of its two projections - both projections' columns count, since the
 // paired launch streams both, and a projection launched on its own must add up the way the paired launch does.
+// Four rows at block 128 on 18432 .. 49151 columns: the shared-activation kernel's window below five rows.
+static bool four_row_wide(const RocmMatMulNBitsArgs* a, int64_t cols)
+{
+    return a->m == 4 && a->block_size == 128 && cols >= 18432 && cols < 49152;
+}
+
 static bool wide_shape(const RocmMatMulNBitsArgs* a, bool pair)
 {
     const int64_t max_rows = a->block_size == 32 ? 16 : a->block_size == 64 ? 32 : 64;
@@ -1407,7 +1413,9 @@ static bool wide_shape(const RocmMatMulNBitsArgs* a, bool pair)
     // on a GPU that runs it well (3584 -> 37888 18.1 -> 17.6 us, 4096 -> 28672 16.0 -> 16.2, 3072 -> 32064 13.8 -> 13.5), and this kernel
     // moved far less from one GPU to the next (on two others the same three calls took 21-22.5 / 18.0-18.3 / 16.8-17.0 us there
     // against 18.8 / 16.5 / 14.9-15.4 at five rows here). More columns lose (4096 -> 128256: 56.4 -> 62.3), and so do three rows.
-    if (a->m == 4 && !pair && a->gamma == nullptr && a->block_size == 128) return a->n >= 18432 && a->n < 49152;
+    // A gate/up pair counts both projections' columns, as below: its single launch went from 20.9 to 18.9 us at four rows on
+    // 3584 -> 2 x 18944 (the unfused call over 37888 columns: 18.5).
+    if (four_row_wide(a, a->n * (pair ? 2 : 1))) return a->gamma == nullptr;
     return a->m >= 5 && a->m <= max_rows && a->n * (pair ? 2 : 1) >= min_cols;
 }
 
@@ -1455,6 +1463,10 @@ extern "C" int rocm_launch_pack_decode(const RocmMatMulNBitsArgs* a, void* packe
 extern "C" int rocm_decode_packed_fuses_norm(const RocmMatMulNBitsArgs* a)
 {
     if (!a->gamma || a->m > 4 || a->k % 128 != 0 || !rocm_decode_packed_eligible(a)) return 0;      // (with gamma, up to four rows never take the shared-activation kernel)
+    // Where four rows take the shared-activation kernel (alone, or as one projection of a pair), the rows are normalized by a
+    // launch of their own: a pair's first call runs its projections over normalized rows, and the later single launch has to
+    // add up in the same order.
+    if (four_row_wide(a, a->n) || four_row_wide(a, 2 * a->n)) return 0;
     if (a->gamma_dtype != ROCM_DT_F32 && a->gamma_dtype != a->a_dtype) return 0;
     return (reinterpret_cast<uintptr_t>(a->gamma) & 15) == 0;
 }
