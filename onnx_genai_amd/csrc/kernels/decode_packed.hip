@@ -1391,10 +1391,12 @@ static int packed_chunk_bytes(const RocmMatMulNBitsArgs* a)
 // (16 rows at block size 32, 32 at 64, 64 at 128: more row blocks than that do not fit the register file)
 // `pair`: the call is the fused gate/up launch or one of its two projections - both projections' columns count, since the
 // paired launch streams both, and a projection launched on its own must add up the way the paired launch does.
-// Four rows at block 128 on 18432 .. 49151 columns: the shared-activation kernel's window below five rows.
-static bool four_row_wide(const RocmMatMulNBitsArgs* a, int64_t cols)
+// The shared-activation kernel's window below five rows: block 128 on 18432 .. 49151 columns, four rows of a plain call, two to
+// four of a gate/up pair (whose columns count together).
+static bool few_row_wide(const RocmMatMulNBitsArgs* a, bool pair)
 {
-    return a->m == 4 && a->block_size == 128 && cols >= 18432 && cols < 49152;
+    const int64_t cols = a->n * (pair ? 2 : 1);
+    return a->m <= 4 && a->m >= (pair ? 2 : 4) && a->block_size == 128 && cols >= 18432 && cols < 49152;
 }
 
 static bool wide_shape(const RocmMatMulNBitsArgs* a, bool pair)
@@ -1413,9 +1415,11 @@ static bool wide_shape(const RocmMatMulNBitsArgs* a, bool pair)
     // on a GPU that runs it well (3584 -> 37888 18.1 -> 17.6 us, 4096 -> 28672 16.0 -> 16.2, 3072 -> 32064 13.8 -> 13.5), and this kernel
     // moved far less from one GPU to the next (on two others the same three calls took 21-22.5 / 18.0-18.3 / 16.8-17.0 us there
     // against 18.8 / 16.5 / 14.9-15.4 at five rows here). More columns lose (4096 -> 128256: 56.4 -> 62.3), and so do three rows.
-    // A gate/up pair counts both projections' columns, as below: its single launch went from 20.9 to 18.9 us at four rows on
-    // 3584 -> 2 x 18944 (the unfused call over 37888 columns: 18.5).
-    if (four_row_wide(a, a->n * (pair ? 2 : 1))) return a->gamma == nullptr;
+    // A gate/up pair counts both projections' columns, as below, and comes here from two rows: the paired four-row split-K
+    // launch is further behind than the plain one (3584 -> 2 x 18944 at 2 / 3 / 4 rows: 20.2-21.2 / 20.5-21.1 / 20.9 -> 17.9 / 18.5 /
+    // 18.9 us, the unfused call over 37888 columns 18.5 at four; 5120 -> 2 x 13824: 20.0 / 20.4-21.3 -> 18.6-18.9 / 19.0-19.7;
+    // 4096 -> 2 x 14336 level).
+    if (few_row_wide(a, pair)) return a->gamma == nullptr;
     return a->m >= 5 && a->m <= max_rows && a->n * (pair ? 2 : 1) >= min_cols;
 }
 
@@ -1463,10 +1467,10 @@ extern "C" int rocm_launch_pack_decode(const RocmMatMulNBitsArgs* a, void* packe
 extern "C" int rocm_decode_packed_fuses_norm(const RocmMatMulNBitsArgs* a)
 {
     if (!a->gamma || a->m > 4 || a->k % 128 != 0 || !rocm_decode_packed_eligible(a)) return 0;      // (with gamma, up to four rows never take the shared-activation kernel)
-    // Where four rows take the shared-activation kernel (alone, or as one projection of a pair), the rows are normalized by a
-    // launch of their own: a pair's first call runs its projections over normalized rows, and the later single launch has to
-    // add up in the same order.
-    if (four_row_wide(a, a->n) || four_row_wide(a, 2 * a->n)) return 0;
+    // Where up to four rows take the shared-activation kernel (alone, or as one projection of a pair), the rows are normalized
+    // by a launch of their own: a pair's first call runs its projections over normalized rows, and the later single launch has
+    // to add up in the same order.
+    if (few_row_wide(a, false) || few_row_wide(a, true)) return 0;
     if (a->gamma_dtype != ROCM_DT_F32 && a->gamma_dtype != a->a_dtype) return 0;
     return (reinterpret_cast<uintptr_t>(a->gamma) & 15) == 0;
 }

@@ -844,6 +844,8 @@ def test_gate_up_swiglu_single_launch(ep, port, a_dt, s_dt, bs, zero_points, m, 
     (E.BF16, E.BF16, 128, 16, 18944, 3584, False),    # the 7B pair: fewer workgroups than CUs per projection alone (weights and windows ahead)
     (E.BF16, E.BF16, 128, 4, 18944, 3584, True),      # four rows at block 128 with 18432 .. 49151 columns in the pair: this kernel too
     (E.F16, E.F16, 128, 4, 9216, 512, False),          # ... its lower edge
+    (E.BF16, E.BF16, 128, 2, 18944, 1024, False),     # ... a pair from two rows
+    (E.F16, E.F32, 128, 3, 9300, 640, True),
     (E.BF16, E.BF16, 128, 5, 14336, 512, True),
     (E.F16, E.F16, 64, 9, 14400, 640, False),         # ragged: the last workgroup's waves run out of column groups
     (E.F16, E.F32, 32, 16, 14336, 256, False),
