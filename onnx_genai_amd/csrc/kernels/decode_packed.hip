@@ -1,4 +1,4 @@
-// Decode path of MatMulNBits over weights repacked for streaming (f16/bf16 activations; M <= 4, or M <= 64 when N is large).
+// Decode path of MatMulNBits over weights repacked for streaming (f16/bf16 activations; M <= 16 at every width, up to 64 rows when N is large).
 //
 // When B, scales and zero points are constant initializers, the kernel object repacks them once into
 // the order in which the split-K MFMA kernel consumes them, so that every vector load of a wave is

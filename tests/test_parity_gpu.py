@@ -236,7 +236,7 @@ def test_decode_matches_oracle(ep, ep_unpacked, port, prepack, a_dt, s_dt, bs, z
     # f32 output: the arithmetic itself, before any narrowing
     y32, variant = run_op(ep, a, a_dt, b, s, s_dt, zp, n, k, bs, bias=bias, bias_dtype=a_dt, y_dtype=E.F32)
     if m <= 16:
-        # up to 16 rows read the repacked stream at every width (the shared-activation kernel from 14336 columns and 5 rows)
+        # up to 16 rows read the repacked stream at every width (the split-K kernel, or the shared-activation kernel where the call is wide enough)
         assert variant == ("decode_mfma_packed" if prepack else "decode_mfma_splitk")
     else:
         # m <= 32: two row blocks through the decode kernel where that beats the tiled kernel (block 128, few columns or rows)
