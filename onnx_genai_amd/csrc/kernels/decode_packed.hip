@@ -1620,6 +1620,12 @@ static int launch_decode_packed(const RocmMatMulNBitsArgs* a, const void* packed
             }
         }
     }
+    // A projection of a gate/up pair takes at most half a workgroup's waves where that leaves a wave five tile groups or fewer,
+    // so that the pair runs as one launch and not as two and the epilogue (bf16, one / two / four rows: 3072 -> 2 x 8192 at block 32
+    // 14.3 -> 9.1 us at one row; 5120 -> 2 x 13824 at block 32 25.5 / 30.9 / 32.6 -> 20.6 / 25.4 / 25.7, at block 64 24.1 / 26.5 / 28.0 ->
+    // 18.8 / 21.7 / 22.8; 8192 -> 2 x 8192 at block 64 22.5 / 25.3 / 26.8 -> 17.7 / 18.6 / 19.9). The projection launched alone on a
+    // pair's first call takes the same count, as everything here.
+    if (pair_member && a->m <= 4 && waves <= 0 && 2 * w > w_max && (p.groups + w_max / 2 - 1) / (w_max / 2) <= 5) w = w_max / 2;
     const int gpw = (p.groups + w - 1) / w;
     w = (p.groups + gpw - 1) / gpw;
     p.groups_per_wave = gpw;

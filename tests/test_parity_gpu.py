@@ -801,7 +801,9 @@ def test_gate_up_swiglu(ep_unpacked, port, a_dt, s_dt, bs, zero_points, m, n, k,
 
 @pytest.mark.parametrize("a_dt,s_dt,bs,zero_points,m,n,k,decomposed", [c for c in SWIGLU_CASES if c[4] <= 4] + [
     (E.BF16, E.BF16, 128, True, 1, 18944, 3584, False),      # the 7B gate/up pair at full size: seven waves per projection
-    (E.F16, E.F16, 32, True, 2, 96, 4096, False),            # more waves per projection than half a workgroup holds: stays on two launches
+    (E.F16, E.F16, 32, True, 2, 96, 4096, False),            # more waves per projection than half a workgroup holds: each takes half, two tile groups a wave
+    (E.BF16, E.BF16, 64, True, 1, 520, 8192 + 64, True),     # ... five tile groups a wave, the last one partial
+    (E.F16, E.F16, 32, True, 2, 96, 16384, False),           # eight tile groups a wave would be too many: stays on two launches
 ])
 def test_gate_up_swiglu_single_launch(ep, port, a_dt, s_dt, bs, zero_points, m, n, k, decomposed):
     """From the second call on, up to four rows over constant weights run as one launch over both repacked copies, with
@@ -817,7 +819,8 @@ def test_gate_up_swiglu_single_launch(ep, port, a_dt, s_dt, bs, zero_points, m, 
         assert ops.kernel.last_variant() == "gate_up_swiglu[decode_mfma_packed]"
         ep.copy_from_host(yb, np.full(m * n * 2, 0xFF, np.uint8))
         ops.run(ab, a_dt, m, yb)
-        single = k <= 2048 or bs == 128
+        half_workgroup = 8 if bs == 128 and s_dt != E.F32 else 4           # waves a projection may take in the paired launch
+        single = -(-(-(-k // 512)) // half_workgroup) <= 5
         assert ops.kernel.last_variant() == ("gate_up_swiglu_packed" if single else "gate_up_swiglu[decode_mfma_packed]")
         assert np.array_equal(ep.download(yb, (m, n), np.uint16), first)
         ep.sync()
