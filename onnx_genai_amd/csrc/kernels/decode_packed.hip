@@ -1578,14 +1578,15 @@ static int launch_decode_packed(const RocmMatMulNBitsArgs* a, const void* packed
     // block 32: 15.8 against 21.7). Two sets keep:
     //  * two to four rows on small grids, where the second set's first fetch, issued before anything else, is worth 1-3 %
     //    (block 128, 3584 -> 4608: 5.56 against 5.72 us; 18944 -> 3584 at block 32: 13.3 against 13.9) - below 256 column groups at
-    //    block 32, else below 640, or below 320 when K is more than eight groups;
+    //    block 32, else up to 512 (two workgroups per CU: 4096 -> 8192 6.4 against 6.5 us at two rows, but 4096 -> 9216 7.7 against
+    //    7.3 and 3072 -> 9216 7.75 against 6.8), or below 320 when K is more than eight groups;
     //  * one row at block size 32 with more groups than a workgroup has waves, on small grids: sixteen scale steps per group
     //    leave enough arithmetic between a wave's loads that fetching ahead pays (18944 -> 3584 12.4 -> 11.8 us; with 1024
     //    column groups it loses, 5120 -> 16384: 17.3 against 12.2; at block 128 one set stays ahead, 9.5 against 9.9 us).
     bool single_set;
     if (one_row) single_set = !(a->block_size == 32 && p.groups > w_max && wgs <= 256);
     else if (a->block_size == 32) single_set = wgs >= 256;
-    else single_set = wgs >= 640 || (wgs >= 320 && p.groups > 8);
+    else single_set = wgs > 512 || (wgs >= 320 && p.groups > 8);
     if (w > w_max) w = w_max;
     if (w > p.groups) w = p.groups;
     // Mid-size grids: a launch whose waves do not all fit the chip at once queues workgroups behind each other, and
