@@ -1604,13 +1604,20 @@ static int launch_decode_packed(const RocmMatMulNBitsArgs* a, const void* packed
         const int per_simd = waves_per_simd(a, f32_scales);
         const int64_t fit = 256 * 4 * per_simd / wgs;
         const int64_t least = a->m <= 1 ? 6 : a->m <= 4 ? 4 : 1;
-        if (fit >= least && w > fit) {
-            w = static_cast<int>(fit);
+        // A count within that bound can still be too many once the waves' places on the SIMDs are counted (576 workgroups of six
+        // waves at five waves per SIMD: two workgroups a CU, 3072 slots for 3456 waves). Then the count that holds the most is
+        // taken as well, if it leaves a wave two tile groups at most (block 32, two / four rows: 3072 -> 9216 8.9 / 8.9 -> 8.3 / 8.7 us,
+        // 3072 -> 12288 10.0 / 10.1 -> 8.5 / 9.0; block 128, five / eight rows: 3072 -> 12288 9.2 -> 8.1; with three groups a wave it
+        // lost, 5120 -> 10240 at block 32: 10.1 -> 10.8).
+        const bool crowded = per_simd <= 5 && w <= fit && wgs * w > 256 * static_cast<int64_t>(per_simd / ((w + 3) / 4) * w);
+        if (fit >= least && (w > fit || crowded)) {
+            if (w > fit) w = static_cast<int>(fit);
+            const int limit = w;
             if (per_simd <= 5) {                       // (with six or more waves per SIMD the plain count is as good or better: 4 rows at block 128, 6144 -> 16384: six waves 14.2 us, four 15.4)
                 int best = -1;
                 for (int g = 1; g <= p.groups; ++g) {
                     const int cand = (p.groups + g - 1) / g;
-                    if (cand > fit) continue;
+                    if (cand > limit || (crowded && g > 2)) continue;
                     const int held = per_simd / ((cand + 3) / 4) * cand;
                     if (held > best) {                 // (ties: the first found, which has the most waves)
                         best = held;
