@@ -286,6 +286,10 @@ OrtStatus* ORT_API_CALL compute_compute(OrtNodeComputeInfo* this_ptr, void* comp
                 if (md && (host.ep_api->MemoryDevice_GetDeviceType(md) != OrtMemoryInfoDeviceType_GPU || host.ep_api->MemoryDevice_GetVendorId(md) != kAmdVendorId))
                     return host.status(ORT_INVALID_ARGUMENT, "MatMulNBits: input " + std::to_string(i) + " is not in ROCm device memory (the session must allocate "
                                                              "this node's tensors with the ROCm execution provider's allocator)");
+                if (md && host.ep_api->MemoryDevice_GetDeviceId && host.ep_api->MemoryDevice_GetDeviceId(md) != device)
+                    return host.status(ORT_INVALID_ARGUMENT, "MatMulNBits: input " + std::to_string(i) + " lives on GPU " +
+                                                             std::to_string(host.ep_api->MemoryDevice_GetDeviceId(md)) + ", this execution provider runs on GPU " +
+                                                             std::to_string(device));
             }
             v.data = const_cast<void*>(data);
             v.dtype = static_cast<uint32_t>(et);
@@ -675,6 +679,12 @@ OrtStatus* CreateEpFactories(const char* registration_name, const OrtApiBase* ap
 {
     if (num_factories) *num_factories = 0;
     if (!api_base || !api_base->GetApi) return nullptr;        // no host API: there is nothing to build a status with
+#if !defined(NXRT_ORT_REAL_HEADERS)
+    // Built against the subset header: OrtApi / OrtEpApi members sit at that header's offsets, not at onnxruntime's. Only a
+    // host that announces the same layout is called through them; any other gets no factory and no call into its tables.
+    const char* host_version = api_base->GetVersionString ? api_base->GetVersionString() : nullptr;
+    if (!host_version || !std::strstr(host_version, ORT_SUBSET_LAYOUT_MARKER)) return nullptr;
+#endif
     const OrtApi* api = api_base->GetApi(ORT_API_VERSION);
     if (!api) return nullptr;                                   // the host is older than the API this plugin was built for
     Host host;

@@ -16,81 +16,9 @@
 #include <type_traits>
 
 #include <cmath>
-#include "mfma_common.hiph"
+#include "prefill_common.hiph"
 
 namespace mnb {
-
-typedef __attribute__((ext_vector_type(8))) _Float16 half8_t;
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
-typedef __attribute__((ext_vector_type(16))) float float16_t;
-typedef __attribute__((ext_vector_type(2))) _Float16 half2_t;
-
-struct PrefillParams {
-    const uint16_t* a;
-    const uint8_t* b;
-    const void* scales;
-    const uint8_t* zp;
-    const void* bias;
-    void* y;
-    int64_t m, n, k, kb;
-    int64_t row_bytes, zp_row;
-    int bs_log2;
-    int scale_dtype, bias_dtype, y_dtype;
-    int steps_per_split;    // K steps of 64 per workgroup along grid.z
-    float* partial;         // [splits][M][N] f32 partial sums when K is split (else NULL: the kernel writes Y itself)
-    // 0x000F000F and the two 16-bit magic exponents, as arguments rather than literals: the mask is moved to a vector
-    // register and the magic stays in a scalar one, which is what lets (x & mask) | magic be one v_and_or_b32
-    uint32_t nibble_mask, magic;
-};
-
-constexpr int kBK = 64;
-constexpr int kPitch = 144;            // bytes per LDS row: 64 halfs + 8 of padding
-
-template <bool BF16>
-__device__ __forceinline__ float16_t mfma32(const uint4& a, const uint4& b, float16_t c)
-{
-    if constexpr (BF16) return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
-    else return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, b), c, 0, 0, 0);
-}
-
-// Two nibbles (elements 2i, 2i+1 of a packed dword) as a pair of 16-bit floats carrying magic + q.
-__device__ __forceinline__ uint32_t magic_pair(uint32_t w, uint32_t w4, uint32_t sel, uint32_t mask, uint32_t magic)
-{
-    return (__builtin_amdgcn_perm(w4, w, sel) & mask) | magic;
-}
-
-// f16, f16 scale: exact subtract, one rounding multiply.
-__device__ __forceinline__ uint32_t finish_f16(uint32_t pair, half2_t neg_off, half2_t scale)
-{
-    const half2_t v = (__builtin_bit_cast(half2_t, pair) + neg_off) * scale;
-    return __builtin_bit_cast(uint32_t, v);
-}
-
-// Eight weights of one packed dword as (q - zp) * scale, computed in f32 and rounded once to the 16-bit type (nearest
-// even), in element order. `shift` is (16 - zp) in every byte: the bytes q + 16 - zp (1..31, no borrow between them)
-// convert to f32 with one instruction each, and t * scale - 16 * scale in one FMA is exactly (q - zp) * scale rounded
-// once, because 16 * scale is exact.
-typedef __attribute__((ext_vector_type(2))) float float2_t;
-typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
-template <bool BF16>
-__device__ __forceinline__ uint4 dequant_dword_f32(uint32_t w, uint32_t shift, float scale, float neg16_scale)
-{
-    uint32_t even = (w & 0x0f0f0f0fu) + shift;            // elements 0, 2, 4, 6, one per byte
-    uint32_t odd = ((w >> 4) & 0x0f0f0f0fu) + shift;      // elements 1, 3, 5, 7
-    asm volatile("" : "+v"(even), "+v"(odd));             // keep the bytes whole: one byte-to-float convert each
-    uint32_t out[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const float lo = fmaf(static_cast<float>((even >> (8 * i)) & 0xffu), scale, neg16_scale);
-        const float hi = fmaf(static_cast<float>((odd >> (8 * i)) & 0xffu), scale, neg16_scale);
-        if constexpr (BF16) {
-            out[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(float2_t{lo, hi}, bf16x2_t));   // v_cvt_pk_bf16_f32
-        } else {
-            out[i] = static_cast<uint32_t>(f32_to_f16_bits(lo)) | (static_cast<uint32_t>(f32_to_f16_bits(hi)) << 16);
-        }
-    }
-    return make_uint4(out[0], out[1], out[2], out[3]);
-}
 
 // BF16: element type. BM x BN: tile of Y per workgroup (128 x 64, 128 x 128, 256 x 128 or 256 x 256). SF32: scales are stored
 // as f32 (otherwise in the activations' 16-bit type). f16 activations with f16 scales dequantize in packed f16,
@@ -280,77 +208,7 @@ __global__ __launch_bounds__(512) void prefill_mfma_kernel(PrefillParams p)
         }
     }
 
-    // Epilogue. A 32x32 accumulator holds, in lane l, column l % 32 and rows 8 q + 4 (l / 32) + r (q, r = 0..3).
-    // The three forms (slice partials, one bias per column, one bias per element) are separate loops behind
-    // wave-uniform branches; the first two are fully unrolled over the accumulators and must stay small, or the
-    // compiler keeps the accumulators of the 256x256 tile in scratch memory for the whole kernel.
-    const int col_in_tile = lane & 31;
-    const int row_group = (lane >> 5) * 4;
-    const bool per_row = (p.bias_dtype & ROCM_BIAS_PER_ROW) != 0;
-    auto for_each = [&](auto&& store) {
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            const int64_t col = n_base + wn * WN + j * 32 + col_in_tile;
-            if (col >= p.n) continue;
-#pragma unroll
-            for (int i = 0; i < TM; ++i) {
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        const int64_t row = m_base + wm * WM + i * 32 + q * 8 + row_group + r;
-                        if (row >= p.m) continue;
-                        store(row, col, acc[i][j][q * 4 + r]);
-                    }
-                }
-            }
-        }
-    };
-    if (p.partial) {                                                                           // slices: the reduce kernel adds the bias
-        float* part = p.partial + static_cast<int64_t>(blockIdx.z) * p.m * p.n;
-        for_each([&](int64_t row, int64_t col, float v) { part[row * p.n + col] = v; });
-    } else if (per_row) {
-        // The bias differs per element, so its load (a choice among three types) sits in a loop that is not
-        // unrolled: sixteen accumulators at a time go through the wave's own 4 KiB of LDS, which gives that loop a
-        // run-time index. The tiles in LDS are dead once every wave is past its last step.
-        __syncthreads();
-        float* stage = reinterpret_cast<float*>(smem) + wave * (16 * 64) + lane;
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            const int64_t col = n_base + wn * WN + j * 32 + col_in_tile;
-#pragma unroll
-            for (int i = 0; i < TM; ++i) {
-#pragma unroll
-                for (int e = 0; e < 16; ++e) stage[e * 64] = acc[i][j][e];
-                if (col >= p.n) continue;
-#pragma unroll 1
-                for (int e = 0; e < 16; ++e) {
-                    const int64_t row = m_base + wm * WM + i * 32 + (e >> 2) * 8 + row_group + (e & 3);
-                    if (row >= p.m) break;
-                    store_from_f32(p.y, p.y_dtype, row * p.n + col, with_bias(stage[e * 64], p.bias, p.bias_dtype, row, p.n, col, p.y_dtype));
-                }
-            }
-        }
-    } else {
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            const int64_t col = n_base + wn * WN + j * 32 + col_in_tile;
-            if (col >= p.n) continue;
-            const BiasTerm bias = load_bias(p.bias, p.bias_dtype, 0, p.n, col);
-#pragma unroll
-            for (int i = 0; i < TM; ++i) {
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        const int64_t row = m_base + wm * WM + i * 32 + q * 8 + row_group + r;
-                        if (row >= p.m) continue;
-                        store_from_f32(p.y, p.y_dtype, row * p.n + col, add_bias(acc[i][j][q * 4 + r], bias, p.y_dtype));
-                    }
-                }
-            }
-        }
-    }
+    store_tile<TM, TN>(p, acc, m_base, n_base, wm * WM, wn * WN, lane, wave, smem);
 }
 
 // Y = sum over slices of the partial sums, in slice order, plus bias; one thread per element.

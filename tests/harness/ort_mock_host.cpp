@@ -203,7 +203,11 @@ static OrtEpApi g_ep_api;
 static OrtApi g_api;
 static const OrtEpApi* api_GetEpApi() { return &g_ep_api; }
 static const OrtApi* base_GetApi(uint32_t version) { return version <= ORT_API_VERSION ? &g_api : nullptr; }
-static const char* base_GetVersionString() { return "1.23.0-mock"; }
+static const char* base_GetVersionString() { return "1.23.0-mock " ORT_SUBSET_LAYOUT_MARKER; }
+// What a real onnxruntime answers: no marker. Its tables must never be touched by a subset build.
+static int g_foreign_get_api_calls = 0;
+static const OrtApi* foreign_GetApi(uint32_t) { ++g_foreign_get_api_calls; return nullptr; }
+static const char* foreign_GetVersionString() { return "1.23.0"; }
 
 static void fill_tables()
 {
@@ -285,6 +289,12 @@ int main(int argc, char** argv)
     CHECK(is_error(create("x", &base, nullptr, factories, 0, &n), ORT_INVALID_ARGUMENT, "room for no factory") && n == 0);
     CHECK(is_error(create("x", &base, nullptr, nullptr, 2, &n), ORT_INVALID_ARGUMENT, "null output"));
     CHECK(release(nullptr) == nullptr);
+    // a host that does not announce the subset layout (a real onnxruntime): no factory, and not one call into its tables
+    const OrtApiBase real_host{foreign_GetApi, foreign_GetVersionString};
+    n = 7;
+    factories[0] = reinterpret_cast<OrtEpFactory*>(1);
+    CHECK(create("x", &real_host, nullptr, factories, 2, &n) == nullptr && n == 0 && g_foreign_get_api_calls == 0);
+    CHECK(factories[0] == reinterpret_cast<OrtEpFactory*>(1));
 
     // ---- a factory under the default name and one under the registration name ----
     CHECK(is_ok(create(nullptr, &base, nullptr, factories, 2, &n)) && n == 1 && factories[1] == nullptr);
@@ -462,6 +472,11 @@ int main(int argc, char** argv)
         OrtValue host_a{va->info, a.data(), host_mem, va->bytes};
         OrtKernelContext bad{{&host_a, vb, vs, vz, nullptr, vbias}, &y, alloc0, 4};
         CHECK(is_error(info[0]->Compute(info[0], state, &bad), ORT_INVALID_ARGUMENT, "not in ROCm device memory"));
+        // nor is one that another AMD GPU holds
+        const OrtMemoryDevice other_gpu{OrtMemoryInfoDeviceType_GPU, 0x1002, 5};
+        OrtValue far_a{va->info, va->data, other_gpu, va->bytes};
+        OrtKernelContext far{{&far_a, vb, vs, vz, nullptr, vbias}, &y, alloc0, 4};
+        CHECK(is_error(info[0]->Compute(info[0], state, &far), ORT_INVALID_ARGUMENT, "lives on GPU 5"));
         alloc0->Free(alloc0, y.data);
         for (OrtValue* v : {va, vb, vs, vz, vbias}) {
             alloc0->Free(alloc0, v->data);

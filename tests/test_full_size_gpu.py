@@ -48,10 +48,11 @@ def sampled_f64(port, a_f32, b, s_f32, zp, cols, k, bs, rows=None):
 
 DECODE_SHAPES = [
     # name, dtype, block, zero points, K, N, rows, scale range
-    ("7b lm_head", E.BF16, 128, True, 3584, 152064, (1, 16), (0.002, 0.01)),
-    ("7b down", E.BF16, 128, True, 18944, 3584, (1, 5, 16), (0.002, 0.01)),
-    ("7b qkv", E.BF16, 128, True, 3584, 4608, (1, 9, 16), (0.002, 0.01)),
-    ("7b gate_up", E.BF16, 128, True, 3584, 37888, (4, 8), (0.002, 0.01)),
+    ("7b lm_head", E.BF16, 128, True, 3584, 152064, (1, 4, 8, 16), (0.002, 0.01)),
+    ("7b down", E.BF16, 128, True, 18944, 3584, (1, 4, 5, 8, 16), (0.002, 0.01)),
+    ("7b qkv", E.BF16, 128, True, 3584, 4608, (1, 4, 8, 9, 16), (0.002, 0.01)),
+    ("7b o", E.BF16, 128, True, 3584, 3584, (1, 4, 8, 16), (0.002, 0.01)),
+    ("7b gate_up", E.BF16, 128, True, 3584, 37888, (1, 4, 8, 16), (0.002, 0.01)),
     ("0.5b lm_head", E.F16, 32, True, 896, 151936, (1,), (0.002, 0.01)),
 ]
 
@@ -81,7 +82,7 @@ def test_decode_configs_at_full_size(ep, port, name, dt, bs, zero_points, k, n, 
         ops.free()
 
 
-PREFILL_SHAPES = [(4096, 14336, 2048), (14336, 4096, 2048), (4096, 14336, 8192), (14336, 4096, 512)]
+PREFILL_SHAPES = [(4096, 14336, 512), (14336, 4096, 512), (4096, 14336, 2048), (14336, 4096, 2048), (4096, 14336, 8192), (14336, 4096, 8192)]
 
 
 @pytest.mark.parametrize("route", ["hand_written", "default"])
@@ -113,7 +114,8 @@ def test_prefill_configs_at_full_size(ep, ep_tiled, port, route, k, n, m):
     assert helpers.rel_l2(y[np.ix_(rows, cols)].astype(np.float64), want) <= TOL_HALF, variant
 
 
-ACC4_SHAPES = [(8192, 28672, 1), (8192, 28672, 8), (28672, 8192, 16), (8192, 28672, 256), (28672, 8192, 1), (28672, 8192, 256), (8192, 10240, 4096)]
+ACC4_SHAPES = [(8192, 28672, 1), (8192, 28672, 8), (28672, 8192, 16), (8192, 28672, 256), (28672, 8192, 1), (28672, 8192, 256), (8192, 10240, 4096),
+               (8192, 28672, 4096), (28672, 8192, 4096), (8192, 10240, 1), (8192, 10240, 256)]
 
 
 @pytest.mark.parametrize("k,n,m", ACC4_SHAPES)

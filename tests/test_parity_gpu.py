@@ -501,9 +501,12 @@ def test_prefill_matches_oracle(ep_tiled, port, a_dt, s_dt, bs, zero_points, m, 
 
 @pytest.mark.parametrize("tile", [1, 2, 3, 4])
 @pytest.mark.parametrize("a_dt,s_dt,bs,zero_points", [(E.F16, E.F16, 32, True), (E.BF16, E.F32, 128, False), (E.BF16, E.BF16, 64, True)])
-def test_prefill_tile_shapes_agree(port, tile, a_dt, s_dt, bs, zero_points):
-    """Every workgroup tile (128 x 128, 256 x 128, 256 x 256, 128 x 64) on a shape with ragged edges in M and N."""
-    m, n, k = 300, 520, 1024
+@pytest.mark.parametrize("n", [520, 515])
+def test_prefill_tile_shapes_agree(port, tile, a_dt, s_dt, bs, zero_points, n):
+    """Every workgroup tile (128 x 128, 256 x 128, 256 x 256, 128 x 64) on a shape with ragged edges in M and N. With N a
+    multiple of 8 the 16-bit outputs leave through the wide stores (16 bytes per lane after a turn through LDS), otherwise
+    element by element: both against the same expectations."""
+    m, k = 300, 1024
     provider = E.RocmExecutionProvider(0, {"prefill_tile": str(tile)})
     try:
         b, s, zp = synth.make_weights(n, k, bs, 41, zero_points=zero_points, scale_lo=0.002, scale_hi=0.01, scale_dtype=s_dt)
