@@ -106,7 +106,7 @@ def build(force: bool = True) -> str:
     spilled = {n: u for n, u in usage.items() if u.get("ScratchSize [bytes/lane]", 0) or u.get("VGPRs Spill", 0)}
     if spilled:
         raise RuntimeError("kernels that use scratch memory:\n" + "\n".join(f"  {n}: {u}" for n, u in sorted(spilled.items())))
-    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs, "-L/opt/rocm/lib", "-lhipblaslt", "-Wl,-z,defs", "-Wl,--exclude-libs,ALL"])
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs, "-ldl", "-Wl,-z,defs", "-Wl,--exclude-libs,ALL"])
     return LIB
 
 

@@ -255,11 +255,15 @@ bool use_packed(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& args, int& r
     return true;
 }
 
-// Tall 16-bit calls: expand the weights to a dense [N, K] matrix of the activations' type and run the library GEMM (the
-// CUDA provider's route for M >= 8, onnx-runtime-ep-cuda/src/kernels/matmul_nbits.rs:6176-6222). Returns false with
-// nothing launched when the route does not apply or is not ready (then the tiled kernel takes the call): too few rows,
-// another dtype mix, a dense copy beyond the configured size, no library kernel for the shape, or a first use while a
-// graph capture is open (nothing may allocate then).
+// Tall 16-bit calls over a dense [N, K] copy of the weights in the activations' type, expanded by a launch of its own. Two users:
+//  * the opt-in library route (dense_gemm_min_rows > 0): the product is the library GEMM, as in the CUDA provider for M >= 8
+//    (onnx-runtime-ep-cuda/src/kernels/matmul_nbits.rs:6176-6222);
+//  * by default, calls of more than 16 rows whose weights the tile loader does not read - bits = 2 / 8 and weights with g_idx
+//    (matmul_nbits.rs:2035, 3636-3658): the product is this provider's own tiled kernel over the dense copy, instead of a
+//    one-wave-per-column GEMV that reads all M rows of A per column.
+// Returns false with nothing launched when the route does not apply or is not ready (then the caller's next route takes the
+// call): too few rows, another dtype mix, a dense copy beyond the configured size, no library kernel for the shape, or a first
+// use while a graph capture is open (nothing may allocate then).
 bool dense_route(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& args, int& rc)
 {
     rc = 0;
@@ -268,22 +272,28 @@ bool dense_route(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& args, int& 
     // other bit widths have no tiled kernel to fall back on, only the plain GEMV: the route pays from a few dozen rows
     const bool plain_only = kn.bits != 4 || args.g_idx != nullptr;
     const int64_t min_rows = !plain_only ? ep.dense_gemm_min_rows : (ep.dense_gemm_min_rows < 32 ? ep.dense_gemm_min_rows : 32);
-    if (ep.dense_gemm_min_rows <= 0 || args.m < min_rows) return false;
-    if ((args.a_dtype != ROCM_DT_F16 && args.a_dtype != ROCM_DT_BF16) || args.y_dtype != args.a_dtype || (args.k & 7) != 0) return false;
-    if ((reinterpret_cast<uintptr_t>(args.a) & 15) != 0 || (reinterpret_cast<uintptr_t>(args.y) & 15) != 0 || (reinterpret_cast<uintptr_t>(args.b) & 3) != 0) return false;
+    bool library = ep.dense_gemm_min_rows > 0 && args.m >= min_rows;
+    if ((args.a_dtype != ROCM_DT_F16 && args.a_dtype != ROCM_DT_BF16) || (args.k & 7) != 0) return false;
+    if ((reinterpret_cast<uintptr_t>(args.a) & 15) != 0 || (reinterpret_cast<uintptr_t>(args.b) & 3) != 0) return false;
     const uint64_t need = static_cast<uint64_t>(args.n) * static_cast<uint64_t>(args.k) * 2;
     if (need > ep.dense_gemm_max_bytes) return false;
-    if (args.bias && (args.bias_dtype & (ROCM_BIAS_POST_ROUND | ROCM_BIAS_PER_ROW))) return false;      // the library's epilogue adds a [N] bias before the one rounding
+    // what the library cannot take: another output type, an unaligned Y, a bias its epilogue does not add before the one rounding
+    if (args.y_dtype != args.a_dtype || (reinterpret_cast<uintptr_t>(args.y) & 15) != 0 ||
+        (args.bias && (args.bias_dtype & (ROCM_BIAS_POST_ROUND | ROCM_BIAS_PER_ROW))))
+        library = false;
+    const bool own = plain_only && rocm_prefill_dense16_eligible(&args);      // (more than 16 rows, K a multiple of 64)
+    if (!library && !own) return false;
     const int bias_dtype = args.bias ? args.bias_dtype : -1;
 
     std::lock_guard<std::mutex> lock(ep.dense_mu);
-    if (!ep.dense) {
-        if (ep.capturing || rocm_dense_gemm_create(&ep.dense) != 0) {
+    if (library) {
+        if (!ep.dense && (ep.capturing || rocm_dense_gemm_create(&ep.dense) != 0)) {
             ep.dense = nullptr;
-            return false;
+            library = false;
         }
+        if (library && !rocm_dense_gemm_ready(ep.dense, args.m, args.n, args.k, args.a_dtype, bias_dtype, ep.capturing ? 0 : 1)) library = false;
+        if (!library && !own) return false;      // no library kernel for the shape: the tiled kernel over the dense copy where it applies
     }
-    if (!rocm_dense_gemm_ready(ep.dense, args.m, args.n, args.k, args.a_dtype, bias_dtype, ep.capturing ? 0 : 1)) return false;
 
     const bool constant = kn.constant_inputs[1] && kn.constant_inputs[2] && (!args.zp || kn.constant_inputs[3]) && !args.g_idx;
     auto expand = [&](void* dst) {
@@ -316,7 +326,7 @@ bool dense_route(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& args, int& 
             kn.dense_scale_dtype = args.scale_dtype;
         }
         w16 = kn.dense;
-        kn.variant = "dense_resident_blaslt";
+        kn.variant = library ? "dense_resident_blaslt" : "dense_resident_tiled";
     } else {
         if (ep.dense_scratch_bytes < need) {
             if (ep.capturing) return false;
@@ -324,9 +334,11 @@ bool dense_route(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& args, int& 
         }
         rc = expand(ep.dense_scratch);
         w16 = ep.dense_scratch;
-        kn.variant = "dense_transient_blaslt";
+        kn.variant = library ? "dense_transient_blaslt" : "dense_transient_tiled";
     }
-    if (rc == 0) rc = rocm_dense_gemm_run(ep.dense, w16, args.a, args.y, args.bias, args.bias_dtype, args.m, args.n, args.k, args.a_dtype, ep.stream);
+    if (rc != 0) return true;
+    if (library) rc = rocm_dense_gemm_run(ep.dense, w16, args.a, args.y, args.bias, args.bias_dtype, args.m, args.n, args.k, args.a_dtype, ep.stream);
+    else rc = rocm_launch_prefill_dense16(&args, w16, ep.prefill_tile, nullptr, 0, ep.stream);       // (no slices of K: they would want scratch of their own)
     return true;
 }
 

@@ -30,9 +30,13 @@ const char* rocm_ffi_error_string(int err);
 int rocm_ffi_device_count(int* count);
 int rocm_ffi_set_device(int device);
 int rocm_ffi_device_info(int device, char* arch, size_t arch_len, int* compute_units, size_t* total_mem);
+/* Compute units of the current device (asked once per device and kept); 256, the MI355X's count, when it cannot be asked.
+ * The launchers size grids and wave counts to it. */
+int rocm_ffi_compute_units(void);
 int rocm_ffi_malloc(void** ptr, size_t bytes);
 int rocm_ffi_free(void* ptr);
-/* How many times rocm_ffi_malloc has been called in this process (every device allocation of the library goes through it). */
+/* How many times rocm_ffi_malloc has been called in this process. Every device allocation of the library goes through it, the
+ * library GEMM route's workspace and the g_idx range check's flag included. */
 uint64_t rocm_ffi_malloc_calls(void);
 /* Device address and size of the library's static scratch array on `device` (a __device__ array of the code object, 256-byte
  * aligned, one per GPU, never freed). The first call for a device makes that device current and resolves the address; later
@@ -141,6 +145,19 @@ int rocm_decode_packed_eligible(const RocmMatMulNBitsArgs* args);
 uint64_t rocm_decode_packed_bytes(const RocmMatMulNBitsArgs* args);
 int rocm_launch_pack_decode(const RocmMatMulNBitsArgs* args, void* packed, rocm_stream_t stream);
 int rocm_launch_decode_packed(const RocmMatMulNBitsArgs* args, const void* packed, int waves, rocm_stream_t stream);
+/* What rocm_launch_decode_packed would launch for `args` on a chip of `compute_units` CUs, without launching anything (only the
+ * shape, dtypes, block size and gamma of `args` are read). pair_member: 0 = a plain call, 1 = one projection of a gate/up pair
+ * launched alone, 2 = the paired launch. -1: the shape does not take this route. */
+typedef struct RocmDecodePackedPlan {
+  int shared_activations;   /* 1: the kernel that shares one LDS copy of the activations; 0: the split-K kernel */
+  int rows_build;           /* rows the build stages: 1, 4, 8 or 16 (shared activations: 16, 32 or 64) */
+  int waves;                /* per workgroup (split-K kernel: per projection) */
+  int groups_per_wave;      /* tile groups of 512 k a wave walks */
+  int register_sets;        /* sets of load registers in flight: 1 or 2 (shared activations: 1 + weights ahead + windows two ahead) */
+  int activation_sums;      /* 1: offset and zero point leave through the block activation sums; 0: through a second MFMA */
+  int64_t workgroups;
+} RocmDecodePackedPlan;
+int rocm_decode_packed_plan(const RocmMatMulNBitsArgs* args, int waves, int pair_member, int compute_units, RocmDecodePackedPlan* out);
 /* 1 when the launch above (and the paired one below) applies args->gamma inside the kernel: up to 4 rows, K % 128 == 0, gamma f32 or
  * of the activations' type and 16-byte aligned, and a shape the split-K kernel takes (not the shared-activation one). */
 int rocm_decode_packed_fuses_norm(const RocmMatMulNBitsArgs* args);
@@ -171,6 +188,11 @@ int rocm_prefill_mfma_plan(const RocmMatMulNBitsArgs* args, int tile_choice, uin
 int rocm_launch_slice_reduce(const float* partial, int slices, int64_t m, int64_t n, const void* bias, int bias_dtype, void* y, int y_dtype,
                              rocm_stream_t stream);
 int rocm_launch_prefill_mfma(const RocmMatMulNBitsArgs* args, int tile_choice, void* scratch, uint64_t scratch_bytes, rocm_stream_t stream);
+/* The same tiled kernel over weights that a launch of their own has expanded to a dense [N, K] matrix of the activations' 16-bit
+ * type (w16_nk, 16-byte aligned; K % 64 == 0): the tall route of bits = 2 / 8 and of weights with g_idx, whose packed forms the
+ * tile loader does not read. args->b / scales / zp are not read; tiles of 128 columns at most. */
+int rocm_prefill_dense16_eligible(const RocmMatMulNBitsArgs* args);
+int rocm_launch_prefill_dense16(const RocmMatMulNBitsArgs* args, const void* w16_nk, int tile_choice, void* scratch, uint64_t scratch_bytes, rocm_stream_t stream);
 
 /* accuracy_level 4. rounding: 0 = ties to even (MLAS rule), 1 = ties away (native Rust rule).
  * qa: int8 [M, kb*bs]; qscale: f32 [M, kb]; qsum: int32 [M, kb] (sum of codes per block). */
@@ -209,6 +231,9 @@ int rocm_acc4_packed_eligible(const RocmMatMulNBitsArgs* args);
  * K % 8 == 0, 16-byte aligned) with the given rounding rule; otherwise codes and pairs come from the workspace. */
 int rocm_acc4_packed_fuses_quantizer(const RocmMatMulNBitsArgs* args);
 int rocm_launch_acc4_packed(const RocmMatMulNBitsArgs* args, const void* packed, const RocmAcc4Workspace* ws, int rounding, int waves, rocm_stream_t stream);
+/* The split of K that launch takes on a chip of `compute_units` CUs (no GPU work): waves per workgroup, tile groups of 512 k per
+ * wave, register sets (1 or 2). -1: the shape does not take this route. */
+int rocm_acc4_packed_plan(const RocmMatMulNBitsArgs* args, int waves, int compute_units, int* waves_out, int* groups_per_wave, int* register_sets);
 
 #ifdef __cplusplus
 }

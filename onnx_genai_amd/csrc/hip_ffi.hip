@@ -6,12 +6,13 @@
 #include <mutex>
 
 #include "hip_ffi.h"
+#include "../../include/nxrt_ep_rocm.h"      // NXRT_ROCM_STATIC_SCRATCH_BYTES: the size the public header promises is the size of the array
 
 namespace {
 // Scratch for the entry point that may not allocate (rocm_ffi_static_scratch): one array per GPU, part of the code object,
 // alive from the moment the library is loaded on a device until the process ends. Host code never uses this name as an
 // address - it is a host-side stand-in; the device address is asked for once per device (hipGetSymbolAddress) and kept.
-constexpr size_t kStaticScratchBytes = 8u << 20;
+constexpr size_t kStaticScratchBytes = NXRT_ROCM_STATIC_SCRATCH_BYTES;
 __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 constexpr int kMaxScratchDevices = 64;
 void* g_scratch_ptr[kMaxScratchDevices] = {};
@@ -73,6 +74,18 @@ int rocm_ffi_device_info(int device, char* arch, size_t arch_len, int* compute_u
     if (compute_units) *compute_units = prop.multiProcessorCount;
     if (total_mem) *total_mem = prop.totalGlobalMem;
     return 0;
+}
+
+int rocm_ffi_compute_units(void)
+{
+    static std::atomic<int> cached[64];
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return 256;
+    int cus = cached[device].load(std::memory_order_relaxed);
+    if (cus > 0) return cus;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus <= 0) return 256;
+    cached[device].store(cus, std::memory_order_relaxed);
+    return cus;
 }
 
 int rocm_ffi_malloc(void** ptr, size_t bytes)

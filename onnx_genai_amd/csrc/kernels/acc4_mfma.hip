@@ -617,7 +617,8 @@ static int acc4_prefill_slices(int64_t m, int64_t n, int64_t padded_k, int block
 {
     const int64_t tiles = ((n + kTile - 1) / kTile) * ((m + kTile - 1) / kTile);
     const int64_t steps = (padded_k + kStep - 1) / kStep;
-    const int64_t resident = block_size < 64 ? 256 : 512;
+    const int64_t cus = rocm_ffi_compute_units();
+    const int64_t resident = block_size < 64 ? cus : 2 * cus;
     // Two slices pay at block size 32 (4096 -> 14336, 17..128 rows: 70-78 -> 44-56 us) and not from 64 up, where they
     // fill the second workgroup slot of each CU (8192 -> 28672 at block 64, 64 / 128 rows: 112 -> 120 us, 123 -> 137 us).
     if (tiles > (block_size < 64 ? resident / 2 : resident / 3)) return 1;
@@ -641,7 +642,7 @@ static int launch_acc4_prefill(const Acc4PrefillParams& p, int slices, hipStream
 {
     const dim3 grid(static_cast<unsigned>((p.n + kTile - 1) / kTile), static_cast<unsigned>((p.m + kTile - 1) / kTile), static_cast<unsigned>(slices));
     const size_t lds = 2 * (2 * kTile * kPitch8 + 2 * (NBS == 2 ? 2 : 1) * kTile * 4);
-    const bool deep = NBS == 2 || static_cast<uint64_t>(grid.x) * grid.y * grid.z <= 256;    // at most one workgroup per CU anyway
+    const bool deep = NBS == 2 || static_cast<uint64_t>(grid.x) * grid.y * grid.z <= static_cast<uint64_t>(rocm_ffi_compute_units());    // at most one workgroup per CU anyway
     if (p.acc_probe) {
         // (block size 32 with four register sets in flight has no room left for the probe's stores: its probe build keeps two -
         // the depth of the load pipeline changes when a step's operands arrive, not what is computed from them)

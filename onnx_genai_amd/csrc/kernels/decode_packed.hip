@@ -866,45 +866,100 @@ void decode_wide_kernel(PackedParams p)
     }
 }
 
-template <bool BF16, typename ST>
-static int launch_wide_bs(const PackedParams& p, int bs, hipStream_t stream)
+// What launch_wide_bs launches for a shape: the build (row blocks, sums or second MFMA, weights / windows ahead, the
+// workgroup's most waves), the waves per workgroup and the grid. No GPU work: a CPU test holds the answers for the model
+// shapes against a committed table, so that a change made for one shape cannot move another unnoticed.
+struct WidePlan {
+    int rb;            // blocks of 16 rows per wave: 1, 2 or 4
+    bool sums, pf, deep;
+    int wmax;          // kWideWaves or kWideWavesMax
+    int waves;         // per workgroup
+    unsigned grid;
+    bool ok;           // false: no build for this call (the dispatch does not send it here)
+};
+
+static WidePlan plan_wide(int64_t m, int64_t n, int bs, bool st16, bool pair, int64_t cus)
 {
-    const int64_t col_groups = (p.n + 15) / 16;
-    const bool pair = p.packed_up != nullptr;
-    constexpr int64_t kCus = 256;
+    WidePlan w{};
+    const int64_t col_groups = (n + 15) / 16;
     const int64_t all_groups = pair ? 2 * col_groups : col_groups;
     // A grid between one and one and a half workgroups of eight waves per CU (3584 -> 37888: 296 workgroups on 256 CUs)
     // leaves some CUs with two workgroups while the others run one, and the launch lasts as long as the doubly loaded ones.
-    const bool in_between = all_groups > kCus * kWideWaves && all_groups <= kCus * kWideWavesMax;
-    const unsigned alone = static_cast<unsigned>((col_groups + kWideWaves - 1) / kWideWaves);
+    const bool in_between = all_groups > cus * kWideWaves && all_groups <= cus * kWideWavesMax;
+    const int64_t alone = (col_groups + kWideWaves - 1) / kWideWaves;
     // How offset and zero point leave the accumulator (it shows in the last bits, so it is decided as for a launch of one
     // projection alone, and a pair follows its projections). Through the block activation sums, except:
     //  * grids of three or more workgroups per CU (3584 -> 152064 at 16 rows: 59 against 64 us);
-    //  * block size 32: the sums build takes 185-196 registers there, one workgroup per CU, and a grid above 256
-    //    workgroups runs in two rounds (3584 -> 37888 at 8 rows: 37.8 us; the second-MFMA build with the next group's
+    //  * block size 32: the sums build takes 185-196 registers there, one workgroup per CU, and a grid above one workgroup
+    //    per CU runs in two rounds (3584 -> 37888 at 8 rows: 37.8 us; the second-MFMA build with the next group's
     //    weights in flight 26.2, 4096 -> 14336 21.6 -> 17.2, 4096 -> 28672 24.0 -> 20.2);
     //  * block size 64 where a launch of the projection gets a balanced grid (below): the sums build with weights ahead
     //    takes 218 registers, too many for more than eight waves a workgroup.
-    const bool sums = alone < 768 && bs != 32 && !(bs == 64 && sizeof(ST) == 2 && col_groups > kCus * kWideWaves && col_groups <= kCus * kWideWavesMax);
+    w.sums = alone < 3 * cus && bs != 32 && !(bs == 64 && st16 && col_groups > cus * kWideWaves && col_groups <= cus * kWideWavesMax);
     // Waves (= column groups) per workgroup: eight, unless the grid is in between and a build for more waves exists - then
     // as many as spread the column groups over one workgroup per CU, up to twelve (3584 -> 37888 at block 128: ten waves,
     // 237 workgroups, 22.6 -> 18.0 us at 8 rows; at block 64 23.7 -> 21.2). Larger workgroups lose where the grid is several
     // times the CUs (3584 -> 152064 65 -> 80 us with ten). A paired launch holds half of its waves' column groups from each
     // projection. The builds for twelve waves: block 128 with the sums, block 64 without (16-bit scales).
     int ww = kWideWaves;
-    if (p.m <= 16 && sizeof(ST) == 2 && in_between && ((bs == 128 && sums) || (bs == 64 && !sums && !pair))) {
-        ww = static_cast<int>((all_groups + kCus - 1) / kCus);
+    if (m <= 16 && st16 && in_between && ((bs == 128 && w.sums) || (bs == 64 && !w.sums && !pair))) {
+        ww = static_cast<int>((all_groups + cus - 1) / cus);
         if (pair && (ww & 1)) ++ww;
         if (ww > kWideWavesMax) ww = kWideWaves;
     }
     const int per_wg = pair ? ww / 2 : ww;
-    const dim3 grid(static_cast<unsigned>((col_groups + per_wg - 1) / per_wg));
+    w.waves = ww;
+    w.grid = static_cast<unsigned>((col_groups + per_wg - 1) / per_wg);
+    w.wmax = ww > kWideWaves ? kWideWavesMax : kWideWaves;
+    w.rb = m <= 16 ? 1 : m <= 32 ? 2 : 4;
+    w.ok = true;
+    if (m <= 16) {
+        // The build by grid size. Measured at 8 / 16 rows (3584 -> 152064, 3584 -> 37888, 4096 -> 16384): three or more
+        // workgroups per CU run best with the windows two ahead (68 -> 64 us); fewer workgroups than CUs with weights and
+        // windows both ahead (17.2 -> 14.5 us); in between neither helps the sums build (20.6 us either way; with both ahead
+        // it spills at block size 32).
+        if (ww > kWideWaves) {
+            // a balanced grid has at most one workgroup per CU: the builds for few workgroups, compiled for twelve waves
+            if (bs == 128 && st16) {
+                w.pf = w.deep = w.grid < cus;
+            } else if (bs == 64 && st16 && !pair) {
+                w.pf = w.deep = true;              // (sums is false here)
+            } else {
+                w.ok = false;
+            }
+        } else if (!w.sums) {
+            w.deep = true;
+            w.pf = !(alone >= 3 * cus && bs != 32);
+        } else if (bs != 32) {
+            w.pf = w.deep = w.grid < cus;
+        } else {
+            w.ok = false;                          // (block size 32 never takes the sums)
+        }
+    } else {
+        // More row blocks per wave only where they fit the register file: two from block size 64, four at 128. The
+        // spilling forms ran several times slower than the routes that take those calls instead (3584 -> 37888: 153 us
+        // at block 32 and 32 rows against 2 x 37 us in blocks of 16 rows; 258 us at block 64 and 64 rows against 83 us
+        // in the tiled kernel). The paired form takes up to 16 rows.
+        w.sums = true;
+        w.pf = w.deep = false;
+        if (pair || bs == 32 || (m > 32 && bs == 64)) w.ok = false;
+    }
+    return w;
+}
+
+template <bool BF16, typename ST>
+static int launch_wide_bs(const PackedParams& p, int bs, int64_t cus, hipStream_t stream)
+{
+    const bool pair = p.packed_up != nullptr;
+    const WidePlan w = plan_wide(p.m, p.n, bs, sizeof(ST) == 2, pair, cus);
+    if (!w.ok) return -1;
+    const dim3 grid(w.grid);
     auto go = [&](auto kernel, size_t lds) {
         if (lds > 65536) {
             const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
             if (e != hipSuccess) return static_cast<int>(e);
         }
-        hipLaunchKernelGGL(kernel, grid, dim3(ww * 64), lds, stream, p);
+        hipLaunchKernelGGL(kernel, grid, dim3(w.waves * 64), lds, stream, p);
         return static_cast<int>(hipGetLastError());
     };
     auto by_rows = [&](auto bs_tag) {
@@ -912,16 +967,11 @@ static int launch_wide_bs(const PackedParams& p, int bs, hipStream_t stream)
         // two window buffers of rows x (tiles x 256 + 16) bytes, then two tables of (blocks per window) x rows f32 sums
         constexpr int NBT = 128 / BS;
         constexpr size_t lds16 = 2 * 16 * (4 * 256 + 16), sums16 = 2 * 4 * NBT * 16 * 4;
-        // up to 16 rows, PAIR or not: the build by grid size. Measured at 8 / 16 rows (3584 -> 152064, 3584 -> 37888,
-        // 4096 -> 16384): three or more workgroups per CU run best with the windows two ahead (68 -> 64 us); fewer
-        // workgroups than CUs with weights and windows both ahead (17.2 -> 14.5 us); in between neither helps the sums build
-        // (20.6 us either way; with both ahead it spills at block size 32).
         auto upto16 = [&](auto pair_tag) {
             constexpr bool P = decltype(pair_tag)::value;
-            if (ww > kWideWaves) {
-                // a balanced grid has at most one workgroup per CU: the builds for few workgroups, compiled for twelve waves
+            if (w.wmax > kWideWaves) {
                 if constexpr (BS == 128 && sizeof(ST) == 2) {
-                    if (grid.x < 256) return go(decode_wide_kernel<BF16, BS, ST, 1, true, true, true, P, kWideWavesMax>, lds16 + sums16);
+                    if (w.pf) return go(decode_wide_kernel<BF16, BS, ST, 1, true, true, true, P, kWideWavesMax>, lds16 + sums16);
                     return go(decode_wide_kernel<BF16, BS, ST, 1, true, false, false, P, kWideWavesMax>, lds16 + sums16);
                 } else if constexpr (BS == 64 && sizeof(ST) == 2 && !P) {
                     return go(decode_wide_kernel<BF16, BS, ST, 1, false, true, true, false, kWideWavesMax>, lds16);
@@ -929,23 +979,18 @@ static int launch_wide_bs(const PackedParams& p, int bs, hipStream_t stream)
                     return -1;
                 }
             }
-            if (!sums) {
-                if (alone >= 768 && bs != 32) return go(decode_wide_kernel<BF16, BS, ST, 1, false, false, true, P>, lds16);
+            if (!w.sums) {
+                if (!w.pf) return go(decode_wide_kernel<BF16, BS, ST, 1, false, false, true, P>, lds16);
                 return go(decode_wide_kernel<BF16, BS, ST, 1, false, true, true, P>, lds16);
             }
             if constexpr (BS != 32) {
-                if (grid.x < 256) return go(decode_wide_kernel<BF16, BS, ST, 1, true, true, true, P>, lds16 + sums16);
+                if (w.pf) return go(decode_wide_kernel<BF16, BS, ST, 1, true, true, true, P>, lds16 + sums16);
                 return go(decode_wide_kernel<BF16, BS, ST, 1, true, false, false, P>, lds16 + sums16);
             } else {
-                return -1;                                 // (block size 32 never takes the sums)
+                return -1;
             }
         };
         if (p.m <= 16) return pair ? upto16(std::true_type{}) : upto16(std::false_type{});
-        if (pair) return -1;                               // the paired form takes up to 16 rows
-        // More row blocks per wave only where they fit the register file: two from block size 64, four at 128. The
-        // spilling forms ran several times slower than the routes that take those calls instead (3584 -> 37888: 153 us
-        // at block 32 and 32 rows against 2 x 37 us in blocks of 16 rows; 258 us at block 64 and 64 rows against 83 us
-        // in the tiled kernel).
         if constexpr (BS == 32) return -1;
         else {
             if (p.m <= 32) return go(decode_wide_kernel<BF16, BS, ST, 2, true, false, false>, 2 * 32 * (4 * 256 + 16) + 2 * 4 * NBT * 32 * 4);
@@ -1504,10 +1549,149 @@ static int w_max_of(const RocmMatMulNBitsArgs* a, bool f32_scales)
     return (a->block_size == 128 && !f32_scales && (a->m <= 8 || a->a_dtype == ROCM_DT_BF16)) ? 16 : 8;
 }
 
+// What rocm_launch_decode_packed launches for a shape, without launching it: which kernel, which build of it, how many waves
+// split K and over how many register sets. Everything below is arithmetic on the shape and the chip's CU count (the
+// thresholds were measured on 256 CUs and are written as multiples of that count), so a CPU test can hold the answers for
+// the model shapes against a committed table: a change made for one shape cannot move another unnoticed.
+struct PackedPlan {
+    bool wide;          // the shared-activation kernel (plan in `w`); otherwise the split-K kernel
+    mnb::WidePlan w;
+    int rows_build;     // split-K kernel: rows the build stages (1, 4, 8, 16)
+    int waves;          // per projection and workgroup
+    int groups_per_wave;
+    bool single_set;
+};
+
+static PackedPlan plan_decode_packed(const RocmMatMulNBitsArgs* a, int waves, bool pair_member, bool paired_launch, int64_t cus)
+{
+    PackedPlan plan{};
+    const bool f32_scales = a->scale_dtype == ROCM_DT_F32;
+    if (wide_shape(a, pair_member)) {
+        plan.wide = true;
+        plan.w = mnb::plan_wide(a->m, a->n, a->block_size, !f32_scales, paired_launch, cus);
+        plan.groups_per_wave = mnb::packed_groups(a);
+        plan.waves = plan.w.waves;
+        return plan;
+    }
+    const int groups = mnb::packed_groups(a);
+    // Waves per workgroup (they split K in whole tile groups). Many column groups (thousands of waves even at four per
+    // group): short waves of at most two tile groups. Few column groups: enough waves per group to reach about 8k in
+    // flight. Then the adjustments below: register sets, and wave counts that fit the chip.
+    const int64_t wgs = (a->n + 15) / 16 * ((pair_member && a->m <= 4) ? 2 : 1);      // (a pair shares a launch up to four rows here)
+    int w = waves;
+    const int w_max = w_max_of(a, f32_scales);
+    // One row: one tile group per wave where the workgroup can hold that many waves, no prefetch, offset and zero point
+    // through the activation sums. Every byte of the call is then requested as soon as its wave starts, and what a wave
+    // computes between its loads and the reduction is the least any variant here does. Measured against the few-wave
+    // prefetching build it replaced on the small shapes (bf16, block 128): 3584 -> 4608 5.06 -> 4.78 us, 3584 -> 3584
+    // 4.17 -> 3.97, 18944 -> 3584 9.94 -> 9.41, 3584 -> 37888 15.81 -> 15.48.
+    // (a gate/up pair keeps the few-wave split: with fourteen waves a workgroup the paired launch measured 17.8 us against 15.5)
+    const bool one_row = a->m <= 1 && !pair_member;
+    const bool large_grid = wgs * 4 >= 24 * cus;
+    if (w <= 0) {
+        if (one_row) {
+            w = groups;
+        } else if (large_grid) {
+            w = (groups + 1) / 2;
+        } else {
+            const int want = static_cast<int>((32 * cus + wgs - 1) / wgs);
+            w = want < groups ? want : groups;               // at least one group per wave
+        }
+        if (w < 1) w = 1;
+    }
+    // One register set or two (the second holds the next group's loads while the current one is multiplied, at the price
+    // of waves per SIMD). Swept over 384 .. 1024 column groups x K = 3584 .. 8192 x 1 / 2 / 4 rows x block 32 / 128: one set is
+    // ahead or level nearly everywhere, by up to 30 % from K = 5120 (block 128, 4 rows, 5120 -> 16384: 12.4 against 16.5 us;
+    // block 32: 15.8 against 21.7). Two sets keep:
+    //  * two to four rows on small grids, where the second set's first fetch, issued before anything else, is worth 1-3 %
+    //    (block 128, 3584 -> 4608: 5.56 against 5.72 us; 18944 -> 3584 at block 32: 13.3 against 13.9) - below 256 column groups at
+    //    block 32, else up to 512 (two workgroups per CU: 4096 -> 8192 6.4 against 6.5 us at two rows, but 4096 -> 9216 7.7 against
+    //    7.3 and 3072 -> 9216 7.75 against 6.8), or below 320 when K is more than eight groups;
+    //  * one row at block size 32 with more groups than a workgroup has waves, on small grids: sixteen scale steps per group
+    //    leave enough arithmetic between a wave's loads that fetching ahead pays (18944 -> 3584 12.4 -> 11.8 us; with 1024
+    //    column groups it loses, 5120 -> 16384: 17.3 against 12.2; at block 128 one set stays ahead, 9.5 against 9.9 us).
+    bool single_set;
+    if (one_row) single_set = !(a->block_size == 32 && groups > w_max && wgs <= cus);
+    else if (a->block_size == 32) single_set = wgs >= cus;
+    else single_set = wgs > 2 * cus || (wgs >= cus + cus / 4 && groups > 8);
+    if (w > w_max) w = w_max;
+    if (w > groups) w = groups;
+    // Mid-size grids: a launch whose waves do not all fit the chip at once queues workgroups behind each other, and
+    // workgroups of 6, 10 or 12 waves leave slots of a CU empty on top; fewer waves of more groups each run it faster
+    // (16 rows, block 128: 3072 -> 16384 13.8 -> 12.2 us, 5120 -> 13824 21.0 -> 17.6, 6144 -> 16384 24.6 -> 21.1, 5120 -> 17920
+    // 24.1 -> 21.7; 8 rows: 16.2 -> 13.9 on 5120 -> 13824; one row: 7168 -> 16384 16.2 -> 14.3; 4 rows at block 32: 3584 -> 16384
+    // 12.5 -> 11.4). Workgroups of eight waves of one group each fill a CU's slots exactly and stay (K = 4096, 16 rows: 14336
+    // columns 13.9 against 14.9 us with four waves, 11008 11.3 against 11.6), and so do the large grids, whose waves are
+    // short enough for the queue not to show (one row, 3584 -> 37888: seven waves of one group, 15.5 against 15.8 us).
+    // Which of the wave counts that fit: a workgroup's waves go round the four SIMDs, so k workgroups of w waves put
+    // k * ceil(w / 4) of them on the first SIMD, and with three to five waves per SIMD a workgroup of 5, 6 or 10 waves keeps
+    // a CU from filling up (16 rows, 5120 -> 13824: five waves 21.4 us, four 17.5, ten 21.0; 2 rows at block 32, 8192 -> 12288:
+    // six waves 18.9 us, four 16.6). Builds of up to five waves per SIMD take the count that holds the most waves per CU that way.
+    if (waves <= 0 && !(w == 8 && groups == 8)) {
+        const int per_simd = waves_per_simd(a, f32_scales);
+        const int64_t fit = cus * 4 * per_simd / wgs;
+        const int64_t least = a->m <= 1 ? 6 : a->m <= 4 ? 4 : 1;
+        // A count within that bound can still be too many once the waves' places on the SIMDs are counted (576 workgroups of six
+        // waves at five waves per SIMD: two workgroups a CU, 3072 slots for 3456 waves). Then the count that holds the most is
+        // taken as well, if it leaves a wave two tile groups at most (block 32, two / four rows: 3072 -> 9216 8.9 / 8.9 -> 8.3 / 8.7 us,
+        // 3072 -> 12288 10.0 / 10.1 -> 8.5 / 9.0; block 128, five / eight rows: 3072 -> 12288 9.2 -> 8.1; with three groups a wave it
+        // lost, 5120 -> 10240 at block 32: 10.1 -> 10.8).
+        const bool crowded = per_simd <= 5 && w <= fit && wgs * w > cus * static_cast<int64_t>(per_simd / ((w + 3) / 4) * w);
+        if (fit >= least && (w > fit || crowded)) {
+            if (w > fit) w = static_cast<int>(fit);
+            const int limit = w;
+            if (per_simd <= 5) {                       // (with six or more waves per SIMD the plain count is as good or better: 4 rows at block 128, 6144 -> 16384: six waves 14.2 us, four 15.4)
+                int best = -1;
+                for (int g = 1; g <= groups; ++g) {
+                    const int cand = (groups + g - 1) / g;
+                    if (cand > limit || (crowded && g > 2)) continue;
+                    const int held = per_simd / ((cand + 3) / 4) * cand;
+                    if (held > best) {                 // (ties: the first found, which has the most waves)
+                        best = held;
+                        w = cand;
+                    }
+                    if (cand == 1) break;
+                }
+            }
+        }
+    }
+    // A projection of a gate/up pair takes at most half a workgroup's waves where that leaves a wave five tile groups or fewer,
+    // so that the pair runs as one launch and not as two and the epilogue (bf16, one / two / four rows: 3072 -> 2 x 8192 at block 32
+    // 14.3 -> 9.1 us at one row; 5120 -> 2 x 13824 at block 32 25.5 / 30.9 / 32.6 -> 20.6 / 25.4 / 25.7, at block 64 24.1 / 26.5 / 28.0 ->
+    // 18.8 / 21.7 / 22.8; 8192 -> 2 x 8192 at block 64 22.5 / 25.3 / 26.8 -> 17.7 / 18.6 / 19.9). The projection launched alone on a
+    // pair's first call takes the same count, as everything here.
+    if (pair_member && a->m <= 4 && waves <= 0 && 2 * w > w_max && (groups + w_max / 2 - 1) / (w_max / 2) <= 5) w = w_max / 2;
+    const int gpw = (groups + w - 1) / w;
+    w = (groups + gpw - 1) / gpw;
+        plan.rows_build = a->m <= 1 ? 1 : a->m <= 4 ? 4 : a->m <= 8 ? 8 : 16;
+    plan.waves = w;
+    plan.groups_per_wave = gpw;
+    plan.single_set = a->m > 4 || single_set || (a->m > 1 && a->gamma != nullptr);
+    return plan;
+}
+
+extern "C" int rocm_decode_packed_plan(const RocmMatMulNBitsArgs* a, int waves, int pair_member, int compute_units, RocmDecodePackedPlan* out)
+{
+    if (!a || !out || compute_units <= 0 || !rocm_decode_packed_eligible(a)) return -1;
+    const PackedPlan plan = plan_decode_packed(a, waves, pair_member != 0, pair_member == 2, compute_units);
+    if (plan.wide && !plan.w.ok) return -1;
+    const int64_t col_groups = (a->n + 15) / 16;
+    out->shared_activations = plan.wide;
+    out->rows_build = plan.wide ? plan.w.rb * 16 : plan.rows_build;
+    out->waves = plan.waves;
+    out->groups_per_wave = plan.groups_per_wave;
+    out->register_sets = plan.wide ? ((plan.w.pf ? 1 : 0) + (plan.w.deep ? 1 : 0) + 1) : (plan.single_set ? 1 : 2);
+    out->activation_sums = plan.wide ? plan.w.sums : (plan.rows_build == 1 && plan.single_set);
+    out->workgroups = plan.wide ? static_cast<int64_t>(plan.w.grid) : col_groups;
+    return 0;
+}
+
 static int launch_decode_packed(const RocmMatMulNBitsArgs* a, const void* packed, const void* packed_up, int decomposed, int waves, bool probe_only,
                                 bool pair_member, rocm_stream_t stream)
 {
     if (!rocm_decode_packed_eligible(a)) return probe_only ? 0 : -1;
+    const int64_t cus = rocm_ffi_compute_units();
+    const PackedPlan plan = plan_decode_packed(a, waves, pair_member, packed_up != nullptr, cus);
     mnb::PackedParams p;
     p.a = static_cast<const uint16_t*>(a->a);
     p.packed = static_cast<const uint8_t*>(packed);
@@ -1538,105 +1722,18 @@ static int launch_decode_packed(const RocmMatMulNBitsArgs* a, const void* packed
 
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool f32_scales = a->scale_dtype == ROCM_DT_F32;
-    if (wide_shape(a, pair_member)) {
+    if (plan.wide) {
         // the shared-activation kernel's paired form takes up to 16 rows (one block of rows per wave)
         if (probe_only) return a->m <= 16 ? 1 : 0;
         if (packed_up && a->m > 16) return -1;
         p.groups_per_wave = p.groups;
-        if (bf16) return f32_scales ? mnb::launch_wide_bs<true, float>(p, a->block_size, s) : mnb::launch_wide_bs<true, uint16_t>(p, a->block_size, s);
-        return f32_scales ? mnb::launch_wide_bs<false, float>(p, a->block_size, s) : mnb::launch_wide_bs<false, uint16_t>(p, a->block_size, s);
+        if (bf16) return f32_scales ? mnb::launch_wide_bs<true, float>(p, a->block_size, cus, s) : mnb::launch_wide_bs<true, uint16_t>(p, a->block_size, cus, s);
+        return f32_scales ? mnb::launch_wide_bs<false, float>(p, a->block_size, cus, s) : mnb::launch_wide_bs<false, uint16_t>(p, a->block_size, cus, s);
     }
-
-    // Waves per workgroup (they split K in whole tile groups). Many column groups (thousands of waves even at four per
-    // group): short waves of at most two tile groups. Few column groups: enough waves per group to reach about 8k in
-    // flight. Then the adjustments below: register sets, and wave counts that fit the chip.
-    const int64_t wgs = (a->n + 15) / 16 * ((pair_member && a->m <= 4) ? 2 : 1);      // (a pair shares a launch up to four rows here)
-    int w = waves;
+    const int w = plan.waves;
     const int w_max = w_max_of(a, f32_scales);
-    // One row: one tile group per wave where the workgroup can hold that many waves, no prefetch, offset and zero point
-    // through the activation sums. Every byte of the call is then requested as soon as its wave starts, and what a wave
-    // computes between its loads and the reduction is the least any variant here does. Measured against the few-wave
-    // prefetching build it replaced on the small shapes (bf16, block 128): 3584 -> 4608 5.06 -> 4.78 us, 3584 -> 3584
-    // 4.17 -> 3.97, 18944 -> 3584 9.94 -> 9.41, 3584 -> 37888 15.81 -> 15.48.
-    // (a gate/up pair keeps the few-wave split: with fourteen waves a workgroup the paired launch measured 17.8 us against 15.5)
-    const bool one_row = a->m <= 1 && !pair_member;
-    const bool large_grid = wgs * 4 >= 6144;
-    if (w <= 0) {
-        if (one_row) {
-            w = p.groups;
-        } else if (large_grid) {
-            w = (p.groups + 1) / 2;
-        } else {
-            const int want = static_cast<int>((8192 + wgs - 1) / wgs);
-            w = want < p.groups ? want : p.groups;               // at least one group per wave
-        }
-        if (w < 1) w = 1;
-    }
-    // One register set or two (the second holds the next group's loads while the current one is multiplied, at the price
-    // of waves per SIMD). Swept over 384 .. 1024 column groups x K = 3584 .. 8192 x 1 / 2 / 4 rows x block 32 / 128: one set is
-    // ahead or level nearly everywhere, by up to 30 % from K = 5120 (block 128, 4 rows, 5120 -> 16384: 12.4 against 16.5 us;
-    // block 32: 15.8 against 21.7). Two sets keep:
-    //  * two to four rows on small grids, where the second set's first fetch, issued before anything else, is worth 1-3 %
-    //    (block 128, 3584 -> 4608: 5.56 against 5.72 us; 18944 -> 3584 at block 32: 13.3 against 13.9) - below 256 column groups at
-    //    block 32, else up to 512 (two workgroups per CU: 4096 -> 8192 6.4 against 6.5 us at two rows, but 4096 -> 9216 7.7 against
-    //    7.3 and 3072 -> 9216 7.75 against 6.8), or below 320 when K is more than eight groups;
-    //  * one row at block size 32 with more groups than a workgroup has waves, on small grids: sixteen scale steps per group
-    //    leave enough arithmetic between a wave's loads that fetching ahead pays (18944 -> 3584 12.4 -> 11.8 us; with 1024
-    //    column groups it loses, 5120 -> 16384: 17.3 against 12.2; at block 128 one set stays ahead, 9.5 against 9.9 us).
-    bool single_set;
-    if (one_row) single_set = !(a->block_size == 32 && p.groups > w_max && wgs <= 256);
-    else if (a->block_size == 32) single_set = wgs >= 256;
-    else single_set = wgs > 512 || (wgs >= 320 && p.groups > 8);
-    if (w > w_max) w = w_max;
-    if (w > p.groups) w = p.groups;
-    // Mid-size grids: a launch whose waves do not all fit the chip at once queues workgroups behind each other, and
-    // workgroups of 6, 10 or 12 waves leave slots of a CU empty on top; fewer waves of more groups each run it faster
-    // (16 rows, block 128: 3072 -> 16384 13.8 -> 12.2 us, 5120 -> 13824 21.0 -> 17.6, 6144 -> 16384 24.6 -> 21.1, 5120 -> 17920
-    // 24.1 -> 21.7; 8 rows: 16.2 -> 13.9 on 5120 -> 13824; one row: 7168 -> 16384 16.2 -> 14.3; 4 rows at block 32: 3584 -> 16384
-    // 12.5 -> 11.4). Workgroups of eight waves of one group each fill a CU's slots exactly and stay (K = 4096, 16 rows: 14336
-    // columns 13.9 against 14.9 us with four waves, 11008 11.3 against 11.6), and so do the large grids, whose waves are
-    // short enough for the queue not to show (one row, 3584 -> 37888: seven waves of one group, 15.5 against 15.8 us).
-    // Which of the wave counts that fit: a workgroup's waves go round the four SIMDs, so k workgroups of w waves put
-    // k * ceil(w / 4) of them on the first SIMD, and with three to five waves per SIMD a workgroup of 5, 6 or 10 waves keeps
-    // a CU from filling up (16 rows, 5120 -> 13824: five waves 21.4 us, four 17.5, ten 21.0; 2 rows at block 32, 8192 -> 12288:
-    // six waves 18.9 us, four 16.6). Builds of up to five waves per SIMD take the count that holds the most waves per CU that way.
-    if (waves <= 0 && !(w == 8 && p.groups == 8)) {
-        const int per_simd = waves_per_simd(a, f32_scales);
-        const int64_t fit = 256 * 4 * per_simd / wgs;
-        const int64_t least = a->m <= 1 ? 6 : a->m <= 4 ? 4 : 1;
-        // A count within that bound can still be too many once the waves' places on the SIMDs are counted (576 workgroups of six
-        // waves at five waves per SIMD: two workgroups a CU, 3072 slots for 3456 waves). Then the count that holds the most is
-        // taken as well, if it leaves a wave two tile groups at most (block 32, two / four rows: 3072 -> 9216 8.9 / 8.9 -> 8.3 / 8.7 us,
-        // 3072 -> 12288 10.0 / 10.1 -> 8.5 / 9.0; block 128, five / eight rows: 3072 -> 12288 9.2 -> 8.1; with three groups a wave it
-        // lost, 5120 -> 10240 at block 32: 10.1 -> 10.8).
-        const bool crowded = per_simd <= 5 && w <= fit && wgs * w > 256 * static_cast<int64_t>(per_simd / ((w + 3) / 4) * w);
-        if (fit >= least && (w > fit || crowded)) {
-            if (w > fit) w = static_cast<int>(fit);
-            const int limit = w;
-            if (per_simd <= 5) {                       // (with six or more waves per SIMD the plain count is as good or better: 4 rows at block 128, 6144 -> 16384: six waves 14.2 us, four 15.4)
-                int best = -1;
-                for (int g = 1; g <= p.groups; ++g) {
-                    const int cand = (p.groups + g - 1) / g;
-                    if (cand > limit || (crowded && g > 2)) continue;
-                    const int held = per_simd / ((cand + 3) / 4) * cand;
-                    if (held > best) {                 // (ties: the first found, which has the most waves)
-                        best = held;
-                        w = cand;
-                    }
-                    if (cand == 1) break;
-                }
-            }
-        }
-    }
-    // A projection of a gate/up pair takes at most half a workgroup's waves where that leaves a wave five tile groups or fewer,
-    // so that the pair runs as one launch and not as two and the epilogue (bf16, one / two / four rows: 3072 -> 2 x 8192 at block 32
-    // 14.3 -> 9.1 us at one row; 5120 -> 2 x 13824 at block 32 25.5 / 30.9 / 32.6 -> 20.6 / 25.4 / 25.7, at block 64 24.1 / 26.5 / 28.0 ->
-    // 18.8 / 21.7 / 22.8; 8192 -> 2 x 8192 at block 64 22.5 / 25.3 / 26.8 -> 17.7 / 18.6 / 19.9). The projection launched alone on a
-    // pair's first call takes the same count, as everything here.
-    if (pair_member && a->m <= 4 && waves <= 0 && 2 * w > w_max && (p.groups + w_max / 2 - 1) / (w_max / 2) <= 5) w = w_max / 2;
-    const int gpw = (p.groups + w - 1) / w;
-    w = (p.groups + gpw - 1) / gpw;
-    p.groups_per_wave = gpw;
+    const bool single_set = plan.single_set;
+    p.groups_per_wave = plan.groups_per_wave;
     // a paired launch keeps each projection's own split of K (so that it adds up in the same order) and needs twice the waves
     if (probe_only) return a->m <= 4 && 2 * w <= w_max ? 1 : 0;
     if (packed_up && (a->m > 4 || 2 * w > w_max)) return -1;
@@ -1690,6 +1787,54 @@ extern "C" int rocm_acc4_packed_fuses_quantizer(const RocmMatMulNBitsArgs* a)
     return a->m <= 4 && !a->acc_probe && work <= 4096;
 }
 
+// Waves per workgroup, tile groups per wave and register sets of rocm_launch_acc4_packed for a shape on a chip of `cus` CUs
+// (thresholds measured on 256 CUs, written as multiples of the count). No GPU work.
+static void plan_acc4_packed(const RocmMatMulNBitsArgs* a, int waves, int64_t cus, int* waves_out, int* groups_per_wave, bool* one_set)
+{
+    const int groups = mnb::packed_groups(a);
+    const int64_t wgs = (a->n + 15) / 16;
+    int w = waves;
+    bool single_set = wgs * 4 >= 24 * cus;
+    if (w <= 0) {
+        if (single_set) {
+            w = (groups + 1) / 2;
+        } else {
+            const int want = static_cast<int>((32 * cus + wgs - 1) / wgs);
+            w = want < groups ? want : groups;
+        }
+        if (w < 1) w = 1;
+    } else {
+        single_set = wgs * w >= 24 * cus;
+    }
+    if (w > 8) w = 8;
+    if (w > groups) w = groups;
+    const int gpw = (groups + w - 1) / w;
+    w = (groups + gpw - 1) / gpw;
+    // One register set (one-row launches; the builds for several rows have no other): with one group per wave a second set
+    // has nothing to fetch ahead (4096 -> 14336: 14.3 -> 9.8 us at block 32, 9.7 -> 8.8 at 64, 9.2 -> 8.4 at 128); at block 32 the
+    // two-set build holds three waves per SIMD against eight (5120 -> 13824 21.4 -> 11.6 us, 6144 -> 16384 23.8 -> 14.4,
+    // 8192 -> 8192 14.1 -> 10.5); and from a few hundred column groups on the other block sizes are level or ahead with one
+    // (13824 -> 5120 at block 128: 12.3 -> 11.2; 8192 -> 10240 at 64: 12.3 -> 11.5). Small K-heavy grids keep two (18944 -> 3584 at
+    // block 128: 9.3 against 10.2 us).
+    if (gpw == 1 || a->block_size == 32 || wgs > cus) single_set = true;
+
+    *waves_out = w;
+    *groups_per_wave = gpw;
+    *one_set = single_set;
+}
+
+extern "C" int rocm_acc4_packed_plan(const RocmMatMulNBitsArgs* a, int waves, int compute_units, int* waves_out, int* groups_per_wave, int* register_sets)
+{
+    if (!a || compute_units <= 0 || !rocm_acc4_packed_eligible(a)) return -1;
+    int w = 0, gpw = 0;
+    bool one_set = false;
+    plan_acc4_packed(a, waves, compute_units, &w, &gpw, &one_set);
+    if (waves_out) *waves_out = w;
+    if (groups_per_wave) *groups_per_wave = gpw;
+    if (register_sets) *register_sets = (one_set || a->m > 1) ? 1 : 2;
+    return 0;
+}
+
 extern "C" int rocm_launch_acc4_packed(const RocmMatMulNBitsArgs* a, const void* packed, const RocmAcc4Workspace* ws, int rounding, int waves, rocm_stream_t stream)
 {
     if (!rocm_acc4_packed_eligible(a)) return -1;
@@ -1717,32 +1862,10 @@ extern "C" int rocm_launch_acc4_packed(const RocmMatMulNBitsArgs* a, const void*
     p.scales_bf16 = a->scale_dtype == ROCM_DT_BF16;
     p.acc_probe = a->acc_probe;
 
-    const int64_t wgs = (a->n + 15) / 16;
-    int w = waves;
-    bool single_set = wgs * 4 >= 6144;
-    if (w <= 0) {
-        if (single_set) {
-            w = (p.groups + 1) / 2;
-        } else {
-            const int want = static_cast<int>((8192 + wgs - 1) / wgs);
-            w = want < p.groups ? want : p.groups;
-        }
-        if (w < 1) w = 1;
-    } else {
-        single_set = wgs * w >= 6144;
-    }
-    if (w > 8) w = 8;
-    if (w > p.groups) w = p.groups;
-    const int gpw = (p.groups + w - 1) / w;
-    w = (p.groups + gpw - 1) / gpw;
+    int w = 0, gpw = 0;
+    bool single_set = false;
+    plan_acc4_packed(a, waves, rocm_ffi_compute_units(), &w, &gpw, &single_set);
     p.groups_per_wave = gpw;
-    // One register set (one-row launches; the builds for several rows have no other): with one group per wave a second set
-    // has nothing to fetch ahead (4096 -> 14336: 14.3 -> 9.8 us at block 32, 9.7 -> 8.8 at 64, 9.2 -> 8.4 at 128); at block 32 the
-    // two-set build holds three waves per SIMD against eight (5120 -> 13824 21.4 -> 11.6 us, 6144 -> 16384 23.8 -> 14.4,
-    // 8192 -> 8192 14.1 -> 10.5); and from a few hundred column groups on the other block sizes are level or ahead with one
-    // (13824 -> 5120 at block 128: 12.3 -> 11.2; 8192 -> 10240 at 64: 12.3 -> 11.5). Small K-heavy grids keep two (18944 -> 3584 at
-    // block 128: 9.3 against 10.2 us).
-    if (gpw == 1 || a->block_size == 32 || wgs > 256) single_set = true;
 
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool f32_scales = a->scale_dtype == ROCM_DT_F32;

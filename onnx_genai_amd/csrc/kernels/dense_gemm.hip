@@ -10,11 +10,62 @@
 
 #include <hipblaslt/hipblaslt.h>
 
+#include <dlfcn.h>
+
 #include <map>
 #include <mutex>
 #include <tuple>
+#include <type_traits>
 
 namespace mnb {
+
+// The library is an opt-in route (dense_gemm_min_rows, dense_weights = resident): it is opened when a provider first asks
+// for it and is no link-time dependency of this library. The header only supplies the types.
+struct BlasLt {
+    decltype(&hipblasLtCreate) Create = nullptr;
+    decltype(&hipblasLtDestroy) Destroy = nullptr;
+    decltype(&hipblasLtMatmulDescCreate) MatmulDescCreate = nullptr;
+    decltype(&hipblasLtMatmulDescDestroy) MatmulDescDestroy = nullptr;
+    decltype(&hipblasLtMatmulDescSetAttribute) MatmulDescSetAttribute = nullptr;
+    decltype(&hipblasLtMatrixLayoutCreate) MatrixLayoutCreate = nullptr;
+    decltype(&hipblasLtMatrixLayoutDestroy) MatrixLayoutDestroy = nullptr;
+    decltype(&hipblasLtMatmulPreferenceCreate) MatmulPreferenceCreate = nullptr;
+    decltype(&hipblasLtMatmulPreferenceDestroy) MatmulPreferenceDestroy = nullptr;
+    decltype(&hipblasLtMatmulPreferenceSetAttribute) MatmulPreferenceSetAttribute = nullptr;
+    decltype(&hipblasLtMatmulAlgoGetHeuristic) MatmulAlgoGetHeuristic = nullptr;
+    decltype(&hipblasLtMatmul) Matmul = nullptr;
+    bool ok = false;
+};
+
+static const BlasLt& blaslt()
+{
+    static const BlasLt table = [] {
+        BlasLt t;
+        void* lib = dlopen("libhipblaslt.so", RTLD_NOW | RTLD_LOCAL);
+        if (!lib) lib = dlopen("/opt/rocm/lib/libhipblaslt.so", RTLD_NOW | RTLD_LOCAL);
+        if (!lib) return t;
+        bool all = true;
+        auto get = [&](auto& fn, const char* name) {
+            fn = reinterpret_cast<std::remove_reference_t<decltype(fn)>>(dlsym(lib, name));
+            all = all && fn != nullptr;
+        };
+        get(t.Create, "hipblasLtCreate");
+        get(t.Destroy, "hipblasLtDestroy");
+        get(t.MatmulDescCreate, "hipblasLtMatmulDescCreate");
+        get(t.MatmulDescDestroy, "hipblasLtMatmulDescDestroy");
+        get(t.MatmulDescSetAttribute, "hipblasLtMatmulDescSetAttribute");
+        get(t.MatrixLayoutCreate, "hipblasLtMatrixLayoutCreate");
+        get(t.MatrixLayoutDestroy, "hipblasLtMatrixLayoutDestroy");
+        get(t.MatmulPreferenceCreate, "hipblasLtMatmulPreferenceCreate");
+        get(t.MatmulPreferenceDestroy, "hipblasLtMatmulPreferenceDestroy");
+        get(t.MatmulPreferenceSetAttribute, "hipblasLtMatmulPreferenceSetAttribute");
+        get(t.MatmulAlgoGetHeuristic, "hipblasLtMatmulAlgoGetHeuristic");
+        get(t.Matmul, "hipblasLtMatmul");
+        t.ok = all;
+        return t;
+    }();
+    return table;
+}
 
 // Each thread expands one packed dword (8 consecutive k of one column) into one 16-byte store. K % 8 == 0.
 template <bool BF16>
@@ -76,10 +127,10 @@ static hipDataType hip_type(int dtype) { return dtype == ROCM_DT_BF16 ? HIP_R_16
 
 static void destroy_plan(GemmPlan& p)
 {
-    if (p.lay_w) hipblasLtMatrixLayoutDestroy(p.lay_w);
-    if (p.lay_a) hipblasLtMatrixLayoutDestroy(p.lay_a);
-    if (p.lay_y) hipblasLtMatrixLayoutDestroy(p.lay_y);
-    if (p.desc) hipblasLtMatmulDescDestroy(p.desc);
+    if (p.lay_w) mnb::blaslt().MatrixLayoutDestroy(p.lay_w);
+    if (p.lay_a) mnb::blaslt().MatrixLayoutDestroy(p.lay_a);
+    if (p.lay_y) mnb::blaslt().MatrixLayoutDestroy(p.lay_y);
+    if (p.desc) mnb::blaslt().MatmulDescDestroy(p.desc);
     p = GemmPlan();
 }
 
@@ -88,34 +139,34 @@ static GemmPlan make_plan(RocmDenseGemm& g, int64_t m, int64_t n, int64_t k, int
 {
     GemmPlan p;
     const hipDataType t = hip_type(dtype);
-    bool ok = hipblasLtMatmulDescCreate(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F) == HIPBLAS_STATUS_SUCCESS;
+    bool ok = mnb::blaslt().MatmulDescCreate(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F) == HIPBLAS_STATUS_SUCCESS;
     const hipblasOperation_t op_t = HIPBLAS_OP_T, op_n = HIPBLAS_OP_N;
-    ok = ok && hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &op_t, sizeof(op_t)) == HIPBLAS_STATUS_SUCCESS;
-    ok = ok && hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &op_n, sizeof(op_n)) == HIPBLAS_STATUS_SUCCESS;
+    ok = ok && mnb::blaslt().MatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &op_t, sizeof(op_t)) == HIPBLAS_STATUS_SUCCESS;
+    ok = ok && mnb::blaslt().MatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &op_n, sizeof(op_n)) == HIPBLAS_STATUS_SUCCESS;
     if (ok && bias_dtype >= 0) {
         const hipblasLtEpilogue_t epi = HIPBLASLT_EPILOGUE_BIAS;
         const int32_t bt = static_cast<int32_t>(hip_type(bias_dtype));
-        ok = hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_EPILOGUE, &epi, sizeof(epi)) == HIPBLAS_STATUS_SUCCESS &&
-             hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_DATA_TYPE, &bt, sizeof(bt)) == HIPBLAS_STATUS_SUCCESS;
+        ok = mnb::blaslt().MatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_EPILOGUE, &epi, sizeof(epi)) == HIPBLAS_STATUS_SUCCESS &&
+             mnb::blaslt().MatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_DATA_TYPE, &bt, sizeof(bt)) == HIPBLAS_STATUS_SUCCESS;
     }
-    ok = ok && hipblasLtMatrixLayoutCreate(&p.lay_w, t, static_cast<uint64_t>(k), static_cast<uint64_t>(n), k) == HIPBLAS_STATUS_SUCCESS;
-    ok = ok && hipblasLtMatrixLayoutCreate(&p.lay_a, t, static_cast<uint64_t>(k), static_cast<uint64_t>(m), k) == HIPBLAS_STATUS_SUCCESS;
-    ok = ok && hipblasLtMatrixLayoutCreate(&p.lay_y, t, static_cast<uint64_t>(n), static_cast<uint64_t>(m), n) == HIPBLAS_STATUS_SUCCESS;
+    ok = ok && mnb::blaslt().MatrixLayoutCreate(&p.lay_w, t, static_cast<uint64_t>(k), static_cast<uint64_t>(n), k) == HIPBLAS_STATUS_SUCCESS;
+    ok = ok && mnb::blaslt().MatrixLayoutCreate(&p.lay_a, t, static_cast<uint64_t>(k), static_cast<uint64_t>(m), k) == HIPBLAS_STATUS_SUCCESS;
+    ok = ok && mnb::blaslt().MatrixLayoutCreate(&p.lay_y, t, static_cast<uint64_t>(n), static_cast<uint64_t>(m), n) == HIPBLAS_STATUS_SUCCESS;
     hipblasLtMatmulPreference_t pref = nullptr;
-    ok = ok && hipblasLtMatmulPreferenceCreate(&pref) == HIPBLAS_STATUS_SUCCESS;
+    ok = ok && mnb::blaslt().MatmulPreferenceCreate(&pref) == HIPBLAS_STATUS_SUCCESS;
     if (ok) {
         const uint64_t cap = g.workspace_bytes;
         hipblasLtMatmulHeuristicResult_t found[1];
         int count = 0;
-        ok = hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &cap, sizeof(cap)) == HIPBLAS_STATUS_SUCCESS &&
-             hipblasLtMatmulAlgoGetHeuristic(g.handle, p.desc, p.lay_w, p.lay_a, p.lay_y, p.lay_y, pref, 1, found, &count) == HIPBLAS_STATUS_SUCCESS &&
+        ok = mnb::blaslt().MatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &cap, sizeof(cap)) == HIPBLAS_STATUS_SUCCESS &&
+             mnb::blaslt().MatmulAlgoGetHeuristic(g.handle, p.desc, p.lay_w, p.lay_a, p.lay_y, p.lay_y, pref, 1, found, &count) == HIPBLAS_STATUS_SUCCESS &&
              count > 0 && found[0].state == HIPBLAS_STATUS_SUCCESS && found[0].workspaceSize <= g.workspace_bytes;
         if (ok) {
             p.algo = found[0].algo;
             p.workspace = found[0].workspaceSize;
         }
     }
-    if (pref) hipblasLtMatmulPreferenceDestroy(pref);
+    if (pref) mnb::blaslt().MatmulPreferenceDestroy(pref);
     if (!ok) {
         destroy_plan(p);
         return p;
@@ -151,13 +202,17 @@ extern "C" int rocm_dense_gemm_create(RocmDenseGemm** out)
     *out = nullptr;
     RocmDenseGemm* g = new (std::nothrow) RocmDenseGemm();
     if (!g) return static_cast<int>(hipErrorOutOfMemory);
-    if (hipblasLtCreate(&g->handle) != HIPBLAS_STATUS_SUCCESS) {
+    if (!mnb::blaslt().ok) {                       // the library is not on this machine: the caller keeps the tiled kernel
+        delete g;
+        return static_cast<int>(hipErrorSharedObjectInitFailed);
+    }
+    if (mnb::blaslt().Create(&g->handle) != HIPBLAS_STATUS_SUCCESS) {
         delete g;
         return static_cast<int>(hipErrorNotInitialized);
     }
-    const hipError_t e = hipMalloc(&g->workspace, mnb::kGemmWorkspace);
+    const hipError_t e = static_cast<hipError_t>(rocm_ffi_malloc(&g->workspace, mnb::kGemmWorkspace));                 // (counted with the library's other allocations)
     if (e != hipSuccess) {
-        hipblasLtDestroy(g->handle);
+        mnb::blaslt().Destroy(g->handle);
         delete g;
         return static_cast<int>(e);
     }
@@ -170,8 +225,8 @@ extern "C" void rocm_dense_gemm_destroy(RocmDenseGemm* g)
 {
     if (!g) return;
     for (auto& kv : g->plans) mnb::destroy_plan(kv.second);
-    if (g->workspace) (void)hipFree(g->workspace);
-    if (g->handle) hipblasLtDestroy(g->handle);
+    if (g->workspace) (void)rocm_ffi_free(g->workspace);
+    if (g->handle) mnb::blaslt().Destroy(g->handle);
     delete g;
 }
 
@@ -201,10 +256,10 @@ extern "C" int rocm_dense_gemm_run(RocmDenseGemm* g, const void* w_nk, const voi
     auto it = g->plans.find(std::make_tuple(m, n, k, dtype, bias ? bias_dtype : -1));
     if (it == g->plans.end() || !it->second.usable) return static_cast<int>(hipErrorInvalidValue);
     mnb::GemmPlan& p = it->second;
-    if (bias && hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias, sizeof(bias)) != HIPBLAS_STATUS_SUCCESS)
+    if (bias && mnb::blaslt().MatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias, sizeof(bias)) != HIPBLAS_STATUS_SUCCESS)
         return 10000 + static_cast<int>(HIPBLAS_STATUS_INVALID_VALUE);
     const float one = 1.f, zero = 0.f;
-    const hipblasStatus_t st = hipblasLtMatmul(g->handle, p.desc, &one, w_nk, p.lay_w, a, p.lay_a, &zero, y, p.lay_y, y, p.lay_y, &p.algo,
+    const hipblasStatus_t st = mnb::blaslt().Matmul(g->handle, p.desc, &one, w_nk, p.lay_w, a, p.lay_a, &zero, y, p.lay_y, y, p.lay_y, &p.algo,
                                                g->workspace, g->workspace_bytes, static_cast<hipStream_t>(stream));
     return st == HIPBLAS_STATUS_SUCCESS ? 0 : 10000 + static_cast<int>(st);
 }

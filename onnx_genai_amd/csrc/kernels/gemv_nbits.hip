@@ -213,7 +213,7 @@ extern "C" int rocm_g_idx_first_bad(const int32_t* g_idx, int64_t count, int64_t
     *first_bad = -1;
     if (count <= 0) return 0;
     unsigned long long* dev = nullptr;
-    hipError_t e = hipMalloc(&dev, sizeof(unsigned long long));
+    hipError_t e = static_cast<hipError_t>(rocm_ffi_malloc(reinterpret_cast<void**>(&dev), sizeof(unsigned long long)));      // (counted with the library's other allocations)
     if (e != hipSuccess) return static_cast<int>(e);
     unsigned long long host = static_cast<unsigned long long>(count);
     hipStream_t s = static_cast<hipStream_t>(stream);
@@ -226,7 +226,7 @@ extern "C" int rocm_g_idx_first_bad(const int32_t* g_idx, int64_t count, int64_t
     }
     if (e == hipSuccess) e = hipMemcpyAsync(&host, dev, sizeof(host), hipMemcpyDeviceToHost, s);
     if (e == hipSuccess) e = hipStreamSynchronize(s);
-    (void)hipFree(dev);
+    (void)rocm_ffi_free(dev);
     if (e == hipSuccess && host < static_cast<unsigned long long>(count)) *first_bad = static_cast<int64_t>(host);
     return static_cast<int>(e);
 }

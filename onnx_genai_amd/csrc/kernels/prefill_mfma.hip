@@ -23,17 +23,22 @@ namespace mnb {
 // BF16: element type. BM x BN: tile of Y per workgroup (128 x 64, 128 x 128, 256 x 128 or 256 x 256). SF32: scales are stored
 // as f32 (otherwise in the activations' 16-bit type). f16 activations with f16 scales dequantize in packed f16,
 // everything else in f32.
-template <bool BF16, int BM, int BN, bool SF32>
+// DENSE: B is not packed 4-bit weights but a [N, K] matrix of the activations' 16-bit type (weights of another width or with
+// g_idx, expanded by a launch of their own): a lane copies its 16-byte pieces to LDS as they are; no scales, no zero points.
+template <bool BF16, int BM, int BN, bool SF32, bool DENSE = false>
 __global__ __launch_bounds__(512) void prefill_mfma_kernel(PrefillParams p)
 {
+    static_assert(!DENSE || (BN <= 128 && !SF32), "dense weights: four times the bytes per column, so only the narrower tiles have the registers");
     constexpr bool F32MATH = BF16 || SF32;
     constexpr int WM = BM / 4;             // wave sub-tile rows
     constexpr int WN = BN / 2;             // and columns
     constexpr int TM = WM / 32;            // 32x32 MFMA tiles per wave along M
     constexpr int TN = WN / 32;            // and along N
     constexpr int A_LOADS = BM / 64;       // 16-byte pieces of A per lane per step
-    constexpr int B_DW = BN / 64;          // packed dwords of B per lane per step (1, 2 or 4)
-    constexpr int B_PIECES = 8 / B_DW;     // lanes that share one column's 32 bytes of a step
+    constexpr int B_DW = BN / 64;          // packed dwords of B per lane per step (1, 2 or 4); dense: 16-byte pieces
+    constexpr int B_PIECES = 8 / B_DW;     // lanes that share one column's 32 (dense: 128) bytes of a step
+    constexpr int B_REGS = DENSE ? 4 * B_DW : B_DW;
+    constexpr uint32_t kBStep = DENSE ? 128u : 32u;            // bytes of one column per step
     const uint32_t nib_mask = __builtin_amdgcn_mov_dpp(p.nibble_mask, 0xE4, 0xf, 0xf, false);
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     unsigned char* lds_a = smem;                                   // [2][BM][kPitch]
@@ -63,7 +68,7 @@ __global__ __launch_bounds__(512) void prefill_mfma_kernel(PrefillParams p)
     const uint32_t a_gstep = 64u * static_cast<uint32_t>(p.k) * 2u;
     const uint32_t a_loff = static_cast<uint32_t>((t >> 3) * kPitch + (t & 7) * 16);
     const int bcol = t / B_PIECES, bpiece = t % B_PIECES;
-    const uint32_t b_goff = static_cast<uint32_t>(bcol) * static_cast<uint32_t>(p.row_bytes) + static_cast<uint32_t>(bpiece * B_DW * 4);
+    const uint32_t b_goff = static_cast<uint32_t>(bcol) * static_cast<uint32_t>(p.row_bytes) + static_cast<uint32_t>(bpiece * B_DW * (DENSE ? 16 : 4));
     const uint32_t b_loff = static_cast<uint32_t>(bcol * kPitch + bpiece * B_DW * 16);
     const uint32_t s_goff = static_cast<uint32_t>(bcol) * static_cast<uint32_t>(p.kb) * kScaleBytes;
     const uint32_t z_goff = static_cast<uint32_t>(bcol) * static_cast<uint32_t>(p.zp_row);
@@ -88,7 +93,7 @@ __global__ __launch_bounds__(512) void prefill_mfma_kernel(PrefillParams p)
     constexpr int D = BN == 256 ? 3 : 4;   // the 256 x 256 tile has no registers left for a fourth set
     struct Regs {
         uint4 a[A_LOADS];
-        uint32_t b[B_DW];
+        uint32_t b[B_REGS];
         uint32_t s;      // raw scale bits; converted when the step is dequantized, so that no load is waited for early
         uint32_t z;      // raw zero-point byte
         uint32_t zsh;    // shift of the nibble to take from it
@@ -98,6 +103,18 @@ __global__ __launch_bounds__(512) void prefill_mfma_kernel(PrefillParams p)
     auto load_global = [&](Regs& r, int kt) {
 #pragma unroll
         for (int i = 0; i < A_LOADS; ++i) r.a[i] = load16(srd_a, a_goff + static_cast<uint32_t>(i) * a_gstep, static_cast<uint32_t>(kt) * 128u);
+        if constexpr (DENSE) {
+#pragma unroll
+            for (int i = 0; i < B_DW; ++i) {
+                const uint4 bw = load16(srd_b, b_goff + static_cast<uint32_t>(i) * 16u, static_cast<uint32_t>(kt) * kBStep);
+                r.b[4 * i] = bw.x;
+                r.b[4 * i + 1] = bw.y;
+                r.b[4 * i + 2] = bw.z;
+                r.b[4 * i + 3] = bw.w;
+            }
+            r.s = r.z = r.zsh = 0;
+            return;
+        }
         if constexpr (B_DW == 1) {
             r.b[0] = __builtin_amdgcn_raw_buffer_load_b32(srd_b, static_cast<int>(b_goff), static_cast<int>(kt * 32), 0);
         } else if constexpr (B_DW == 2) {
@@ -129,6 +146,10 @@ __global__ __launch_bounds__(512) void prefill_mfma_kernel(PrefillParams p)
         if ((B_DW == 2 && (part & 1)) || (B_DW == 1 && part != 0)) return;
         const int dw = B_DW == 4 ? part : (part >> 1);
         unsigned char* lb = lds_b + buf * (BN * kPitch) + b_loff;
+        if constexpr (DENSE) {
+            *reinterpret_cast<uint4*>(lb + dw * 16) = make_uint4(r.b[4 * dw], r.b[4 * dw + 1], r.b[4 * dw + 2], r.b[4 * dw + 3]);
+            return;
+        }
         const uint32_t w = r.b[dw];
         const uint32_t zq = ((r.z >> r.zsh) & zp_mask) | zp_default;
         if constexpr (F32MATH) {
@@ -223,12 +244,12 @@ __global__ __launch_bounds__(256) void prefill_reduce_kernel(const float* __rest
     }
 }
 
-template <bool BF16, int BM, int BN, bool SF32>
+template <bool BF16, int BM, int BN, bool SF32, bool DENSE = false>
 static int launch_prefill(const PrefillParams& p, int splits, hipStream_t stream)
 {
     const dim3 grid(static_cast<unsigned>((p.n + BN - 1) / BN), static_cast<unsigned>((p.m + BM - 1) / BM), static_cast<unsigned>(splits));
     const size_t lds = 2 * static_cast<size_t>(BM + BN) * kPitch;
-    auto kernel = prefill_mfma_kernel<BF16, BM, BN, SF32>;
+    auto kernel = prefill_mfma_kernel<BF16, BM, BN, SF32, DENSE>;
     if (lds > 65536) {
         const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
         if (e != hipSuccess) return static_cast<int>(e);
@@ -264,6 +285,7 @@ struct PrefillPlan {
 PrefillPlan plan_prefill(const RocmMatMulNBitsArgs* a, int tile_choice, uint64_t scratch_bytes)
 {
     const int steps = static_cast<int>(a->k / 64);
+    const int64_t cus = rocm_ffi_compute_units();      // (256 where no device can be asked: the plan of a host without a GPU is the MI355X's)
     const uint64_t per_split = static_cast<uint64_t>(a->m) * static_cast<uint64_t>(a->n) * 4;
     auto workgroups = [&](int tile) {
         const int bm = (tile == 1 || tile == 2) ? 256 : 128;
@@ -274,7 +296,7 @@ PrefillPlan plan_prefill(const RocmMatMulNBitsArgs* a, int tile_choice, uint64_t
     // more than the scratch holds
     auto slices = [&](int tile) {
         const int64_t wgs = workgroups(tile);
-        int want = static_cast<int>((384 + wgs - 1) / wgs);
+        int want = static_cast<int>((cus + cus / 2 + wgs - 1) / wgs);
         if (want > steps / 8) want = steps / 8;
         if (want > 16) want = 16;
         while (want > 1 && static_cast<uint64_t>(want) * per_split > scratch_bytes) --want;
@@ -285,13 +307,13 @@ PrefillPlan plan_prefill(const RocmMatMulNBitsArgs* a, int tile_choice, uint64_t
     if (tile_choice >= 1 && tile_choice <= 4) {
         plan.tile = tile_choice == 4 ? 3 : tile_choice - 1;
         plan.splits = slices(plan.tile);
-    } else if (a->m >= 256 && workgroups(2) >= 256) {
+    } else if (a->m >= 256 && workgroups(2) >= cus) {
         plan.tile = 2;
-    } else if (a->m >= 256 && workgroups(1) >= 256) {
+    } else if (a->m >= 256 && workgroups(1) >= cus) {
         plan.tile = 1;
-    } else if (workgroups(0) >= 256) {
+    } else if (workgroups(0) >= cus) {
         plan.tile = 0;
-    } else if (a->m >= 512 && workgroups(0) * slices(0) >= 256) {
+    } else if (a->m >= 512 && workgroups(0) * slices(0) >= cus) {
         plan.tile = 0;                       // few tiles of Y but a long K: 128 x 128 tiles over slices of K (below 512 rows 128 x 64 is ahead)
         plan.splits = slices(0);
     } else {
@@ -303,7 +325,7 @@ PrefillPlan plan_prefill(const RocmMatMulNBitsArgs* a, int tile_choice, uint64_t
     // better in larger tiles over more slices (18944 -> 3584 at M = 1536: 336 tiles of 128 x 128, one per CU, two rounds,
     // 423 us; 256 x 128 tiles over three slices 300 us), and one round of larger tiles that leaves some CUs idle beats two
     // rounds of smaller ones (4096 -> 14336 at M = 1024: 224 tiles of 256 x 256 152 us, 448 of 256 x 128 177 us) - a workgroup
-    // runs faster when fewer of them share the memory system. The model: workgroups go round by round over 256 CUs; a round
+    // runs faster when fewer of them share the memory system. The model: workgroups go round by round over the CUs (256 where it was fitted); a round
     // costs (steps per slice) x (the tile's time per step: 2.52 / 1.42 / 0.78 us for 256 x 256 / 256 x 128 / 128 x 128 with every
     // CU busy, 0.45 for 128 x 64; two of the small tiles share a CU) x (0.4 + 0.6 x the fraction of CUs busy) + 8 us for the
     // ends of a workgroup, and the reduction adds its bytes at 4 TB/s. Fitted to 160 timings of 60 shapes (K = 3584 ..
@@ -316,12 +338,12 @@ PrefillPlan plan_prefill(const RocmMatMulNBitsArgs* a, int tile_choice, uint64_t
             const int occ = tile == 3 ? 2 : (tile == 0 && !bf16) ? 2 : 1;                 // workgroups per CU
             const int sps = (steps + splits - 1) / splits;
             const int sl = (steps + sps - 1) / sps;
-            const int64_t total = workgroups(tile) * sl, cap = 256 * occ;
+            const int64_t total = workgroups(tile) * sl, cap = cus * occ;
             const int64_t full = total / cap, rem = total % cap;
             const double work = sps * step_us[tile];
             double t = full * (work * occ + 8.0);
-            if (rem > 256) t += work * 2 * (0.4 + 0.6 * rem / 512.0) + 8.0;                // (occ = 2: pairs share CUs)
-            else if (rem > 0) t += work * (0.4 + 0.6 * rem / 256.0) + 8.0;
+            if (rem > cus) t += work * 2 * (0.4 + 0.6 * rem / (2.0 * cus)) + 8.0;                // (occ = 2: pairs share CUs)
+            else if (rem > 0) t += work * (0.4 + 0.6 * rem / static_cast<double>(cus)) + 8.0;
             if (sl > 1) t += sl * static_cast<double>(a->m) * static_cast<double>(a->n) * 4.0 / 4e6 + 3.0;
             return t;
         };
@@ -364,9 +386,9 @@ extern "C" int rocm_prefill_mfma_plan(const RocmMatMulNBitsArgs* a, int tile_cho
     return 0;
 }
 
-extern "C" int rocm_launch_prefill_mfma(const RocmMatMulNBitsArgs* a, int tile_choice, void* scratch, uint64_t scratch_bytes, rocm_stream_t stream)
+// The launch of both entry points below. `dense`: a->b is a [N, K] matrix of the activations' 16-bit type instead of packed weights.
+static int launch_tiled(const RocmMatMulNBitsArgs* a, bool dense, int tile_choice, void* scratch, uint64_t scratch_bytes, rocm_stream_t stream)
 {
-    if (!rocm_prefill_mfma_eligible(a)) return -1;
     mnb::PrefillParams p;
     p.a = static_cast<const uint16_t*>(a->a);
     p.b = a->b;
@@ -378,7 +400,7 @@ extern "C" int rocm_launch_prefill_mfma(const RocmMatMulNBitsArgs* a, int tile_c
     p.n = a->n;
     p.k = a->k;
     p.kb = (a->k + a->block_size - 1) / a->block_size;
-    p.row_bytes = p.kb * a->block_size / 2;
+    p.row_bytes = dense ? a->k * 2 : p.kb * a->block_size / 2;
     p.zp_row = (p.kb + 1) / 2;
     p.bs_log2 = __builtin_ctz(static_cast<unsigned>(a->block_size));
     p.scale_dtype = a->scale_dtype;
@@ -386,7 +408,8 @@ extern "C" int rocm_launch_prefill_mfma(const RocmMatMulNBitsArgs* a, int tile_c
     p.y_dtype = a->y_dtype;
     p.nibble_mask = 0x000F000Fu;
     p.magic = a->a_dtype == ROCM_DT_BF16 ? 0x43004300u : 0x64006400u;
-    const PrefillPlan plan = plan_prefill(a, tile_choice, scratch ? scratch_bytes : 0);
+    PrefillPlan plan = plan_prefill(a, tile_choice, scratch ? scratch_bytes : 0);
+    if (dense && plan.tile == 2) plan.tile = 1;          // dense weights: no 256 x 256 build (four times the bytes per column in registers)
     p.steps_per_split = plan.steps_per_split;
     p.partial = plan.splits > 1 ? static_cast<float*>(scratch) : nullptr;
     hipStream_t s = static_cast<hipStream_t>(stream);
@@ -399,13 +422,48 @@ extern "C" int rocm_launch_prefill_mfma(const RocmMatMulNBitsArgs* a, int tile_c
         if (plan.tile == 3) return mnb::launch_prefill<B, 128, 64, S>(p, plan.splits, s);
         return mnb::launch_prefill<B, 128, 128, S>(p, plan.splits, s);
     };
+    auto go_dense = [&](auto bf) {
+        constexpr bool B = decltype(bf)::value;
+        if (plan.tile == 1) return mnb::launch_prefill<B, 256, 128, false, true>(p, plan.splits, s);
+        if (plan.tile == 3) return mnb::launch_prefill<B, 128, 64, false, true>(p, plan.splits, s);
+        return mnb::launch_prefill<B, 128, 128, false, true>(p, plan.splits, s);
+    };
     int rc;
-    if (bf16 && sf32) rc = go(std::true_type{}, std::true_type{});
+    if (dense) rc = bf16 ? go_dense(std::true_type{}) : go_dense(std::false_type{});
+    else if (bf16 && sf32) rc = go(std::true_type{}, std::true_type{});
     else if (bf16) rc = go(std::true_type{}, std::false_type{});
     else if (sf32) rc = go(std::false_type{}, std::true_type{});
     else rc = go(std::false_type{}, std::false_type{});
     if (rc != 0 || plan.splits == 1) return rc;
     return rocm_launch_slice_reduce(static_cast<const float*>(scratch), plan.splits, a->m, a->n, a->bias, a->bias_dtype, a->y, a->y_dtype, stream);
+}
+
+extern "C" int rocm_launch_prefill_mfma(const RocmMatMulNBitsArgs* a, int tile_choice, void* scratch, uint64_t scratch_bytes, rocm_stream_t stream)
+{
+    if (!rocm_prefill_mfma_eligible(a)) return -1;
+    return launch_tiled(a, false, tile_choice, scratch, scratch_bytes, stream);
+}
+
+extern "C" int rocm_prefill_dense16_eligible(const RocmMatMulNBitsArgs* a)
+{
+    const bool half_in = a->a_dtype == ROCM_DT_F16 || a->a_dtype == ROCM_DT_BF16;
+    // From eight rows: what this route replaces is a GEMV of one wave per column that reads every row of A per column
+    // (8 bits, 3584 -> 18944: 28 us at one row, 660 us at sixteen; expansion and tiled kernel together 114 us at 32 rows).
+    if (!(half_in && a->m >= 8 && a->n >= 1 && a->k >= 64 && a->k % 64 == 0)) return 0;
+    if (256 * a->k * 2 >= 0x7fffffff) return 0;                                                  // 32-bit offsets inside one tile
+    return (reinterpret_cast<uintptr_t>(a->a) & 15) == 0;
+}
+
+extern "C" int rocm_launch_prefill_dense16(const RocmMatMulNBitsArgs* a, const void* w16_nk, int tile_choice, void* scratch, uint64_t scratch_bytes, rocm_stream_t stream)
+{
+    if (!rocm_prefill_dense16_eligible(a) || (reinterpret_cast<uintptr_t>(w16_nk) & 15) != 0) return -1;
+    RocmMatMulNBitsArgs d = *a;
+    d.b = static_cast<const uint8_t*>(w16_nk);
+    d.scales = nullptr;
+    d.zp = nullptr;
+    d.scale_dtype = a->a_dtype;
+    d.block_size = 64;                      // (the planner only reads it through the eligibility of the packed form)
+    return launch_tiled(&d, true, tile_choice, scratch, scratch_bytes, stream);
 }
 
 extern "C" int rocm_launch_slice_reduce(const float* partial, int slices, int64_t m, int64_t n, const void* bias, int bias_dtype, void* y, int y_dtype,

@@ -330,7 +330,7 @@ GRAPH_CASES = [
     (E.F16, 64, 4, 5, 96, 512),            # accuracy_level 4 with the caller's workspace: quantizer + int8 MFMA
     (E.F16, 64, 4, 130, 200, 576),
     (E.F16, 64, 4, 130, 200, 2048),        # the same over slices of K: partial sums in the workspace + reduce
-    (E.BF16, 128, 0, 1024, 136, 512),      # tall call: weights expanded to 16 bits + the library GEMM
+    (E.BF16, 128, 0, 1024, 136, 512),      # tall call: the tiled kernel in 256-row tiles (the library GEMM route is opt-in)
 ]
 
 
@@ -675,6 +675,7 @@ NBITS_CASES = [
     (E.BF16, E.BF16, 128, True, 5, 200, 3584),
     (E.F16, E.F32, 16, True, 13, 64, 200),        # K ends inside a block
     (E.F16, E.F16, 64, True, 40, 136, 512),       # tall enough for the dense route at these widths
+    (E.F16, E.F16, 32, True, 9, 100, 640),        # nine rows: already the tiled kernel over the dense copy by default
     (E.BF16, E.BF16, 128, True, 300, 256, 1024),
     (E.F32, E.F16, 64, True, 20, 72, 256),        # f32 activations stay on the plain kernel at any height
     (E.BF16, E.BF16, 128, True, 1, 1030, 3584),   # 8 bits: the 16-byte-load GEMV (one row), ragged column count
@@ -683,18 +684,24 @@ NBITS_CASES = [
 ]
 
 
+@pytest.mark.parametrize("route", ["default", "library"])
 @pytest.mark.parametrize("bits", [2, 8])
 @pytest.mark.parametrize("a_dt,s_dt,bs,zero_points,m,n,k", NBITS_CASES)
-def test_other_bit_widths_match_oracle(ep, ep_dense, port, bits, a_dt, s_dt, bs, zero_points, m, n, k):
-    tall = a_dt != E.F32 and m >= 32 and k % 8 == 0
-    if tall:
-        ep = ep_dense                                  # with the opt-in dense route tall calls leave the plain kernel
+def test_other_bit_widths_match_oracle(ep, ep_dense, port, route, bits, a_dt, s_dt, bs, zero_points, m, n, k):
+    """bits = 2 and 8. Up to 16 rows (and f32 activations at any height) the plain kernel; taller 16-bit calls expand the weights
+    to the activations' type and run this provider's tiled kernel over the dense copy - or, where the provider was created with
+    the opt-in library route, the library GEMM."""
+    tall = a_dt != E.F32 and m >= (32 if route == "library" else 8) and k % 64 == 0
+    if route == "library":
+        if not tall:
+            pytest.skip("the library route only differs on tall calls")
+        ep = ep_dense
     b, s, zp = synth.make_weights_bits(n, k, bs, bits, 50 + bits + n, zero_points=zero_points, scale_lo=0.002 if bits == 8 else 0.02,
                                        scale_hi=0.004 if bits == 8 else 0.04, scale_dtype=s_dt)
     a = synth.make_activation(m, k, 51 + m, a_dt)
     bias = synth.to_dtype(np.linspace(-1, 1, n).astype(np.float32), a_dt)
     y, variant = run_op(ep, a, a_dt, b, s, s_dt, zp, n, k, bs, bias=bias, bias_dtype=a_dt, bits=bits)
-    assert variant == ("dense_transient_blaslt" if tall else "gemv_nbits_f32")
+    assert variant == (("dense_transient_blaslt" if route == "library" else "dense_transient_tiled") if tall else "gemv_nbits_f32")
     want = port.matmul_f64_bits(synth.to_f32(a, a_dt), b, synth.to_f32(s, s_dt), zp, n, k, bs, bits, bias=synth.to_f32(bias, a_dt))
     assert helpers.rel_l2(synth.to_f32(y, a_dt), want) <= (TOL_F32 if a_dt == E.F32 else TOL_HALF)
 
@@ -706,10 +713,16 @@ def test_other_bit_widths_match_oracle(ep, ep_dense, port, bits, a_dt, s_dt, bs,
     (E.BF16, 128, True, 16, 72, 1024, False),
     (E.F16, 64, True, 48, 136, 512, True),          # tall: dense route over weights expanded with their groups
 ])
-def test_g_idx_matches_oracle(ep, ep_dense, port, bits, a_dt, bs, zero_points, m, n, k, with_bias):
-    """Act-order weights (g_idx at input 4): scale and zero point of element k come from group g_idx[k] (matmul_nbits.rs:3636-3658)."""
-    if m >= 32 and a_dt != E.F32:
-        ep = ep_dense                                  # the opt-in dense route; the default provider runs the plain kernel at any height
+@pytest.mark.parametrize("route", ["default", "library"])
+def test_g_idx_matches_oracle(ep, ep_dense, port, route, bits, a_dt, bs, zero_points, m, n, k, with_bias):
+    """Act-order weights (g_idx at input 4): scale and zero point of element k come from group g_idx[k] (matmul_nbits.rs:3636-3658).
+    Tall 16-bit calls expand the weights with their groups and run the tiled kernel over the dense copy (default) or the
+    library GEMM (opt-in)."""
+    tall = m >= (32 if route == "library" else 8) and a_dt != E.F32 and k % 64 == 0
+    if route == "library":
+        if not tall:
+            pytest.skip("the library route only differs on tall calls")
+        ep = ep_dense
     kb = k // bs
     if bits == 4:
         b, s, zp = synth.make_weights(n, k, bs, 60 + n, zero_points=zero_points, scale_lo=0.005, scale_hi=0.02, scale_dtype=a_dt)
@@ -719,7 +732,7 @@ def test_g_idx_matches_oracle(ep, ep_dense, port, bits, a_dt, bs, zero_points, m
     a = synth.make_activation(m, k, 61 + m, a_dt)
     bias = synth.to_dtype(np.linspace(-1, 1, n).astype(np.float32), a_dt) if with_bias else None
     y, variant = run_op(ep, a, a_dt, b, s, a_dt, zp, n, k, bs, bias=bias, bias_dtype=a_dt, bits=bits, g_idx=g)
-    assert variant == ("dense_transient_blaslt" if (m >= 32 and a_dt != E.F32) else "gemv_nbits_f32")
+    assert variant == (("dense_transient_blaslt" if route == "library" else "dense_transient_tiled") if tall else "gemv_nbits_f32")
     w = port.dequantize_nk_gidx(b, synth.to_f32(s, a_dt), zp, g, n, k, bs, bits).astype(np.float64)
     want = synth.to_f32(a, a_dt).astype(np.float64) @ w.T + (synth.to_f32(bias, a_dt).astype(np.float64) if with_bias else 0.0)
     assert helpers.rel_l2(synth.to_f32(y, a_dt), want) <= (TOL_F32 if a_dt == E.F32 else TOL_HALF)

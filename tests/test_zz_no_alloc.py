@@ -63,6 +63,63 @@ def test_execute_static_matches_execute_and_allocates_nothing():
         provider.shutdown()
 
 
+def test_execute_static_on_a_default_provider_after_the_copy_exists():
+    """The default configuration: execute makes the repacked copy of the constant weights on its first call; from then on the
+    static entry point runs the same kernels over that copy - the one-row and few-row decode builds, accuracy_level 4 with the
+    row quantized inside the kernel, and with the codes of 2 .. 16 rows written into the static scratch in the copy's order."""
+    provider = E.RocmExecutionProvider(0)
+    try:
+        calls = [
+            (E.BF16, 128, 0, 1, 304, 3584, E.BF16),       # one row over the repacked stream
+            (E.F16, 32, 0, 4, 528, 2048, E.F16),          # four rows
+            (E.BF16, 128, 0, 16, 272, 3584, E.BF16),      # sixteen rows: the build that stages them per wave
+            (E.F16, 64, 4, 1, 320, 8192, E.F32),          # accuracy_level 4, one row quantized in the kernel
+            (E.F16, 64, 4, 8, 320, 4096, E.F32),          # accuracy_level 4, eight rows: codes and pairs in the static scratch
+            (E.F16, 64, 4, 3, 96, 1024, E.F32),           # the same, smaller, over the same scratch
+        ]
+        for i, (a_dt, bs, acc, m, n, k, y_dt) in enumerate(calls):
+            want, got, v1, v2, allocations = _both_ways(provider, a_dt, bs, acc, m, n, k, y_dt, 970 + i)
+            assert v1 == v2 and ("packed" in v1), (calls[i], v1, v2)
+            assert allocations == 0, (calls[i], allocations)
+            assert np.array_equal(want, got), (calls[i], v1)
+    finally:
+        provider.shutdown()
+
+
+def test_execute_static_with_fewer_slices_than_execute(port):
+    """A tall call whose preferred K slices want more partial sums than the static scratch holds runs with fewer slices: another
+    order of summation than execute's, so the two are held to the oracle's bar, not to each other's bits."""
+    from tests import helpers
+    provider = E.RocmExecutionProvider(0, {"prepack": "0", "dense_gemm_min_rows": "0"})
+    try:
+        a_dt, bs, m, n, k = E.F16, 32, 300, 2048, 16384
+        b, s, zp = synth.make_weights(n, k, bs, 990, zero_points=True, scale_lo=0.002, scale_hi=0.01, scale_dtype=a_dt)
+        a = synth.make_activation(m, k, 991, a_dt)
+        ops = E.DeviceOperands(provider, b, s, a_dt, zp, n, k, bs)
+        need, _ = ops.kernel.workspace_requirement([((m, k), a_dt)])
+        assert need > 8 << 20, need                                  # the preferred plan does not fit the 8 MiB array
+        ab, y1, y2 = provider.upload(a), provider.allocate(m * n * 2), provider.allocate(m * n * 2)
+        try:
+            views = ops.views(ab, a_dt, m)
+            ops.kernel.execute(views, [E.TensorView(y1.ptr, a_dt, (m, n))])
+            before = provider.lib.nxrt_rocm_device_allocation_count()
+            ops.kernel.execute_static(views, [E.TensorView(y2.ptr, a_dt, (m, n))])
+            assert provider.lib.nxrt_rocm_device_allocation_count() == before
+            assert ops.kernel.last_variant() == "prefill_mfma_lds"
+            got1, got2 = provider.download(y1, (m, n), np.float16), provider.download(y2, (m, n), np.float16)
+        finally:
+            for buf in (ab, y1, y2):
+                provider.deallocate(buf)
+            ops.free()
+        cols = np.unique(np.linspace(0, n - 1, 96).astype(np.int64))
+        w = port.dequantize_nk(np.ascontiguousarray(b[cols]), np.ascontiguousarray(s.astype(np.float32)[cols]), np.ascontiguousarray(zp[cols]), len(cols), k, bs)
+        want = a.astype(np.float64) @ w.astype(np.float64).T
+        assert helpers.rel_l2(got1[:, cols], want) <= 5e-3
+        assert helpers.rel_l2(got2[:, cols], want) <= 5e-3
+    finally:
+        provider.shutdown()
+
+
 def test_execute_static_refuses_what_does_not_fit():
     provider = E.RocmExecutionProvider(0, {"prepack": "0", "dense_gemm_min_rows": "0"})
     try:
