@@ -110,6 +110,41 @@ def trace_summary(kernel_trace_csv):
     return out
 
 
+def trace_spread(kernel_trace_csv, calls_per_layer=4, layers=LAYERS):
+    """Where the spread of the decode step's launch durations comes from, out of a rocprofv3 `--kernel-trace` file of this
+    benchmark's step (one graph replay = `layers` x `calls_per_layer` launches + lm_head, in that order). Per call of a layer:
+    percentiles over all launches, and the spread split three ways - between layers (each layer has its own weight buffers:
+    a spread that follows the buffer shows here), between replays (clock, temperature), and what is left inside a layer
+    across replays. No GPU work."""
+    import csv
+    import numpy as np
+    rows = sorted(csv.DictReader(open(kernel_trace_csv)), key=lambda r: int(r["Start_Timestamp"]))
+    rows = [r for r in rows if "decode_packed_kernel" in r["Kernel_Name"] or "decode_wide_kernel" in r["Kernel_Name"]]
+    wgs = lambda r: int(r["Grid_Size_X"]) // max(int(r["Workgroup_Size_X"]), 1)
+    per_replay = layers * calls_per_layer + 1
+    largest = max(wgs(r) for r in rows)
+    ends = [i for i, r in enumerate(rows) if wgs(r) == largest and i >= per_replay - 1]
+    replays = [rows[i - per_replay + 1:i + 1] for i in ends][2:]            # (without the eager pass and the first warm-up replay)
+    dur = np.array([[int(r["End_Timestamp"]) - int(r["Start_Timestamp"]) for r in rep] for rep in replays], dtype=float) / 1e3
+    out = []
+    for j in range(calls_per_layer):
+        sub = dur[:, [calls_per_layer * l + j for l in range(layers)]]        # [replay][layer]
+        by_layer = sub.mean(axis=0)
+        slow = np.argsort(by_layer)[::-1][:3]
+        out.append({"call_of_layer": j, "workgroups": wgs(replays[0][j]), "launches": int(sub.size), "mean_us": round(float(sub.mean()), 2),
+                    "min_us": round(float(sub.min()), 2), "p10_us": round(float(np.percentile(sub, 10)), 2), "p50_us": round(float(np.percentile(sub, 50)), 2),
+                    "p90_us": round(float(np.percentile(sub, 90)), 2), "max_us": round(float(sub.max()), 2),
+                    "mean_over_min": round(float(sub.mean() / sub.min()), 3),
+                    "std_between_layers_us": round(float(by_layer.std()), 3), "std_between_replays_us": round(float(sub.mean(axis=1).std()), 3),
+                    "std_inside_a_layer_us": round(float(sub.std(axis=0).mean()), 3),
+                    "slowest_layers": [{"layer": int(l), "mean_us": round(float(by_layer[l]), 2)} for l in slow]})
+    lm = dur[:, -1]
+    out.append({"call_of_layer": "lm_head", "workgroups": largest, "launches": int(lm.size), "mean_us": round(float(lm.mean()), 2), "min_us": round(float(lm.min()), 2),
+                "max_us": round(float(lm.max()), 2), "mean_over_min": round(float(lm.mean() / lm.min()), 3)})
+    out.append({"replays": len(replays), "sum_of_means_us": round(float(dur.mean(axis=0).sum()), 1), "sum_of_minima_us": round(float(dur.min(axis=0).sum()), 1)})
+    return out
+
+
 def measured_traffic(kernel_template_hint):
     """HBM bytes per launch of the gate/up decode kernel from the tracked counter summary, or None when there is none
     or it was taken on another kernel."""
@@ -381,8 +416,12 @@ def main():
                     help="run only the prefill and accuracy_level=4 tables, one JSON line per row (the command their profiles are taken from)")
     ap.add_argument("--traffic-from", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
                     help="no GPU work: turn two rocprofv3 counter files of --only-roofline runs (FETCH_SIZE, WRITE_SIZE) into profiles/decode_gate_up_m1_traffic.txt")
+    ap.add_argument("--trace-spread", metavar="KERNEL_TRACE_CSV",
+                    help="no GPU work: per call of a layer, the percentiles of the step's launch durations in a rocprofv3 kernel trace and how their spread splits between layers, replays and the rest")
     ap.add_argument("--trace-summary", metavar="KERNEL_TRACE_CSV",
                     help="no GPU work: per kernel and launch shape of a rocprofv3 --kernel-trace file of this benchmark, one JSON line each")
+    ap.add_argument("--lds-probe", action="store_true",
+                    help="only measure what one CU's LDS moves per clock (reads, writes, global memory straight into LDS, mixed) and print one JSON line")
     ap.add_argument("--read-floor", action="store_true",
                     help="run only the yardstick: a plain read of each decode shape's bytes, one launch per layer buffer in a graph, beside the decode kernel's time on the same buffers")
     ap.add_argument("--row-sweep", action="store_true",
@@ -396,6 +435,10 @@ def main():
     if args.traffic_from:
         print(json.dumps(traffic_from_counters(*args.traffic_from)), flush=True)
         return
+    if args.trace_spread:
+        for row in trace_spread(args.trace_spread, layers=args.layers):
+            print(json.dumps(row), flush=True)
+        return
     if args.trace_summary:
         for row in trace_summary(args.trace_summary):
             print(json.dumps(row), flush=True)
@@ -405,6 +448,13 @@ def main():
     info = ep.device_info()
     if args.only_roofline:
         return roofline_only(ep, args)
+    if args.lds_probe:
+        names = {0: "ds_read_b128", 1: "ds_write_b128", 2: "buffer_load_dwordx4 ... lds", 3: "half the waves read, half write"}
+        table = [{"access": names[mode], "waves_per_cu": waves, "bytes_per_clock_per_cu": round(ep.lds_probe(mode, waves), 1)}
+                 for mode in (0, 1, 2, 3) for waves in (1, 4, 8, 16)]
+        print(json.dumps({"lds_probe": table}))
+        ep.shutdown()
+        return
     if args.read_floor:
         for row in read_floor(ep, args):
             print(json.dumps(row), flush=True)

@@ -75,6 +75,10 @@ NxrtStatus nxrt_rocm_ep_sync(NxrtRocmEp* ep);
  * loads, four in flight per lane, one workgroup per 16 KiB) and keeps nothing. Its time is the least any kernel can spend
  * pulling that many bytes from HBM; bench.py --read-floor reports it beside the decode kernels' times. */
 NxrtStatus nxrt_rocm_ep_read_probe(NxrtRocmEp* ep, const void* src_device, size_t bytes);
+/* Diagnostic for benchmarks (no counterpart in the reference): bytes per clock one CU's LDS moves with `waves` waves (1..16)
+ * of a workgroup repeating 16-byte accesses. mode 0: reads; 1: writes; 2: global memory straight into LDS; 3: half the waves
+ * read while the others write. Synchronous; allocates and frees its own small buffers. */
+NxrtStatus nxrt_rocm_ep_lds_probe(NxrtRocmEp* ep, uint32_t mode, uint32_t waves, uint32_t iters, double* bytes_per_clock);
 /* The nxrt EP vtable whose ctx is this provider (what NxrtEpFactoryVtable.create_ep hands out);
  * the inverse recovers the provider from a vtable obtained through the plugin exports. */
 NxrtRocmEp* nxrt_rocm_ep_from_vtable(const NxrtEpVtable* vtable);
@@ -175,6 +179,10 @@ NxrtStatus nxrt_rocm_matmul_nbits_execute_static(NxrtRocmMatMulNBits* kernel, co
 uint64_t nxrt_rocm_matmul_nbits_estimated_flops(const NxrtRocmMatMulNBits* kernel);
 /* record_kernel_variant (kernel.rs:361): which kernel served the last execute. */
 const char* nxrt_rocm_matmul_nbits_last_variant(const NxrtRocmMatMulNBits* kernel);
+/* record_kernel_metrics (onnx-runtime-ep-api/src/kernel.rs:243-267, called at matmul_nbits.rs:1588-1597): what the last plain
+ * execute moved and computed by the reference's count - bytes = the bytes of every present input tensor + the output's;
+ * flops = 2*M*N*K, + M*N with a bias. Zero before the first call. */
+void nxrt_rocm_matmul_nbits_last_metrics(const NxrtRocmMatMulNBits* kernel, uint64_t* flops, uint64_t* bytes);
 void nxrt_rocm_matmul_nbits_release(NxrtRocmMatMulNBits* kernel);
 /* The same kernel behind the nxrt kernel vtable (raw pointers only: the shapes are those given at
  * create time, M taken from input_shapes[0]). The host calls release(ctx) once. */

@@ -146,6 +146,7 @@ struct NxrtRocmMatMulNBits {
     std::mutex norm_mu;                  // held across a normalized call: `norm` feeds the kernels enqueued under it
     bool constant_inputs[6] = {false, false, false, false, false, false};
     std::string variant = "none";
+    uint64_t last_flops = 0, last_bytes = 0;   // of the last plain MatMulNBits call: what the CPU provider's record_kernel_metrics notes (matmul_nbits.rs:1588-1597)
     void* scratch = nullptr;             // kernel-owned workspace, grown on demand
     size_t scratch_bytes = 0;
     std::vector<void*> retired;          // outgrown workspaces: kept until the kernel dies, since a HIP graph recorded earlier may still name them
@@ -547,6 +548,20 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
 
     uint64_t M = 1;
     for (uint32_t i = 0; i + 1 < A.ndim; ++i) M *= A.shape[i];
+    {
+        // record_kernel_metrics (onnx-runtime-ep-api/src/kernel.rs:243-267): bytes = every present input's bytes + the output's;
+        // flops = 2 M N K, + M N with a bias (matmul_nbits.rs:1588-1597)
+        uint64_t bytes = 0;
+        for (const Named& t : all) {
+            if (!t.v) continue;
+            uint64_t elems = 1;
+            for (uint32_t i = 0; i < t.v->ndim; ++i) elems *= t.v->shape[i];
+            const uint32_t dt = t.v->dtype;
+            bytes += elems * (dt == NXRT_DT_FLOAT32 || dt == NXRT_DT_INT32 ? 4u : dt == NXRT_DT_UINT8 ? 1u : 2u);
+        }
+        kn.last_bytes = bytes;
+        kn.last_flops = 2ull * M * static_cast<uint64_t>(kn.n) * static_cast<uint64_t>(kn.k) + (BIAS ? M * static_cast<uint64_t>(kn.n) : 0ull);
+    }
     if (M == 0) return ok();
     // A required tensor without memory behind it would reach a kernel as address 0: a GPU memory fault instead of a status.
     for (const Named& t : {Named{"A", &A}, Named{"B", &B}, Named{"scales", &S}, Named{"Y", &Y}})
@@ -1155,6 +1170,12 @@ uint64_t nxrt_rocm_matmul_nbits_estimated_flops(const NxrtRocmMatMulNBits* kerne
 }
 
 const char* nxrt_rocm_matmul_nbits_last_variant(const NxrtRocmMatMulNBits* kernel) { return kernel ? kernel->variant.c_str() : ""; }
+
+void nxrt_rocm_matmul_nbits_last_metrics(const NxrtRocmMatMulNBits* kernel, uint64_t* flops, uint64_t* bytes)
+{
+    if (flops) *flops = kernel ? kernel->last_flops : 0;
+    if (bytes) *bytes = kernel ? kernel->last_bytes : 0;
+}
 
 void nxrt_rocm_matmul_nbits_release(NxrtRocmMatMulNBits* kernel) { vtable_release(kernel); }
 

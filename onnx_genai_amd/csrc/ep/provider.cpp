@@ -219,6 +219,16 @@ NxrtStatus nxrt_rocm_ep_read_probe(NxrtRocmEp* ep, const void* src, size_t bytes
     });
 }
 
+NxrtStatus nxrt_rocm_ep_lds_probe(NxrtRocmEp* ep, uint32_t mode, uint32_t waves, uint32_t iters, double* bytes_per_clock)
+{
+    return fenced([&]() -> NxrtStatus {
+        if (!ep || !bytes_per_clock) return make_status(NXRT_INVALID_ARGUMENT, "lds_probe: null pointer");
+        NxrtStatus st = ep->bind();
+        if (st.code != NXRT_OK) return st;
+        return hip_status(rocm_ffi_lds_probe(static_cast<int>(mode), static_cast<int>(waves), static_cast<int>(iters), bytes_per_clock), "LDS probe");
+    });
+}
+
 NxrtStatus nxrt_rocm_ep_sync(NxrtRocmEp* ep)
 {
     return fenced([&]() -> NxrtStatus {

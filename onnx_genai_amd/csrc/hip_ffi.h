@@ -47,6 +47,10 @@ int rocm_ffi_memcpy_d2h(void* dst, const void* src, size_t bytes, rocm_stream_t 
 /* Reads `bytes` (a multiple of 16 is read) of device memory and keeps nothing: the time of the plainest kernel that pulls
  * that many bytes, for benchmarks to hold other kernels against. `sink`: 4 writable bytes, or NULL. */
 int rocm_ffi_read_probe(const void* src, size_t bytes, void* sink, rocm_stream_t stream);
+/* Bytes per clock one CU's LDS moves when `waves` waves (1..16) of one workgroup per CU each repeat eight 16-byte accesses
+ * per lane `iters` times. mode 0: ds_read_b128; 1: ds_write_b128; 2: global memory straight into LDS; 3: even waves read, odd
+ * waves write (the figure is the sum of both). Synchronous, allocates its own small buffers: a diagnostic, not a kernel path. */
+int rocm_ffi_lds_probe(int mode, int waves, int iters, double* bytes_per_clock);
 int rocm_ffi_memcpy_d2d(void* dst, const void* src, size_t bytes, rocm_stream_t stream);
 int rocm_ffi_stream_create(rocm_stream_t* stream);
 int rocm_ffi_stream_destroy(rocm_stream_t stream);

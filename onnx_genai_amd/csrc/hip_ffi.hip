@@ -43,9 +43,96 @@ __global__ __launch_bounds__(256) void read_probe_kernel(const uint4* __restrict
     for (int i = 0; i < 4; ++i) x ^= v[i].x ^ v[i].y ^ v[i].z ^ v[i].w;
     if (x == 0x9e3779b9u && sink) *sink = x;
 }
+
+// What one CU's LDS moves per clock, by kind of access: every workgroup (one per CU, `waves` waves) repeats eight 16-byte
+// accesses per lane and waits for them, `iters` times; lane 0 of each wave notes the cycles it took. MODE 0: ds_read_b128;
+// 1: ds_write_b128; 2: global memory straight into LDS (buffer_load_dwordx4 ... lds, from a small buffer that stays in
+// cache); 3: even waves read while odd waves write. The tiled kernels' step is sized against these figures.
+typedef __attribute__((ext_vector_type(4))) uint32_t lds_u32x4_t;
+template <int MODE>
+__global__ __launch_bounds__(1024) void lds_probe_kernel(unsigned long long* cycles, const uint32_t* src, int iters)
+{
+    extern __shared__ __attribute__((aligned(16))) unsigned char probe_smem[];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    for (int i = threadIdx.x; i < 16384; i += blockDim.x) reinterpret_cast<uint32_t*>(probe_smem)[i] = i;
+    __syncthreads();
+    lds_u32x4_t srd;
+    const uint64_t base = reinterpret_cast<uint64_t>(src);
+    srd.x = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(base));
+    srd.y = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(base >> 32));
+    srd.z = 1u << 20;
+    srd.w = 0x00020000u;
+    const uint32_t off = lane * 16;
+    lds_u32x4_t acc = {1, 2, 3, 4};
+    const int role = MODE == 3 ? (wave & 1) : MODE;
+    const unsigned long long t0 = __builtin_readcyclecounter();
+    for (int it = 0; it < iters; ++it) {
+        if (role == 0) {
+            lds_u32x4_t v[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const uint32_t a = (off + ((j + wave) & 7) * 4096 + ((it & 1) << 10)) & 0xfff0;
+                asm volatile("ds_read_b128 %0, %1" : "=v"(v[j]) : "v"(a));
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                asm volatile("" ::"v"(v[j]));
+                acc.x ^= v[j].x;
+            }
+        } else if (role == 1) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const uint32_t a = (off + ((j + wave) & 7) * 4096 + ((it & 1) << 10)) & 0xfff0;
+                asm volatile("ds_write_b128 %0, %1" ::"v"(a), "v"(acc));
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const uint32_t lds = __builtin_amdgcn_readfirstlane((((j + wave) & 7) * 4096 + ((it & 1) << 10)) & 0xffff);
+                const uint32_t soff = (j * 1024 + wave * 8192 + blockIdx.x * 131072) & 0xfffff;
+                asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds" ::"s"(lds), "v"(off), "s"(srd), "s"(soff) : "memory");
+            }
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
+    }
+    const unsigned long long t1 = __builtin_readcyclecounter();
+    if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x12345) cycles[1000] = 1;
+    if (lane == 0) cycles[blockIdx.x * 16 + wave] = t1 - t0;
+}
 }  // namespace
 
 extern "C" {
+
+int rocm_ffi_lds_probe(int mode, int waves, int iters, double* bytes_per_clock)
+{
+    if (mode < 0 || mode > 3 || waves < 1 || waves > 16 || iters < 1 || !bytes_per_clock) return static_cast<int>(hipErrorInvalidValue);
+    constexpr int kBlocks = 256;
+    unsigned long long* dev = nullptr;
+    uint32_t* src = nullptr;
+    hipError_t e = static_cast<hipError_t>(rocm_ffi_malloc(reinterpret_cast<void**>(&dev), (kBlocks * 16 + 1024) * sizeof(unsigned long long)));
+    if (e == hipSuccess) e = static_cast<hipError_t>(rocm_ffi_malloc(reinterpret_cast<void**>(&src), 1u << 21));
+    if (e == hipSuccess) e = hipMemset(src, 1, 1u << 21);
+    if (e == hipSuccess) {
+        const dim3 grid(kBlocks), block(static_cast<unsigned>(waves * 64));
+        if (mode == 0) hipLaunchKernelGGL(lds_probe_kernel<0>, grid, block, 65536, nullptr, dev, src, iters);
+        else if (mode == 1) hipLaunchKernelGGL(lds_probe_kernel<1>, grid, block, 65536, nullptr, dev, src, iters);
+        else if (mode == 2) hipLaunchKernelGGL(lds_probe_kernel<2>, grid, block, 65536, nullptr, dev, src, iters);
+        else hipLaunchKernelGGL(lds_probe_kernel<3>, grid, block, 65536, nullptr, dev, src, iters);
+        e = hipGetLastError();
+    }
+    unsigned long long host[16] = {};
+    if (e == hipSuccess) e = hipDeviceSynchronize();
+    if (e == hipSuccess) e = hipMemcpy(host, dev, sizeof(host), hipMemcpyDeviceToHost);
+    if (dev) (void)rocm_ffi_free(dev);
+    if (src) (void)rocm_ffi_free(src);
+    if (e != hipSuccess) return static_cast<int>(e);
+    unsigned long long longest = 1;
+    for (int w = 0; w < waves; ++w) longest = host[w] > longest ? host[w] : longest;
+    *bytes_per_clock = static_cast<double>(waves) * iters * 8.0 * 64.0 * 16.0 / static_cast<double>(longest);
+    return 0;
+}
 
 int rocm_ffi_read_probe(const void* src, size_t bytes, void* sink, rocm_stream_t stream)
 {

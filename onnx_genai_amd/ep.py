@@ -99,6 +99,8 @@ def load_library() -> C.CDLL:
     L.nxrt_rocm_ep_copy.argtypes = [v, v, v, sz]
     L.nxrt_rocm_ep_read_probe.restype = S
     L.nxrt_rocm_ep_read_probe.argtypes = [v, v, sz]
+    L.nxrt_rocm_ep_lds_probe.restype = S
+    L.nxrt_rocm_ep_lds_probe.argtypes = [v, u32, u32, u32, C.POINTER(C.c_double)]
     L.nxrt_rocm_ep_sync.restype = S
     L.nxrt_rocm_ep_sync.argtypes = [v]
     L.nxrt_rocm_ep_from_vtable.restype = v
@@ -121,6 +123,8 @@ def load_library() -> C.CDLL:
     L.nxrt_rocm_matmul_nbits_estimated_flops.argtypes = [v]
     L.nxrt_rocm_matmul_nbits_last_variant.restype = C.c_char_p
     L.nxrt_rocm_matmul_nbits_last_variant.argtypes = [v]
+    L.nxrt_rocm_matmul_nbits_last_metrics.restype = None
+    L.nxrt_rocm_matmul_nbits_last_metrics.argtypes = [v, C.POINTER(u64), C.POINTER(u64)]
     L.nxrt_rocm_matmul_nbits_release.restype = None
     L.nxrt_rocm_matmul_nbits_release.argtypes = [v]
     L.nxrt_rocm_matmul_nbits_set_block_acc_probe.restype = S
@@ -293,6 +297,12 @@ class RocmExecutionProvider:
         """Enqueues a plain read of `nbytes` of `src` (a benchmark's yardstick: the least time a kernel can take to pull them)."""
         self.lib.nxrt_rocm_ep_read_probe(self.handle, src.ptr, nbytes).check()
 
+    def lds_probe(self, mode: int, waves: int, iters: int = 2000) -> float:
+        """Bytes per clock one CU's LDS moves (mode 0 reads, 1 writes, 2 global memory straight into LDS, 3 reads and writes mixed)."""
+        out = C.c_double()
+        self.lib.nxrt_rocm_ep_lds_probe(self.handle, mode, waves, iters, C.byref(out)).check()
+        return out.value
+
     def sync(self) -> None:
         self.lib.nxrt_rocm_ep_sync(self.handle).check()
 
@@ -454,6 +464,12 @@ class MatMulNBitsKernel:
 
     def last_variant(self) -> str:
         return self.lib.nxrt_rocm_matmul_nbits_last_variant(self.handle).decode()
+
+    def last_metrics(self) -> tuple[int, int]:
+        """(flops, bytes) of the last plain call, by the reference's count (record_kernel_metrics)."""
+        flops, nbytes = C.c_uint64(), C.c_uint64()
+        self.lib.nxrt_rocm_matmul_nbits_last_metrics(self.handle, C.byref(flops), C.byref(nbytes))
+        return flops.value, nbytes.value
 
     def set_block_acc_probe(self, buf: DeviceBuffer | None) -> None:
         """accuracy_level 4: later executes also store their int32 block accumulators [M, N, kb] into `buf` (None clears)."""

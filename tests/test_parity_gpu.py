@@ -1564,6 +1564,30 @@ def test_execute_validation_messages(ep):
     ops.free()
 
 
+def test_last_call_metrics_follow_the_reference_count(ep):
+    """record_kernel_metrics (onnx-runtime-ep-api/src/kernel.rs:243-267, matmul_nbits.rs:1588-1597): bytes = every present input's
+    bytes plus the output's; flops = 2 M N K, plus M N with a bias."""
+    a_dt, bs, m, n, k = E.BF16, 128, 3, 80, 512
+    kb = k // bs
+    b, s, zp = synth.make_weights(n, k, bs, 35, zero_points=True, scale_lo=0.002, scale_hi=0.01, scale_dtype=a_dt)
+    bias = synth.to_dtype(np.linspace(-1, 1, n).astype(np.float32), a_dt)
+    for with_bias in (False, True):
+        ops = E.DeviceOperands(ep, b, s, a_dt, zp, n, k, bs, bias=bias if with_bias else None, bias_dtype=a_dt)
+        assert ops.kernel.last_metrics() == (0, 0)
+        ab, yb = ep.upload(synth.make_activation(m, k, 36, a_dt)), ep.allocate(m * n * 2)
+        try:
+            ops.run(ab, a_dt, m, yb)
+            ep.sync()
+            flops, nbytes = ops.kernel.last_metrics()
+        finally:
+            ep.deallocate(ab)
+            ep.deallocate(yb)
+            ops.free()
+        want_bytes = m * k * 2 + n * kb * (bs // 2) + n * kb * 2 + n * ((kb + 1) // 2) + (n * 2 if with_bias else 0) + m * n * 2
+        assert flops == 2 * m * n * k + (m * n if with_bias else 0)
+        assert nbytes == want_bytes
+
+
 def test_kernel_vtable_execute(ep, port):
     """The nxrt kernel vtable (raw pointers only) runs the same kernel with the create-time shapes."""
     import ctypes as C
