@@ -223,6 +223,20 @@ int grow_buffer(void*& buf, size_t& bytes, uint64_t need, std::vector<void*>& re
     return 0;
 }
 
+// A copy of the weights (repacked or dense) that a call with other weights has replaced. Once the provider has recorded a
+// HIP graph, a graph may still replay through the copy, so it is kept until the kernel dies. Before that, nothing can name
+// it after the stream has drained, and it is freed: a host that alternates a node between weight sets without recording
+// graphs holds one copy, not one per switch. (Never called while frozen.)
+void drop_weight_copy(NxrtRocmMatMulNBits& kn, void* old)
+{
+    if (kn.ep->captures.load() != 0) {
+        kn.retired.push_back(old);
+        return;
+    }
+    rocm_ffi_stream_sync(kn.ep->stream);
+    rocm_ffi_free(old);
+}
+
 // True when the call can run on the repacked copy of constant weights; makes that copy on first use (never while a
 // graph capture is open: a capture may neither allocate nor should it record the one-time repack). `rc` receives a
 // HIP error of the repack.
@@ -236,7 +250,7 @@ bool use_packed(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& args, int& r
     if (current) return true;
     if (frozen(kn)) return false;
     if (kn.packed) {
-        kn.retired.push_back(kn.packed);    // not freed: a HIP graph recorded over the old weights may still replay through it
+        drop_weight_copy(kn, kn.packed);
         kn.packed = nullptr;
     }
     if (rocm_ffi_malloc(&kn.packed, rocm_decode_packed_bytes(&args)) != 0) {
@@ -312,7 +326,7 @@ bool dense_route(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& args, int& 
         if (!current) {
             if (ep.capturing) return false;
             if (kn.dense) {
-                kn.retired.push_back(kn.dense);     // kept for graphs recorded over the old weights
+                drop_weight_copy(kn, kn.dense);
                 kn.dense = nullptr;
             }
             if (rocm_ffi_malloc(&kn.dense, need) != 0) {

@@ -289,7 +289,10 @@ NxrtStatus nxrt_rocm_ep_capture_begin(NxrtRocmEp* ep)
         if (st.code != NXRT_OK) return st;
         if (ep->capturing) return make_status(NXRT_INVALID_ARGUMENT, "capture_begin: a capture is already open on this provider");
         st = hip_status(rocm_ffi_capture_begin(ep->stream), "hipStreamBeginCapture");
-        if (st.code == NXRT_OK) ep->capturing = true;
+        if (st.code == NXRT_OK) {
+            ep->capturing = true;
+            ep->captures.fetch_add(1);
+        }
         return st;
     });
 }

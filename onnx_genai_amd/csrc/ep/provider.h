@@ -37,6 +37,7 @@ struct NxrtRocmEp {
     void* static_scratch = nullptr;               // this GPU's static scratch array (device address), resolved when the provider is created
     size_t static_scratch_bytes = 0;
     bool capturing = false;                       // a stream capture is open: nothing may allocate or synchronise
+    std::atomic<uint64_t> captures{0};            // stream captures opened on this provider so far: while 0, no HIP graph can name a buffer of its kernels
     // The host may release the provider, its kernels and its allocators in any order (each vtable is released exactly
     // once, independently): every kernel object and allocator handle holds one reference, the creator holds the first,
     // and the provider dies with the last.

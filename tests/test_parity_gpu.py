@@ -416,31 +416,50 @@ def test_graph_survives_a_later_larger_call(ep_tiled):
         ops.free()
 
 
-def test_packed_copy_follows_the_weights(ep, port):
-    """One kernel object, two different weight tensors in turn: the repacked copy is rebuilt when the pointers change."""
+def test_packed_copy_follows_the_weights(port):
+    """One kernel object, two weight tensors in turn: the repacked copy is rebuilt when the pointers change. The replaced
+    copy is freed while the provider has recorded no graph, and kept once it has (a graph may replay through it)."""
+    ep = E.RocmExecutionProvider(0)
     a_dt, bs, m, n, k = E.F16, 128, 1, 96, 1024
     a = synth.make_activation(m, k, 5, a_dt)
-    ab, yb = ep.upload(a), ep.allocate(m * n * 4)
+    ab, yb, yg = ep.upload(a), ep.allocate(m * n * 4), ep.allocate(m * n * 4)
     b1, s1, zp1 = synth.make_weights(n, k, bs, 31, zero_points=True, scale_lo=0.002, scale_hi=0.01, scale_dtype=a_dt)
     first = E.DeviceOperands(ep, b1, s1, a_dt, zp1, n, k, bs)
     b2, s2, zp2 = synth.make_weights(n, k, bs, 32, zero_points=True, scale_lo=0.002, scale_hi=0.01, scale_dtype=a_dt)
     other = [ep.upload(b2), ep.upload(s2), ep.upload(zp2)]
     kb = k // bs
-    first.kernel.execute(first.views(ab, a_dt, m), [E.TensorView(yb.ptr, E.F32, (m, n))])
-    y1 = ep.download(yb, (m, n), np.float32)
+    views1 = first.views(ab, a_dt, m)
     views2 = [E.TensorView(ab.ptr, a_dt, (m, k)), E.TensorView(other[0].ptr, E.U8, (n, kb, bs // 2)),
               E.TensorView(other[1].ptr, a_dt, (n, kb)), E.TensorView(other[2].ptr, E.U8, (n, (kb + 1) // 2))]
+    want1 = oracle_f64(port, a, a_dt, b1, s1, a_dt, zp1, n, k, bs)
+    want2 = oracle_f64(port, a, a_dt, b2, s2, a_dt, zp2, n, k, bs)
+    first.kernel.execute(views1, [E.TensorView(yb.ptr, E.F32, (m, n))])
+    assert helpers.rel_l2(ep.download(yb, (m, n), np.float32), want1) <= 1e-4
+    for _ in range(3):                        # back and forth without a graph: every replaced copy is freed
+        first.kernel.execute(views2, [E.TensorView(yb.ptr, E.F32, (m, n))])
+        assert first.kernel.last_variant() == "decode_mfma_packed"
+        assert helpers.rel_l2(ep.download(yb, (m, n), np.float32), want2) <= 1e-4
+        first.kernel.execute(views1, [E.TensorView(yb.ptr, E.F32, (m, n))])
+        assert helpers.rel_l2(ep.download(yb, (m, n), np.float32), want1) <= 1e-4
     assert first.kernel.retired_buffers() == 0
+    ep.sync()
+    ep.capture_begin()
+    try:
+        first.kernel.execute(views1, [E.TensorView(yg.ptr, E.F32, (m, n))])
+    finally:
+        graph = ep.capture_end()
+    # the graph reads the copy made from the first weights: a call with the second keeps that copy
     first.kernel.execute(views2, [E.TensorView(yb.ptr, E.F32, (m, n))])
-    assert first.kernel.last_variant() == "decode_mfma_packed"
-    # the copy made from the first weights is kept, not freed: a graph recorded over it may still be replayed
     assert first.kernel.retired_buffers() == 1
-    y2 = ep.download(yb, (m, n), np.float32)
-    assert helpers.rel_l2(y1, oracle_f64(port, a, a_dt, b1, s1, a_dt, zp1, n, k, bs)) <= 1e-4
-    assert helpers.rel_l2(y2, oracle_f64(port, a, a_dt, b2, s2, a_dt, zp2, n, k, bs)) <= 1e-4
-    for buf in other + [ab, yb]:
+    assert helpers.rel_l2(ep.download(yb, (m, n), np.float32), want2) <= 1e-4
+    graph.replay()
+    ep.sync()
+    assert helpers.rel_l2(ep.download(yg, (m, n), np.float32), want1) <= 1e-4
+    graph.release()
+    for buf in other + [ab, yb, yg]:
         ep.deallocate(buf)
     first.free()
+    ep.shutdown()
 
 
 def test_decode_is_deterministic(ep):
