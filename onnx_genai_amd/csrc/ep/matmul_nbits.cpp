@@ -273,7 +273,7 @@ bool use_packed(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& args, int& r
 // Tall 16-bit calls over a dense [N, K] copy of the weights in the activations' type, expanded by a launch of its own. Two users:
 //  * the opt-in library route (dense_gemm_min_rows > 0): the product is the library GEMM, as in the CUDA provider for M >= 8
 //    (onnx-runtime-ep-cuda/src/kernels/matmul_nbits.rs:6176-6222);
-//  * by default, calls of more than 16 rows whose weights the tile loader does not read - bits = 2 / 8 and weights with g_idx
+//  * by default, calls from five rows whose weights the tile loader does not read - bits = 2 / 8 and weights with g_idx
 //    (matmul_nbits.rs:2035, 3636-3658): the product is this provider's own tiled kernel over the dense copy, instead of a
 //    one-wave-per-column GEMV that reads all M rows of A per column.
 // Returns false with nothing launched when the route does not apply or is not ready (then the caller's next route takes the
@@ -296,7 +296,7 @@ bool dense_route(NxrtRocmMatMulNBits& kn, const RocmMatMulNBitsArgs& args, int& 
     if (args.y_dtype != args.a_dtype || (reinterpret_cast<uintptr_t>(args.y) & 15) != 0 ||
         (args.bias && (args.bias_dtype & (ROCM_BIAS_POST_ROUND | ROCM_BIAS_PER_ROW))))
         library = false;
-    const bool own = plain_only && rocm_prefill_dense16_eligible(&args);      // (more than 16 rows, K a multiple of 64)
+    const bool own = plain_only && rocm_prefill_dense16_eligible(&args);      // (five rows or more, K a multiple of 64)
     if (!library && !own) return false;
     const int bias_dtype = args.bias ? args.bias_dtype : -1;
 
@@ -645,8 +645,8 @@ NxrtStatus execute_impl(NxrtRocmMatMulNBits& kn, const NxrtRocmTensorView* in, u
         kn.g_idx_checked = args.g_idx;
     }
     if (kn.bits != 4 || G) {
-        // 2 and 8 bits, and act-order weights of any width: tall 16-bit calls expand the weights and run the library GEMM,
-        // everything else the plain f32 GEMV
+        // 2 and 8 bits, and act-order weights of any width: 16-bit calls from five rows expand the weights and run the tiled
+        // kernel over the dense copy (or, opt-in, the library GEMM), everything else the plain f32 GEMV
         if (!dense_route(kn, args, rc)) {
             rc = rocm_launch_gemv_nbits(&args, static_cast<int>(kn.bits), stream);
             kn.variant = "gemv_nbits_f32";

@@ -447,9 +447,11 @@ extern "C" int rocm_launch_prefill_mfma(const RocmMatMulNBitsArgs* a, int tile_c
 extern "C" int rocm_prefill_dense16_eligible(const RocmMatMulNBitsArgs* a)
 {
     const bool half_in = a->a_dtype == ROCM_DT_F16 || a->a_dtype == ROCM_DT_BF16;
-    // From eight rows: what this route replaces is a GEMV of one wave per column that reads every row of A per column
-    // (8 bits, 3584 -> 18944: 28 us at one row, 660 us at sixteen; expansion and tiled kernel together 114 us at 32 rows).
-    if (!(half_in && a->m >= 8 && a->n >= 1 && a->k >= 64 && a->k % 64 == 0)) return 0;
+    // From five rows: what this route replaces is a GEMV of one wave per column that reads every row of A per column
+    // (8 bits, 3584 -> 18944: 28 us at one row, 306 us at seven; 2 bits, 4096 -> 14336: 115 and 720 us), while expansion and
+    // tiled kernel together cost the same at every height up to a few dozen rows (110-115 us and 166-170 us on those two).
+    // Up to four rows the 8-bit GEMV with 16-byte loads is the better one.
+    if (!(half_in && a->m >= 5 && a->n >= 1 && a->k >= 64 && a->k % 64 == 0)) return 0;
     if (256 * a->k * 2 >= 0x7fffffff) return 0;                                                  // 32-bit offsets inside one tile
     return (reinterpret_cast<uintptr_t>(a->a) & 15) == 0;
 }

@@ -694,7 +694,7 @@ NBITS_CASES = [
     (E.BF16, E.BF16, 128, True, 5, 200, 3584),
     (E.F16, E.F32, 16, True, 13, 64, 200),        # K ends inside a block
     (E.F16, E.F16, 64, True, 40, 136, 512),       # tall enough for the dense route at these widths
-    (E.F16, E.F16, 32, True, 9, 100, 640),        # nine rows: already the tiled kernel over the dense copy by default
+    (E.F16, E.F16, 32, True, 9, 100, 640),        # nine rows: the tiled kernel over the dense copy by default (from five)
     (E.BF16, E.BF16, 128, True, 300, 256, 1024),
     (E.F32, E.F16, 64, True, 20, 72, 256),        # f32 activations stay on the plain kernel at any height
     (E.BF16, E.BF16, 128, True, 1, 1030, 3584),   # 8 bits: the 16-byte-load GEMV (one row), ragged column count
@@ -707,10 +707,10 @@ NBITS_CASES = [
 @pytest.mark.parametrize("bits", [2, 8])
 @pytest.mark.parametrize("a_dt,s_dt,bs,zero_points,m,n,k", NBITS_CASES)
 def test_other_bit_widths_match_oracle(ep, ep_dense, port, route, bits, a_dt, s_dt, bs, zero_points, m, n, k):
-    """bits = 2 and 8. Up to 16 rows (and f32 activations at any height) the plain kernel; taller 16-bit calls expand the weights
+    """bits = 2 and 8. Up to four rows (and f32 activations, or K not a multiple of 64, at any height) the plain kernel; taller 16-bit calls expand the weights
     to the activations' type and run this provider's tiled kernel over the dense copy - or, where the provider was created with
     the opt-in library route, the library GEMM."""
-    tall = a_dt != E.F32 and m >= (32 if route == "library" else 8) and k % 64 == 0
+    tall = a_dt != E.F32 and m >= (32 if route == "library" else 5) and k % 64 == 0
     if route == "library":
         if not tall:
             pytest.skip("the library route only differs on tall calls")
@@ -737,7 +737,7 @@ def test_g_idx_matches_oracle(ep, ep_dense, port, route, bits, a_dt, bs, zero_po
     """Act-order weights (g_idx at input 4): scale and zero point of element k come from group g_idx[k] (matmul_nbits.rs:3636-3658).
     Tall 16-bit calls expand the weights with their groups and run the tiled kernel over the dense copy (default) or the
     library GEMM (opt-in)."""
-    tall = m >= (32 if route == "library" else 8) and a_dt != E.F32 and k % 64 == 0
+    tall = m >= (32 if route == "library" else 5) and a_dt != E.F32 and k % 64 == 0
     if route == "library":
         if not tall:
             pytest.skip("the library route only differs on tall calls")
