@@ -1,8 +1,9 @@
 // MatMulNBits at the bit widths other than 4 that the CPU provider takes (2 and 8; NBitsLayout,
 // onnx-runtime-ep-cpu/src/kernels/matmul_nbits.rs:1276-1321): element i of a packed row sits in byte i / (8 / bits) at
 // bit (i % (8 / bits)) * bits, zero points are packed the same way (default 1 << (bits - 1)), w = (q - zp) * scale with one
-// f32 multiply. These widths get the plain kernels only: dequantization (f32 for the parity probe, 16 bits for the dense
-// route's library GEMM) and an f32 GEMV with one wave per output column; the tuned kernels are 4-bit.
+// f32 multiply. These widths get plain kernels: dequantization (f32 for the parity probe, 16 bits for the tall route's
+// dense copy) and f32 GEMVs with one wave per output column - one that loads a dword per lane and takes any shape, and
+// for up to four f16 / bf16 rows one per width that moves 16 bytes per load; the tuned kernels are 4-bit.
 #include "common.hiph"
 
 namespace mnb {
@@ -170,6 +171,60 @@ __global__ __launch_bounds__(256) void gemv_q8_kernel(RocmMatMulNBitsArgs p, int
     }
 }
 
+// 2 bits, f16 / bf16 activations, up to four rows, K % 64 == 0: one wave per output column, 64 weights (one 16-byte load)
+// and 64 activations per row (eight 16-byte loads, served by the caches: every wave reads the same rows) per lane and
+// step, every load of the step issued before the arithmetic. f32 math in the plain kernel's order of operations per
+// element ((q - zp) * scale rounded, then one FMA); a dword of 16 weights never straddles a block (block >= 16).
+template <bool BF16, int ROWS>
+__global__ __launch_bounds__(256) void gemv_q2_kernel(RocmMatMulNBitsArgs p, int bs_log2, int64_t kb)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t col = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+    if (col >= p.n) return;
+    const int64_t row_bytes = (kb << bs_log2) >> 2;
+    const uint4* brow = reinterpret_cast<const uint4*>(p.b + col * row_bytes);
+    const uint8_t* zrow = p.zp ? p.zp + col * ((kb * 2 + 7) >> 3) : nullptr;
+    const uint16_t* a = static_cast<const uint16_t*>(p.a);
+    const int64_t runs = p.k >> 6;                         // 64-weight runs in K
+    float acc[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) acc[r] = 0.0f;
+    auto widen = [](uint32_t pair, int hi) { const uint16_t h = static_cast<uint16_t>(hi ? pair >> 16 : pair); return BF16 ? bf16_bits_to_f32(h) : f16_bits_to_f32(h); };
+    for (int64_t run = lane; run < runs; run += 64) {
+        const uint4 w = brow[run];
+        uint4 av[ROWS][8];
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) {
+            const uint4* arow = reinterpret_cast<const uint4*>(a + (r < p.m ? r : 0) * p.k) + run * 8;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) av[r][i] = arow[i];
+        }
+        const uint32_t wd[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            const int64_t blk = ((run << 6) + d * 16) >> bs_log2;
+            const float s = load_as_f32(p.scales, p.scale_dtype, col * kb + blk);
+            const float z = zero_point_bits<2>(zrow, blk);
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const float wv = __fmul_rn(static_cast<float>((wd[d] >> (2 * i)) & 3u) - z, s);
+                const int e = d * 16 + i;                                  // element of the run
+#pragma unroll
+                for (int r = 0; r < ROWS; ++r) {
+                    const uint4& piece = av[r][e >> 3];
+                    const uint32_t pr[4] = {piece.x, piece.y, piece.z, piece.w};
+                    acc[r] = fmaf(widen(pr[(e & 7) >> 1], e & 1), wv, acc[r]);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+        const float total = wave_sum(acc[r]);
+        if (lane == 0 && r < p.m) store_from_f32(p.y, p.y_dtype, r * p.n + col, with_bias(total, p.bias, p.bias_dtype, r, p.n, col, p.y_dtype));
+    }
+}
+
 template <int BITS>
 static int launch_dequant(const uint8_t* b, const void* scales, int scale_dtype, const uint8_t* zp, const int32_t* g, int64_t n, int64_t k, int block_size,
                           int out_dtype, void* out, hipStream_t s)
@@ -273,6 +328,23 @@ extern "C" int rocm_launch_gemv_nbits(const RocmMatMulNBitsArgs* args, int bits,
             else hipLaunchKernelGGL((mnb::gemv_q8_kernel<false, 4>), grid, dim3(256), 0, s, *args, bs_log2, kb);
         }
         return static_cast<int>(hipGetLastError());
+    }
+    if (bits == 2 && !args->g_idx && half_in && args->m <= 4 && args->k % 64 == 0 && (reinterpret_cast<uintptr_t>(args->a) & 15) == 0 &&
+        (reinterpret_cast<uintptr_t>(args->b) & 15) == 0) {
+        const int bs_log2 = __builtin_ctz(static_cast<unsigned>(args->block_size));
+        const int64_t kb = (args->k + args->block_size - 1) / args->block_size;
+        if ((((kb << bs_log2) >> 2) & 15) == 0) {              // every column's row of weights starts on 16 bytes
+            const dim3 grid(static_cast<unsigned>((args->n + 3) / 4));
+            const bool bf16 = args->a_dtype == ROCM_DT_BF16;
+            if (args->m == 1) {
+                if (bf16) hipLaunchKernelGGL((mnb::gemv_q2_kernel<true, 1>), grid, dim3(256), 0, s, *args, bs_log2, kb);
+                else hipLaunchKernelGGL((mnb::gemv_q2_kernel<false, 1>), grid, dim3(256), 0, s, *args, bs_log2, kb);
+            } else {
+                if (bf16) hipLaunchKernelGGL((mnb::gemv_q2_kernel<true, 4>), grid, dim3(256), 0, s, *args, bs_log2, kb);
+                else hipLaunchKernelGGL((mnb::gemv_q2_kernel<false, 4>), grid, dim3(256), 0, s, *args, bs_log2, kb);
+            }
+            return static_cast<int>(hipGetLastError());
+        }
     }
     if (bits == 2) return mnb::launch_gemv<2>(args, s);
     if (bits == 4) return mnb::launch_gemv<4>(args, s);            // 4 bits come here with g_idx only

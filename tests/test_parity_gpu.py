@@ -700,6 +700,8 @@ NBITS_CASES = [
     (E.BF16, E.BF16, 128, True, 1, 1030, 3584),   # 8 bits: the 16-byte-load GEMV (one row), ragged column count
     (E.F16, E.F16, 16, False, 4, 70, 1040),       # 8 bits: four rows, a K that leaves the last step half empty
     (E.F16, E.F16, 32, True, 3, 40, 72),          # K % 16 != 0: the plain kernel
+    (E.F16, E.F16, 32, True, 3, 72, 1024),        # 2 bits: three rows through the 16-byte-load GEMV (K % 64 == 0)
+    (E.BF16, E.F32, 16, True, 2, 50, 4096 + 64),  # ... block 16: four blocks per load, f32 scales
 ]
 
 
