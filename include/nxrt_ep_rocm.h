@@ -170,8 +170,12 @@ NxrtStatus nxrt_rocm_matmul_nbits_execute(NxrtRocmMatMulNBits* kernel, const Nxr
  *   - nothing is set up on the fly: constant weights that have no repacked copy yet are streamed in the caller's layout, the
  *     library GEMM route is not taken, a g_idx tensor must have been range-checked by an earlier execute;
  *   - every call on one GPU shares that GPU's array, which keeps the last call's contents (the kernels overwrite all they
- *     read). Calls through one provider are ordered by its stream; calls through different providers on the same GPU, or a
- *     static call concurrent with another one's kernels still running on another stream, race on the array. */
+ *     read). Calls through one provider are ordered by its stream. Calls through different providers on the same GPU are
+ *     chained on the GPU: each call records an event behind its launches, and a call on another stream waits for it
+ *     (hipStreamWaitEvent) before its own - they run one after the other, in the order in which the host made them. The
+ *     exception is a call made while its provider has a graph capture open: it neither waits nor records (an event from
+ *     outside a capture cannot be waited for inside one), so graphs recorded through several providers of one GPU must not
+ *     be replayed at the same time; the host orders them. */
 #define NXRT_ROCM_STATIC_SCRATCH_BYTES (8u << 20)
 NxrtStatus nxrt_rocm_matmul_nbits_execute_static(NxrtRocmMatMulNBits* kernel, const NxrtRocmTensorView* inputs, uint32_t n_inputs,
                                                  NxrtRocmTensorView* outputs, uint32_t n_outputs);

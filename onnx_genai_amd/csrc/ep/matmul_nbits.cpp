@@ -1173,7 +1173,23 @@ NxrtStatus nxrt_rocm_matmul_nbits_execute_static(NxrtRocmMatMulNBits* kernel, co
                                                           "call execute with a workspace"));
         NxrtRocmEp* ep = kernel->ep;
         if (!ep->static_scratch) return make_status(NXRT_INTERNAL_ERROR, err("the static scratch of this GPU was not resolved when the provider was created"));
-        return execute_impl(*kernel, inputs, n_inputs, outputs, n_outputs, ep->static_scratch, ep->static_scratch_bytes, true);
+        // Every provider of a GPU shares the array: a call behind another provider's call (another stream) waits for it on
+        // the GPU. Under an open capture neither the wait nor the record can be taken (an event from outside a capture
+        // cannot be waited for inside one): graphs recorded through several providers of one GPU are the host's to order.
+        if (ep->capturing) return execute_impl(*kernel, inputs, n_inputs, outputs, n_outputs, ep->static_scratch, ep->static_scratch_bytes, true);
+        NxrtStatus st = ep->bind();
+        if (st.code != NXRT_OK) return st;
+        st = hip_status(rocm_ffi_static_scratch_begin(static_cast<int>(ep->device), ep->stream), "hipStreamWaitEvent(static scratch)");
+        if (st.code != NXRT_OK) return st;
+        NxrtStatus run;
+        try {
+            run = execute_impl(*kernel, inputs, n_inputs, outputs, n_outputs, ep->static_scratch, ep->static_scratch_bytes, true);
+        } catch (...) {
+            rocm_ffi_static_scratch_end(static_cast<int>(ep->device), ep->stream);
+            throw;
+        }
+        st = hip_status(rocm_ffi_static_scratch_end(static_cast<int>(ep->device), ep->stream), "hipEventRecord(static scratch)");
+        return run.code != NXRT_OK ? run : st;
     });
 }
 

@@ -40,8 +40,16 @@ int rocm_ffi_free(void* ptr);
 uint64_t rocm_ffi_malloc_calls(void);
 /* Device address and size of the library's static scratch array on `device` (a __device__ array of the code object, 256-byte
  * aligned, one per GPU, never freed). The first call for a device makes that device current and resolves the address; later
- * calls only read it back. Shared by every caller on that GPU and never cleared: contents are whatever the last user left. */
+ * calls only read it back. Shared by every caller on that GPU and never cleared: contents are whatever the last user left.
+ * The first call also creates the event that chains the array's users (below). */
 int rocm_ffi_static_scratch(int device, void** ptr, size_t* bytes);
+/* Bracket the launches of one user of that array. `begin` takes the device's host lock and, if the previous user enqueued
+ * on another stream, makes `stream` wait (on the GPU, hipStreamWaitEvent) for the event that user recorded; `end` records
+ * the event on `stream` and drops the lock: users on different streams of one GPU run one after the other, in the order
+ * of their `begin`. Neither allocates device memory. Not for a stream under capture (events from outside a capture cannot
+ * be waited for inside one): a caller skips both there. A failed `begin` holds no lock. */
+int rocm_ffi_static_scratch_begin(int device, rocm_stream_t stream);
+int rocm_ffi_static_scratch_end(int device, rocm_stream_t stream);
 int rocm_ffi_memcpy_h2d(void* dst, const void* src, size_t bytes, rocm_stream_t stream);
 int rocm_ffi_memcpy_d2h(void* dst, const void* src, size_t bytes, rocm_stream_t stream);
 /* Reads `bytes` (a multiple of 16 is read) of device memory and keeps nothing: the time of the plainest kernel that pulls

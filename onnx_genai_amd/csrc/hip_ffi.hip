@@ -17,6 +17,12 @@ __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 constexpr int kMaxScratchDevices = 64;
 void* g_scratch_ptr[kMaxScratchDevices] = {};
 std::mutex g_scratch_mu;
+// Users of one GPU's scratch array are chained on the GPU: each records this event when its launches are enqueued, and a
+// user on another stream waits for it first.
+hipEvent_t g_scratch_event[kMaxScratchDevices] = {};
+hipStream_t g_scratch_last_stream[kMaxScratchDevices] = {};
+bool g_scratch_event_recorded[kMaxScratchDevices] = {};
+std::mutex g_scratch_use_mu[kMaxScratchDevices];
 std::atomic<uint64_t> g_device_allocations{0};
 
 __global__ void fill_u32_kernel(uint32_t* dst, uint32_t value, size_t count)
@@ -193,11 +199,43 @@ int rocm_ffi_static_scratch(int device, void** ptr, size_t* bytes)
         if (e == hipSuccess) e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
         if (e != hipSuccess) return static_cast<int>(e);
         if (!p) return static_cast<int>(hipErrorInvalidSymbol);
+        hipEvent_t ev = nullptr;
+        e = hipEventCreateWithFlags(&ev, hipEventDisableTiming);
+        if (e != hipSuccess) return static_cast<int>(e);
+        g_scratch_event[device] = ev;
         g_scratch_ptr[device] = p;
     }
     *ptr = g_scratch_ptr[device];
     *bytes = kStaticScratchBytes;
     return 0;
+}
+
+int rocm_ffi_static_scratch_begin(int device, rocm_stream_t stream)
+{
+    if (device < 0 || device >= kMaxScratchDevices || !g_scratch_event[device]) return static_cast<int>(hipErrorInvalidValue);
+    g_scratch_use_mu[device].lock();
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (g_scratch_event_recorded[device] && g_scratch_last_stream[device] != s) {
+        const hipError_t e = hipStreamWaitEvent(s, g_scratch_event[device], 0);
+        if (e != hipSuccess) {
+            g_scratch_use_mu[device].unlock();
+            return static_cast<int>(e);
+        }
+    }
+    return 0;
+}
+
+int rocm_ffi_static_scratch_end(int device, rocm_stream_t stream)
+{
+    if (device < 0 || device >= kMaxScratchDevices || !g_scratch_event[device]) return static_cast<int>(hipErrorInvalidValue);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const hipError_t e = hipEventRecord(g_scratch_event[device], s);
+    if (e == hipSuccess) {
+        g_scratch_event_recorded[device] = true;
+        g_scratch_last_stream[device] = s;
+    }
+    g_scratch_use_mu[device].unlock();
+    return static_cast<int>(e);
 }
 int rocm_ffi_free(void* ptr) { return static_cast<int>(hipFree(ptr)); }
 

@@ -151,3 +151,41 @@ def test_execute_static_refuses_what_does_not_fit():
             fused.free()
     finally:
         provider.shutdown()
+
+
+def test_static_calls_through_two_providers_of_one_gpu_do_not_race():
+    """Two providers share the GPU's static scratch and have a stream each. Calls that use the scratch heavily (int8 codes
+    of a tall accuracy_level 4 call) are made through both in turn without any host synchronization in between; each must
+    give what it gives alone. The library chains them on the GPU (an event recorded behind each call, waited for by the next
+    call on another stream)."""
+    p1, p2 = E.RocmExecutionProvider(0, {"prepack": "0"}), E.RocmExecutionProvider(0, {"prepack": "0"})
+    try:
+        jobs = []
+        for i, (prov, m, n, k) in enumerate([(p1, 96, 256, 8192), (p2, 80, 320, 8192)]):
+            a_dt, bs = E.F16, 64
+            b, s, zp = synth.make_weights(n, k, bs, 990 + i, zero_points=True, scale_lo=0.002, scale_hi=0.01, scale_dtype=a_dt)
+            a = synth.make_activation(m, k, 995 + i, a_dt)
+            ops = E.DeviceOperands(prov, b, s, a_dt, zp, n, k, bs, accuracy_level=4)
+            ab, y_ref, y = prov.upload(a), prov.allocate(m * n * 4), prov.allocate(m * n * 4)
+            views = ops.views(ab, a_dt, m)
+            ops.kernel.execute_static(views, [E.TensorView(y_ref.ptr, E.F32, (m, n))])
+            prov.sync()
+            jobs.append((prov, ops, views, ab, y_ref, y, m, n))
+        alone = [job[0].download(job[4], (job[6], job[7]), np.float32) for job in jobs]
+        before = p1.lib.nxrt_rocm_device_allocation_count()
+        for _ in range(20):                                    # 40 calls, alternating providers, no synchronization in between
+            for prov, ops, views, ab, y_ref, y, m, n in jobs:
+                ops.kernel.execute_static(views, [E.TensorView(y.ptr, E.F32, (m, n))])
+        assert p1.lib.nxrt_rocm_device_allocation_count() == before
+        p1.sync()
+        p2.sync()
+        for (prov, ops, views, ab, y_ref, y, m, n), want in zip(jobs, alone):
+            assert np.array_equal(prov.download(y, (m, n), np.float32), want)
+        for prov, ops, views, ab, y_ref, y, m, n in jobs:
+            for buf in (ab, y_ref, y):
+                prov.deallocate(buf)
+            ops.free()
+    finally:
+        p1.shutdown()
+        p2.shutdown()
+
